@@ -1,0 +1,346 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 quantized-linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one pass of the hot path over one batch: every quantized nn.Linear
+of one denoising step of the FLUX.1-dev-shaped MMDiT (BASELINE config 2: 19
+double-stream + 38 single-stream blocks, 4096 image + 512 text tokens, hidden
+3072, MLP 12288 with GELU-tanh) run back to back at its real shape with its own
+weights -- per Linear: per-token e4m3 activation quantization, FP8 GEMM, fused
+scale/bias/(GELU) epilogue, bf16 out. 494 Linears, 5.95e13 FLOP. Inputs are
+synthetic (~N(0,1) bf16 activations, random e4m3 weights) and resident in HBM
+before the timed region.
+
+Prints ONE JSON line. `value` is the whole-step linear throughput in TFLOP/s
+(sum of 2MKN / step time). Beside it: the headline-shape kernel figures
+(`linear_headline`: GEMM and quantizer at M=4608 K=3072 N=12288), `roofline`
+for the dominant kernel (the FP8 GEMM, timed with HIP events on the launch
+stream), the full synthetic-transformer forward (`dit_step_ms`, attention and
+glue included) and `cpu_baseline`: the CPU restatement of the reference path
+(PyTorch CPU ops) timed on this box's host cores on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+FP8_PEAK_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
+BF16_PEAK_TFLOPS = 2500.0
+HBM_PEAK_GBPS = 8000.0
+HEADLINE = (4608, 3072, 12288)  # M, K, N
+
+
+def flux_step_linears():
+  """(name, M, K, N, gelu, count) of every quantized Linear of one FLUX-shaped
+  step; layer names as in diffusers' FluxTransformer2DModel."""
+  img, txt, both, d, mlp = 4096, 512, 4608, 3072, 12288
+  double = [
+      ("attn.to_q", img, d, d, False), ("attn.to_k", img, d, d, False),
+      ("attn.to_v", img, d, d, False), ("attn.to_out.0", img, d, d, False),
+      ("ff.net.0.proj", img, d, mlp, True), ("ff.net.2", img, mlp, d, False),
+      ("norm1.linear", 1, d, 6 * d, False),
+      ("attn.add_q_proj", txt, d, d, False), ("attn.add_k_proj", txt, d, d, False),
+      ("attn.add_v_proj", txt, d, d, False), ("attn.to_add_out", txt, d, d, False),
+      ("ff_context.net.0.proj", txt, d, mlp, True), ("ff_context.net.2", txt, mlp, d, False),
+      ("norm1_context.linear", 1, d, 6 * d, False),
+  ]
+  single = [
+      ("attn.to_q", both, d, d, False), ("attn.to_k", both, d, d, False),
+      ("attn.to_v", both, d, d, False), ("proj_mlp", both, d, mlp, True),
+      ("proj_out", both, d + mlp, d, False), ("norm.linear", 1, d, 3 * d, False),
+  ]
+  out = []
+  for i in range(19):
+    out += [(f"transformer_blocks.{i}.{n}", M, K, N, g) for n, M, K, N, g in double]
+  for i in range(38):
+    out += [(f"single_transformer_blocks.{i}.{n}", M, K, N, g) for n, M, K, N, g in single]
+  return out
+
+
+def _rand_fp8(shape, gen, device):
+  import torch
+  # random e4m3 codes with |value| <= 1.75 (exponent field <= 7): no NaN codes
+  bits = torch.randint(0, 256, shape, dtype=torch.uint8, device=device, generator=gen)
+  return (bits & 0xBF).view(torch.float8_e4m3fn)
+
+
+class HotPath:
+  """All quantized Linears of one step, each with its own weight."""
+
+  def __init__(self, device):
+    import torch
+    from cache_dit_amd import _native
+    self.torch = torch
+    self.native = _native
+    g = torch.Generator(device=device).manual_seed(0)
+    self.layers = []
+    self.flop = 0
+    max_mk, max_mn = {}, 0
+    for name, M, K, N, gelu in flux_step_linears():
+      w = _rand_fp8((N, K), g, device)
+      ws = torch.rand(N, device=device, generator=g) * 1e-3 + 1e-4
+      b = (torch.randn(N, device=device, generator=g) * 0.01).to(torch.bfloat16)
+      self.layers.append((M, K, N, w, ws, b, 1 if gelu else 0))
+      self.flop += 2 * M * K * N
+      max_mk[(M, K)] = None
+      max_mn = max(max_mn, M * N)
+    # activations: one bf16 input per distinct (M, K); scratch for codes/scales/output
+    self.x = {mk: torch.randn(mk, device=device, generator=g).to(torch.bfloat16) for mk in max_mk}
+    self.q = {mk: torch.empty(mk, dtype=torch.float8_e4m3fn, device=device) for mk in max_mk}
+    self.s = {mk: torch.empty(mk[0], dtype=torch.float32, device=device) for mk in max_mk}
+    self.out = torch.empty(max_mn, dtype=torch.bfloat16, device=device)
+
+  def step(self):
+    from cache_dit_amd import ops
+    for M, K, N, w, ws, b, epi in self.layers:
+      x, q, s = self.x[(M, K)], self.q[(M, K)], self.s[(M, K)]
+      out = self.out[:M * N].view(M, N)
+      ops.quant_rowwise_into(x, q, s, 0)
+      ops.gemm_rowwise_into(q, s, w, ws, b, out, epi)
+
+
+def _time_events(fn, iters, warmup):
+  """Average duration in ms of fn() over `iters` calls, HIP events on the current
+  stream (the stream the kernels are launched on)."""
+  import torch
+  for _ in range(warmup):
+    fn()
+  torch.cuda.synchronize()
+  e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  e0.record()
+  for _ in range(iters):
+    fn()
+  e1.record()
+  torch.cuda.synchronize()
+  return e0.elapsed_time(e1) / iters
+
+
+def headline_kernels(device):
+  """GEMM and quantizer alone at the headline shape, rotating over enough distinct
+  buffers that the 256 MiB last-level cache cannot serve repeats."""
+  import torch
+  from cache_dit_amd import ops
+  M, K, N = HEADLINE
+  g = torch.Generator(device=device).manual_seed(1)
+  nbuf = 8
+  xs = [torch.randn(M, K, device=device, generator=g).to(torch.bfloat16) for _ in range(nbuf)]
+  qs = [torch.empty(M, K, dtype=torch.float8_e4m3fn, device=device) for _ in range(nbuf)]
+  ss = [torch.empty(M, dtype=torch.float32, device=device) for _ in range(nbuf)]
+  ws = [_rand_fp8((N, K), g, device) for _ in range(nbuf)]
+  wsc = torch.rand(N, device=device, generator=g) * 1e-3 + 1e-4
+  b = (torch.randn(N, device=device, generator=g) * 0.01).to(torch.bfloat16)
+  outs = [torch.empty(M, N, dtype=torch.bfloat16, device=device) for _ in range(2)]
+  for i in range(nbuf):
+    ops.quant_rowwise_into(xs[i], qs[i], ss[i], 0)
+  it = {"i": 0}
+
+  def gemm():
+    i = it["i"] = (it["i"] + 1) % nbuf
+    ops.gemm_rowwise_into(qs[i], ss[i], ws[i], wsc, b, outs[i & 1], 1)
+
+  def quant():
+    i = it["i"] = (it["i"] + 1) % nbuf
+    ops.quant_rowwise_into(xs[i], qs[i], ss[i], 0)
+
+  gemm_ms = _time_events(gemm, 50, 10)
+  quant_ms = _time_events(quant, 200, 20)
+  res = {
+      "shape": {"M": M, "K": K, "N": N},
+      "gemm_ms": gemm_ms,
+      "gemm_tflops": 2.0 * M * K * N / gemm_ms / 1e9,
+      "quant_ms": quant_ms,
+      "quant_gbps": (3.0 * M * K + 4.0 * M) / quant_ms / 1e6,
+  }
+  res["gemm_frac_fp8_peak"] = res["gemm_tflops"] / FP8_PEAK_TFLOPS
+  res["quant_frac_hbm_peak"] = res["quant_gbps"] / HBM_PEAK_GBPS
+  res["linear_tflops"] = 2.0 * M * K * N / (gemm_ms + quant_ms) / 1e9
+  # the vendor library on the same codes, as a comparator (not a baseline)
+  try:
+    a_s = ss[0].reshape(M, 1)
+    w_s = wsc.reshape(1, N)
+
+    def vendor():
+      torch._scaled_mm(qs[0], ws[0].t(), scale_a=a_s, scale_b=w_s, bias=b,
+                       out_dtype=torch.bfloat16)
+
+    v_ms = _time_events(vendor, 20, 5)
+    res["hipblaslt_scaled_mm_tflops"] = 2.0 * M * K * N / v_ms / 1e9
+  except Exception as e:  # not every build has row-wise _scaled_mm
+    res["hipblaslt_scaled_mm_tflops"] = None
+    res["hipblaslt_note"] = str(e)[:120]
+  # weight-only mode at the same shape
+  try:
+    def w8a16():
+      i = it["i"] = (it["i"] + 1) % nbuf
+      ops.w8a16_into(xs[i], ws[i], wsc, b, outs[i & 1], 1)
+
+    w_ms = _time_events(w8a16, 30, 5)
+    res["w8a16_ms"] = w_ms
+    res["w8a16_tflops"] = 2.0 * M * K * N / w_ms / 1e9
+    res["w8a16_frac_bf16_peak"] = res["w8a16_tflops"] / BF16_PEAK_TFLOPS
+  except Exception as e:
+    res["w8a16_note"] = str(e)[:120]
+  return res
+
+
+def cpu_baseline():
+  """The CPU restatement of the reference path (oracle.torch_oracle: eager PyTorch
+  CPU ops) on BASELINE config 1 (M=4608, K=3072, N=3072): activation quantization +
+  scaled matmul + bias, weights pre-quantized. 1 warm-up + 3 timed runs, median."""
+  import torch
+  from oracle import torch_oracle as to
+  cores = os.cpu_count() or 1
+  torch.set_num_threads(cores)
+  g = torch.Generator().manual_seed(0)
+  M, K, N = 4608, 3072, 3072
+  x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+  w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
+  b = (torch.randn(N, generator=g) * 0.01).to(torch.bfloat16)
+  wq, ws = to.quantize_rowwise(w)
+  times, qtimes = [], []
+  for i in range(4):
+    t0 = time.perf_counter()
+    xq, xs = to.quantize_rowwise(x)
+    t1 = time.perf_counter()
+    to.scaled_mm_rowwise(xq, xs, wq, ws, b)
+    t2 = time.perf_counter()
+    if i:
+      times.append(t2 - t0)
+      qtimes.append(t1 - t0)
+  times.sort()
+  qtimes.sort()
+  t, tq = times[len(times) // 2], qtimes[len(qtimes) // 2]
+  return {
+      "value": 2.0 * M * K * N / t / 1e12,
+      "unit": "TFLOP/s",
+      "cores": torch.get_num_threads(),
+      "kind": "port",
+      "sample": f"BASELINE config 1 linear (M={M} K={K} N={N}): per-token quant + scaled matmul "
+                f"+ bias in eager PyTorch CPU ops, median of 3 runs, {t*1e3:.0f} ms/linear",
+      "quant_gbps": (3.0 * M * K + 4.0 * M) / tq / 1e9,
+      "ms_per_linear": t * 1e3,
+  }
+
+
+def dit_forward_ms(device):
+  """Full synthetic FLUX-shaped transformer forward (attention, norms, RoPE and
+  residual glue included), quantized with float8_per_row."""
+  try:
+    import torch
+    import cache_dit_amd
+    from cache_dit_amd.testing.dit_shapes import FluxLikeTransformer, flux_like_inputs
+  except Exception as e:
+    return None, f"synthetic transformer unavailable: {e}"[:160]
+  torch.manual_seed(0)
+  with torch.device(device):
+    model = FluxLikeTransformer().to(torch.bfloat16)
+  cache_dit_amd.quantize(model, cache_dit_amd.QuantizeConfig(quant_type="float8_per_row"))
+  cache_dit_amd.testing.dit_shapes.fuse_gelu_epilogues(model)
+  inputs = flux_like_inputs(device)
+  with torch.inference_mode():
+    ms = _time_events(lambda: model(**inputs), 5, 2)
+  return ms, None
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=10)
+  ap.add_argument("--warmup", type=int, default=3)
+  ap.add_argument("--skip-cpu", action="store_true", help="skip the cpu_baseline leg")
+  ap.add_argument("--skip-dit", action="store_true", help="skip the full-transformer forward")
+  args = ap.parse_args()
+  if args.gpus != 1:
+    sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
+             "use --gpus 1")
+  import torch
+  if not torch.cuda.is_available():
+    sys.exit("bench.py: no GPU visible; the hot path has no CPU fallback")
+  from cache_dit_amd import _native
+  device = torch.device("cuda", 0)
+  torch.cuda.set_device(device)
+  arch = _native.device_arch()
+
+  hot = HotPath(device)
+  for _ in range(args.warmup):
+    hot.step()
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(args.steps):
+    hot.step()
+  torch.cuda.synchronize()
+  dt = time.perf_counter() - t0
+  ms_per_step = dt / args.steps * 1e3
+  value = hot.flop / (dt / args.steps) / 1e12
+  n_layers = len(hot.layers)
+  step_flop = hot.flop
+  del hot
+  torch.cuda.empty_cache()
+
+  head = headline_kernels(device)
+  M, K, N = HEADLINE
+  roofline = {
+      "kernel": "gemm_fp8_tiled (w8a8 GEMM + epilogue) at M=4608 K=3072 N=12288",
+      "bound": "mfma",
+      "achieved": head["gemm_tflops"],
+      "peak": FP8_PEAK_TFLOPS,
+      "unit": "TFLOP/s",
+      "frac": head["gemm_tflops"] / FP8_PEAK_TFLOPS,
+      "traffic": None,
+  }
+  roofline_quant = {
+      "kernel": "quant_rowwise_regs at M=4608 K=3072",
+      "bound": "hbm",
+      "achieved": head["quant_gbps"],
+      "peak": HBM_PEAK_GBPS,
+      "unit": "GB/s",
+      "frac": head["quant_gbps"] / HBM_PEAK_GBPS,
+      "traffic": None,
+  }
+  dit_ms, dit_note = (None, "skipped") if args.skip_dit else dit_forward_ms(device)
+  cpu = None if args.skip_cpu else cpu_baseline()
+
+  line = {
+      "metric": "fp8_w8a8_linear_tflops",
+      "value": value,
+      "unit": "TFLOP/s",
+      "n_gpus": 1,
+      "steps": args.steps,
+      "warmup": args.warmup,
+      "ms_per_step": ms_per_step,
+      "higher_is_better": True,
+      "scaling": "weak",
+      "vs_baseline": None,
+      "dtype": "fp8_e4m3 (fp32 accumulate, bf16 out)",
+      "data": "synthetic",
+      "config": {
+          "workload": "flux1_dev_shaped_step: all quantized Linears of one denoising step "
+                      "(19 double + 38 single blocks, 4096 img + 512 txt tokens), "
+                      "per-token quant + FP8 GEMM + epilogue each",
+          "quant_type": "float8_per_row",
+          "linears_per_step": n_layers,
+          "linear_flop_per_step": step_flop,
+          "batch": 1,
+      },
+      "frac_fp8_peak": value / FP8_PEAK_TFLOPS,
+      "linear_headline": head,
+      "dit_step_ms": dit_ms,
+      "dit_step_note": dit_note,
+      "roofline": roofline,
+      "roofline_quant": roofline_quant,
+      "cpu_baseline": cpu,
+      "device": arch,
+  }
+  print(json.dumps(line))
+
+
+if __name__ == "__main__":
+  main()

@@ -1,0 +1,218 @@
+// extern "C" layer of libcdit_hip.so: argument validation, device check,
+// error reporting. Declarations and their reference citations: include/cdit_hip.h.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "cdit_internal.h"
+
+namespace cdit {
+
+namespace {
+thread_local char g_err[512] = "";
+int g_gemm_variant = -1;
+
+// gfx950 check, cached per device ordinal (the answer cannot change).
+int check_arch() {
+  static int cached[64];  // 0 unknown, 1 ok, 2 wrong arch
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    set_error("hipGetDevice: %s", hipGetErrorString(e));
+    return CDIT_EHIP;
+  }
+  if (dev >= 0 && dev < 64 && cached[dev] == 1) return CDIT_OK;
+  hipDeviceProp_t p;
+  e = hipGetDeviceProperties(&p, dev);
+  if (e != hipSuccess) {
+    set_error("hipGetDeviceProperties: %s", hipGetErrorString(e));
+    return CDIT_EHIP;
+  }
+  const bool ok = strncmp(p.gcnArchName, "gfx950", 6) == 0;
+  if (dev >= 0 && dev < 64) cached[dev] = ok ? 1 : 2;
+  if (!ok) {
+    set_error("device %d is %s; libcdit_hip.so is built for gfx950 only (its FP8 is OCP e4m3fn, "
+              "older CDNA parts use e4m3fnuz)", dev, p.gcnArchName);
+    return CDIT_EARCH;
+  }
+  return CDIT_OK;
+}
+
+int after_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+    return CDIT_EHIP;
+  }
+  return CDIT_OK;
+}
+
+int check_gemm(const char* fn, const void* a, const void* b, const float* b_scale,
+               const void* out, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+               int64_t ldo, int epilogue, int out_dtype_id) {
+  if (M < 0 || N < 0 || K < 0) {
+    set_error("%s: negative dimension (M=%lld N=%lld K=%lld)", fn, (long long)M, (long long)N,
+              (long long)K);
+    return CDIT_EINVAL;
+  }
+  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) {
+    set_error("%s: dimension exceeds int32", fn);
+    return CDIT_EINVAL;
+  }
+  if (out_dtype_id != CDIT_DT_BF16) {
+    set_error("%s: out_dtype_id %d not built (only 1 = bf16)", fn, out_dtype_id);
+    return CDIT_EINVAL;
+  }
+  if (epilogue & ~CDIT_EPI_GELU_TANH) {
+    set_error("%s: unknown epilogue bits 0x%x", fn, epilogue);
+    return CDIT_EINVAL;
+  }
+  if (K % 16 != 0) {
+    set_error("%s: K=%lld is not a multiple of 16", fn, (long long)K);
+    return CDIT_EINVAL;
+  }
+  if (lda < K || ldb < K || ldo < N) {
+    set_error("%s: leading dimension smaller than the row (lda=%lld ldb=%lld ldo=%lld)", fn,
+              (long long)lda, (long long)ldb, (long long)ldo);
+    return CDIT_EINVAL;
+  }
+  if (M > 0 && N > 0 && (!out || !b_scale || (K > 0 && (!a || !b)))) {
+    set_error("%s: null pointer argument", fn);
+    return CDIT_EINVAL;
+  }
+  return CDIT_OK;
+}
+
+}  // namespace
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+}  // namespace cdit
+
+using namespace cdit;
+
+extern "C" {
+
+int cdit_abi_version(void) { return CDIT_ABI_VERSION; }
+
+const char* cdit_last_error(void) { return g_err; }
+
+int cdit_device_arch(char* buf, int buf_len) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  hipDeviceProp_t p;
+  if (e == hipSuccess) e = hipGetDeviceProperties(&p, dev);
+  if (e != hipSuccess) {
+    set_error("cdit_device_arch: %s", hipGetErrorString(e));
+    return CDIT_EHIP;
+  }
+  if (buf && buf_len > 0) {
+    strncpy(buf, p.gcnArchName, (size_t)buf_len - 1);
+    buf[buf_len - 1] = '\0';
+  }
+  return check_arch();
+}
+
+int cdit_set_gemm_variant(int variant) {
+  int prev = g_gemm_variant;
+  g_gemm_variant = variant;
+  return prev;
+}
+
+int cdit_fp8_quant_rowwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_x, void* q_e4m3,
+                           int64_t ld_q, float* scale, int scale_mode, void* stream) {
+  const char* fn = "cdit_fp8_quant_rowwise";
+  if (M < 0 || K < 0 || M > INT32_MAX || K > INT32_MAX) {
+    set_error("%s: bad shape M=%lld K=%lld", fn, (long long)M, (long long)K);
+    return CDIT_EINVAL;
+  }
+  if (scale_mode != CDIT_SCALE_BF16DIV && scale_mode != CDIT_SCALE_FP32DIV) {
+    set_error("%s: unknown scale_mode %d", fn, scale_mode);
+    return CDIT_EINVAL;
+  }
+  if (M == 0) return CDIT_OK;
+  if (ld_x < K || ld_q < K) {
+    set_error("%s: leading dimension smaller than K (ld_x=%lld ld_q=%lld K=%lld)", fn,
+              (long long)ld_x, (long long)ld_q, (long long)K);
+    return CDIT_EINVAL;
+  }
+  if (!scale || (K > 0 && (!x_bf16 || !q_e4m3))) {
+    set_error("%s: null pointer argument", fn);
+    return CDIT_EINVAL;
+  }
+  int rc = check_arch();
+  if (rc) return rc;
+  rc = launch_quant_rowwise(x_bf16, M, K, ld_x, q_e4m3, ld_q, scale, scale_mode,
+                            static_cast<hipStream_t>(stream));
+  return rc ? rc : after_launch(fn);
+}
+
+int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale, const void* b_q,
+                          const float* b_scale, const void* bias_bf16, void* out, int64_t M,
+                          int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldo,
+                          int epilogue, int out_dtype_id, void* stream) {
+  const char* fn = "cdit_fp8_gemm_rowwise";
+  int rc = check_gemm(fn, a_q, b_q, b_scale, out, M, N, K, lda, ldb, ldo, epilogue, out_dtype_id);
+  if (rc) return rc;
+  if (M == 0 || N == 0) return CDIT_OK;
+  if (!a_scale) {
+    set_error("%s: a_scale is null", fn);
+    return CDIT_EINVAL;
+  }
+  rc = check_arch();
+  if (rc) return rc;
+  GemmArgs g;
+  g.a = a_q;
+  g.a_scale = a_scale;
+  g.b = static_cast<const uint8_t*>(b_q);
+  g.b_scale = b_scale;
+  g.bias = static_cast<const uint16_t*>(bias_bf16);
+  g.out = static_cast<uint16_t*>(out);
+  g.M = (int)M;
+  g.N = (int)N;
+  g.K = (int)K;
+  g.lda = lda;
+  g.ldb = ldb;
+  g.ldo = ldo;
+  g.epilogue = epilogue;
+  rc = launch_gemm_fp8(g, g_gemm_variant, static_cast<hipStream_t>(stream));
+  return rc ? rc : after_launch(fn);
+}
+
+int cdit_w8a16_gemm(const void* x_bf16, const void* b_q, const float* b_scale,
+                    const void* bias_bf16, void* out, int64_t M, int64_t N, int64_t K,
+                    int64_t lda, int64_t ldb, int64_t ldo, int epilogue, int out_dtype_id,
+                    void* stream) {
+  const char* fn = "cdit_w8a16_gemm";
+  int rc =
+      check_gemm(fn, x_bf16, b_q, b_scale, out, M, N, K, lda, ldb, ldo, epilogue, out_dtype_id);
+  if (rc) return rc;
+  if (M == 0 || N == 0) return CDIT_OK;
+  rc = check_arch();
+  if (rc) return rc;
+  GemmArgs g;
+  g.a = x_bf16;
+  g.a_scale = nullptr;
+  g.b = static_cast<const uint8_t*>(b_q);
+  g.b_scale = b_scale;
+  g.bias = static_cast<const uint16_t*>(bias_bf16);
+  g.out = static_cast<uint16_t*>(out);
+  g.M = (int)M;
+  g.N = (int)N;
+  g.K = (int)K;
+  g.lda = lda;
+  g.ldb = ldb;
+  g.ldo = ldo;
+  g.epilogue = epilogue;
+  rc = launch_gemm_w8a16(g, g_gemm_variant, static_cast<hipStream_t>(stream));
+  return rc ? rc : after_launch(fn);
+}
+
+}  // extern "C"

@@ -1,0 +1,36 @@
+// Internal declarations shared by the kernel files and the C-ABI layer.
+#ifndef CDIT_INTERNAL_H_
+#define CDIT_INTERNAL_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "cdit_hip.h"
+
+namespace cdit {
+
+// Each launcher validates nothing: capi.hip checks shapes, strides, alignment
+// and the device before calling. They return 0 or a CDIT_E* code.
+int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void* q,
+                         int64_t ld_q, float* scale, int scale_mode, hipStream_t stream);
+
+struct GemmArgs {
+  const void* a;         // fp8 [M,K] (w8a8) or bf16 [M,K] (w8a16)
+  const float* a_scale;  // [M] (w8a8) or nullptr (w8a16)
+  const uint8_t* b;      // fp8 [N,K]
+  const float* b_scale;  // [N]
+  const uint16_t* bias;  // bf16 [N] or nullptr
+  uint16_t* out;         // bf16 [M,N]
+  int M, N, K;
+  int64_t lda, ldb, ldo;
+  int epilogue;
+};
+
+// variant < 0: choose by shape.
+int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream);
+int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream);
+
+void set_error(const char* fmt, ...);
+
+}  // namespace cdit
+#endif

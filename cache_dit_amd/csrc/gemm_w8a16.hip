@@ -1,0 +1,245 @@
+// Weight-only FP8 GEMM (w8a16) for gfx950: bf16 activations x e4m3 weights,
+// the weights dequantized to bf16 inside the mainloop, fp32 accumulate,
+// per-output-channel scale + bias + optional GELU-tanh + bf16 in the epilogue.
+//
+//   out[m,n] = epi((sum_k x[m,k] float(b[n,k])) * b_scale[n] + bias[n])
+//
+// Every e4m3 value is exactly representable in bf16, so the in-loop conversion
+// (v_cvt_scalef32_pk_bf16_fp8 with scale 1) is lossless and the weight never
+// exists in HBM at 16 bits: B costs 1 byte per element of traffic instead of
+// the 1 (read) + 2 (write) + 2 (read) of dequantize-then-GEMM.
+//
+// MFMA: v_mfma_f32_32x32x16_bf16; per lane 8 consecutive K elements of row
+// (lane&31), K-group h = lane>>5. The K order inside a 32-element block is
+// free as long as A and B agree, so lane group h takes elements [16h, 16h+16)
+// of the block: one 16-byte read of B (two MFMA steps of 8 bytes) and one
+// 32-byte read of A.
+//
+// Tile: BM x BN outputs, BK = 64 elements per pipeline step: A panel rows are
+// 128 bytes (8 chunks, chunk c of row r at position c ^ (r&7)), B panel rows
+// are 64 bytes (4 chunks, chunk c of row r at position c ^ ((r>>1)&3), two
+// rows per 128-byte line), both conflict free for 16-byte accesses. Panels
+// are staged with 128-bit LDS-DMA loads, double buffered.
+//
+// Replaces F.linear(x, W.dequantize(), bias) of the reference's
+// float8_weight_only mode (src/cache_dit/quantization/torchao/quantize_ao.py:604-610).
+#include "gemm_common.h"
+
+namespace cdit {
+namespace {
+
+constexpr int BKE = 64;  // K elements per pipeline step
+
+template <int BM_, int BN_, int WGM_, int WGN_, bool EPI_LDS_, int GROUP_M_>
+struct CfgW {
+  static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
+  static constexpr bool EPI_LDS = EPI_LDS_;
+  static constexpr int GROUP_M = GROUP_M_;
+  static constexpr int WAVES = WGM * WGN;
+  static constexpr int THREADS = WAVES * 64;
+  static constexpr int WM = BM / WGM, WN = BN / WGN;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int A_ROW = BKE * 2, B_ROW = BKE;  // bytes per panel row
+  static constexpr int A_BYTES = BM * A_ROW, B_BYTES = BN * B_ROW;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int EPI_PITCH = WN * 2 + 16;
+  static constexpr int EPI_BYTES = EPI_LDS ? WAVES * WM * EPI_PITCH : 0;
+  static constexpr int LDS_BYTES = (2 * STAGE_BYTES > EPI_BYTES) ? 2 * STAGE_BYTES : EPI_BYTES;
+  // LDS-DMA instructions per wave and stage (1 KiB each)
+  static constexpr int A_DMA = A_BYTES / 1024 / WAVES, B_DMA = B_BYTES / 1024 / WAVES;
+  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
+  static_assert(A_BYTES % (1024 * WAVES) == 0 && B_BYTES % (1024 * WAVES) == 0,
+                "panel/waves mismatch");
+};
+
+template <class C>
+__global__ __launch_bounds__(C::THREADS) void gemm_w8a16_tiled(GemmArgs g, int tiles_m,
+                                                               int tiles_n) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / C::WGN, wn = wave % C::WGN;
+
+  int tm, tn;
+  tile_of_block<C::GROUP_M>(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
+  const int m0 = tm * C::BM, n0 = tn * C::BN;
+  const uint8_t* __restrict__ A =
+      static_cast<const uint8_t*>(g.a) + (int64_t)m0 * g.lda * 2;  // bf16: 2 bytes/element
+  const uint8_t* __restrict__ B = g.b + (int64_t)n0 * g.ldb;
+  const int rows_a = g.M - m0, rows_b = g.N - n0;
+
+  // ---- LDS-DMA maps: a wave instruction fills 1 KiB = 8 A rows or 16 B rows;
+  // lane l lands on (row l/8, position l%8) resp. (row l/4, position l%4) and
+  // fetches the logical chunk that the swizzle puts there.
+  uint32_t a_off[C::A_DMA], b_off[C::B_DMA];
+#pragma unroll
+  for (int p = 0; p < C::A_DMA; ++p) {
+    const int row = (wave * C::A_DMA + p) * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ (row & 7);
+    a_off[p] = (uint32_t)min(row, rows_a - 1) * (uint32_t)(g.lda * 2) + c * 16;
+  }
+#pragma unroll
+  for (int p = 0; p < C::B_DMA; ++p) {
+    const int row = (wave * C::B_DMA + p) * 16 + (lane >> 2);
+    const int c = (lane & 3) ^ ((row >> 1) & 3);
+    b_off[p] = (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
+  }
+
+  // ---- operand read maps; kb = 32-element K block inside the step (0..1)
+  const int h = lane >> 5;
+  uint32_t rd_a[2][2], rd_b[2];
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) {
+    const int ra_row = wm * C::WM + (lane & 31);
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+      rd_a[kb][e] = ra_row * C::A_ROW + (((4 * kb + 2 * h + e) ^ (lane & 7)) << 4);
+    const int rb_row = wn * C::WN + (lane & 31);
+    rd_b[kb] = C::A_BYTES + rb_row * C::B_ROW + (((2 * kb + h) ^ ((lane >> 1) & 3)) << 4);
+  }
+
+  v16f acc[C::TM][C::TN];
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int KT = g.K / BKE;
+
+  auto fetch = [&](int kt, int stage) {
+    const uint8_t* Ak = A + (int64_t)kt * C::A_ROW;
+    const uint8_t* Bk = B + (int64_t)kt * C::B_ROW;
+    uint8_t* st = smem + stage * C::STAGE_BYTES;
+#pragma unroll
+    for (int p = 0; p < C::A_DMA; ++p)
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(Ak + a_off[p]),
+          (__attribute__((address_space(3))) void*)(st + (wave * C::A_DMA + p) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int p = 0; p < C::B_DMA; ++p)
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(Bk + b_off[p]),
+          (__attribute__((address_space(3))) void*)(st + C::A_BYTES +
+                                                    (wave * C::B_DMA + p) * 1024),
+          16, 0, 0);
+  };
+
+  auto compute = [&](int stage) {
+    const uint8_t* st = smem + stage * C::STAGE_BYTES;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      v8bf a_lo[C::TM], a_hi[C::TM];  // MFMA steps 0 and 1 of this block
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i) {
+        a_lo[i] = *reinterpret_cast<const v8bf*>(st + rd_a[kb][0] + i * 32 * C::A_ROW);
+        a_hi[i] = *reinterpret_cast<const v8bf*>(st + rd_a[kb][1] + i * 32 * C::A_ROW);
+      }
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j) {
+        const uint4 w = *reinterpret_cast<const uint4*>(st + rd_b[kb] + j * 32 * C::B_ROW);
+        // 16 e4m3 bytes -> 16 bf16 (exact), two at a time
+        v2bf c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.x, 1.0f, false);
+        v2bf c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.x, 1.0f, true);
+        v2bf c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.y, 1.0f, false);
+        v2bf c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.y, 1.0f, true);
+        v2bf c4 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.z, 1.0f, false);
+        v2bf c5 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.z, 1.0f, true);
+        v2bf c6 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.w, 1.0f, false);
+        v2bf c7 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.w, 1.0f, true);
+        const v8bf b_lo = {c0[0], c0[1], c1[0], c1[1], c2[0], c2[1], c3[0], c3[1]};
+        const v8bf b_hi = {c4[0], c4[1], c5[0], c5[1], c6[0], c6[1], c7[0], c7[1]};
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) {
+          // operands swapped: result rows follow B (n), result columns follow A (m)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_lo, a_lo[i], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_hi, a_hi[i], acc[i][j], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  fetch(0, 0);
+  for (int kt = 0; kt < KT; ++kt) {
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of step kt is in LDS
+    __syncthreads();                     // ... and everyone's; stage (kt+1)&1 is free again
+    if (kt + 1 < KT) fetch(kt + 1, (kt + 1) & 1);
+    compute(kt & 1);
+  }
+
+  tile_epilogue<C>(acc, g, smem, m0, n0, wm, wn, lane, wave);
+}
+
+// Any shape: one output element per thread, scalar decode + FMA.
+__global__ __launch_bounds__(256) void gemm_w8a16_generic(GemmArgs g) {
+  const int n = blockIdx.x * 16 + (threadIdx.x & 15);
+  const int m = blockIdx.y * 16 + (threadIdx.x >> 4);
+  if (m >= g.M || n >= g.N) return;
+  const uint16_t* a = static_cast<const uint16_t*>(g.a) + (int64_t)m * g.lda;
+  const uint8_t* b = g.b + (int64_t)n * g.ldb;
+  float acc = 0.0f;
+  for (int k = 0; k < g.K; ++k) {
+    const float x = __uint_as_float((uint32_t)a[k] << 16);
+    const float w = __builtin_amdgcn_cvt_f32_fp8((int)b[k], 0);
+    acc = fmaf(x, w, acc);
+  }
+  float v = acc * g.b_scale[n];
+  if (g.bias) v += __uint_as_float((uint32_t)g.bias[n] << 16);
+  if (g.epilogue & CDIT_EPI_GELU_TANH) v = gelu_tanh(v);
+  g.out[(int64_t)m * g.ldo + n] = (uint16_t)f32_to_bf16_bits(v);
+}
+
+template <class C>
+int launch_tiled(const GemmArgs& g, hipStream_t stream) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_w8a16_tiled<C>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(%d bytes LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
+      return CDIT_EHIP;
+    }
+    attr_set = true;
+  }
+  const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
+  hipLaunchKernelGGL(gemm_w8a16_tiled<C>, dim3(tiles_m * tiles_n), dim3(C::THREADS), C::LDS_BYTES,
+                     stream, g, tiles_m, tiles_n);
+  return 0;
+}
+
+bool tiled_ok(const GemmArgs& g) {
+  return g.K >= BKE && g.K % BKE == 0 && g.N % 8 == 0 && g.lda % 8 == 0 && g.ldb % 16 == 0 &&
+         g.ldo % 8 == 0 && reinterpret_cast<uintptr_t>(g.a) % 16 == 0 &&
+         reinterpret_cast<uintptr_t>(g.b) % 16 == 0 &&
+         reinterpret_cast<uintptr_t>(g.out) % 16 == 0 &&
+         (int64_t)1024 * g.lda < (int64_t)1 << 31 && (int64_t)512 * g.ldb < (int64_t)1 << 31;
+}
+
+}  // namespace
+
+typedef CfgW<256, 256, 2, 2, true, 8> W0;
+typedef CfgW<256, 256, 2, 2, false, 8> W1;
+typedef CfgW<256, 128, 2, 2, true, 8> W2;
+typedef CfgW<128, 128, 2, 2, true, 8> W3;
+
+int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
+  if (!tiled_ok(g) || variant == 100) {
+    dim3 grid((g.N + 15) / 16, (g.M + 15) / 16);
+    hipLaunchKernelGGL(gemm_w8a16_generic, grid, dim3(256), 0, stream, g);
+    return 0;
+  }
+  if (variant < 0) variant = 0;
+  switch (variant) {
+    case 0: return launch_tiled<W0>(g, stream);
+    case 1: return launch_tiled<W1>(g, stream);
+    case 2: return launch_tiled<W2>(g, stream);
+    case 3: return launch_tiled<W3>(g, stream);
+    default:
+      set_error("cdit_w8a16_gemm: unknown kernel variant %d", variant);
+      return CDIT_EINVAL;
+  }
+}
+
+}  // namespace cdit

@@ -1,0 +1,258 @@
+"""Operator boundary: `torch.ops.cdit.*`, backed by libcdit_hip.so.
+
+Mirrors the reference's own op for this path,
+`cache_dit_torchao_ops::float8_inference_scaled_mm`
+(src/cache_dit/quantization/torchao/_scaled_mm.py:94-137): same argument
+order and meaning (a_data [M,K] e4m3 row-major, a_scale [M,1], b_data [K,N] =
+`qweight.t()` column-major, b_scale [1,N], optional bias, out dtype id 0/1/2 =
+fp16/bf16/fp32, use_fast_accum), same fake-impl shape rule, same error types.
+On top of it the quantizer (torchao's per-row `Float8Tensor.from_hp`) and the
+weight-only matmul are ops of their own.
+
+Ownership and stream conventions follow the reference's native extension
+(src/cache_dit/kernels/cuda/_ops_registery.py:35-59): this wrapper allocates
+every output with torch.empty and launches on the current torch stream.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _native
+
+_DTYPE_TO_ID = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}
+_ID_TO_DTYPE = {v: k for k, v in _DTYPE_TO_ID.items()}
+FP8 = torch.float8_e4m3fn
+
+
+def encode_output_dtype(output_dtype: torch.dtype) -> int:
+  dtype_id = _DTYPE_TO_ID.get(output_dtype)
+  if dtype_id is None:
+    raise ValueError(f"Unsupported float8 inference output dtype: {output_dtype}")
+  return dtype_id
+
+
+def decode_output_dtype(dtype_id: int) -> torch.dtype:
+  output_dtype = _ID_TO_DTYPE.get(dtype_id)
+  if output_dtype is None:
+    raise ValueError(f"Unsupported float8 inference output dtype id: {dtype_id}")
+  return output_dtype
+
+
+def _stream_ptr(t: torch.Tensor) -> int:
+  return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_cuda(name: str, *tensors: Optional[torch.Tensor]) -> None:
+  for t in tensors:
+    if t is not None and not t.is_cuda:
+      raise RuntimeError(f"{name}: expected tensors on the GPU, got a {t.device} tensor "
+                         "(there is no CPU path)")
+
+
+# --------------------------------------------------------------------------- raw launchers
+# These take already-validated 2-D tensors and write into caller-provided outputs.
+
+
+def quant_rowwise_into(x2: torch.Tensor, q: torch.Tensor, scale: torch.Tensor,
+                       scale_mode_id: int) -> None:
+  M, K = x2.shape
+  with torch.cuda.device(x2.device):
+    _native.check(_native.load().cdit_fp8_quant_rowwise(x2.data_ptr(), M, K, x2.stride(0),
+                                                        q.data_ptr(), q.stride(0),
+                                                        scale.data_ptr(), scale_mode_id,
+                                                        _stream_ptr(x2)))
+
+
+def gemm_rowwise_into(a: torch.Tensor, a_scale: torch.Tensor, w: torch.Tensor,
+                      w_scale: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                      epilogue: int) -> None:
+  """a [M,K] e4m3, w [N,K] e4m3 (row-major), scales fp32 contiguous, out [M,N] bf16."""
+  M, K = a.shape
+  N = w.shape[0]
+  with torch.cuda.device(a.device):
+    _native.check(_native.load().cdit_fp8_gemm_rowwise(
+        a.data_ptr(), a_scale.data_ptr(), w.data_ptr(), w_scale.data_ptr(),
+        bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, K, a.stride(0),
+        w.stride(0), out.stride(0), epilogue, _native.DT_BF16, _stream_ptr(a)))
+
+
+def w8a16_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
+               bias: Optional[torch.Tensor], out: torch.Tensor, epilogue: int) -> None:
+  M, K = x2.shape
+  N = w.shape[0]
+  with torch.cuda.device(x2.device):
+    _native.check(_native.load().cdit_w8a16_gemm(
+        x2.data_ptr(), w.data_ptr(), w_scale.data_ptr(),
+        bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, K, x2.stride(0),
+        w.stride(0), out.stride(0), epilogue, _native.DT_BF16, _stream_ptr(x2)))
+
+
+# --------------------------------------------------------------------------- op definitions
+
+torch.library.define(
+    "cdit::fp8_rowwise_quant",
+    "(Tensor x, int scale_mode=0) -> (Tensor, Tensor)",
+)
+torch.library.define(
+    "cdit::float8_inference_scaled_mm",
+    "(Tensor a_data, Tensor a_scale, Tensor b_data, Tensor b_scale, Tensor? bias, "
+    "int out_dtype_id, bool use_fast_accum, int epilogue=0) -> Tensor",
+)
+torch.library.define(
+    "cdit::w8a16_mm",
+    "(Tensor x, Tensor b_data, Tensor b_scale, Tensor? bias, int out_dtype_id, "
+    "int epilogue=0) -> Tensor",
+)
+
+
+def _as_rows(x: torch.Tensor) -> torch.Tensor:
+  x2 = x.reshape(-1, x.shape[-1])
+  if x2.stride(-1) != 1:
+    x2 = x2.contiguous()
+  return x2
+
+
+@torch.library.impl("cdit::fp8_rowwise_quant", "CUDA")
+def _fp8_rowwise_quant(x: torch.Tensor, scale_mode: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+  if x.dtype != torch.bfloat16:
+    raise ValueError(f"cdit::fp8_rowwise_quant: x must be bfloat16, got {x.dtype}")
+  if x.dim() < 1:
+    raise ValueError("cdit::fp8_rowwise_quant: x must have at least one dimension")
+  if scale_mode not in (0, 1):
+    raise ValueError(f"cdit::fp8_rowwise_quant: scale_mode must be 0 or 1, got {scale_mode}")
+  x2 = _as_rows(x)
+  q = torch.empty(x2.shape, dtype=FP8, device=x.device)
+  scale = torch.empty((x2.shape[0], ), dtype=torch.float32, device=x.device)
+  if x2.numel() > 0 or x2.shape[0] > 0:
+    quant_rowwise_into(x2, q, scale, scale_mode)
+  return q.reshape(x.shape), scale.reshape(*x.shape[:-1], 1)
+
+
+@torch.library.register_fake("cdit::fp8_rowwise_quant")
+def _fake_fp8_rowwise_quant(x, scale_mode=0):
+  return (x.new_empty(x.shape, dtype=FP8), x.new_empty((*x.shape[:-1], 1), dtype=torch.float32))
+
+
+def _weight_rows(b_data: torch.Tensor, name: str) -> torch.Tensor:
+  """b_data is [K,N]; the kernels want the [N,K] row-major weight it is the
+  transpose of (the reference passes `qweight.t()`, stride (1, K))."""
+  if b_data.dim() != 2:
+    raise ValueError(f"{name}: b_data must be 2-D [K,N], got shape {tuple(b_data.shape)}")
+  w = b_data.t()
+  if w.stride(-1) != 1:
+    # a row-major [K,N] operand: materialise the K-contiguous layout once.
+    w = w.contiguous()
+  return w
+
+
+@torch.library.impl("cdit::float8_inference_scaled_mm", "CUDA")
+def _float8_inference_scaled_mm(a_data, a_scale, b_data, b_scale, bias, out_dtype_id,
+                                use_fast_accum, epilogue=0):
+  del use_fast_accum  # a cuBLASLt hint; fp32 accumulation is the only mode here
+  name = "cdit::float8_inference_scaled_mm"
+  out_dtype = decode_output_dtype(out_dtype_id)
+  if out_dtype != torch.bfloat16:
+    raise ValueError(f"{name}: only bfloat16 output is built, got {out_dtype}")
+  if a_data.dtype != FP8 or b_data.dtype != FP8:
+    raise ValueError(f"{name}: a_data/b_data must be float8_e4m3fn, got {a_data.dtype}/"
+                     f"{b_data.dtype}")
+  w = _weight_rows(b_data, name)
+  a2 = _as_rows(a_data)
+  M, K = a2.shape
+  N = w.shape[0]
+  if w.shape[1] != K:
+    raise ValueError(f"{name}: shape mismatch a {tuple(a_data.shape)} x b {tuple(b_data.shape)}")
+  if a_scale.numel() != M or b_scale.numel() != N:
+    raise ValueError(f"{name}: expected a_scale with {M} and b_scale with {N} elements, got "
+                     f"{a_scale.numel()} and {b_scale.numel()}")
+  a_s = a_scale.reshape(-1).to(torch.float32).contiguous()
+  b_s = b_scale.reshape(-1).to(torch.float32).contiguous()
+  if bias is not None:
+    if bias.numel() != N:
+      raise ValueError(f"{name}: bias must have {N} elements")
+    bias = bias.reshape(-1).to(torch.bfloat16).contiguous()
+  out = torch.empty((M, N), dtype=torch.bfloat16, device=a_data.device)
+  gemm_rowwise_into(a2, a_s, w, b_s, bias, out, int(epilogue))
+  return out.reshape(*a_data.shape[:-1], N)
+
+
+@torch.library.register_fake("cdit::float8_inference_scaled_mm")
+def _fake_float8_inference_scaled_mm(a_data, a_scale, b_data, b_scale, bias, out_dtype_id,
+                                     use_fast_accum, epilogue=0):
+  return a_data.new_empty((*a_data.shape[:-1], b_data.shape[-1]),
+                          dtype=decode_output_dtype(out_dtype_id))
+
+
+@torch.library.impl("cdit::w8a16_mm", "CUDA")
+def _w8a16_mm(x, b_data, b_scale, bias, out_dtype_id, epilogue=0):
+  name = "cdit::w8a16_mm"
+  out_dtype = decode_output_dtype(out_dtype_id)
+  if out_dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
+    raise ValueError(f"{name}: only bfloat16 activations and output are built, got {x.dtype} -> "
+                     f"{out_dtype}")
+  if b_data.dtype != FP8:
+    raise ValueError(f"{name}: b_data must be float8_e4m3fn, got {b_data.dtype}")
+  w = _weight_rows(b_data, name)
+  x2 = _as_rows(x)
+  M, K = x2.shape
+  N = w.shape[0]
+  if w.shape[1] != K:
+    raise ValueError(f"{name}: shape mismatch x {tuple(x.shape)} x b {tuple(b_data.shape)}")
+  if b_scale.numel() != N:
+    raise ValueError(f"{name}: b_scale must have {N} elements")
+  b_s = b_scale.reshape(-1).to(torch.float32).contiguous()
+  if bias is not None:
+    bias = bias.reshape(-1).to(torch.bfloat16).contiguous()
+  out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+  w8a16_into(x2, w, b_s, bias, out, int(epilogue))
+  return out.reshape(*x.shape[:-1], N)
+
+
+@torch.library.register_fake("cdit::w8a16_mm")
+def _fake_w8a16_mm(x, b_data, b_scale, bias, out_dtype_id, epilogue=0):
+  return x.new_empty((*x.shape[:-1], b_data.shape[-1]), dtype=decode_output_dtype(out_dtype_id))
+
+
+# --------------------------------------------------------------------------- python-level API
+
+
+def fp8_rowwise_quant(x: torch.Tensor,
+                      scale_mode: str = "bf16div") -> Tuple[torch.Tensor, torch.Tensor]:
+  """Per-row dynamic e4m3 quantization of a bf16 tensor -> (codes, scale[...,1])."""
+  _require_cuda("fp8_rowwise_quant", x)
+  return torch.ops.cdit.fp8_rowwise_quant(x, _native.SCALE_MODE_IDS[scale_mode])
+
+
+def float8_inference_scaled_mm(
+    a_data: torch.Tensor,
+    a_scale: torch.Tensor,
+    b_data: torch.Tensor,
+    b_scale: torch.Tensor,
+    output_dtype: torch.dtype,
+    output_scale: Optional[torch.Tensor] = None,
+    bias: Optional[torch.Tensor] = None,
+    use_fast_accum: bool = False,
+    epilogue: int = 0,
+) -> torch.Tensor:
+  """Same signature as the reference's `_opaque_addmm_float8_unwrapped_inference`
+  (src/cache_dit/quantization/torchao/_scaled_mm.py:140-162), incl. its refusal of
+  `output_scale`."""
+  if output_scale is not None:
+    raise NotImplementedError("float8 scaled_mm wrapper does not support scale_result yet.")
+  _require_cuda("float8_inference_scaled_mm", a_data, b_data)
+  return torch.ops.cdit.float8_inference_scaled_mm(a_data, a_scale, b_data, b_scale, bias,
+                                                   encode_output_dtype(output_dtype),
+                                                   use_fast_accum, epilogue)
+
+
+def w8a16_mm(x: torch.Tensor,
+             b_data: torch.Tensor,
+             b_scale: torch.Tensor,
+             bias: Optional[torch.Tensor] = None,
+             output_dtype: torch.dtype = torch.bfloat16,
+             epilogue: int = 0) -> torch.Tensor:
+  _require_cuda("w8a16_mm", x, b_data)
+  return torch.ops.cdit.w8a16_mm(x, b_data, b_scale, bias, encode_output_dtype(output_dtype),
+                                 epilogue)

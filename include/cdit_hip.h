@@ -1,0 +1,143 @@
+/*
+ * cdit_hip.h -- C ABI of libcdit_hip.so: MI355X (gfx950 / CDNA4) kernels for
+ * the FP8 quantized-linear hot path of cache-dit's `float8_per_row`
+ * (w8a8, dynamic per-token activation scales) and `float8_weight_only`
+ * (w8a16) quantize modes.
+ *
+ * Conventions (they follow the native-op conventions of the reference's own
+ * extension, csrc/kernels/svdq/torch.h:9-24 and
+ * src/cache_dit/kernels/cuda/_ops_registery.py:35-59):
+ *   - the caller owns every buffer; nothing here allocates or frees device
+ *     memory and no pointer is retained after the call returns;
+ *   - all pointers are device pointers on the current HIP device;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); work
+ *     is enqueued on it and the call returns without synchronising;
+ *   - every function returns 0 on success and a non-zero CDIT_E* code on
+ *     failure; cdit_last_error() then returns a thread-local message;
+ *   - FP8 means OCP e4m3fn (bias 7, max 448, NaN 0x7F/0xFF, no inf), the
+ *     format torch.float8_e4m3fn names; bf16 buffers are raw uint16 bits;
+ *   - matrices are row-major with a leading dimension in ELEMENTS.
+ *
+ * Only plain C types cross this boundary: a maintainer binds it with ctypes,
+ * cffi, pybind or a torch extension as they prefer.
+ */
+#ifndef CDIT_HIP_H_
+#define CDIT_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CDIT_ABI_VERSION 1
+
+enum cdit_status {
+  CDIT_OK = 0,
+  CDIT_EINVAL = 1,  /* bad shape, stride, alignment, mode or null pointer */
+  CDIT_EARCH = 2,   /* current device is not gfx950                       */
+  CDIT_EHIP = 3     /* a HIP runtime call failed (message has the reason) */
+};
+
+/* How the per-row scale amax/448 is rounded (the reference leaves this to
+ * torchao's _choose_scale_float8, call site
+ * src/cache_dit/quantization/torchao/quantize_ao.py:54-70):
+ *   BF16DIV: fp32 true divide, round-to-nearest-even to bf16, widen to fp32
+ *            (what an un-upcast bf16 `amax / 448.0` does in eager PyTorch);
+ *   FP32DIV: fp32 true divide, kept in fp32. */
+enum cdit_scale_mode { CDIT_SCALE_BF16DIV = 0, CDIT_SCALE_FP32DIV = 1 };
+
+/* Epilogue flags of the GEMM entry points (bit mask). */
+enum cdit_epilogue {
+  CDIT_EPI_NONE = 0,
+  CDIT_EPI_GELU_TANH = 1 /* 0.5 v (1 + tanh(0.79788456 (v + 0.044715 v^3))),
+                            the diffusers nn.GELU(approximate="tanh") that follows
+                            proj_mlp / ff.net.0.proj (reference dataflow:
+                            src/cache_dit/caching/patch_functors/functor_flux.py:48-80;
+                            formula precedent csrc/kernels/svdq/gemm_utils.cuh:363-378) */
+};
+
+/* Output element type ids, the reference's numbering
+ * (src/cache_dit/quantization/torchao/_scaled_mm.py:38-43). */
+enum cdit_dtype_id { CDIT_DT_F16 = 0, CDIT_DT_BF16 = 1, CDIT_DT_F32 = 2 };
+
+/* ABI version of the loaded library (== CDIT_ABI_VERSION it was built with). */
+int cdit_abi_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* cdit_last_error(void);
+
+/* Writes the gcnArchName of the current device (e.g. "gfx950:sramecc+:xnack-")
+ * into buf. Returns CDIT_OK, or CDIT_EARCH when it is not a gfx950. */
+int cdit_device_arch(char* buf, int buf_len);
+
+/*
+ * Per-row (per-token / per-output-channel) dynamic FP8 quantizer.
+ * Replaces torchao's _choose_scale_float8 + _quantize_affine_float8 as called
+ * through Float8Tensor.from_hp(x, PerRow()) -- reference call sites
+ * src/cache_dit/quantization/torchao/quantize_ao.py:54-70 (scale, with the
+ * zero-scale patch :65-67) and tests/kernels/test_opaque_scaled_mm.py:68-73.
+ *
+ *   amax[m]  = max_k |x[m,k]|                      (bf16, exact)
+ *   scale[m] = amax/448 rounded per scale_mode; 0 -> 1
+ *   q[m,k]   = e4m3fn_rne(clamp(float(x[m,k]) / scale[m], -448, 448))
+ *
+ * x: bf16 [M,K], leading dimension ld_x; q: e4m3 bytes [M,K], leading
+ * dimension ld_q; scale: fp32 [M]. The division is IEEE correctly rounded.
+ * M == 0 or K == 0 is a no-op that returns CDIT_OK. NaN/Inf inputs are outside
+ * the bit-exact contract.
+ */
+int cdit_fp8_quant_rowwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_x,
+                           void* q_e4m3, int64_t ld_q, float* scale,
+                           int scale_mode, void* stream);
+
+/*
+ * Row-wise scaled FP8 GEMM with fused epilogue. Replaces
+ * torch._scaled_mm(a, b, scale_a, scale_b, bias, out_dtype) as called by
+ * _run_float8_inference_scaled_mm, src/cache_dit/quantization/torchao/_scaled_mm.py:62-91
+ * (op schema :94-98).
+ *
+ *   out[m,n] = epi( (sum_k a[m,k] * b[n,k]) * a_scale[m] * b_scale[n] + bias[n] )
+ *
+ * a_q: e4m3 [M,K] row-major (lda); b_q: e4m3 [N,K] row-major (ldb) -- the
+ * quantized nn.Linear weight as stored, i.e. the reference's column-major
+ * [K,N] `qweight.t()`; a_scale fp32 [M]; b_scale fp32 [N]; bias bf16 [N] or
+ * NULL; out [M,N] (ldo) of out_dtype_id (only CDIT_DT_BF16 is built).
+ * Accumulation is fp32. Requires K % 16 == 0 (as the reference's FP8 matmul
+ * does) and 16-byte aligned a_q/b_q rows.
+ */
+int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale,
+                          const void* b_q, const float* b_scale,
+                          const void* bias_bf16, void* out,
+                          int64_t M, int64_t N, int64_t K,
+                          int64_t lda, int64_t ldb, int64_t ldo,
+                          int epilogue, int out_dtype_id, void* stream);
+
+/*
+ * Weight-only FP8 GEMM (w8a16): bf16 activations, e4m3 weights dequantized in
+ * the mainloop, per-output-channel scale applied in the epilogue. Replaces
+ * F.linear(x, W.dequantize(), bias) of torchao's Float8WeightOnlyConfig
+ * (reference selection: src/cache_dit/quantization/torchao/quantize_ao.py:604-610).
+ *
+ *   out[m,n] = epi( (sum_k x[m,k] * float(b[n,k])) * b_scale[n] + bias[n] )
+ *
+ * x_bf16 [M,K] (lda); b_q e4m3 [N,K] (ldb); b_scale fp32 [N]; bias bf16 [N] or
+ * NULL; out bf16 [M,N] (ldo). Requires K % 16 == 0.
+ */
+int cdit_w8a16_gemm(const void* x_bf16, const void* b_q, const float* b_scale,
+                    const void* bias_bf16, void* out,
+                    int64_t M, int64_t N, int64_t K,
+                    int64_t lda, int64_t ldb, int64_t ldo,
+                    int epilogue, int out_dtype_id, void* stream);
+
+/*
+ * Tuning hook used by the benchmark and the tests: forces the kernel variant
+ * the two GEMM entry points pick (-1 = automatic choice by shape). Returns
+ * the previous value. Process-global; not meant for concurrent use.
+ */
+int cdit_set_gemm_variant(int variant);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CDIT_HIP_H_ */

@@ -1,0 +1,193 @@
+"""GPU parity of the row-wise scaled FP8 GEMM (w8a8) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import bits_u8, config1_inputs, elementwise_ok, max_rel_err
+from oracle import c_oracle
+from oracle import torch_oracle as to
+
+pytestmark = pytest.mark.gpu
+FP8 = torch.float8_e4m3fn
+REL_TOL = 1e-2  # BASELINE north star: max relative error 1e-2, bf16 out, fp32 accumulate
+
+
+@pytest.fixture(autouse=True)
+def _auto_variant():
+  from cache_dit_amd import _native
+  _native.set_gemm_variant(-1)
+  yield
+  _native.set_gemm_variant(-1)
+
+
+def _rand_problem(M, N, K, seed, bias=True, outliers=True):
+  g = torch.Generator().manual_seed(seed)
+  x = torch.randn(M, K, generator=g)
+  if outliers and K >= 16:
+    x[:, torch.randperm(K, generator=g)[:max(1, K // 1000)]] *= 20
+  w = torch.randn(N, K, generator=g) * 0.02
+  b = (torch.randn(N, generator=g) * 0.01).to(torch.bfloat16) if bias else None
+  xq, xs = to.quantize_rowwise(x.to(torch.bfloat16))
+  wq, ws = to.quantize_rowwise(w.to(torch.bfloat16))
+  return xq, xs, wq, ws, b
+
+
+def _run(xq, xs, wq, ws, b, epilogue=0):
+  from cache_dit_amd import ops
+  out = ops.float8_inference_scaled_mm(xq.cuda(), xs.cuda(), wq.cuda().t(), ws.cuda().t(),
+                                       torch.bfloat16, bias=None if b is None else b.cuda(),
+                                       use_fast_accum=True, epilogue=epilogue)
+  torch.cuda.synchronize()
+  return out
+
+
+def _assert_close(out, ref):
+  assert out.dtype == torch.bfloat16 and out.shape == ref.shape
+  assert torch.isfinite(out.float()).all()
+  e = max_rel_err(out, ref)
+  assert e <= REL_TOL, f"max rel err {e:.3e} > {REL_TOL}"
+  assert elementwise_ok(out, ref, REL_TOL)
+
+
+TILED_VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7]
+
+
+@pytest.mark.parametrize("variant", TILED_VARIANTS + [100])
+@pytest.mark.parametrize("M,N,K", [(512, 768, 1024), (300, 520, 256), (1, 264, 128),
+                                   (257, 8, 384)])
+def test_variants_with_tails(variant, M, N, K):
+  from cache_dit_amd import _native
+  p = _rand_problem(M, N, K, seed=M + N + K)
+  ref = to.scaled_mm_rowwise(*p)
+  _native.set_gemm_variant(variant)
+  _assert_close(_run(*p), ref)
+
+
+@pytest.mark.parametrize("variant", TILED_VARIANTS + [100])
+def test_exact_small_integers(variant):
+  """Integer-valued codes and power-of-two scales: every partial sum is exact in
+  fp32 whatever the order, so the output must equal the oracle bit for bit."""
+  from cache_dit_amd import _native
+  g = torch.Generator().manual_seed(11)
+  M, N, K = 320, 264, 512
+  a = torch.randint(-4, 5, (M, K), generator=g).float().to(FP8)
+  w = torch.randint(-4, 5, (N, K), generator=g).float().to(FP8)
+  a_s = torch.full((M, 1), 0.5)
+  w_s = torch.full((N, 1), 0.25)
+  ref = to.scaled_mm_rowwise(a, a_s, w, w_s)
+  _native.set_gemm_variant(variant)
+  out = _run(a, a_s, w, w_s, None)
+  assert torch.equal(out.cpu(), ref)
+
+
+def test_k_position_sensitivity():
+  """One non-zero per row of A at a different K position per row against a weight
+  whose value encodes its K index: a K-permutation mismatch between the A and B
+  operand layouts would show up as a wrong (not just noisy) answer."""
+  M, N, K = 256, 256, 256
+  a = torch.zeros(M, K)
+  a[torch.arange(M), torch.arange(M) % K] = 1.0
+  w = ((torch.arange(K) % 15) + 1).float().repeat(N, 1) * (1 + (torch.arange(N) % 2)).reshape(-1, 1)
+  ones_m, ones_n = torch.ones(M, 1), torch.ones(N, 1)
+  ref = to.scaled_mm_rowwise(a.to(FP8), ones_m, w.to(FP8), ones_n)
+  out = _run(a.to(FP8), ones_m, w.to(FP8), ones_n, None)
+  assert torch.equal(out.cpu(), ref)
+
+
+def test_reference_smoke_shape_w32x64_x4x64():
+  # tests/kernels/test_opaque_scaled_mm.py:67-74 of the reference: W[32,64], x[4,64], seed 0
+  torch.manual_seed(0)
+  w = torch.randn(32, 64).to(torch.bfloat16)
+  x = torch.randn(4, 64).to(torch.bfloat16)
+  xq, xs = to.quantize_rowwise(x)
+  wq, ws = to.quantize_rowwise(w)
+  ref = to.scaled_mm_rowwise(xq, xs, wq, ws)
+  out = _run(xq, xs, wq, ws, None)
+  assert out.shape == (4, 32)
+  _assert_close(out, ref)
+
+
+def test_reference_partition_shape_m512_k3072_n3072():
+  # tests/kernels/test_rowwise_cudagraph_partition.py:35-37 of the reference
+  p = _rand_problem(512, 3072, 3072, seed=2)
+  _assert_close(_run(*p), to.scaled_mm_rowwise(*p))
+
+
+def test_config1_full():
+  x, w, b = config1_inputs()
+  xq, xs = to.quantize_rowwise(x[0])
+  wq, ws = to.quantize_rowwise(w)
+  ref = to.scaled_mm_rowwise(xq, xs, wq, ws, b)
+  _assert_close(_run(xq, xs, wq, ws, b), ref)
+
+
+@pytest.mark.parametrize("M,N,K", [(333, 512, 1024), (64, 256, 3072)])
+def test_against_c_oracle(M, N, K):
+  """The plain-C restatement (double accumulation) as a second checker."""
+  xq, xs, wq, ws, b = _rand_problem(M, N, K, seed=5)
+  ref_bits = c_oracle.gemm_rowwise(bits_u8(xq), xs.numpy(), bits_u8(wq), ws.numpy(),
+                                   b.view(torch.int16).numpy().view(np.uint16))
+  ref = torch.from_numpy(ref_bits.view(np.int16)).view(torch.bfloat16)
+  _assert_close(_run(xq, xs, wq, ws, b), ref)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 7, 100])
+def test_gelu_tanh_epilogue(variant):
+  from cache_dit_amd import _native
+  p = _rand_problem(384, 512, 1024, seed=9)
+  # make the pre-activation O(1) so that GELU is exercised away from zero
+  p = (p[0], p[1] * 8, p[2], p[3], p[4])
+  fused = to.scaled_mm_rowwise(*p, gelu="fused")
+  unfused = to.scaled_mm_rowwise(*p, gelu="unfused")
+  _native.set_gemm_variant(variant)
+  out = _run(*p, epilogue=1)
+  _assert_close(out, fused)
+  _assert_close(out, unfused)  # one bf16 rounding apart: inside the same bar
+
+
+def test_against_torch_scaled_mm_on_gpu():
+  """torch._scaled_mm (hipBLASLt row-wise FP8, a library routine) fed with the same
+  codes and scales: a second witness for the GEMM at the FLUX MLP shape."""
+  M, N, K = 4608, 12288, 3072
+  g = torch.Generator(device="cuda").manual_seed(3)
+  a = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
+  w = (torch.randn(N, K, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+  b = (torch.randn(N, generator=g, device="cuda") * 0.01).to(torch.bfloat16)
+  from cache_dit_amd import ops
+  aq, a_s = ops.fp8_rowwise_quant(a)
+  wq, w_s = ops.fp8_rowwise_quant(w)
+  out = ops.float8_inference_scaled_mm(aq, a_s, wq.t(), w_s.t(), torch.bfloat16, bias=b)
+  try:
+    ref = torch._scaled_mm(aq, wq.t(), scale_a=a_s, scale_b=w_s.t(), bias=b,
+                           out_dtype=torch.bfloat16)
+  except Exception as e:  # pragma: no cover - depends on the box's hipBLASLt
+    pytest.skip(f"torch._scaled_mm row-wise not available here: {e}")
+  assert max_rel_err(out, ref) <= REL_TOL
+  # linearity in the scales (size-independent property at the full shape)
+  out2 = ops.float8_inference_scaled_mm(aq, a_s * 2, wq.t(), w_s.t() * 0.5, torch.bfloat16,
+                                        bias=b)
+  assert torch.equal(out2, out)
+
+
+def test_error_paths():
+  from cache_dit_amd import ops
+  a = torch.zeros(4, 64, device="cuda").to(FP8)
+  w = torch.zeros(32, 64, device="cuda").to(FP8)
+  s_a, s_w = torch.ones(4, 1, device="cuda"), torch.ones(1, 32, device="cuda")
+  with pytest.raises(NotImplementedError):
+    ops.float8_inference_scaled_mm(a, s_a, w.t(), s_w, torch.bfloat16, output_scale=s_a)
+  with pytest.raises(ValueError):
+    ops.float8_inference_scaled_mm(a, s_a, w.t(), s_w, torch.float64)
+  with pytest.raises(ValueError):
+    ops.float8_inference_scaled_mm(a, s_a, w.t(), s_w, torch.float32)  # not built
+  with pytest.raises(ValueError):
+    ops.float8_inference_scaled_mm(a, s_a[:2], w.t(), s_w, torch.bfloat16)
+  from cache_dit_amd import _native
+  L = _native.load()
+  o = torch.zeros(4, 32, dtype=torch.bfloat16, device="cuda")
+  rc = L.cdit_fp8_gemm_rowwise(a.data_ptr(), s_a.data_ptr(), w.data_ptr(), s_w.data_ptr(), None,
+                               o.data_ptr(), 4, 32, 40, 64, 64, 32, 0, 1, None)
+  assert rc == 1 and b"multiple of 16" in L.cdit_last_error()
+  rc = L.cdit_fp8_gemm_rowwise(a.data_ptr(), s_a.data_ptr(), w.data_ptr(), s_w.data_ptr(), None,
+                               o.data_ptr(), 0, 32, 64, 64, 64, 32, 0, 1, None)
+  assert rc == 0  # empty M is a no-op

@@ -1,0 +1,117 @@
+"""GPU parity of the weight-only (w8a16) GEMM against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import bits_u8, elementwise_ok, max_rel_err
+from oracle import c_oracle
+from oracle import torch_oracle as to
+
+pytestmark = pytest.mark.gpu
+FP8 = torch.float8_e4m3fn
+REL_TOL = 1e-2
+
+
+@pytest.fixture(autouse=True)
+def _auto_variant():
+  from cache_dit_amd import _native
+  _native.set_gemm_variant(-1)
+  yield
+  _native.set_gemm_variant(-1)
+
+
+def _problem(M, N, K, seed, bias=True):
+  g = torch.Generator().manual_seed(seed)
+  x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+  w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
+  b = (torch.randn(N, generator=g) * 0.01).to(torch.bfloat16) if bias else None
+  wq, ws = to.quantize_rowwise(w)
+  return x, wq, ws, b
+
+
+def _run(x, wq, ws, b, epilogue=0):
+  from cache_dit_amd import ops
+  out = ops.w8a16_mm(x.cuda(), wq.cuda().t(), ws.cuda(), None if b is None else b.cuda(),
+                     torch.bfloat16, epilogue)
+  torch.cuda.synchronize()
+  return out
+
+
+def _assert_close(out, ref):
+  assert out.dtype == torch.bfloat16 and out.shape == ref.shape
+  e = max_rel_err(out, ref)
+  assert e <= REL_TOL, f"max rel err {e:.3e}"
+  assert elementwise_ok(out, ref, REL_TOL)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 100])
+@pytest.mark.parametrize("M,N,K", [(512, 768, 1024), (300, 520, 192), (1, 264, 64), (257, 8, 384)])
+def test_variants_with_tails(variant, M, N, K):
+  from cache_dit_amd import _native
+  p = _problem(M, N, K, seed=M + N + K)
+  _native.set_gemm_variant(variant)
+  out = _run(*p)
+  _assert_close(out, to.w8a16_linear(*p, fused=True))
+  _assert_close(out, to.w8a16_linear(*p, fused=False))  # the reference's dequantize-first form
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 100])
+def test_exact_small_integers(variant):
+  from cache_dit_amd import _native
+  g = torch.Generator().manual_seed(12)
+  M, N, K = 320, 264, 512
+  x = torch.randint(-4, 5, (M, K), generator=g).to(torch.bfloat16)
+  w = torch.randint(-4, 5, (N, K), generator=g).float().to(FP8)
+  ws = torch.full((N, 1), 0.25)
+  _native.set_gemm_variant(variant)
+  out = _run(x, w, ws, None)
+  assert torch.equal(out.cpu(), to.w8a16_linear(x, w, ws, fused=True))
+
+
+def test_k_position_sensitivity():
+  M, N, K = 256, 256, 256
+  x = torch.zeros(M, K)
+  x[torch.arange(M), torch.arange(M) % K] = 1.0
+  w = ((torch.arange(K) % 15) + 1).float().repeat(N, 1)
+  ones = torch.ones(N, 1)
+  out = _run(x.to(torch.bfloat16), w.to(FP8), ones, None)
+  assert torch.equal(out.cpu(), to.w8a16_linear(x.to(torch.bfloat16), w.to(FP8), ones, fused=True))
+
+
+def test_every_e4m3_code_dequantizes_exactly():
+  """x = identity picks out single weights: out[m, n] = float(code) for all 256 codes
+  (NaN codes excluded), so the in-loop e4m3 -> bf16 conversion is checked value by value."""
+  codes = torch.arange(256, dtype=torch.uint8)
+  keep = (codes & 0x7f) != 0x7f
+  codes = codes[keep]
+  K = 256
+  N = 256
+  w = torch.zeros(N, K, dtype=torch.uint8)
+  w[torch.arange(codes.numel()), torch.arange(codes.numel())] = codes
+  wq = w.view(FP8)
+  x = torch.eye(K).to(torch.bfloat16)
+  out = _run(x, wq, torch.ones(N, 1), None)
+  expect = wq.float().t().to(torch.bfloat16)  # exact: every e4m3 value is a bf16 value
+  assert torch.equal(out.cpu(), expect)
+
+
+@pytest.mark.parametrize("K,N", [(3072, 3072), (3072, 9216), (3072, 12288), (12288, 3072),
+                                 (15360, 3072)])
+def test_flux_shapes_m4608(K, N):
+  M = 4608
+  x, wq, ws, b = _problem(M, N, K, seed=K + N)
+  out = _run(x, wq, ws, b)
+  rows = torch.arange(0, M, 37)  # every 37th row against the oracle
+  ref = to.w8a16_linear(x[rows], wq, ws, b, fused=True)
+  _assert_close(out[rows.cuda()], ref)
+
+
+def test_against_c_oracle_and_gelu():
+  x, wq, ws, b = _problem(200, 256, 512, seed=8)
+  xb = x.view(torch.int16).numpy().view(np.uint16)
+  bb = b.view(torch.int16).numpy().view(np.uint16)
+  for gelu in (0, 1):
+    ref_bits = c_oracle.w8a16(xb, bits_u8(wq), ws.numpy(), bb, gelu=gelu, dequant_bf16=False)
+    ref = torch.from_numpy(ref_bits.view(np.int16)).view(torch.bfloat16)
+    _assert_close(_run(x, wq, ws * (8 if gelu else 1), b, epilogue=gelu), ref if not gelu else
+                  to.w8a16_linear(x, wq, ws * 8, b, gelu="fused", fused=True))
