@@ -28,14 +28,19 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
 }
 
-// tanh-approximated GELU, the formula of torch.nn.functional.gelu(approximate="tanh").
+// tanh-approximated GELU, the formula of torch.nn.functional.gelu(approximate="tanh"):
+// 0.5 v (1 + tanh(u)), u = sqrt(2/pi) (v + 0.044715 v^3). Since
+// 0.5 (1 + tanh(u)) = 1 / (1 + exp(-2u)), it is evaluated as v * rcp(1 + exp2(c u))
+// with the hardware exp2 and reciprocal (about 1 ulp each; the result is rounded
+// to bf16 afterwards). exp2 overflow gives v * 0 = -0 for very negative v and
+// exp2 underflow gives v * 1 for very positive v, the correct limits.
 __device__ __forceinline__ float gelu_tanh(float v) {
   const float kAlpha = 0.7978845608028654f;  // sqrt(2/pi)
   const float kBeta = 0.044715f;
-  float u = kAlpha * (v + kBeta * v * v * v);
-  // tanh(u) = 1 - 2/(exp(2u)+1); exp overflow to +inf gives 1, underflow gives -1.
-  float t = 1.0f - 2.0f / (__expf(2.0f * u) + 1.0f);
-  return 0.5f * v * (1.0f + t);
+  const float kM2Log2e = -2.8853900817779268f;  // -2 * log2(e)
+  const float u = kAlpha * (v + kBeta * v * v * v);
+  const float e = __builtin_amdgcn_exp2f(kM2Log2e * u);
+  return v * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 // Workgroup id -> output tile. Workgroups are handed to the 8 XCDs round-robin

@@ -286,7 +286,11 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     hipLaunchKernelGGL(gemm_fp8_generic, grid, dim3(256), 0, stream, g);
     return 0;
   }
-  if (variant < 0) variant = 0;
+  if (variant < 0) {
+    // enough 256x256 tiles to cover the 256 CUs: the 8-wave kernel; else smaller tiles
+    const int64_t big_tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
+    variant = big_tiles >= 200 ? 7 : 6;
+  }
   switch (variant) {
     case 0: return launch_tiled<V0>(g, stream);
     case 1: return launch_tiled<V1>(g, stream);

@@ -230,7 +230,7 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
     hipLaunchKernelGGL(gemm_w8a16_generic, grid, dim3(256), 0, stream, g);
     return 0;
   }
-  if (variant < 0) variant = 0;
+  if (variant < 0) variant = 3;
   switch (variant) {
     case 0: return launch_tiled<W0>(g, stream);
     case 1: return launch_tiled<W1>(g, stream);
