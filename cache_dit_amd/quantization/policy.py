@@ -94,16 +94,17 @@ class QuantizeContext:
 
   # -- construction -----------------------------------------------------------
   @staticmethod
-  def from_config(config: QuantizeConfig, module: nn.Module, **kwargs) -> "QuantizeContext":
+  def from_config(quantize_config: QuantizeConfig, module: nn.Module,
+                  **kwargs) -> "QuantizeContext":
     return QuantizeContext(
         module_ref=module,
-        quant_type=config.quant_type,
-        regional_quantize=config.regional_quantize,
-        repeated_blocks=config.repeated_blocks,
-        exclude_layers=config.exclude_layers,
-        precision_plan=config.precision_plan,
-        per_tensor_fallback=config.per_tensor_fallback,
-        verbose=config.verbose,
+        quant_type=quantize_config.quant_type,
+        regional_quantize=quantize_config.regional_quantize,
+        repeated_blocks=quantize_config.repeated_blocks,
+        exclude_layers=quantize_config.exclude_layers,
+        precision_plan=quantize_config.precision_plan,
+        per_tensor_fallback=quantize_config.per_tensor_fallback,
+        verbose=quantize_config.verbose,
         kwargs=copy.deepcopy(kwargs),
     ).normalize()
 
@@ -413,16 +414,13 @@ def quantize_ao(module: nn.Module, quantize_config: QuantizeConfig,
   convert = _convert_fn
   if convert is None:
     _check_platform(ctx)
-    convert = _default_convert
 
-    def convert_checked(linear: nn.Linear, qt: str) -> None:
+    def convert(linear: nn.Linear, qt: str) -> None:
       if qt not in BUILT_QUANTIZE_TYPES:
         raise NotImplementedError(
             f"quant_type {qt!r} has no MI355X kernel in this build (built: "
             f"{BUILT_QUANTIZE_TYPES})")
       _default_convert(linear, qt)
-
-    convert = convert_checked
 
   def basic(qt_override: Optional[str] = None):
     return lambda m, name: basic_filter(m, name, ctx, qt_override)

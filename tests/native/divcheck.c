@@ -44,7 +44,7 @@ int main(int argc, char** argv) {
           const float ref = x / s;
           const float q0 = x * r;
           const float e = fmaf(-q0, s, x);
-          const float q1 = fmaf(e, r, q0);
+          const float q1 = copysignf(fmaf(e, r, q0), x);
           ++checked;
           if (f2u(q1) != f2u(ref)) {
             ++bad_q;

@@ -1,0 +1,90 @@
+"""The C ABI library loads and exports every symbol include/cdit_hip.h declares;
+argument validation that needs no GPU; fake (meta) implementations of the ops."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+  text = open(os.path.join(ROOT, "include", "cdit_hip.h")).read()
+  text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+  return sorted(set(re.findall(r"\b(cdit_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported():
+  from cache_dit_amd import _native
+  if not _native.is_built():
+    pytest.skip("libcdit_hip.so not built (run __graft_entry__.build())")
+  names = _declared()
+  assert sorted(_native.EXPORTS) == names
+  L = ctypes.CDLL(_native.LIB_PATH)
+  for n in names:
+    assert hasattr(L, n), n
+  assert _native.load().cdit_abi_version() == _native.ABI_VERSION == 1
+
+
+def test_argument_validation_without_gpu():
+  from cache_dit_amd import _native
+  if not _native.is_built():
+    pytest.skip("libcdit_hip.so not built")
+  L = _native.load()
+  assert L.cdit_fp8_quant_rowwise(None, -1, 8, 8, None, 8, None, 0, None) == 1
+  assert b"bad shape" in L.cdit_last_error()
+  assert L.cdit_fp8_quant_rowwise(None, 4, 8, 8, None, 8, None, 5, None) == 1
+  assert b"scale_mode" in L.cdit_last_error()
+  assert L.cdit_fp8_quant_rowwise(None, 0, 8, 8, None, 8, None, 0, None) == 0  # empty: no-op
+  one = ctypes.c_void_p(16)
+  assert L.cdit_fp8_gemm_rowwise(one, one, one, one, None, one, 4, 4, 24, 24, 24, 4, 0, 1, None) == 1
+  assert b"multiple of 16" in L.cdit_last_error()
+  assert L.cdit_fp8_gemm_rowwise(one, one, one, one, None, one, 4, 4, 32, 32, 32, 4, 0, 2, None) == 1
+  assert b"out_dtype_id" in L.cdit_last_error()
+  assert L.cdit_fp8_gemm_rowwise(one, one, one, one, None, one, 4, 4, 32, 32, 32, 4, 8, 1, None) == 1
+  assert L.cdit_fp8_gemm_rowwise(one, one, one, one, None, one, 4, 4, 32, 16, 32, 4, 0, 1, None) == 1
+  assert b"leading dimension" in L.cdit_last_error()
+  assert L.cdit_w8a16_gemm(one, one, None, None, one, 4, 4, 32, 32, 32, 4, 0, 1, None) == 1
+  assert b"null pointer" in L.cdit_last_error()
+  assert L.cdit_w8a16_gemm(one, one, one, None, one, 0, 4, 32, 32, 32, 4, 0, 1, None) == 0
+  assert L.cdit_set_gemm_variant(3) == -1 and L.cdit_set_gemm_variant(-1) == 3
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+  from cache_dit_amd import _native
+  monkeypatch.setattr(_native, "_lib", None)
+  monkeypatch.setenv("CDIT_HIP_LIB", str(tmp_path / "nope.so"))
+  with pytest.raises(_native.CditNativeError, match="no fallback"):
+    _native.load()
+
+
+def test_fake_impls_shapes_and_dtypes():
+  import cache_dit_amd.ops  # noqa: F401  (registers torch.ops.cdit)
+  from torch._subclasses.fake_tensor import FakeTensorMode
+  FP8 = torch.float8_e4m3fn
+  with FakeTensorMode():
+    x = torch.empty(2, 77, 3072, dtype=torch.bfloat16, device="cuda")
+    q, s = torch.ops.cdit.fp8_rowwise_quant(x, 0)
+    assert q.shape == (2, 77, 3072) and q.dtype == FP8 and q.device.type == "cuda"
+    assert s.shape == (2, 77, 1) and s.dtype == torch.float32
+    a = torch.empty(154, 3072, dtype=FP8, device="cuda")
+    b = torch.empty(12288, 3072, dtype=FP8, device="cuda").t()
+    for dt_id, dt in ((0, torch.float16), (1, torch.bfloat16), (2, torch.float32)):
+      y = torch.ops.cdit.float8_inference_scaled_mm(a, s.reshape(-1, 1), b,
+                                                    torch.empty(1, 12288, device="cuda"), None,
+                                                    dt_id, True)
+      assert y.shape == (154, 12288) and y.dtype == dt
+    y = torch.ops.cdit.w8a16_mm(x, b, torch.empty(12288, device="cuda"), None, 1, 1)
+    assert y.shape == (2, 77, 12288) and y.dtype == torch.bfloat16
+
+
+def test_dtype_id_codec():
+  from cache_dit_amd import ops
+  assert [ops.encode_output_dtype(d) for d in (torch.float16, torch.bfloat16, torch.float32)] == [0, 1, 2]
+  assert ops.decode_output_dtype(1) is torch.bfloat16
+  with pytest.raises(ValueError, match="output dtype"):
+    ops.encode_output_dtype(torch.float64)
+  with pytest.raises(ValueError, match="dtype id"):
+    ops.decode_output_dtype(9)

@@ -1,0 +1,204 @@
+"""GPU end-to-end: quantize() on real modules, golden vectors, and the single-step
+transformer output against the same model run with the oracle's ops."""
+import copy
+import logging
+import os
+
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+from helpers import bits_u8, cosine, max_rel_err
+from oracle import torch_oracle as to
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+logging.getLogger("CACHE_DIT_AMD").setLevel(logging.WARNING)
+
+
+def _bf(a):
+  return torch.from_numpy(a.view(np.int16)).view(torch.bfloat16)
+
+
+def test_golden_vectors_on_gpu():
+  from cache_dit_amd import ops
+  z = np.load(os.path.join(GOLD, "quant_vectors.npz"))
+  x = _bf(z["x"]).cuda()
+  for mode in ("bf16div", "fp32div"):
+    q, s = ops.fp8_rowwise_quant(x, mode)
+    assert (bits_u8(q) == z[f"q_{mode}"]).all()
+    assert (s.reshape(-1).cpu().numpy().view(np.uint32) == z[f"s_{mode}"].view(np.uint32)).all()
+  z = np.load(os.path.join(GOLD, "linear_vectors.npz"))
+  x, b = _bf(z["x"]).cuda(), _bf(z["bias"]).cuda()
+  wq = torch.from_numpy(z["wq"]).view(torch.float8_e4m3fn).cuda()
+  ws = torch.from_numpy(z["ws"]).cuda()
+  xq, xs = ops.fp8_rowwise_quant(x)
+  assert (bits_u8(xq) == z["xq"]).all() and (xs.reshape(-1).cpu().numpy() == z["xs"]).all()
+  y = ops.float8_inference_scaled_mm(xq, xs, wq.t(), ws.reshape(1, -1), torch.bfloat16, bias=b)
+  assert max_rel_err(y, _bf(z["y_w8a8"])) <= 1e-2
+  yg = ops.float8_inference_scaled_mm(xq, xs, wq.t(), ws.reshape(1, -1), torch.bfloat16, bias=b,
+                                      epilogue=1)
+  assert max_rel_err(yg, _bf(z["y_w8a8_gelu_fused"])) <= 1e-2
+  assert max_rel_err(yg, _bf(z["y_w8a8_gelu_unfused"])) <= 1e-2
+  yw = ops.w8a16_mm(x, wq.t(), ws, b)
+  assert max_rel_err(yw, _bf(z["y_w8a16_ref"])) <= 1e-2
+  assert max_rel_err(yw, _bf(z["y_w8a16_fused"])) <= 1e-2
+
+
+class _Blk(nn.Module):
+
+  def __init__(self, d):
+    super().__init__()
+    self.to_q = nn.Linear(d, d)
+    self.proj_mlp = nn.Linear(d, 4 * d)
+    self.act_mlp = nn.GELU(approximate="tanh")
+    self.proj_out = nn.Linear(4 * d, d, bias=False)
+    self.mod = nn.Linear(d, d)
+
+  def forward(self, x):
+    return x + self.proj_out(self.act_mlp(self.proj_mlp(self.to_q(x) + self.mod(x))))
+
+
+class _Net(nn.Module):
+  _repeated_blocks = ["_Blk"]
+
+  def __init__(self, d=256):
+    super().__init__()
+    self.blocks = nn.ModuleList([_Blk(d), _Blk(d)])
+
+  def forward(self, x):
+    for b in self.blocks:
+      x = b(x)
+    return x
+
+
+@pytest.mark.parametrize("quant_type", ["float8_per_row", "float8_weight_only"])
+@pytest.mark.parametrize("where", ["gpu", "cpu_then_gpu"])
+def test_quantize_module_in_place(quant_type, where):
+  """Weights quantized on the GPU, or on the CPU before `.to(device)` as the
+  reference's CLI flow does: same codes either way, equal to the oracle's."""
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd.nn import Fp8DynamicLinear, Fp8WeightOnlyLinear
+  torch.manual_seed(0)
+  net = _Net().to(torch.bfloat16)
+  ref = copy.deepcopy(net)
+  if where == "gpu":
+    net = net.cuda()
+  out = cache_dit.quantize(net, cache_dit.QuantizeConfig(quant_type=quant_type))
+  assert out is net and net._is_quantized
+  net = net.cuda()
+  cls = Fp8DynamicLinear if quant_type == "float8_per_row" else Fp8WeightOnlyLinear
+  for blk, rblk in zip(net.blocks, ref.blocks):
+    assert type(blk.mod) is nn.Linear and blk.mod.weight.dtype == torch.bfloat16  # excluded
+    for name in ("to_q", "proj_mlp", "proj_out"):
+      lin, rlin = getattr(blk, name), getattr(rblk, name)
+      assert isinstance(lin, cls) and isinstance(lin, nn.Linear) and lin._is_inner_quantized
+      wq, ws = to.quantize_rowwise(rlin.weight.detach())
+      assert lin.weight.dtype == torch.float8_e4m3fn and not lin.weight.requires_grad
+      assert (bits_u8(lin.weight) == bits_u8(wq)).all()
+      assert torch.equal(lin.weight_scale.cpu(), ws)
+  x = torch.randn(2, 50, 256, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+  y = net(x.cuda())
+  assert y.shape == x.shape and y.dtype == torch.bfloat16
+  # the same network with the oracle's ops on the CPU
+  f = to.w8a8_linear if quant_type == "float8_per_row" else to.w8a16_linear
+  h = x
+  for rblk in ref.blocks:
+    q = {n: to.quantize_rowwise(getattr(rblk, n).weight.detach()) for n in ("to_q", "proj_mlp",
+                                                                           "proj_out")}
+    t = f(h, *q["to_q"], rblk.to_q.bias.detach()) + rblk.mod(h)
+    t = rblk.act_mlp(f(t, *q["proj_mlp"], rblk.proj_mlp.bias.detach()))
+    h = h + f(t, *q["proj_out"], None)
+  assert cosine(y, h) >= 0.9999 and max_rel_err(y, h) <= 2e-2
+  assert "quant_type=" + quant_type in repr(net.blocks[0].to_q)
+  sd = net.state_dict()
+  assert sd["blocks.0.to_q.weight"].dtype == torch.float8_e4m3fn
+  assert sd["blocks.0.to_q.weight_scale"].shape == (256, 1)
+
+
+def test_input_checks_of_the_quantized_linear():
+  import cache_dit_amd as cache_dit
+  net = _Net().to(torch.bfloat16).cuda()
+  cache_dit.quantize(net, cache_dit.QuantizeConfig())
+  lin = net.blocks[0].to_q
+  with pytest.raises(ValueError, match="bfloat16"):
+    lin(torch.zeros(4, 256, device="cuda"))
+  with pytest.raises(RuntimeError, match="no CPU path"):
+    lin(torch.zeros(4, 256, dtype=torch.bfloat16))
+  assert lin(torch.zeros(0, 256, dtype=torch.bfloat16, device="cuda")).shape == (0, 256)
+  y = lin(torch.zeros(3, 5, 256, dtype=torch.bfloat16, device="cuda"))  # zero rows: scale 1
+  assert torch.equal(y, lin.bias.expand(3, 5, 256))
+  xs = torch.randn(8, 512, device="cuda").to(torch.bfloat16)[:, ::2]  # non-contiguous input
+  assert torch.equal(lin(xs), lin(xs.contiguous()))
+
+
+def _oracle_ops_forward(model, inputs, device):
+  """Runs `model` with every quantized Linear replaced by the oracle's w8a8
+  arithmetic written in plain torch ops on `device`."""
+  from cache_dit_amd.nn import _Fp8LinearBase
+
+  def fwd(self, x):
+    return to.w8a8_linear(x, self.weight, self.weight_scale, self.bias,
+                          gelu="fused" if self.epilogue else None)
+
+  saved = _Fp8LinearBase.forward
+  from cache_dit_amd import nn as cnn
+  old = cnn.Fp8DynamicLinear.forward
+  cnn.Fp8DynamicLinear.forward = fwd
+  try:
+    with torch.inference_mode():
+      return model(**inputs)
+  finally:
+    cnn.Fp8DynamicLinear.forward = old
+
+
+def test_small_flux_like_step_cosine_vs_oracle_ops():
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd.testing import dit_shapes as ds
+  torch.manual_seed(0)
+  kw = dict(dim=512, heads=4, mlp=2048, n_double=2, n_single=3, in_channels=64, text_dim=256,
+            pooled_dim=128)
+  model = ds.FluxLikeTransformer(**kw).to(torch.bfloat16).cuda()
+  bf16_model = copy.deepcopy(model)
+  cache_dit.quantize(model, cache_dit.QuantizeConfig())
+  inputs = ds.flux_like_inputs("cuda", n_img=320, n_txt=64, in_channels=64, text_dim=256,
+                               pooled_dim=128)
+  with torch.inference_mode():
+    y = model(**inputs)
+    y_bf16 = bf16_model(**inputs)
+  y_ref = _oracle_ops_forward(model, inputs, "cuda")
+  assert torch.isfinite(y.float()).all()
+  assert cosine(y, y_ref) >= 0.999, cosine(y, y_ref)
+  assert cosine(y, y_bf16) >= 0.99, cosine(y, y_bf16)
+  # fusing GELU into the epilogue keeps the output inside the same bar
+  n = ds.fuse_gelu_epilogues(model)
+  assert n == 2 * 2 + 3
+  with torch.inference_mode():
+    y_fused = model(**inputs)
+  assert cosine(y_fused, y_ref) >= 0.999
+
+
+def test_full_flux_shaped_step_cosine():
+  """BASELINE config 2 at full size (19 + 38 blocks, 4096 + 512 tokens): the HIP
+  path against the oracle's arithmetic in torch ops on the same GPU, and against
+  the unquantized bf16 model."""
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd.testing import dit_shapes as ds
+  torch.manual_seed(0)
+  with torch.device("cuda"):
+    model = ds.FluxLikeTransformer().to(torch.bfloat16)
+  inputs = ds.flux_like_inputs("cuda")
+  with torch.inference_mode():
+    y_bf16 = model(**inputs)
+  cache_dit.quantize(model, cache_dit.QuantizeConfig())
+  total, quantized = ds.count_linears(model)
+  assert quantized == 494
+  with torch.inference_mode():
+    y = model(**inputs)
+  y_ref = _oracle_ops_forward(model, inputs, "cuda")
+  c_ref, c_bf16 = cosine(y, y_ref), cosine(y, y_bf16)
+  print(f"full FLUX-shaped step: cosine vs oracle ops {c_ref:.6f}, vs bf16 {c_bf16:.6f}")
+  assert torch.isfinite(y.float()).all()
+  assert c_ref >= 0.999, c_ref
+  assert c_bf16 >= 0.99, c_bf16

@@ -1,0 +1,150 @@
+"""Pins the quantizer oracle: the plain-C restatement against the PyTorch-op
+restatement, both against closed forms, invariants, the committed golden vectors
+and the known answers of the BASELINE config-1 recipe."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import bits_u32, bits_u8, config1_inputs
+from oracle import c_oracle
+from oracle import torch_oracle as to
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+MODES = {"bf16div": 0, "fp32div": 1}
+
+
+def _u16(t):
+  return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+def test_c_and_torch_restatements_agree(mode):
+  g = torch.Generator().manual_seed(0)
+  x = torch.randn(300, 768, generator=g) * torch.logspace(-30, 30, 300).reshape(-1, 1)
+  x[::7, 5] *= 50
+  x[3] = 0
+  x = x.to(torch.bfloat16)
+  q, s = to.quantize_rowwise(x, mode)
+  qc, sc = c_oracle.quant_rowwise(_u16(x), MODES[mode])
+  assert (bits_u8(q) == qc).all()
+  assert (bits_u32(s.reshape(-1)) == sc.view(np.uint32)).all()
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+def test_golden_vectors(mode):
+  z = np.load(os.path.join(GOLD, "quant_vectors.npz"))
+  x = torch.from_numpy(z["x"].view(np.int16)).view(torch.bfloat16)
+  q, s = to.quantize_rowwise(x, mode)
+  assert (bits_u8(q) == z[f"q_{mode}"]).all()
+  assert (s.reshape(-1).numpy().view(np.uint32) == z[f"s_{mode}"].view(np.uint32)).all()
+  qc, sc = c_oracle.quant_rowwise(z["x"], MODES[mode])
+  assert (qc == z[f"q_{mode}"]).all() and (sc.view(np.uint32) == z[f"s_{mode}"].view(np.uint32)).all()
+
+
+def test_scale_closed_forms():
+  L = c_oracle.lib()
+  one = 0x3F80  # bf16 1.0
+  # fp32div: exactly fl32(amax/448); bf16div: that, rounded to 8 significant bits
+  assert L.oracle_row_scale(one, 1) == np.float32(1.0) / np.float32(448.0)
+  s0 = L.oracle_row_scale(one, 0)
+  assert (np.float32(s0).view(np.uint32) & 0xFFFF) == 0
+  assert abs(s0 - 1 / 448) <= 2.0**-9 * (1 / 448)  # within half a bf16 ulp (relative 2^-9)
+  # amax = 448 * 2^k gives scale exactly 2^k in both modes
+  for k in (-20, 0, 7):
+    am = int(torch.tensor(448.0 * 2.0**k).to(torch.bfloat16).view(torch.int16)) & 0xFFFF
+    assert L.oracle_row_scale(am, 0) == L.oracle_row_scale(am, 1) == 2.0**k
+  assert L.oracle_row_scale(0, 0) == 1.0 and L.oracle_row_scale(0, 1) == 1.0  # zero row -> 1
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+def test_invariants(mode):
+  g = torch.Generator().manual_seed(2)
+  x = (torch.randn(64, 1024, generator=g) * 5).to(torch.bfloat16)
+  x[0] = 0
+  x[1, 1:] = 0  # single non-zero
+  q, s = to.quantize_rowwise(x, mode)
+  qb = q.view(torch.uint8)
+  assert float(s[0]) == 1.0 and int(qb[0].max()) == 0
+  top = (qb & 0x7F).amax(-1)
+  assert bool(((top[1:] == 0x7E) | (top[1:] == 0x7D)).all())  # amax element -> +-448 or one below
+  assert int(((qb & 0x7F) == 0x7F).sum()) == 0  # never NaN
+  # |dequant - x| <= half an e4m3 step at |x/s| (3 mantissa bits; subnormal step 2^-9),
+  # except where the clamp cut (|x/s| > 448 can only happen by the rounding of s)
+  y = x.float() / s
+  step = torch.exp2(torch.floor(torch.log2(y.abs().clamp_min(2.0**-6)))) / 8
+  inside = y.abs() <= 448
+  err = (q.float() - y).abs()
+  assert bool((err[inside] <= 0.5 * step[inside]).all())
+  # sign symmetry and power-of-two equivariance
+  q2, s2 = to.quantize_rowwise(-x, mode)
+  assert bool((q2.view(torch.uint8)[1:] == (qb[1:] ^ 0x80)).all()) and torch.equal(s2, s)
+  q3, s3 = to.quantize_rowwise((x.float() * 4).to(torch.bfloat16), mode)
+  assert torch.equal(q3.view(torch.uint8), qb) and torch.equal(s3[1:], s[1:] * 4)
+
+
+def test_config1_known_answers():
+  """Numbers of the BASELINE config-1 recipe (global seed 0): which channels are
+  outliers, the amax range, how the two scale modes differ, and how many codes a
+  reciprocal multiply would flip. A missing bf16 rounding of the scale, an fp32
+  instead of bf16 amax or a reciprocal in place of the division changes them."""
+  ka = json.load(open(os.path.join(GOLD, "survey_known_answers.json")))
+  assert ka["outlier_idx"] == [1586, 2987, 108] and ka["rows_scale_differs"] == 3978
+  assert ka["codes_differ"] == 227812 and ka["recip_mul_codes_differ_bf16div"] == 1284
+  assert ka["recip_mul_codes_differ_fp32div"] == 6382
+  torch.manual_seed(0)
+  x = torch.randn(1, 4608, 3072)
+  idx = torch.randperm(3072)[:3]
+  assert idx.tolist() == ka["outlier_idx"]
+  x[..., idx] *= 20
+  x = x.to(torch.bfloat16)
+  amax = x.abs().amax(-1).float()
+  assert float(amax.min()) == ka["amax_min"] and float(amax.max()) == ka["amax_max"]
+  qa, sa = to.quantize_rowwise(x, "bf16div")
+  qb, sb = to.quantize_rowwise(x, "fp32div")
+  assert int((sa != sb).sum()) == ka["rows_scale_differs"]
+  assert int((qa.view(torch.uint8) != qb.view(torch.uint8)).sum()) == ka["codes_differ"]
+  for q, s, key in ((qa, sa, "bf16div"), (qb, sb, "fp32div")):
+    rc = (x.float() * (1.0 / s)).clamp(-448, 448).to(torch.float8_e4m3fn)
+    assert int((rc.view(torch.uint8) != q.view(torch.uint8)).sum()) == ka[f"recip_mul_codes_differ_{key}"]
+  assert int(((qa.view(torch.uint8) & 0x7F).amax(-1) == 0x7E).sum()) == ka["rows_hitting_448"] == 4608
+  # the generator-local recipe the other tests use yields the same bits
+  x2, _, _ = config1_inputs()
+  assert torch.equal(x2, x)
+  # and the plain-C restatement agrees on a slice of it
+  qc, sc = c_oracle.quant_rowwise(_u16(x[0, :256]), 0)
+  assert (qc == bits_u8(qa[0, :256])).all() and (sc.view(np.uint32) == bits_u32(sa[0, :256].reshape(-1))).all()
+
+
+def test_brute_force_tiny():
+  """Pure-Python loop over a tiny input, written from the spec, vs both restatements."""
+  import math
+  vals = [0.0, -0.0, 1.0, -3.5, 0.0078125, 448.0, -1000.0, 1e-5, 7.0, 0.33]
+  x = torch.tensor([vals, [v * 0.001 for v in vals]], dtype=torch.float32).to(torch.bfloat16)
+  L = c_oracle.lib()
+  for mode, mid in MODES.items():
+    q, s = to.quantize_rowwise(x, mode)
+    for r in range(x.shape[0]):
+      row = [float(v) for v in x[r].float()]
+      amax = max(abs(v) for v in row)
+      sc = np.float32(amax) / np.float32(448.0)
+      if mode == "bf16div":
+        sc = np.float32(float(torch.tensor(float(sc)).to(torch.bfloat16)))
+      if sc == 0:
+        sc = np.float32(1.0)
+      assert np.float32(s[r, 0].item()) == sc
+      for k, v in enumerate(row):
+        y = np.float32(v) / sc
+        y = min(max(y, np.float32(-448.0)), np.float32(448.0))
+        assert int(q.view(torch.uint8)[r, k]) == L.oracle_e4m3_encode(float(y))
+
+
+def test_nan_and_inf_inputs_follow_torch():
+  x = torch.tensor([[1.0, float("nan"), 2.0], [1.0, float("inf"), -2.0]]).to(torch.bfloat16)
+  q, s = to.quantize_rowwise(x)
+  qc, sc = c_oracle.quant_rowwise(_u16(x), 0)
+  assert np.isnan(sc[0]) and np.isnan(float(s[0]))
+  assert ((qc[0] & 0x7F) == 0x7F).all() and ((bits_u8(q)[0] & 0x7F) == 0x7F).all()
+  assert np.isinf(sc[1]) and (qc[1] == bits_u8(q)[1]).all()
