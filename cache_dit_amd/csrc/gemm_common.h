@@ -24,8 +24,11 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   return u >> 16;
 }
 
+// two fp32 -> packed bf16 with the hardware converter (v_cvt_pk_bf16_f32, RNE).
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  const v2f v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf));
 }
 
 // tanh-approximated GELU, the formula of torch.nn.functional.gelu(approximate="tanh"):
@@ -67,71 +70,78 @@ __device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m,
 // Epilogue shared by the tiled kernels. The MFMAs were issued with the
 // operands swapped, so acc[i][j][4*gq+e] is out[m][n] with
 //   m = m0 + wm*WM + 32i + (lane&31),  n = n0 + wn*WN + 32j + 8*gq + 4*(lane>>5) + e:
-// four consecutive columns per lane. They are scaled, biased, optionally
-// GELU'd, packed to bf16 and stored 8 bytes at a time, or (EPI_LDS) transposed
-// through a per-wave LDS tile and stored 16 bytes per lane along rows.
-// a_scale may be null (weight-only mode): then it is 1.
+// four consecutive columns per lane. Per element: one multiply by a_scale[m], one
+// FMA with b_scale[n] and bias[n], optional GELU, hardware bf16 pack. With
+// EPI_LDS each 32-row block of the wave tile is transposed through a wave-private
+// LDS tile (32 rows x EPI_PITCH bytes at `et`; no workgroup barrier needed) so that
+// every lane stores 16 bytes along a row; otherwise lanes store their 8 bytes
+// directly. a_scale may be null (weight-only mode): then it is 1.
 template <class C>
 __device__ __forceinline__ void tile_epilogue(v16f (&acc)[C::TM][C::TN], const GemmArgs& g,
-                                              uint8_t* smem, int m0, int n0, int wm, int wn,
-                                              int lane, int wave) {
-  const int h = lane >> 5;
+                                              uint8_t* et, int m0, int n0, int wm, int wn,
+                                              int lane) {
+  const int h = lane >> 5, r = lane & 31;
   const bool gelu = (g.epilogue & CDIT_EPI_GELU_TANH) != 0;
-  float as[C::TM];
+  const int nw = n0 + wn * C::WN;  // first column of the wave tile
+  const int mw = m0 + wm * C::WM;
+  v4f bs[C::TN][4], bi[C::TN][4];
 #pragma unroll
-  for (int i = 0; i < C::TM; ++i) {
-    const int m = m0 + wm * C::WM + 32 * i + (lane & 31);
-    as[i] = (g.a_scale && m < g.M) ? g.a_scale[m] : 1.0f;
-  }
-  if constexpr (C::EPI_LDS) __syncthreads();  // all waves are done with the stage buffers
-  uint8_t* et = smem + wave * (C::WM * C::EPI_PITCH);
-#pragma unroll
-  for (int j = 0; j < C::TN; ++j) {
+  for (int j = 0; j < C::TN; ++j)
 #pragma unroll
     for (int gq = 0; gq < 4; ++gq) {
-      const int nl = 32 * j + 8 * gq + 4 * h;  // column inside the wave tile
-      const int n = n0 + wn * C::WN + nl;
-      float bs[4], bi[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const bool ok = n + e < g.N;
-        bs[e] = ok ? g.b_scale[n + e] : 0.0f;
-        bi[e] = (ok && g.bias) ? __uint_as_float((uint32_t)g.bias[n + e] << 16) : 0.0f;
+      const int n = nw + 32 * j + 8 * gq + 4 * h;  // N % 8 == 0: a group of 4 is all in or out
+      v4f s4 = {0.0f, 0.0f, 0.0f, 0.0f}, b4 = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (n < g.N) {
+        s4 = *reinterpret_cast<const v4f*>(g.b_scale + n);
+        if (g.bias) {
+          const uint2 bb = *reinterpret_cast<const uint2*>(g.bias + n);
+          b4[0] = __uint_as_float(bb.x << 16);
+          b4[1] = __uint_as_float(bb.x & 0xffff0000u);
+          b4[2] = __uint_as_float(bb.y << 16);
+          b4[3] = __uint_as_float(bb.y & 0xffff0000u);
+        }
       }
+      bs[j][gq] = s4;
+      bi[j][gq] = b4;
+    }
 #pragma unroll
-      for (int i = 0; i < C::TM; ++i) {
+  for (int i = 0; i < C::TM; ++i) {
+    const int m = mw + 32 * i + r;
+    const float as = g.a_scale ? (m < g.M ? g.a_scale[m] : 0.0f) : 1.0f;
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) {
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          v[e] = acc[i][j][4 * gq + e] * as[i] * bs[e] + bi[e];
+          v[e] = __fmaf_rn(acc[i][j][4 * gq + e] * as, bs[j][gq][e], bi[j][gq][e]);
           if (gelu) v[e] = gelu_tanh(v[e]);
         }
         uint2 pk;
         pk.x = pack_bf16x2(v[0], v[1]);
         pk.y = pack_bf16x2(v[2], v[3]);
-        const int ml = 32 * i + (lane & 31);  // row inside the wave tile
+        const int nl = 32 * j + 8 * gq + 4 * h;  // column inside the wave tile
         if constexpr (C::EPI_LDS) {
-          *reinterpret_cast<uint2*>(et + ml * C::EPI_PITCH + nl * 2) = pk;
+          *reinterpret_cast<uint2*>(et + r * C::EPI_PITCH + nl * 2) = pk;
         } else {
-          const int m = m0 + wm * C::WM + ml;
-          if (m < g.M && n < g.N)  // N % 8 == 0, so a group of 4 is all in or all out
-            *reinterpret_cast<uint2*>(g.out + (int64_t)m * g.ldo + n) = pk;
+          if (m < g.M && nw + nl < g.N)
+            *reinterpret_cast<uint2*>(g.out + (int64_t)m * g.ldo + nw + nl) = pk;
         }
       }
-    }
-  }
-  if constexpr (C::EPI_LDS) {
-    // Each wave re-reads its own tile row-wise: 16 bytes (8 columns) per lane.
-    constexpr int LANES_PER_ROW = C::WN / 8;
-    constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
-    const int cl = (lane % LANES_PER_ROW) * 8;
-    const int n = n0 + wn * C::WN + cl;
+    if constexpr (C::EPI_LDS) {
+      // read the 32 x WN block back row-wise, 16 bytes (8 columns) per lane
+      constexpr int CPR = C::WN / 8;         // 16-byte chunks per row
+      constexpr int PER_LANE = 32 * CPR / 64;  // chunks per lane
+      static_assert((32 * CPR) % 64 == 0, "wave tile width must be a multiple of 16");
 #pragma unroll
-    for (int r0 = 0; r0 < C::WM; r0 += ROWS_PER_PASS) {
-      const int ml = r0 + lane / LANES_PER_ROW;
-      const int m = m0 + wm * C::WM + ml;
-      const uint4 v = *reinterpret_cast<const uint4*>(et + ml * C::EPI_PITCH + cl * 2);
-      if (m < g.M && n < g.N) *reinterpret_cast<uint4*>(g.out + (int64_t)m * g.ldo + n) = v;
+      for (int t = 0; t < PER_LANE; ++t) {
+        const int q = t * 64 + lane;
+        const int row = q / CPR, cc = q % CPR;
+        const uint4 d = *reinterpret_cast<const uint4*>(et + row * C::EPI_PITCH + cc * 16);
+        const int mm = mw + 32 * i + row, nn = nw + cc * 8;
+        if (mm < g.M && nn < g.N) *reinterpret_cast<uint4*>(g.out + (int64_t)mm * g.ldo + nn) = d;
+      }
     }
   }
 }

@@ -16,9 +16,10 @@
 // 32-byte read of A.
 //
 // Tile: BM x BN outputs, BK = 64 elements per pipeline step: A panel rows are
-// 128 bytes (8 chunks, chunk c of row r at position c ^ (r&7)), B panel rows
-// are 64 bytes (4 chunks, chunk c of row r at position c ^ ((r>>1)&3), two
-// rows per 128-byte line), both conflict free for 16-byte accesses. Panels
+// 128 bytes (8 chunks, chunk c of row r at position c ^ ((r>>1)&7)), B panel
+// rows are 64 bytes (4 chunks, chunk c of row r at position c ^ ((r>>2)&3)):
+// with 64 LDS banks of 4 B and 16 lanes served per pass, both are conflict free
+// for the 16-byte operand reads. Panels
 // are staged with 128-bit LDS-DMA loads, double buffered.
 //
 // Replaces F.linear(x, W.dequantize(), bias) of the reference's
@@ -43,7 +44,7 @@ struct CfgW {
   static constexpr int A_BYTES = BM * A_ROW, B_BYTES = BN * B_ROW;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int EPI_PITCH = WN * 2 + 16;
-  static constexpr int EPI_BYTES = EPI_LDS ? WAVES * WM * EPI_PITCH : 0;
+  static constexpr int EPI_BYTES = EPI_LDS ? WAVES * 32 * EPI_PITCH : 0;
   static constexpr int LDS_BYTES = (2 * STAGE_BYTES > EPI_BYTES) ? 2 * STAGE_BYTES : EPI_BYTES;
   // LDS-DMA instructions per wave and stage (1 KiB each)
   static constexpr int A_DMA = A_BYTES / 1024 / WAVES, B_DMA = B_BYTES / 1024 / WAVES;
@@ -76,13 +77,13 @@ __global__ __launch_bounds__(C::THREADS) void gemm_w8a16_tiled(GemmArgs g, int t
 #pragma unroll
   for (int p = 0; p < C::A_DMA; ++p) {
     const int row = (wave * C::A_DMA + p) * 8 + (lane >> 3);
-    const int c = (lane & 7) ^ (row & 7);
+    const int c = (lane & 7) ^ ((row >> 1) & 7);
     a_off[p] = (uint32_t)min(row, rows_a - 1) * (uint32_t)(g.lda * 2) + c * 16;
   }
 #pragma unroll
   for (int p = 0; p < C::B_DMA; ++p) {
     const int row = (wave * C::B_DMA + p) * 16 + (lane >> 2);
-    const int c = (lane & 3) ^ ((row >> 1) & 3);
+    const int c = (lane & 3) ^ ((row >> 2) & 3);
     b_off[p] = (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
   }
 
@@ -94,9 +95,9 @@ __global__ __launch_bounds__(C::THREADS) void gemm_w8a16_tiled(GemmArgs g, int t
     const int ra_row = wm * C::WM + (lane & 31);
 #pragma unroll
     for (int e = 0; e < 2; ++e)
-      rd_a[kb][e] = ra_row * C::A_ROW + (((4 * kb + 2 * h + e) ^ (lane & 7)) << 4);
+      rd_a[kb][e] = ra_row * C::A_ROW + (((4 * kb + 2 * h + e) ^ ((lane >> 1) & 7)) << 4);
     const int rb_row = wn * C::WN + (lane & 31);
-    rd_b[kb] = C::A_BYTES + rb_row * C::B_ROW + (((2 * kb + h) ^ ((lane >> 1) & 3)) << 4);
+    rd_b[kb] = C::A_BYTES + rb_row * C::B_ROW + (((2 * kb + h) ^ ((lane >> 2) & 3)) << 4);
   }
 
   v16f acc[C::TM][C::TN];
@@ -169,7 +170,8 @@ __global__ __launch_bounds__(C::THREADS) void gemm_w8a16_tiled(GemmArgs g, int t
     compute(kt & 1);
   }
 
-  tile_epilogue<C>(acc, g, smem, m0, n0, wm, wn, lane, wave);
+  if constexpr (C::EPI_LDS) __syncthreads();  // all waves are done with the stage buffers
+  tile_epilogue<C>(acc, g, smem + wave * (32 * C::EPI_PITCH), m0, n0, wm, wn, lane);
 }
 
 // Any shape: one output element per thread, scalar decode + FMA.
