@@ -30,6 +30,7 @@ EXPORTS = (
     "cdit_fp8_quant_rowwise",
     "cdit_fp8_gemm_rowwise",
     "cdit_w8a16_gemm",
+    "cdit_fp8_linear_w8a8",
     "cdit_set_gemm_variant",
 )
 
@@ -56,6 +57,9 @@ def _bind(L: ctypes.CDLL) -> None:
   L.cdit_fp8_gemm_rowwise.restype = ci
   L.cdit_fp8_gemm_rowwise.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci,
                                       vp]
+  L.cdit_fp8_linear_w8a8.restype = ci
+  L.cdit_fp8_linear_w8a8.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci,
+                                     ci, vp]
   L.cdit_w8a16_gemm.restype = ci
   L.cdit_w8a16_gemm.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, vp]
 

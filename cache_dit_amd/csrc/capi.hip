@@ -186,6 +186,16 @@ int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale, const void* b_q
   return rc ? rc : after_launch(fn);
 }
 
+int cdit_fp8_linear_w8a8(const void* x_bf16, const void* w_q, const float* w_scale,
+                         const void* bias_bf16, void* out, void* q_ws, float* scale_ws, int64_t M,
+                         int64_t N, int64_t K, int64_t ld_x, int64_t ldw, int64_t ldo,
+                         int scale_mode, int epilogue, int out_dtype_id, void* stream) {
+  int rc = cdit_fp8_quant_rowwise(x_bf16, M, K, ld_x, q_ws, K, scale_ws, scale_mode, stream);
+  if (rc) return rc;
+  return cdit_fp8_gemm_rowwise(q_ws, scale_ws, w_q, w_scale, bias_bf16, out, M, N, K, K, ldw, ldo,
+                               epilogue, out_dtype_id, stream);
+}
+
 int cdit_w8a16_gemm(const void* x_bf16, const void* b_q, const float* b_scale,
                     const void* bias_bf16, void* out, int64_t M, int64_t N, int64_t K,
                     int64_t lda, int64_t ldb, int64_t ldo, int epilogue, int out_dtype_id,

@@ -228,20 +228,25 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_tiled(GemmArgs g, int til
 
 // ---------------------------------------------------------------------------
 // Ping-pong kernel: 8 waves as two groups of 4 (one wave of each group per SIMD).
-// K advances in 64-byte steps through STAGES LDS buffers filled by LDS-DMA three
-// steps ahead. Every wave alternates a memory slot (issue the DMA for step kt+3,
-// read its MFMA operands of step kt from LDS) and a compute slot (its MFMAs of
-// step kt); slots are separated by workgroup barriers and group 1 runs one slot
-// behind group 0, so on every SIMD one wave feeds the matrix core while the
-// other one moves data. Barriers are bare s_barrier with explicit s_waitcnt:
-// a fenced barrier would wait for all DMA in flight and drain the pipeline.
+// K advances in 64-byte steps through STAGES LDS buffers filled by LDS-DMA
+// STAGES-1 steps ahead. Every wave alternates a memory slot (issue the DMA for
+// step kt+STAGES-1, read its MFMA operands of step kt from LDS) and a compute
+// slot (its MFMAs of step kt); slots are separated by workgroup barriers and
+// group 1 runs one slot behind group 0, so on every SIMD one wave feeds the
+// matrix core while the other one moves data. Barriers are bare s_barrier with
+// explicit s_waitcnt: a fenced barrier would wait for all DMA in flight and
+// drain the pipeline.
 //
-// Panel rows are 64 B = 4 chunks; LDS has 64 banks x 4 B, a 16-byte access is
-// served 16 lanes at a time, so 16 consecutive rows (4 per 256-byte bank row)
-// must land on distinct bank quads: chunk c of row r sits at c ^ ((r>>2)&3).
+// Panel rows are 64 B = 4 chunks; LDS has 64 banks x 4 B and serves a 16-byte
+// access 16 lanes per pass, so chunk c of row r sits at c ^ ((r>>2)&3)
+// (measured conflict free).
+//
+// The 1 KiB DMA instructions of a step (A panel first, then B) are dealt to the
+// waves round-robin; when their number is not a multiple of 8 the first waves
+// issue one more than the others, and each wave counts its own (D) for s_waitcnt.
 template <int BM_, int BN_, int STAGES_, bool EPI_LDS_, int GROUP_M_, int DBG_ = 0>
 struct CfgPP {
-  static constexpr int DBG = DBG_;  // timing experiments only: 1 no DMA in loop, 2 no LDS reads, 4 no MFMA, 8 raise wave priority around the MFMAs, 16 clocks
+  static constexpr int DBG = DBG_;  // 16: record clocks into a_scale (timing experiments)
   static constexpr int BM = BM_, BN = BN_, STAGES = STAGES_, WGM = 2, WGN = 4;
   static constexpr bool EPI_LDS = EPI_LDS_;
   static constexpr int GROUP_M = GROUP_M_;
@@ -251,15 +256,16 @@ struct CfgPP {
   static constexpr int BKP = 64;
   static constexpr int A_BYTES = BM * BKP, B_BYTES = BN * BKP;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int A_DMA = A_BYTES / 1024 / WAVES, B_DMA = B_BYTES / 1024 / WAVES;
-  static constexpr int DMA_PER_STAGE = A_DMA + B_DMA;  // per wave
+  static constexpr int NA = A_BYTES / 1024, NB = B_BYTES / 1024, NT = NA + NB;  // DMA per step
+  static constexpr int DMAX = (NT + WAVES - 1) / WAVES;
   static constexpr int EPI_PITCH = WN * 2 + 16;
   static constexpr int EPI_BYTES = EPI_LDS ? WAVES * 32 * EPI_PITCH : 0;
   static constexpr int LDS_BYTES =
       (STAGES * STAGE_BYTES > EPI_BYTES) ? STAGES * STAGE_BYTES : EPI_BYTES;
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
-  static_assert(A_BYTES % (1024 * WAVES) == 0 && B_BYTES % (1024 * WAVES) == 0, "panel/waves");
-  static_assert(STAGES == 4, "the wait counts below assume a prefetch distance of 3");
+  static_assert(BM % 16 == 0 && BN % 16 == 0, "panels are filled 16 rows at a time");
+  static_assert(STAGES == 3 || STAGES == 4, "prefetch distance 2 or 3");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
 
 // s_waitcnt vmcnt(N) lgkmcnt(0) followed by a bare workgroup barrier. The memory
@@ -268,7 +274,83 @@ template <int VM>
 __device__ __forceinline__ void wait_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(VM) : "memory");
 }
+template <int VM>
+__device__ __forceinline__ void wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(VM) : "memory");
+}
 __device__ __forceinline__ void bare_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+// Main loop for a wave that issues D DMA instructions per step.
+template <class C, int D>
+__device__ __forceinline__ void pingpong_loop(v16f (&acc)[C::TM][C::TN], uint8_t* smem,
+                                              const uint8_t* __restrict__ A,
+                                              const uint8_t* __restrict__ B,
+                                              const uint32_t (&off)[C::DMAX], int KT, int wave,
+                                              int group, const uint32_t (&rd_a)[2],
+                                              const uint32_t (&rd_b)[2]) {
+  constexpr int BKP = C::BKP, PD = C::STAGES - 1;
+  auto fetch = [&](int kt) {
+    uint8_t* st = smem + (kt % C::STAGES) * C::STAGE_BYTES;
+#pragma unroll
+    for (int p = 0; p < D; ++p) {
+      const int id = wave + C::WAVES * p;  // A panel: ids [0, NA); B panel: [NA, NT)
+      const uint8_t* src = (id < C::NA ? A : B) + (int64_t)kt * BKP + off[p];
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(st + id * 1024),
+                                       16, 0, 0);
+    }
+  };
+  // prologue: PD steps in flight; step 0 must have landed before the first slot
+#pragma unroll
+  for (int s = 0; s < PD; ++s)
+    if (s < KT) fetch(s);
+  if (KT > PD - 1) {
+    wait_vm<(PD - 1) * D>();
+  } else if (PD == 3 && KT > 1) {
+    wait_vm<D>();
+  } else {
+    wait_vm<0>();
+  }
+  if (group == 1) bare_barrier();  // group 1 runs one slot behind
+
+  for (int kt = 0; kt < KT; ++kt) {
+    bare_barrier();  // ---- memory slot of this wave
+    if (kt + PD < KT) fetch(kt + PD);
+    const uint8_t* st = smem + (kt % C::STAGES) * C::STAGE_BYTES;
+    v8i af[C::TM], bf[C::TN];
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i) {
+      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_a[0] + i * 32 * BKP);
+      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_a[1] + i * 32 * BKP);
+      af[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_b[0] + j * 32 * BKP);
+      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_b[1] + j * 32 * BKP);
+      bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+    // step kt+1 of this wave has landed once only the later steps are in flight
+    const int later = min(kt + PD, KT - 1) - (kt + 1);  // steps issued after kt+1
+    if (later >= 2 && PD >= 3) {
+      wait_and_barrier<2 * D>();
+    } else if (later == 1) {
+      wait_and_barrier<D>();
+    } else {
+      wait_and_barrier<0>();
+    }
+    // ---- compute slot
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[i][j], 0, 0,
+                                                                    0, 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (group == 0) bare_barrier();
+}
 
 template <class C>
 __global__ __launch_bounds__(C::THREADS) void gemm_fp8_pingpong(GemmArgs g, int tiles_m,
@@ -281,7 +363,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_pingpong(GemmArgs g, int 
   constexpr int BKP = C::BKP;
 
   long long dbg_t0 = 0, dbg_r0 = 0;
-  if constexpr (C::DBG & 16) { dbg_t0 = clock64(); dbg_r0 = wall_clock64(); }
+  if constexpr (C::DBG & 16) {
+    dbg_t0 = clock64();
+    dbg_r0 = wall_clock64();
+  }
   int tm, tn;
   tile_of_block<C::GROUP_M>(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
   const int m0 = tm * C::BM, n0 = tn * C::BN;
@@ -289,21 +374,18 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_pingpong(GemmArgs g, int 
   const uint8_t* __restrict__ B = g.b + (int64_t)n0 * g.ldb;
   const int rows_a = g.M - m0, rows_b = g.N - n0;
 
-  // DMA map: instruction p of this wave fills 16 panel rows (1 KiB); lane l lands on
-  // row l/4, position l%4 and fetches the logical chunk the swizzle puts there.
-  uint32_t a_off[C::A_DMA], b_off[C::B_DMA];
+  // DMA map: instruction id fills 16 panel rows (1 KiB); lane l lands on row l/4,
+  // position l%4 and fetches the logical chunk the swizzle puts there.
+  uint32_t off[C::DMAX];
   const int drow = lane >> 2;
 #pragma unroll
-  for (int p = 0; p < C::A_DMA; ++p) {
-    const int row = (wave * C::A_DMA + p) * 16 + drow;
+  for (int p = 0; p < C::DMAX; ++p) {
+    const int id = wave + C::WAVES * p;
+    const bool is_a = id < C::NA;
+    const int row = (is_a ? id : id - C::NA) * 16 + drow;
     const int c = (lane & 3) ^ ((row >> 2) & 3);
-    a_off[p] = (uint32_t)min(row, rows_a - 1) * (uint32_t)g.lda + c * 16;
-  }
-#pragma unroll
-  for (int p = 0; p < C::B_DMA; ++p) {
-    const int row = (wave * C::B_DMA + p) * 16 + drow;
-    const int c = (lane & 3) ^ ((row >> 2) & 3);
-    b_off[p] = (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
+    off[p] = is_a ? (uint32_t)min(row, rows_a - 1) * (uint32_t)g.lda + c * 16
+                  : (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
   }
   // operand read map: row lane&31, K-half h: chunks 2h, 2h+1
   const int h = lane >> 5;
@@ -324,96 +406,34 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_pingpong(GemmArgs g, int 
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   const int KT = g.K / BKP;
-  auto fetch = [&](int kt) {
-    const uint8_t* Ak = A + (int64_t)kt * BKP;
-    const uint8_t* Bk = B + (int64_t)kt * BKP;
-    uint8_t* st = smem + (kt % C::STAGES) * C::STAGE_BYTES;
-#pragma unroll
-    for (int p = 0; p < C::A_DMA; ++p)
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(Ak + a_off[p]),
-          (__attribute__((address_space(3))) void*)(st + (wave * C::A_DMA + p) * 1024), 16, 0, 0);
-#pragma unroll
-    for (int p = 0; p < C::B_DMA; ++p)
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(Bk + b_off[p]),
-          (__attribute__((address_space(3))) void*)(st + C::A_BYTES +
-                                                    (wave * C::B_DMA + p) * 1024),
-          16, 0, 0);
-  };
-  constexpr int D = C::DMA_PER_STAGE;
-
-  // prologue: three steps in flight; step 0 must have landed before the first slot
-  fetch(0);
-  if (KT > 1) fetch(1);
-  if (KT > 2) fetch(2);
-  if (KT > 2) {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * D) : "memory");
-  } else if (KT > 1) {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D) : "memory");
+  if constexpr (C::NT % C::WAVES == 0) {
+    pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
   } else {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (wave < C::NT % C::WAVES) {
+      pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
+    } else {
+      pingpong_loop<C, C::DMAX - 1>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
+    }
   }
-  if (wm == 1) bare_barrier();  // group 1 runs one slot behind
 
-  for (int kt = 0; kt < KT; ++kt) {
-    bare_barrier();  // ---- memory slot of this wave
-    if (!(C::DBG & 1) && kt + 3 < KT) fetch(kt + 3);
-    const uint8_t* st = smem + (kt % C::STAGES) * C::STAGE_BYTES;
-    v8i af[C::TM], bf[C::TN];
-    if constexpr (C::DBG & 2) {
-      for (int i = 0; i < C::TM; ++i) for (int e = 0; e < 8; ++e) af[i][e] = lane + kt;
-      for (int j = 0; j < C::TN; ++j) for (int e = 0; e < 8; ++e) bf[j][e] = lane - kt;
-    } else {
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i) {
-      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_a[0] + i * 32 * BKP);
-      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_a[1] + i * 32 * BKP);
-      af[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-#pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
-      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_b[0] + j * 32 * BKP);
-      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_b[1] + j * 32 * BKP);
-      bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-    }
-    // step kt+1 of this wave has landed once at most the later steps are in flight
-    if (kt + 3 < KT) {
-      wait_and_barrier<2 * D>();
-    } else if (kt + 2 < KT) {
-      wait_and_barrier<D>();
-    } else {
-      wait_and_barrier<0>();
-    }
-    // ---- compute slot
-    __builtin_amdgcn_sched_barrier(0);
-    if (C::DBG & 8) __builtin_amdgcn_s_setprio(1);
-    if constexpr (C::DBG & 4) {
-      for (int i = 0; i < C::TM; ++i) for (int j = 0; j < C::TN; ++j) acc[i][j][0] += (float)(af[i][0] + bf[j][1] + af[i][7] + bf[j][6] + af[i][4] + bf[j][3]);
-    } else {
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-      for (int j = 0; j < C::TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[i][j], 0, 0,
-                                                                    0, 0, 0, 0);
-    }
-    if (C::DBG & 8) __builtin_amdgcn_s_setprio(0);
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  if (wm == 0) bare_barrier();
-
+  // All LDS operand reads and all DMA are complete here (the last slot barrier
+  // follows group 1's last reads), so the stage buffers can hold the epilogue tiles.
+  uint8_t* et = smem + wave * (32 * C::EPI_PITCH);
   if constexpr (C::DBG & 16) {
     long long t1 = clock64(), r1 = wall_clock64();
-    tile_epilogue<C>(acc, g, smem + wave * (32 * C::EPI_PITCH), m0, n0, wm, wn, lane);
+    tile_epilogue<C>(acc, g, et, m0, n0, wm, wn, lane);
     long long t2 = clock64(), r2 = wall_clock64();
     if (tid == 0 && blockIdx.x < 1024) {
       long long* d = reinterpret_cast<long long*>(const_cast<float*>(g.a_scale)) + blockIdx.x * 6;
-      d[0] = t1 - dbg_t0; d[1] = r1 - dbg_r0; d[2] = t2 - t1; d[3] = r2 - r1; d[4] = dbg_r0; d[5] = r2;
+      d[0] = t1 - dbg_t0;
+      d[1] = r1 - dbg_r0;
+      d[2] = t2 - t1;
+      d[3] = r2 - r1;
+      d[4] = dbg_r0;
+      d[5] = r2;
     }
   } else {
-    tile_epilogue<C>(acc, g, smem + wave * (32 * C::EPI_PITCH), m0, n0, wm, wn, lane);
+    tile_epilogue<C>(acc, g, et, m0, n0, wm, wn, lane);
   }
 }
 
@@ -493,15 +513,13 @@ typedef Cfg<256, 128, 2, 2, true, true, 8> V4;
 typedef Cfg<128, 256, 2, 2, true, true, 8> V5;
 typedef Cfg<128, 128, 2, 2, true, true, 8> V6;
 typedef Cfg<256, 256, 2, 4, true, true, 8> V7;  // 8 waves, 128x64 wave tiles
-typedef CfgPP<256, 256, 4, true, 8> V8;         // ping-pong, 4 stages of 64 B
+typedef CfgPP<256, 256, 4, true, 8> V8;   // ping-pong, 4 stages of 64 B
 typedef CfgPP<256, 256, 4, false, 8> V9;
-typedef CfgPP<256, 256, 4, true, 8, 1> D1;
-typedef CfgPP<256, 256, 4, true, 8, 2> D2;
-typedef CfgPP<256, 256, 4, true, 8, 3> D3;
-typedef CfgPP<256, 256, 4, true, 8, 4> D4;
-typedef CfgPP<256, 256, 4, true, 8, 8> D8;
-typedef CfgPP<256, 256, 4, true, 8, 6> D6;
-typedef CfgPP<256, 256, 4, true, 8, 24> D24;
+typedef CfgPP<192, 384, 4, true, 8> V10;  // 96x96 wave tiles
+typedef CfgPP<256, 256, 3, true, 8> V12;
+typedef CfgPP<256, 128, 4, true, 8> V13;  // 128x32 wave tiles
+typedef CfgPP<128, 256, 4, true, 8> V14;  // 64x64 wave tiles
+typedef CfgPP<256, 256, 4, true, 8, 16> D16;
 
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {
@@ -525,13 +543,11 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     case 7: return launch_tiled<V7>(g, stream);
     case 8: return launch_pingpong<V8>(g, stream);
     case 9: return launch_pingpong<V9>(g, stream);
-    case 21: return launch_pingpong<D1>(g, stream);
-    case 22: return launch_pingpong<D2>(g, stream);
-    case 23: return launch_pingpong<D3>(g, stream);
-    case 24: return launch_pingpong<D4>(g, stream);
-    case 28: return launch_pingpong<D8>(g, stream);
-    case 26: return launch_pingpong<D6>(g, stream);
-    case 30: return launch_pingpong<D24>(g, stream);
+    case 10: return launch_pingpong<V10>(g, stream);
+    case 12: return launch_pingpong<V12>(g, stream);
+    case 13: return launch_pingpong<V13>(g, stream);
+    case 14: return launch_pingpong<V14>(g, stream);
+    case 30: return launch_pingpong<D16>(g, stream);
     default:
       set_error("cdit_fp8_gemm_rowwise: unknown kernel variant %d", variant);
       return CDIT_EINVAL;

@@ -76,13 +76,11 @@ class Fp8DynamicLinear(_Fp8LinearBase):
   def forward(self, x: torch.Tensor) -> torch.Tensor:
     x2 = self._check_input(x)
     M = x2.shape[0]
-    dev = x2.device
-    q = torch.empty((M, self.in_features), dtype=FP8, device=dev)
-    s = torch.empty((M, ), dtype=torch.float32, device=dev)
-    out = torch.empty((M, self.out_features), dtype=torch.bfloat16, device=dev)
+    out = torch.empty((M, self.out_features), dtype=torch.bfloat16, device=x2.device)
     if M > 0:
-      ops.quant_rowwise_into(x2, q, s, _native.SCALE_MODE_IDS[self.scale_mode])
-      ops.gemm_rowwise_into(q, s, self.weight, self.weight_scale, self.bias, out, self.epilogue)
+      q, s = ops.activation_workspace(M, self.in_features, x2.device)
+      ops.linear_w8a8_into(x2, self.weight, self.weight_scale, self.bias, out, q, s,
+                           self._scale_mode_id, self.epilogue)
     return out.view(*x.shape[:-1], self.out_features)
 
 
@@ -133,6 +131,7 @@ def convert_linear_(linear: nn.Linear,
     linear.bias = nn.Parameter(bias.detach().contiguous(), requires_grad=False)
   linear.epilogue = _native.EPI_GELU_TANH if gelu_tanh else _native.EPI_NONE
   linear.scale_mode = scale_mode
+  linear._scale_mode_id = _native.SCALE_MODE_IDS[scale_mode]
   linear.quant_type = quant_type
   linear.__class__ = cls
   return linear

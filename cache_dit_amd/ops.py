@@ -41,7 +41,48 @@ def decode_output_dtype(dtype_id: int) -> torch.dtype:
 
 
 def _stream_ptr(t: torch.Tensor) -> int:
-  return torch.cuda.current_stream(t.device).cuda_stream
+  return torch._C._cuda_getCurrentRawStream(t.device.index)
+
+
+class _DeviceOf:
+  """Makes `t`'s device current for the launch when it is not already (the kernels
+  run on the current HIP device); free when it is."""
+  __slots__ = ("guard", )
+
+  def __init__(self, t: torch.Tensor):
+    self.guard = None if t.device.index == torch.cuda.current_device() else torch.cuda.device(
+        t.device)
+
+  def __enter__(self):
+    if self.guard is not None:
+      self.guard.__enter__()
+
+  def __exit__(self, *exc):
+    if self.guard is not None:
+      self.guard.__exit__(*exc)
+
+
+_workspaces: dict = {}
+
+
+def activation_workspace(M: int, K: int, device: torch.device):
+  """(codes [M,K] e4m3, scales [M] fp32) scratch for one Linear forward. Outside
+  graph capture one growable buffer per (device, stream) is reused: every use is
+  ordered on that stream, so the GEMM that consumes it has been enqueued before
+  the next quantizer overwrites it. During capture fresh tensors come from the
+  graph's own pool."""
+  if torch.cuda.is_current_stream_capturing():
+    return (torch.empty((M, K), dtype=FP8, device=device),
+            torch.empty((M, ), dtype=torch.float32, device=device))
+  key = (device.index, torch._C._cuda_getCurrentRawStream(device.index))
+  ws = _workspaces.get(key)
+  if ws is None or ws[0].numel() < M * K or ws[1].numel() < M:
+    nq = max(M * K, ws[0].numel() if ws else 0)
+    ns = max(M, ws[1].numel() if ws else 0)
+    ws = (torch.empty(nq, dtype=FP8, device=device), torch.empty(ns, dtype=torch.float32,
+                                                                device=device))
+    _workspaces[key] = ws
+  return ws[0][:M * K].view(M, K), ws[1][:M]
 
 
 def _require_cuda(name: str, *tensors: Optional[torch.Tensor]) -> None:
@@ -58,7 +99,7 @@ def _require_cuda(name: str, *tensors: Optional[torch.Tensor]) -> None:
 def quant_rowwise_into(x2: torch.Tensor, q: torch.Tensor, scale: torch.Tensor,
                        scale_mode_id: int) -> None:
   M, K = x2.shape
-  with torch.cuda.device(x2.device):
+  with _DeviceOf(x2):
     _native.check(_native.load().cdit_fp8_quant_rowwise(x2.data_ptr(), M, K, x2.stride(0),
                                                         q.data_ptr(), q.stride(0),
                                                         scale.data_ptr(), scale_mode_id,
@@ -71,7 +112,7 @@ def gemm_rowwise_into(a: torch.Tensor, a_scale: torch.Tensor, w: torch.Tensor,
   """a [M,K] e4m3, w [N,K] e4m3 (row-major), scales fp32 contiguous, out [M,N] bf16."""
   M, K = a.shape
   N = w.shape[0]
-  with torch.cuda.device(a.device):
+  with _DeviceOf(a):
     _native.check(_native.load().cdit_fp8_gemm_rowwise(
         a.data_ptr(), a_scale.data_ptr(), w.data_ptr(), w_scale.data_ptr(),
         bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, K, a.stride(0),
@@ -82,11 +123,27 @@ def w8a16_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
                bias: Optional[torch.Tensor], out: torch.Tensor, epilogue: int) -> None:
   M, K = x2.shape
   N = w.shape[0]
-  with torch.cuda.device(x2.device):
+  with _DeviceOf(x2):
     _native.check(_native.load().cdit_w8a16_gemm(
         x2.data_ptr(), w.data_ptr(), w_scale.data_ptr(),
         bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, K, x2.stride(0),
         w.stride(0), out.stride(0), epilogue, _native.DT_BF16, _stream_ptr(x2)))
+
+
+def linear_w8a8_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
+                     bias: Optional[torch.Tensor], out: torch.Tensor, q_ws: torch.Tensor,
+                     s_ws: torch.Tensor, scale_mode_id: int, epilogue: int) -> None:
+  """Quantizer + GEMM of one Linear forward in a single library call."""
+  M, K = x2.shape
+  N = w.shape[0]
+  with _DeviceOf(x2):
+    rc = _native.load().cdit_fp8_linear_w8a8(
+        x2.data_ptr(), w.data_ptr(), w_scale.data_ptr(),
+        bias.data_ptr() if bias is not None else None, out.data_ptr(), q_ws.data_ptr(),
+        s_ws.data_ptr(), M, N, K, x2.stride(0), w.stride(0), out.stride(0), scale_mode_id,
+        epilogue, _native.DT_BF16, _stream_ptr(x2))
+  if rc:
+    _native.check(rc)
 
 
 # --------------------------------------------------------------------------- op definitions

@@ -131,6 +131,25 @@ int cdit_w8a16_gemm(const void* x_bf16, const void* b_q, const float* b_scale,
                     int epilogue, int out_dtype_id, void* stream);
 
 /*
+ * One quantized nn.Linear forward in the w8a8 dynamic mode: the two calls above
+ * back to back on `stream` (per-token quantization of x into the caller's
+ * workspace, then the scaled GEMM), saving one trip through the caller's FFI.
+ * This is what torchao's Float8Tensor `aten.linear` override does for a Linear
+ * that cache-dit converted with `quantize_(..., Float8DynamicActivation
+ * Float8WeightConfig(granularity=(PerRow(), PerRow())))`
+ * (src/cache_dit/quantization/torchao/quantize_ao.py:166-179, :540-558).
+ *
+ * x_bf16 [M,K] (ld_x); w_q e4m3 [N,K] (ldw); w_scale fp32 [N]; bias bf16 [N] or
+ * NULL; out bf16 [M,N] (ldo); q_ws: workspace of M*K bytes (receives the
+ * activation codes, contiguous); scale_ws: workspace of M floats.
+ */
+int cdit_fp8_linear_w8a8(const void* x_bf16, const void* w_q, const float* w_scale,
+                         const void* bias_bf16, void* out, void* q_ws, float* scale_ws,
+                         int64_t M, int64_t N, int64_t K,
+                         int64_t ld_x, int64_t ldw, int64_t ldo,
+                         int scale_mode, int epilogue, int out_dtype_id, void* stream);
+
+/*
  * Tuning hook used by the benchmark and the tests: forces the kernel variant
  * the two GEMM entry points pick (-1 = automatic choice by shape). Returns
  * the previous value. Process-global; not meant for concurrent use.
