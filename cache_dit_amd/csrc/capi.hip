@@ -121,6 +121,10 @@ int cdit_device_arch(char* buf, int buf_len) {
 }
 
 int cdit_set_gemm_variant(int variant) {
+  if (variant >= 1000) {  // 1000 + v selects the quantizer kernel variant instead
+    cdit::g_quant_variant = variant - 1000;
+    return g_gemm_variant;
+  }
   int prev = g_gemm_variant;
   g_gemm_variant = variant;
   return prev;

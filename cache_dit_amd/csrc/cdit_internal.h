@@ -14,6 +14,8 @@ namespace cdit {
 int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void* q,
                          int64_t ld_q, float* scale, int scale_mode, hipStream_t stream);
 
+extern int g_quant_variant;
+
 struct GemmArgs {
   const void* a;         // fp8 [M,K] (w8a8) or bf16 [M,K] (w8a16)
   const float* a_scale;  // [M] (w8a8) or nullptr (w8a16)

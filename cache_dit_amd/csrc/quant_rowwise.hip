@@ -2,8 +2,9 @@
 //
 // One 64-lane wavefront owns one row: it reads the row once from HBM with
 // 128-bit loads and keeps it in VGPRs, reduces |x| to the row amax with a
-// cross-lane max, derives the scale, then divides, clamps, converts with the
-// hardware e4m3 converter (v_cvt_pk_fp8_f32, RNE) and writes 64-bit packs.
+// cross-lane max, derives the scale, then divides, converts with the hardware
+// e4m3 converter (v_cvt_pk_fp8_f32, RNE) and writes 64-bit packs. Loads and
+// stores carry the nontemporal hint: every byte is touched once.
 // Algorithmic traffic is 2 B read + 1 B written per element + 4 B per row.
 //
 // Arithmetic follows torchao's _choose_scale_float8 / _quantize_affine_float8
@@ -40,14 +41,30 @@ __device__ __forceinline__ float round_to_bf16(float f) {
   return __uint_as_float(u & 0xffff0000u);
 }
 
-// max over the wavefront of an unsigned value (order independent, exact).
+// max over the wavefront of an unsigned value (order independent, exact). Four
+// DPP steps reduce each row of 16 lanes (xor 1, xor 2, half mirror, mirror), then
+// the four row results are read into scalars.
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    uint32_t o = (uint32_t)__shfl_xor((int)v, off, 64);
-    v = v > o ? v : o;
-  }
-  return v;
+  auto step = [](uint32_t a, int ctrl_id) {
+    uint32_t o;
+    switch (ctrl_id) {
+      case 0: o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)a, 0xB1, 0xf, 0xf, false); break;
+      case 1: o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)a, 0x4E, 0xf, 0xf, false); break;
+      case 2: o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)a, 0x141, 0xf, 0xf, false); break;
+      default: o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)a, 0x140, 0xf, 0xf, false); break;
+    }
+    return a > o ? a : o;
+  };
+  v = step(v, 0);  // quad_perm [1,0,3,2]
+  v = step(v, 1);  // quad_perm [2,3,0,1]
+  v = step(v, 2);  // row_half_mirror
+  v = step(v, 3);  // row_mirror
+  const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0);
+  const uint32_t b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+  const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32);
+  const uint32_t d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+  const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+  return ab > cd ? ab : cd;
 }
 
 __device__ __forceinline__ float row_scale(uint32_t amax_bits, int scale_mode) {
@@ -81,13 +98,22 @@ __device__ __forceinline__ bool scale_in_fast_window(float s) {
   return e >= 27u && e <= 227u;
 }
 
-// two bf16 pairs (4 elements) -> 4 e4m3 bytes
+// two bf16 pairs (4 elements) -> 4 e4m3 bytes. On the fast path the clamp is
+// implicit: |x| <= amax and scale >= amax/448 * (1 - 2^-9), so |x/scale| < 450,
+// below the tie at 464 where the e4m3 conversion would stop rounding to 448
+// (tests/native/divcheck.c checks the unclamped quotient of every input pair).
 template <bool FAST>
 __device__ __forceinline__ uint32_t quant4(uint32_t w0, uint32_t w1, float s, float r) {
-  float a = clamp448(div_scale<FAST>(bf16_lo(w0), s, r));
-  float b = clamp448(div_scale<FAST>(bf16_hi(w0), s, r));
-  float c = clamp448(div_scale<FAST>(bf16_lo(w1), s, r));
-  float d = clamp448(div_scale<FAST>(bf16_hi(w1), s, r));
+  float a = div_scale<FAST>(bf16_lo(w0), s, r);
+  float b = div_scale<FAST>(bf16_hi(w0), s, r);
+  float c = div_scale<FAST>(bf16_lo(w1), s, r);
+  float d = div_scale<FAST>(bf16_hi(w1), s, r);
+  if constexpr (!FAST) {
+    a = clamp448(a);
+    b = clamp448(b);
+    c = clamp448(c);
+    d = clamp448(d);
+  }
   uint32_t p = 0;
   p = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, p, false);
   p = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, p, true);
@@ -104,8 +130,8 @@ __device__ __forceinline__ uint32_t absmax2(uint32_t m, uint32_t w) {
 }
 
 // Row resident in registers: CH 16-byte chunks per lane (K <= CH*512).
-template <int CH>
-__global__ __launch_bounds__(256) void quant_rowwise_regs(
+template <int CH, bool NT = false>
+__global__ __launch_bounds__(64) void quant_rowwise_regs(
     const uint16_t* __restrict__ x, int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q,
     float* __restrict__ scale, int M, int K, int scale_mode) {
   const int lane = threadIdx.x & 63;
@@ -119,7 +145,17 @@ __global__ __launch_bounds__(256) void quant_rowwise_regs(
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       const int idx = c * 64 + lane;
-      v[c] = idx < nchunks ? xr[idx] : make_uint4(0, 0, 0, 0);
+      if (idx < nchunks) {
+        if constexpr (NT) {
+          typedef unsigned int u4v __attribute__((ext_vector_type(4)));
+          const u4v t = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(xr + idx));
+          v[c] = make_uint4(t[0], t[1], t[2], t[3]);
+        } else {
+          v[c] = xr[idx];
+        }
+      } else {
+        v[c] = make_uint4(0, 0, 0, 0);
+      }
     }
     uint32_t m = 0;
 #pragma unroll
@@ -142,7 +178,13 @@ __global__ __launch_bounds__(256) void quant_rowwise_regs(
           uint2 o;
           o.x = quant4<true>(v[c].x, v[c].y, s, r);
           o.y = quant4<true>(v[c].z, v[c].w, s, r);
-          qr[idx] = o;
+          if constexpr (NT) {
+            typedef unsigned int u2v __attribute__((ext_vector_type(2)));
+            const u2v t = {o.x, o.y};
+            __builtin_nontemporal_store(t, reinterpret_cast<u2v*>(qr + idx));
+          } else {
+            qr[idx] = o;
+          }
         }
       }
     } else {
@@ -161,7 +203,7 @@ __global__ __launch_bounds__(256) void quant_rowwise_regs(
 
 // Any K, any alignment: one wavefront per row, two passes over the row with
 // element-wise loads (the second pass hits L2). Slow path for odd shapes.
-__global__ __launch_bounds__(256) void quant_rowwise_generic(
+__global__ __launch_bounds__(64) void quant_rowwise_generic(
     const uint16_t* __restrict__ x, int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q,
     float* __restrict__ scale, int M, int K, int scale_mode) {
   const int lane = threadIdx.x & 63;
@@ -189,6 +231,8 @@ __global__ __launch_bounds__(256) void quant_rowwise_generic(
 
 }  // namespace
 
+int g_quant_variant = 0;  // 0: streaming (nontemporal) loads and stores, 1: plain
+
 int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void* q,
                          int64_t ld_q, float* scale, int scale_mode, hipStream_t stream) {
   const uint16_t* xp = static_cast<const uint16_t*>(x);
@@ -196,19 +240,25 @@ int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void
   const bool aligned = (K % 8 == 0) && (ld_x % 8 == 0) && (ld_q % 8 == 0) &&
                        (reinterpret_cast<uintptr_t>(x) % 16 == 0) &&
                        (reinterpret_cast<uintptr_t>(q) % 8 == 0);
-  constexpr int kThreads = 256, kWaves = kThreads / 64;
+  // one wavefront per workgroup: rows spread evenly over the CUs whatever M is
+  constexpr int kThreads = 64, kWaves = kThreads / 64;
   int64_t blocks = (M + kWaves - 1) / kWaves;
   // enough blocks to cover the chip many times over; rows beyond that are
   // picked up by the grid-stride loop.
-  const int64_t kMaxBlocks = 256 * 64;
+  const int64_t kMaxBlocks = 256 * 256;
   if (blocks > kMaxBlocks) blocks = kMaxBlocks;
   dim3 grid((unsigned)blocks), block(kThreads);
   const int Mi = (int)M, Ki = (int)K;
   const int need = (int)((K + 511) / 512);  // 16-byte chunks per lane
 #define CDIT_QUANT_CASE(CH)                                                                 \
   if (aligned && need <= CH) {                                                              \
-    hipLaunchKernelGGL(quant_rowwise_regs<CH>, grid, block, 0, stream, xp, ld_x, qp, ld_q,  \
-                       scale, Mi, Ki, scale_mode);                                          \
+    if (g_quant_variant == 0) {                                                             \
+      hipLaunchKernelGGL((quant_rowwise_regs<CH, true>), grid, block, 0, stream, xp, ld_x,  \
+                         qp, ld_q, scale, Mi, Ki, scale_mode);                              \
+    } else {                                                                                \
+      hipLaunchKernelGGL((quant_rowwise_regs<CH, false>), grid, block, 0, stream, xp, ld_x, \
+                         qp, ld_q, scale, Mi, Ki, scale_mode);                              \
+    }                                                                                       \
     return 0;                                                                               \
   }
   CDIT_QUANT_CASE(1)
