@@ -142,7 +142,11 @@ def headline_kernels(device):
     ops.quant_rowwise_into(xs[i], qs[i], ss[i], 0)
   it = {"i": 0}
 
-  def gemm():
+  def gemm():  # scales + bias epilogue: what quantize() installs by default
+    i = it["i"] = (it["i"] + 1) % nbuf
+    ops.gemm_rowwise_into(qs[i], ss[i], ws[i], wsc, b, outs[i & 1], 0)
+
+  def gemm_gelu():  # with the optional GELU-tanh folded in (fuse_gelu_tanh_)
     i = it["i"] = (it["i"] + 1) % nbuf
     ops.gemm_rowwise_into(qs[i], ss[i], ws[i], wsc, b, outs[i & 1], 1)
 
@@ -150,12 +154,16 @@ def headline_kernels(device):
     i = it["i"] = (it["i"] + 1) % nbuf
     ops.quant_rowwise_into(xs[i], qs[i], ss[i], 0)
 
-  gemm_ms = _time_events(gemm, 50, 10)
+  _time_events(gemm, 100, 100)  # bring the clocks to their steady state first
+  gemm_ms = _time_events(gemm, 100, 10)
+  gemm_gelu_ms = _time_events(gemm_gelu, 100, 10)
   quant_ms = _time_events(quant, 200, 20)
   res = {
       "shape": {"M": M, "K": K, "N": N},
       "gemm_ms": gemm_ms,
       "gemm_tflops": 2.0 * M * K * N / gemm_ms / 1e9,
+      "gemm_gelu_ms": gemm_gelu_ms,
+      "gemm_gelu_tflops": 2.0 * M * K * N / gemm_gelu_ms / 1e9,
       "quant_ms": quant_ms,
       "quant_gbps": (3.0 * M * K + 4.0 * M) / quant_ms / 1e6,
   }
@@ -312,7 +320,8 @@ def main():
   head = headline_kernels(device)
   M, K, N = HEADLINE
   roofline = {
-      "kernel": "gemm_fp8_tiled (w8a8 GEMM + epilogue) at M=4608 K=3072 N=12288",
+      "kernel": "gemm_fp8_pingpong<192x384> (w8a8 GEMM + scale/bias epilogue) at M=4608 K=3072 "
+                "N=12288",
       "bound": "mfma",
       "achieved": head["gemm_tflops"],
       "peak": FP8_PEAK_TFLOPS,

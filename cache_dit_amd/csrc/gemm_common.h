@@ -46,6 +46,50 @@ __device__ __forceinline__ float gelu_tanh(float v) {
   return v * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
+// s_waitcnt vmcnt(N) lgkmcnt(0) followed by a bare workgroup barrier. The memory
+// clobber keeps the compiler from moving LDS accesses across it.
+template <int VM>
+__device__ __forceinline__ void wait_and_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(VM) : "memory");
+}
+template <int VM>
+__device__ __forceinline__ void wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(VM) : "memory");
+}
+__device__ __forceinline__ void bare_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+// Waits until at most `later` steps (of D DMA instructions each) are in flight,
+// `later` in [0, MAXL]; the count has to be an immediate, hence the switch.
+template <int D, int MAXL, bool BARRIER>
+__device__ __forceinline__ void wait_steps(int later) {
+#define CDIT_WAIT_CASE(L)                                 \
+  case L:                                                 \
+    if constexpr (L <= MAXL) {                            \
+      if constexpr (BARRIER) {                            \
+        wait_and_barrier<(L * D > 63 ? 63 : L * D)>();    \
+      } else {                                            \
+        wait_vm<(L * D > 63 ? 63 : L * D)>();             \
+      }                                                   \
+    }                                                     \
+    break;
+  switch (later) {
+    CDIT_WAIT_CASE(0)
+    CDIT_WAIT_CASE(1)
+    CDIT_WAIT_CASE(2)
+    CDIT_WAIT_CASE(3)
+    CDIT_WAIT_CASE(4)
+    CDIT_WAIT_CASE(5)
+    CDIT_WAIT_CASE(6)
+    default:
+      if constexpr (BARRIER) {
+        wait_and_barrier<0>();
+      } else {
+        wait_vm<0>();
+      }
+  }
+#undef CDIT_WAIT_CASE
+}
+
 // Workgroup id -> output tile. Workgroups are handed to the 8 XCDs round-robin
 // and each XCD has its own L2, so ids that land on one XCD are first made
 // consecutive, then walked in column-major order inside groups of GROUP_M tile

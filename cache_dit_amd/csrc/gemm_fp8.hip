@@ -33,8 +33,10 @@ namespace {
 
 constexpr int BK = 128;  // bytes of K per pipeline step (two 64-wide MFMA steps)
 
-template <int BM_, int BN_, int WGM_, int WGN_, bool DIRECT_, bool EPI_LDS_, int GROUP_M_>
+template <int BM_, int BN_, int WGM_, int WGN_, bool DIRECT_, bool EPI_LDS_, int GROUP_M_,
+          int STAGES_ = 2>
 struct Cfg {
+  static constexpr int STAGES = STAGES_;  // LDS buffers; more than 2 needs DIRECT staging
   static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
   static constexpr bool DIRECT = DIRECT_, EPI_LDS = EPI_LDS_;
   static constexpr int GROUP_M = GROUP_M_;
@@ -46,7 +48,10 @@ struct Cfg {
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int EPI_PITCH = WN * 2 + 16;  // bytes per row of the per-wave transpose tile
   static constexpr int EPI_BYTES = EPI_LDS ? WAVES * 32 * EPI_PITCH : 0;
-  static constexpr int LDS_BYTES = (2 * STAGE_BYTES > EPI_BYTES) ? 2 * STAGE_BYTES : EPI_BYTES;
+  static constexpr int LDS_BYTES =
+      (STAGES * STAGE_BYTES > EPI_BYTES) ? STAGES * STAGE_BYTES : EPI_BYTES;
+  static_assert(STAGES == 2 || DIRECT, "multi-stage needs LDS-DMA staging");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
   // staging: 16-byte chunks per thread and per wave instruction
   static constexpr int A_CHUNKS = BM * 8 / THREADS, B_CHUNKS = BN * 8 / THREADS;
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
@@ -200,7 +205,22 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_tiled(GemmArgs g, int til
   };
 
   // ---- main loop ----------------------------------------------------------
-  if constexpr (C::DIRECT) {
+  if constexpr (C::DIRECT && C::STAGES > 2) {
+    // STAGES-1 steps in flight; bare barriers with explicit vmcnt so that the
+    // younger DMA keeps flying across them.
+    constexpr int PD = C::STAGES - 1, D = C::A_CHUNKS + C::B_CHUNKS;
+#pragma unroll
+    for (int s = 0; s < PD; ++s)
+      if (s < KT) fetch(s, s);
+    wait_steps<D, PD - 1, true>(min(PD, KT) - 1);
+    for (int kt = 0; kt < KT; ++kt) {
+      // stage (kt+PD)%STAGES was read in iteration kt-1; the barrier that ended it
+      // makes it free
+      if (kt + PD < KT) fetch(kt + PD, (kt + PD) % C::STAGES);
+      compute(kt % C::STAGES);
+      wait_steps<D, PD - 1, true>(max(min(kt + PD, KT - 1) - (kt + 1), 0));
+    }
+  } else if constexpr (C::DIRECT) {
     fetch(0, 0);
     for (int kt = 0; kt < KT; ++kt) {
       // tile kt has landed (this wave's part), then everyone's part; all waves
@@ -244,13 +264,17 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_tiled(GemmArgs g, int til
 // The 1 KiB DMA instructions of a step (A panel first, then B) are dealt to the
 // waves round-robin; when their number is not a multiple of 8 the first waves
 // issue one more than the others, and each wave counts its own (D) for s_waitcnt.
-template <int BM_, int BN_, int STAGES_, bool EPI_LDS_, int GROUP_M_, int DBG_ = 0>
+template <int BM_, int BN_, int STAGES_, bool EPI_LDS_, int GROUP_M_, int DBG_ = 0, int WAVES_ = 8>
 struct CfgPP {
   static constexpr int DBG = DBG_;  // 16: record clocks into a_scale (timing experiments)
-  static constexpr int BM = BM_, BN = BN_, STAGES = STAGES_, WGM = 2, WGN = 4;
+  // WAVES = 8: ping-pong (two groups of four). WAVES = 4: all waves in phase, one
+  // barrier per step; sized (<= 80 KiB LDS, <= 256 VGPRs) so that two such
+  // workgroups share a CU and fill each other's stalls and epilogues.
+  static constexpr bool PINGPONG = WAVES_ == 8;
+  static constexpr int BM = BM_, BN = BN_, STAGES = STAGES_, WGM = 2, WGN = WAVES_ / 2;
   static constexpr bool EPI_LDS = EPI_LDS_;
   static constexpr int GROUP_M = GROUP_M_;
-  static constexpr int WAVES = 8, THREADS = 512;
+  static constexpr int WAVES = WAVES_, THREADS = WAVES_ * 64;
   static constexpr int WM = BM / WGM, WN = BN / WGN;
   static constexpr int TM = WM / 32, TN = WN / 32;
   static constexpr int BKP = 64;
@@ -264,21 +288,9 @@ struct CfgPP {
       (STAGES * STAGE_BYTES > EPI_BYTES) ? STAGES * STAGE_BYTES : EPI_BYTES;
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
   static_assert(BM % 16 == 0 && BN % 16 == 0, "panels are filled 16 rows at a time");
-  static_assert(STAGES == 3 || STAGES == 4, "prefetch distance 2 or 3");
+  static_assert(STAGES >= 3 && STAGES <= 8, "prefetch distance 2..7");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
-
-// s_waitcnt vmcnt(N) lgkmcnt(0) followed by a bare workgroup barrier. The memory
-// clobber keeps the compiler from moving LDS accesses across it.
-template <int VM>
-__device__ __forceinline__ void wait_and_barrier() {
-  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(VM) : "memory");
-}
-template <int VM>
-__device__ __forceinline__ void wait_vm() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(VM) : "memory");
-}
-__device__ __forceinline__ void bare_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
 // Main loop for a wave that issues D DMA instructions per step.
 template <class C, int D>
@@ -304,13 +316,7 @@ __device__ __forceinline__ void pingpong_loop(v16f (&acc)[C::TM][C::TN], uint8_t
 #pragma unroll
   for (int s = 0; s < PD; ++s)
     if (s < KT) fetch(s);
-  if (KT > PD - 1) {
-    wait_vm<(PD - 1) * D>();
-  } else if (PD == 3 && KT > 1) {
-    wait_vm<D>();
-  } else {
-    wait_vm<0>();
-  }
+  wait_steps<D, PD - 1, false>(min(PD, KT) - 1);  // step 0 landed; the later ones may fly
   if (group == 1) bare_barrier();  // group 1 runs one slot behind
 
   for (int kt = 0; kt < KT; ++kt) {
@@ -332,13 +338,7 @@ __device__ __forceinline__ void pingpong_loop(v16f (&acc)[C::TM][C::TN], uint8_t
     }
     // step kt+1 of this wave has landed once only the later steps are in flight
     const int later = min(kt + PD, KT - 1) - (kt + 1);  // steps issued after kt+1
-    if (later >= 2 && PD >= 3) {
-      wait_and_barrier<2 * D>();
-    } else if (later == 1) {
-      wait_and_barrier<D>();
-    } else {
-      wait_and_barrier<0>();
-    }
+    wait_steps<D, PD - 1, true>(max(later, 0));
     // ---- compute slot
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -352,9 +352,66 @@ __device__ __forceinline__ void pingpong_loop(v16f (&acc)[C::TM][C::TN], uint8_t
   if (group == 0) bare_barrier();
 }
 
+// Main loop of the 4-wave flavour: all waves in phase, one barrier per step.
+template <class C, int D>
+__device__ __forceinline__ void inphase_loop(v16f (&acc)[C::TM][C::TN], uint8_t* smem,
+                                             const uint8_t* __restrict__ A,
+                                             const uint8_t* __restrict__ B,
+                                             const uint32_t (&off)[C::DMAX], int KT, int wave,
+                                             const uint32_t (&rd_a)[2],
+                                             const uint32_t (&rd_b)[2]) {
+  constexpr int BKP = C::BKP, PD = C::STAGES - 1;
+  auto fetch = [&](int kt) {
+    uint8_t* st = smem + (kt % C::STAGES) * C::STAGE_BYTES;
+#pragma unroll
+    for (int p = 0; p < D; ++p) {
+      const int id = wave + C::WAVES * p;
+      const uint8_t* src = (id < C::NA ? A : B) + (int64_t)kt * BKP + off[p];
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(st + id * 1024),
+                                       16, 0, 0);
+    }
+  };
+#pragma unroll
+  for (int s = 0; s < PD; ++s)
+    if (s < KT) fetch(s);
+  wait_steps<D, PD - 1, false>(min(PD, KT) - 1);
+  for (int kt = 0; kt < KT; ++kt) {
+    // everyone's part of step kt has landed and everyone has left compute(kt-1),
+    // whose stage the next DMA overwrites
+    bare_barrier();
+    if (kt + PD < KT) fetch(kt + PD);
+    const uint8_t* st = smem + (kt % C::STAGES) * C::STAGE_BYTES;
+    v8i af[C::TM], bf[C::TN];
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i) {
+      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_a[0] + i * 32 * BKP);
+      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_a[1] + i * 32 * BKP);
+      af[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_b[0] + j * 32 * BKP);
+      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_b[1] + j * 32 * BKP);
+      bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[i][j], 0, 0,
+                                                                    0, 0, 0, 0);
+    // own DMA of step kt+1 landed (LDS reads of this step too) before the next barrier
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    wait_steps<D, PD - 1, false>(max(min(kt + PD, KT - 1) - (kt + 1), 0));
+  }
+  bare_barrier();  // all operand reads done: the stage buffers may hold epilogue tiles
+}
+
+// Two waves per SIMD in both flavours (8 waves of one workgroup, or 4 + 4 of two).
 template <class C>
-__global__ __launch_bounds__(C::THREADS) void gemm_fp8_pingpong(GemmArgs g, int tiles_m,
-                                                                int tiles_n) {
+__global__ __launch_bounds__(C::THREADS, 2) void gemm_fp8_pingpong(GemmArgs g, int tiles_m,
+                                                                   int tiles_n) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -406,13 +463,25 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_pingpong(GemmArgs g, int 
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   const int KT = g.K / BKP;
-  if constexpr (C::NT % C::WAVES == 0) {
-    pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
-  } else {
-    if (wave < C::NT % C::WAVES) {
+  if constexpr (C::PINGPONG) {
+    if constexpr (C::NT % C::WAVES == 0) {
       pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
     } else {
-      pingpong_loop<C, C::DMAX - 1>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
+      if (wave < C::NT % C::WAVES) {
+        pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
+      } else {
+        pingpong_loop<C, C::DMAX - 1>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
+      }
+    }
+  } else {
+    if constexpr (C::NT % C::WAVES == 0) {
+      inphase_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, rd_a, rd_b);
+    } else {
+      if (wave < C::NT % C::WAVES) {
+        inphase_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, rd_a, rd_b);
+      } else {
+        inphase_loop<C, C::DMAX - 1>(acc, smem, A, B, off, KT, wave, rd_a, rd_b);
+      }
     }
   }
 
@@ -453,6 +522,79 @@ int launch_pingpong(const GemmArgs& g, hipStream_t stream) {
   hipLaunchKernelGGL(gemm_fp8_pingpong<C>, dim3(tiles_m * tiles_n), dim3(C::THREADS),
                      C::LDS_BYTES, stream, g, tiles_m, tiles_n);
   return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Skinny kernel for M <= 16 (the M = 1 modulation Linears `norm1.linear`,
+// `norm.linear` of every block): pure weight streaming. A workgroup of 4 waves
+// owns 16 output channels; each wave takes a quarter of K and reads its weight
+// rows straight from HBM into MFMA operand registers (lane = row l&15, 32-byte K
+// group l>>4; 16 x 128-byte segments per pair of loads), multiplies by the (zero
+// padded) activation rows with v_mfma_f32_16x16x128_f8f6f4, and the four partial
+// 16x16 tiles are summed through LDS before the epilogue. No LDS staging of the
+// weights: every weight byte is used exactly once.
+__global__ __launch_bounds__(256) void gemm_fp8_skinny(GemmArgs g) {
+  __shared__ float part[4][16][17];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, kg = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int nrow = min(n0 + r, g.N - 1);
+  const int KT = g.K / 128;           // 128-byte steps in total
+  const int per = (KT + 3) / 4;       // steps per wave
+  const int k_begin = wave * per, k_end = min(KT, k_begin + per);
+  const uint8_t* __restrict__ wp = g.b + (int64_t)nrow * g.ldb + kg * 32;
+  const uint8_t* __restrict__ ap =
+      static_cast<const uint8_t*>(g.a) + (int64_t)min(r, g.M - 1) * g.lda + kg * 32;
+  const bool a_valid = r < g.M;
+  v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  constexpr int U = 6;  // steps in flight
+  for (int k0 = k_begin; k0 < k_end; k0 += U) {
+    v4i w[U][2], a[U][2];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kt = min(k0 + u, k_end - 1);  // clamped duplicates are not accumulated
+      const v4i* wq = reinterpret_cast<const v4i*>(wp + (int64_t)kt * 128);
+      w[u][0] = __builtin_nontemporal_load(wq);
+      w[u][1] = __builtin_nontemporal_load(wq + 1);
+      const v4i* aq = reinterpret_cast<const v4i*>(ap + (int64_t)kt * 128);
+      a[u][0] = aq[0];
+      a[u][1] = aq[1];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (k0 + u < k_end) {
+        v8i wf = __builtin_shufflevector(w[u][0], w[u][1], 0, 1, 2, 3, 4, 5, 6, 7);
+        v8i af = __builtin_shufflevector(a[u][0], a[u][1], 0, 1, 2, 3, 4, 5, 6, 7);
+        if (!a_valid) af = v8i{0, 0, 0, 0, 0, 0, 0, 0};
+        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, acc, 0, 0, 0, 0, 0, 0);
+      }
+    }
+  }
+  // acc[e] = partial out[m = lane&15][n0 + 4*(lane>>4) + e]
+#pragma unroll
+  for (int e = 0; e < 4; ++e) part[wave][r][4 * kg + e] = acc[e];
+  __syncthreads();
+  if (wave == 0) {
+    const int m = r, nl = 4 * kg;
+    if (m < g.M && n0 + nl < g.N) {
+      const float as = g.a_scale[m];
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float sum = (part[0][m][nl + e] + part[1][m][nl + e]) +
+                          (part[2][m][nl + e] + part[3][m][nl + e]);
+        const int n = n0 + nl + e;
+        float t = sum * as * g.b_scale[n];
+        if (g.bias) t += __uint_as_float((uint32_t)g.bias[n] << 16);
+        if (g.epilogue & CDIT_EPI_GELU_TANH) t = gelu_tanh(t);
+        v[e] = t;
+      }
+      uint2 pk;
+      pk.x = pack_bf16x2(v[0], v[1]);
+      pk.y = pack_bf16x2(v[2], v[3]);
+      *reinterpret_cast<uint2*>(g.out + (int64_t)m * g.ldo + n0 + nl) = pk;
+    }
+  }
 }
 
 // Any shape, any alignment: a 16x16 output tile per workgroup, one output
@@ -513,13 +655,25 @@ typedef Cfg<256, 128, 2, 2, true, true, 8> V4;
 typedef Cfg<128, 256, 2, 2, true, true, 8> V5;
 typedef Cfg<128, 128, 2, 2, true, true, 8> V6;
 typedef Cfg<256, 256, 2, 4, true, true, 8> V7;  // 8 waves, 128x64 wave tiles
+typedef Cfg<128, 128, 2, 2, true, true, 8, 4> V19;  // small tiles, 4 stages of 128 B
+typedef Cfg<128, 64, 2, 2, true, true, 8, 4> V20;
+typedef Cfg<64, 128, 2, 2, true, true, 8, 4> V21;
+typedef Cfg<128, 128, 2, 4, true, true, 8, 4> V22;  // 8 waves, 64x32 wave tiles
 typedef CfgPP<256, 256, 4, true, 8> V8;   // ping-pong, 4 stages of 64 B
 typedef CfgPP<256, 256, 4, false, 8> V9;
 typedef CfgPP<192, 384, 4, true, 8> V10;  // 96x96 wave tiles
 typedef CfgPP<256, 256, 3, true, 8> V12;
 typedef CfgPP<256, 128, 4, true, 8> V13;  // 128x32 wave tiles
 typedef CfgPP<128, 256, 4, true, 8> V14;  // 64x64 wave tiles
+typedef CfgPP<128, 128, 8, true, 8> V15;   // small tiles, deep prefetch
+typedef CfgPP<128, 256, 6, true, 8> V16;
+typedef CfgPP<64, 256, 6, true, 8> V17;
+typedef CfgPP<64, 128, 8, true, 8> V18;
+typedef CfgPP<192, 192, 3, true, 8, 0, 4> V23;  // 4 waves, 96x96 wave tiles, 2 WGs/CU
+typedef CfgPP<256, 128, 3, true, 8, 0, 4> V24;  // 4 waves, 128x64 wave tiles, 2 WGs/CU
+typedef CfgPP<128, 128, 4, true, 8, 0, 4> V26;  // 4 waves, 64x64 wave tiles
 typedef CfgPP<256, 256, 4, true, 8, 16> D16;
+typedef CfgPP<192, 384, 4, true, 8, 16> D17;
 
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {
@@ -527,10 +681,31 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     hipLaunchKernelGGL(gemm_fp8_generic, grid, dim3(256), 0, stream, g);
     return 0;
   }
+  if ((variant < 0 && g.M <= 16) || variant == 50) {
+    if (g.M > 16) {
+      set_error("cdit_fp8_gemm_rowwise: the skinny kernel takes M <= 16, got %d", g.M);
+      return CDIT_EINVAL;
+    }
+    hipLaunchKernelGGL(gemm_fp8_skinny, dim3((g.N + 15) / 16), dim3(256), 0, stream, g);
+    return 0;
+  }
   if (variant < 0) {
-    // enough 256x256 tiles to cover the 256 CUs: the ping-pong kernel; else smaller tiles
-    const int64_t big_tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
-    variant = big_tiles >= 200 ? 8 : 6;
+    // Cost model: full rounds over the 256 CUs times the tile area. With enough
+    // 256x256 tiles to fill the chip, take whichever of 256x256 and 192x384 needs
+    // fewer CU-rounds of work (ties to 256x256); smaller problems take smaller
+    // tiles: 128x128 (two workgroups per CU) when those fill the chip, else 64x128
+    // with a 4-deep DMA pipeline.
+    auto tiles = [&](int bm, int bn) {
+      return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
+    };
+    auto cost = [&](int bm, int bn) { return ((tiles(bm, bn) + 255) / 256) * bm * bn; };
+    if (tiles(256, 256) >= 200) {
+      variant = cost(192, 384) < cost(256, 256) ? 10 : 8;
+    } else if (tiles(128, 128) >= 256) {
+      variant = 6;
+    } else {
+      variant = 21;
+    }
   }
   switch (variant) {
     case 0: return launch_tiled<V0>(g, stream);
@@ -541,13 +716,25 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     case 5: return launch_tiled<V5>(g, stream);
     case 6: return launch_tiled<V6>(g, stream);
     case 7: return launch_tiled<V7>(g, stream);
+    case 19: return launch_tiled<V19>(g, stream);
+    case 20: return launch_tiled<V20>(g, stream);
+    case 21: return launch_tiled<V21>(g, stream);
+    case 22: return launch_tiled<V22>(g, stream);
     case 8: return launch_pingpong<V8>(g, stream);
     case 9: return launch_pingpong<V9>(g, stream);
     case 10: return launch_pingpong<V10>(g, stream);
     case 12: return launch_pingpong<V12>(g, stream);
     case 13: return launch_pingpong<V13>(g, stream);
     case 14: return launch_pingpong<V14>(g, stream);
+    case 15: return launch_pingpong<V15>(g, stream);
+    case 16: return launch_pingpong<V16>(g, stream);
+    case 17: return launch_pingpong<V17>(g, stream);
+    case 18: return launch_pingpong<V18>(g, stream);
+    case 23: return launch_pingpong<V23>(g, stream);
+    case 24: return launch_pingpong<V24>(g, stream);
+    case 26: return launch_pingpong<V26>(g, stream);
     case 30: return launch_pingpong<D16>(g, stream);
+    case 31: return launch_pingpong<D17>(g, stream);
     default:
       set_error("cdit_fp8_gemm_rowwise: unknown kernel variant %d", variant);
       return CDIT_EINVAL;

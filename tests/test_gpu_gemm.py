@@ -49,7 +49,7 @@ def _assert_close(out, ref):
   assert elementwise_ok(out, ref, REL_TOL)
 
 
-TILED_VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 13, 14]
+TILED_VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 13, 14, 15, 16, 17, 18, 19, 20, 21, 22, 23, 24, 26]
 
 
 @pytest.mark.parametrize("variant", TILED_VARIANTS + [100])
@@ -78,6 +78,36 @@ def test_exact_small_integers(variant):
   _native.set_gemm_variant(variant)
   out = _run(a, a_s, w, w_s, None)
   assert torch.equal(out.cpu(), ref)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 18432, 3072), (1, 9216, 3072), (3, 264, 384), (16, 512, 128),
+                                   (7, 3072, 15360)])
+@pytest.mark.parametrize("gelu", [0, 1])
+def test_skinny_kernel(M, N, K, gelu):
+  """M <= 16 (the M = 1 modulation Linears): automatic choice and forced variant."""
+  from cache_dit_amd import _native
+  p = _rand_problem(M, N, K, seed=M * 7 + N + K)
+  ref = to.scaled_mm_rowwise(*p, gelu="fused" if gelu else None)
+  _assert_close(_run(*p, epilogue=gelu), ref)
+  _native.set_gemm_variant(50)
+  _assert_close(_run(*p, epilogue=gelu), ref)
+
+
+def test_skinny_exact_and_k_positions():
+  from cache_dit_amd import _native
+  g = torch.Generator().manual_seed(13)
+  M, N, K = 5, 272, 1024
+  a = torch.randint(-4, 5, (M, K), generator=g).float().to(FP8)
+  w = torch.randint(-4, 5, (N, K), generator=g).float().to(FP8)
+  a_s, w_s = torch.full((M, 1), 0.5), torch.full((N, 1), 0.25)
+  _native.set_gemm_variant(50)
+  assert torch.equal(_run(a, a_s, w, w_s, None).cpu(), to.scaled_mm_rowwise(a, a_s, w, w_s))
+  a = torch.zeros(M, K)
+  a[torch.arange(M), torch.tensor([0, 33, 130, 517, 1023])] = 1.0
+  w = ((torch.arange(K) % 15) + 1).float().repeat(N, 1)
+  ones_m, ones_n = torch.ones(M, 1), torch.ones(N, 1)
+  assert torch.equal(_run(a.to(FP8), ones_m, w.to(FP8), ones_n, None).cpu(),
+                     to.scaled_mm_rowwise(a.to(FP8), ones_m, w.to(FP8), ones_n))
 
 
 def test_k_position_sensitivity():
