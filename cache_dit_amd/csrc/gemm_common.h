@@ -48,15 +48,27 @@ __device__ __forceinline__ float gelu_tanh(float v) {
 
 // s_waitcnt vmcnt(N) lgkmcnt(0) followed by a bare workgroup barrier. The memory
 // clobber keeps the compiler from moving LDS accesses across it.
+// The s_waitcnt is emitted through the builtin so that the compiler's own wait
+// insertion sees it (it would otherwise re-wait for LDS reads with lgkmcnt(0)).
 template <int VM>
 __device__ __forceinline__ void wait_and_barrier() {
-  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(VM) : "memory");
+  asm volatile("" ::: "memory");
+  // simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
+  __builtin_amdgcn_s_waitcnt((VM & 0xf) | (7 << 4) | (0 << 8) | ((VM >> 4) << 14));
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
 }
 template <int VM>
 __device__ __forceinline__ void wait_vm() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(VM) : "memory");
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt((VM & 0xf) | (7 << 4) | (0xf << 8) | ((VM >> 4) << 14));
+  asm volatile("" ::: "memory");
 }
-__device__ __forceinline__ void bare_barrier() { asm volatile("s_barrier" ::: "memory"); }
+__device__ __forceinline__ void bare_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
 
 // Waits until at most `later` steps (of D DMA instructions each) are in flight,
 // `later` in [0, MAXL]; the count has to be an immediate, hence the switch.

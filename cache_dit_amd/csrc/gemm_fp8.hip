@@ -264,13 +264,17 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_tiled(GemmArgs g, int til
 // The 1 KiB DMA instructions of a step (A panel first, then B) are dealt to the
 // waves round-robin; when their number is not a multiple of 8 the first waves
 // issue one more than the others, and each wave counts its own (D) for s_waitcnt.
-template <int BM_, int BN_, int STAGES_, bool EPI_LDS_, int GROUP_M_, int DBG_ = 0, int WAVES_ = 8>
+template <int BM_, int BN_, int STAGES_, bool EPI_LDS_, int GROUP_M_, int DBG_ = 0, int WAVES_ = 8,
+          bool SWP_ = false>
 struct CfgPP {
+  // SWP: software-pipelined loop (8 waves in phase, operands of step kt+1 read from
+  // LDS into a second register set while the MFMAs of step kt issue).
+  static constexpr bool SWP = SWP_;
   static constexpr int DBG = DBG_;  // 16: record clocks into a_scale (timing experiments)
   // WAVES = 8: ping-pong (two groups of four). WAVES = 4: all waves in phase, one
   // barrier per step; sized (<= 80 KiB LDS, <= 256 VGPRs) so that two such
   // workgroups share a CU and fill each other's stalls and epilogues.
-  static constexpr bool PINGPONG = WAVES_ == 8;
+  static constexpr bool PINGPONG = WAVES_ == 8 && !SWP_;
   static constexpr int BM = BM_, BN = BN_, STAGES = STAGES_, WGM = 2, WGN = WAVES_ / 2;
   static constexpr bool EPI_LDS = EPI_LDS_;
   static constexpr int GROUP_M = GROUP_M_;
@@ -350,6 +354,77 @@ __device__ __forceinline__ void pingpong_loop(v16f (&acc)[C::TM][C::TN], uint8_t
     __builtin_amdgcn_sched_barrier(0);
   }
   if (group == 0) bare_barrier();
+}
+
+// Software-pipelined main loop: all 8 waves in phase, one barrier per 64-byte step.
+// While the MFMAs of step kt issue from one operand register set, the operands of
+// step kt+1 are read from LDS into the other, so neither LDS latency nor the
+// single-wave MFMA issue gap is exposed (two waves per SIMD alternate MFMAs). A
+// stage is free as soon as its operands sit in registers, one step earlier than
+// in the ping-pong loop: DMA runs STAGES steps ahead.
+template <class C, int D>
+__device__ __forceinline__ void swp_loop(v16f (&acc)[C::TM][C::TN], uint8_t* smem,
+                                         const uint8_t* __restrict__ A,
+                                         const uint8_t* __restrict__ B,
+                                         const uint32_t (&off)[C::DMAX], int KT, int wave,
+                                         const uint32_t (&rd_a)[2], const uint32_t (&rd_b)[2]) {
+  constexpr int BKP = C::BKP, S = C::STAGES;
+  auto fetch = [&](int kt) {
+    uint8_t* st = smem + (kt % S) * C::STAGE_BYTES;
+#pragma unroll
+    for (int p = 0; p < D; ++p) {
+      const int id = wave + C::WAVES * p;
+      const uint8_t* src = (id < C::NA ? A : B) + (int64_t)kt * BKP + off[p];
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(st + id * 1024),
+                                       16, 0, 0);
+    }
+  };
+  auto read_frags = [&](int kt, v8i (&fa)[C::TM], v8i (&fb)[C::TN]) {
+    const uint8_t* st = smem + (kt % S) * C::STAGE_BYTES;
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_b[0] + j * 32 * BKP);
+      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_b[1] + j * 32 * BKP);
+      fb[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i) {
+      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_a[0] + i * 32 * BKP);
+      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_a[1] + i * 32 * BKP);
+      fa[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  };
+  auto step = [&](int kt, v8i (&ca)[C::TM], v8i (&cb)[C::TN], v8i (&na)[C::TM],
+                  v8i (&nb)[C::TN]) {
+    // own DMA of step kt+1 landed; own reads of step kt (previous iteration) done
+    wait_steps<D, S - 1, true>(max(min(kt + S - 1, KT - 1) - (kt + 1), 0));
+    if (kt + S < KT) fetch(kt + S);  // into the stage whose operands are in ca/cb
+    read_frags(min(kt + 1, KT - 1), na, nb);  // the last step re-reads itself: unused
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cb[j], ca[i], acc[i][j], 0, 0,
+                                                                    0, 0, 0, 0);
+    // issue order: one MFMA, then two LDS reads, ... so the reads hide under the MFMAs
+#pragma unroll
+    for (int t = 0; t < C::TM * C::TN; ++t) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+  };
+#pragma unroll
+  for (int s = 0; s < S; ++s)
+    if (s < KT) fetch(s);
+  wait_steps<D, S - 1, true>(min(S, KT) - 1);  // step 0 landed everywhere
+  v8i a0[C::TM], b0[C::TN], a1[C::TM], b1[C::TN];
+  read_frags(0, a0, b0);
+  for (int kt = 0; kt < KT; kt += 2) {  // KT is even (K is a multiple of 128)
+    step(kt, a0, b0, a1, b1);
+    step(kt + 1, a1, b1, a0, b0);
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
 // Main loop of the 4-wave flavour: all waves in phase, one barrier per step.
@@ -463,7 +538,17 @@ __global__ __launch_bounds__(C::THREADS, 2) void gemm_fp8_pingpong(GemmArgs g, i
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   const int KT = g.K / BKP;
-  if constexpr (C::PINGPONG) {
+  if constexpr (C::SWP) {
+    if constexpr (C::NT % C::WAVES == 0) {
+      swp_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, rd_a, rd_b);
+    } else {
+      if (wave < C::NT % C::WAVES) {
+        swp_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, rd_a, rd_b);
+      } else {
+        swp_loop<C, C::DMAX - 1>(acc, smem, A, B, off, KT, wave, rd_a, rd_b);
+      }
+    }
+  } else if constexpr (C::PINGPONG) {
     if constexpr (C::NT % C::WAVES == 0) {
       pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
     } else {
@@ -672,6 +757,9 @@ typedef CfgPP<64, 128, 8, true, 8> V18;
 typedef CfgPP<192, 192, 3, true, 8, 0, 4> V23;  // 4 waves, 96x96 wave tiles, 2 WGs/CU
 typedef CfgPP<256, 128, 3, true, 8, 0, 4> V24;  // 4 waves, 128x64 wave tiles, 2 WGs/CU
 typedef CfgPP<128, 128, 4, true, 8, 0, 4> V26;  // 4 waves, 64x64 wave tiles
+typedef CfgPP<256, 256, 3, true, 8, 0, 8, true> V27;  // software-pipelined, 3 stages
+typedef CfgPP<256, 256, 4, true, 8, 0, 8, true> V28;
+typedef CfgPP<192, 384, 3, true, 8, 0, 8, true> V29;
 typedef CfgPP<256, 256, 4, true, 8, 16> D16;
 typedef CfgPP<192, 384, 4, true, 8, 16> D17;
 
@@ -733,6 +821,9 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     case 23: return launch_pingpong<V23>(g, stream);
     case 24: return launch_pingpong<V24>(g, stream);
     case 26: return launch_pingpong<V26>(g, stream);
+    case 27: return launch_pingpong<V27>(g, stream);
+    case 28: return launch_pingpong<V28>(g, stream);
+    case 29: return launch_pingpong<V29>(g, stream);
     case 30: return launch_pingpong<D16>(g, stream);
     case 31: return launch_pingpong<D17>(g, stream);
     default:
