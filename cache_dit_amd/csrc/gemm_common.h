@@ -107,12 +107,11 @@ __device__ __forceinline__ void wait_steps(int later) {
 // consecutive, then walked in column-major order inside groups of GROUP_M tile
 // rows: the 32 workgroups resident on an XCD then share a handful of A and B
 // panels.
+// Linear tile id -> (tile row, tile column): column-major inside groups of GROUP_M
+// tile rows.
 template <int GROUP_M>
-__device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m, int tiles_n,
-                                              int* tm, int* tn) {
-  constexpr int kXcd = 8;
-  int id = bid;
-  if (nblocks % kXcd == 0) id = (bid % kXcd) * (nblocks / kXcd) + bid / kXcd;
+__device__ __forceinline__ void tile_of_linear(int id, int tiles_m, int tiles_n, int* tm,
+                                               int* tn) {
   const int per_group = GROUP_M * tiles_n;
   const int group = id / per_group;
   const int first_m = group * GROUP_M;
@@ -122,6 +121,14 @@ __device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m,
   *tn = in_group / gsize;
 }
 
+template <int GROUP_M>
+__device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m, int tiles_n,
+                                              int* tm, int* tn) {
+  constexpr int kXcd = 8;
+  int id = bid;
+  if (nblocks % kXcd == 0) id = (bid % kXcd) * (nblocks / kXcd) + bid / kXcd;
+  tile_of_linear<GROUP_M>(id, tiles_m, tiles_n, tm, tn);
+}
 
 // Epilogue shared by the tiled kernels. The MFMAs were issued with the
 // operands swapped, so acc[i][j][4*gq+e] is out[m][n] with
@@ -132,6 +139,12 @@ __device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m,
 // LDS tile (32 rows x EPI_PITCH bytes at `et`; no workgroup barrier needed) so that
 // every lane stores 16 bytes along a row; otherwise lanes store their 8 bytes
 // directly. a_scale may be null (weight-only mode): then it is 1.
+// Whether the wave-private epilogue tile has unpadded rows (EPI_PITCH == 2*WN).
+template <class C>
+__device__ __forceinline__ constexpr bool epi_rotated() {
+  return C::EPI_PITCH == C::WN * 2;
+}
+
 template <class C>
 __device__ __forceinline__ void tile_epilogue(v16f (&acc)[C::TM][C::TN], const GemmArgs& g,
                                               uint8_t* et, int m0, int n0, int wm, int wn,
@@ -140,26 +153,32 @@ __device__ __forceinline__ void tile_epilogue(v16f (&acc)[C::TM][C::TN], const G
   const bool gelu = (g.epilogue & CDIT_EPI_GELU_TANH) != 0;
   const int nw = n0 + wn * C::WN;  // first column of the wave tile
   const int mw = m0 + wm * C::WM;
-  v4f bs[C::TN][4], bi[C::TN][4];
-#pragma unroll
-  for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-    for (int gq = 0; gq < 4; ++gq) {
-      const int n = nw + 32 * j + 8 * gq + 4 * h;  // N % 8 == 0: a group of 4 is all in or out
-      v4f s4 = {0.0f, 0.0f, 0.0f, 0.0f}, b4 = {0.0f, 0.0f, 0.0f, 0.0f};
-      if (n < g.N) {
-        s4 = *reinterpret_cast<const v4f*>(g.b_scale + n);
-        if (g.bias) {
-          const uint2 bb = *reinterpret_cast<const uint2*>(g.bias + n);
-          b4[0] = __uint_as_float(bb.x << 16);
-          b4[1] = __uint_as_float(bb.x & 0xffff0000u);
-          b4[2] = __uint_as_float(bb.y << 16);
-          b4[3] = __uint_as_float(bb.y & 0xffff0000u);
-        }
+  // b_scale / bias of this lane's 4-column groups. Wide wave tiles reload them for
+  // every 32-row block (L1 hits) instead of keeping TN*32 registers alive next to
+  // the accumulators.
+  constexpr bool kPreload = C::TN <= 2;
+  auto load_cols = [&](int j, int gq, v4f& s4, v4f& b4) {
+    const int n = nw + 32 * j + 8 * gq + 4 * h;  // N % 8 == 0: a group of 4 is all in or out
+    s4 = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    b4 = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    if (n < g.N) {
+      s4 = *reinterpret_cast<const v4f*>(g.b_scale + n);
+      if (g.bias) {
+        const uint2 bb = *reinterpret_cast<const uint2*>(g.bias + n);
+        b4[0] = __uint_as_float(bb.x << 16);
+        b4[1] = __uint_as_float(bb.x & 0xffff0000u);
+        b4[2] = __uint_as_float(bb.y << 16);
+        b4[3] = __uint_as_float(bb.y & 0xffff0000u);
       }
-      bs[j][gq] = s4;
-      bi[j][gq] = b4;
     }
+  };
+  v4f bs[kPreload ? C::TN : 1][4], bi[kPreload ? C::TN : 1][4];
+  if constexpr (kPreload) {
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) load_cols(j, gq, bs[j][gq], bi[j][gq]);
+  }
 #pragma unroll
   for (int i = 0; i < C::TM; ++i) {
     const int m = mw + 32 * i + r;
@@ -168,10 +187,17 @@ __device__ __forceinline__ void tile_epilogue(v16f (&acc)[C::TM][C::TN], const G
     for (int j = 0; j < C::TN; ++j)
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
+        v4f s4, b4;
+        if constexpr (kPreload) {
+          s4 = bs[j][gq];
+          b4 = bi[j][gq];
+        } else {
+          load_cols(j, gq, s4, b4);
+        }
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          v[e] = __fmaf_rn(acc[i][j][4 * gq + e] * as, bs[j][gq][e], bi[j][gq][e]);
+          v[e] = __fmaf_rn(acc[i][j][4 * gq + e] * as, s4[e], b4[e]);
           if (gelu) v[e] = gelu_tanh(v[e]);
         }
         uint2 pk;
@@ -179,7 +205,13 @@ __device__ __forceinline__ void tile_epilogue(v16f (&acc)[C::TM][C::TN], const G
         pk.y = pack_bf16x2(v[2], v[3]);
         const int nl = 32 * j + 8 * gq + 4 * h;  // column inside the wave tile
         if constexpr (C::EPI_LDS) {
-          *reinterpret_cast<uint2*>(et + r * C::EPI_PITCH + nl * 2) = pk;
+          if constexpr (epi_rotated<C>()) {
+            // unpadded rows: rotate the 16-byte chunks by the row index instead
+            const int chunk = ((nl >> 3) + r) % (C::WN / 8);
+            *reinterpret_cast<uint2*>(et + r * C::EPI_PITCH + chunk * 16 + (nl & 7) * 2) = pk;
+          } else {
+            *reinterpret_cast<uint2*>(et + r * C::EPI_PITCH + nl * 2) = pk;
+          }
         } else {
           if (m < g.M && nw + nl < g.N)
             *reinterpret_cast<uint2*>(g.out + (int64_t)m * g.ldo + nw + nl) = pk;
@@ -194,7 +226,8 @@ __device__ __forceinline__ void tile_epilogue(v16f (&acc)[C::TM][C::TN], const G
       for (int t = 0; t < PER_LANE; ++t) {
         const int q = t * 64 + lane;
         const int row = q / CPR, cc = q % CPR;
-        const uint4 d = *reinterpret_cast<const uint4*>(et + row * C::EPI_PITCH + cc * 16);
+        const int pc = epi_rotated<C>() ? (cc + row) % CPR : cc;
+        const uint4 d = *reinterpret_cast<const uint4*>(et + row * C::EPI_PITCH + pc * 16);
         const int mm = mw + 32 * i + row, nn = nw + cc * 8;
         if (mm < g.M && nn < g.N) *reinterpret_cast<uint4*>(g.out + (int64_t)mm * g.ldo + nn) = d;
       }

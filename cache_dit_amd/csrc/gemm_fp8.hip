@@ -264,21 +264,12 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_tiled(GemmArgs g, int til
 // The 1 KiB DMA instructions of a step (A panel first, then B) are dealt to the
 // waves round-robin; when their number is not a multiple of 8 the first waves
 // issue one more than the others, and each wave counts its own (D) for s_waitcnt.
-template <int BM_, int BN_, int STAGES_, bool EPI_LDS_, int GROUP_M_, int DBG_ = 0, int WAVES_ = 8,
-          bool SWP_ = false>
+template <int BM_, int BN_, int STAGES_, bool EPI_LDS_, int GROUP_M_>
 struct CfgPP {
-  // SWP: software-pipelined loop (8 waves in phase, operands of step kt+1 read from
-  // LDS into a second register set while the MFMAs of step kt issue).
-  static constexpr bool SWP = SWP_;
-  static constexpr int DBG = DBG_;  // 16: record clocks into a_scale (timing experiments)
-  // WAVES = 8: ping-pong (two groups of four). WAVES = 4: all waves in phase, one
-  // barrier per step; sized (<= 80 KiB LDS, <= 256 VGPRs) so that two such
-  // workgroups share a CU and fill each other's stalls and epilogues.
-  static constexpr bool PINGPONG = WAVES_ == 8 && !SWP_;
-  static constexpr int BM = BM_, BN = BN_, STAGES = STAGES_, WGM = 2, WGN = WAVES_ / 2;
+  static constexpr int BM = BM_, BN = BN_, STAGES = STAGES_, WGM = 2, WGN = 4;
   static constexpr bool EPI_LDS = EPI_LDS_;
   static constexpr int GROUP_M = GROUP_M_;
-  static constexpr int WAVES = WAVES_, THREADS = WAVES_ * 64;
+  static constexpr int WAVES = 8, THREADS = 512;
   static constexpr int WM = BM / WGM, WN = BN / WGN;
   static constexpr int TM = WM / 32, TN = WN / 32;
   static constexpr int BKP = 64;
@@ -356,134 +347,7 @@ __device__ __forceinline__ void pingpong_loop(v16f (&acc)[C::TM][C::TN], uint8_t
   if (group == 0) bare_barrier();
 }
 
-// Software-pipelined main loop: all 8 waves in phase, one barrier per 64-byte step.
-// While the MFMAs of step kt issue from one operand register set, the operands of
-// step kt+1 are read from LDS into the other, so neither LDS latency nor the
-// single-wave MFMA issue gap is exposed (two waves per SIMD alternate MFMAs). A
-// stage is free as soon as its operands sit in registers, one step earlier than
-// in the ping-pong loop: DMA runs STAGES steps ahead.
-template <class C, int D>
-__device__ __forceinline__ void swp_loop(v16f (&acc)[C::TM][C::TN], uint8_t* smem,
-                                         const uint8_t* __restrict__ A,
-                                         const uint8_t* __restrict__ B,
-                                         const uint32_t (&off)[C::DMAX], int KT, int wave,
-                                         const uint32_t (&rd_a)[2], const uint32_t (&rd_b)[2]) {
-  constexpr int BKP = C::BKP, S = C::STAGES;
-  auto fetch = [&](int kt) {
-    uint8_t* st = smem + (kt % S) * C::STAGE_BYTES;
-#pragma unroll
-    for (int p = 0; p < D; ++p) {
-      const int id = wave + C::WAVES * p;
-      const uint8_t* src = (id < C::NA ? A : B) + (int64_t)kt * BKP + off[p];
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(st + id * 1024),
-                                       16, 0, 0);
-    }
-  };
-  auto read_frags = [&](int kt, v8i (&fa)[C::TM], v8i (&fb)[C::TN]) {
-    const uint8_t* st = smem + (kt % S) * C::STAGE_BYTES;
-#pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
-      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_b[0] + j * 32 * BKP);
-      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_b[1] + j * 32 * BKP);
-      fb[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i) {
-      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_a[0] + i * 32 * BKP);
-      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_a[1] + i * 32 * BKP);
-      fa[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-  };
-  auto step = [&](int kt, v8i (&ca)[C::TM], v8i (&cb)[C::TN], v8i (&na)[C::TM],
-                  v8i (&nb)[C::TN]) {
-    // own DMA of step kt+1 landed; own reads of step kt (previous iteration) done
-    wait_steps<D, S - 1, true>(max(min(kt + S - 1, KT - 1) - (kt + 1), 0));
-    if (kt + S < KT) fetch(kt + S);  // into the stage whose operands are in ca/cb
-    read_frags(min(kt + 1, KT - 1), na, nb);  // the last step re-reads itself: unused
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-      for (int j = 0; j < C::TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cb[j], ca[i], acc[i][j], 0, 0,
-                                                                    0, 0, 0, 0);
-    // issue order: one MFMA, then two LDS reads, ... so the reads hide under the MFMAs
-#pragma unroll
-    for (int t = 0; t < C::TM * C::TN; ++t) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-    }
-  };
-#pragma unroll
-  for (int s = 0; s < S; ++s)
-    if (s < KT) fetch(s);
-  wait_steps<D, S - 1, true>(min(S, KT) - 1);  // step 0 landed everywhere
-  v8i a0[C::TM], b0[C::TN], a1[C::TM], b1[C::TN];
-  read_frags(0, a0, b0);
-  for (int kt = 0; kt < KT; kt += 2) {  // KT is even (K is a multiple of 128)
-    step(kt, a0, b0, a1, b1);
-    step(kt + 1, a1, b1, a0, b0);
-  }
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
-// Main loop of the 4-wave flavour: all waves in phase, one barrier per step.
-template <class C, int D>
-__device__ __forceinline__ void inphase_loop(v16f (&acc)[C::TM][C::TN], uint8_t* smem,
-                                             const uint8_t* __restrict__ A,
-                                             const uint8_t* __restrict__ B,
-                                             const uint32_t (&off)[C::DMAX], int KT, int wave,
-                                             const uint32_t (&rd_a)[2],
-                                             const uint32_t (&rd_b)[2]) {
-  constexpr int BKP = C::BKP, PD = C::STAGES - 1;
-  auto fetch = [&](int kt) {
-    uint8_t* st = smem + (kt % C::STAGES) * C::STAGE_BYTES;
-#pragma unroll
-    for (int p = 0; p < D; ++p) {
-      const int id = wave + C::WAVES * p;
-      const uint8_t* src = (id < C::NA ? A : B) + (int64_t)kt * BKP + off[p];
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(st + id * 1024),
-                                       16, 0, 0);
-    }
-  };
-#pragma unroll
-  for (int s = 0; s < PD; ++s)
-    if (s < KT) fetch(s);
-  wait_steps<D, PD - 1, false>(min(PD, KT) - 1);
-  for (int kt = 0; kt < KT; ++kt) {
-    // everyone's part of step kt has landed and everyone has left compute(kt-1),
-    // whose stage the next DMA overwrites
-    bare_barrier();
-    if (kt + PD < KT) fetch(kt + PD);
-    const uint8_t* st = smem + (kt % C::STAGES) * C::STAGE_BYTES;
-    v8i af[C::TM], bf[C::TN];
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i) {
-      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_a[0] + i * 32 * BKP);
-      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_a[1] + i * 32 * BKP);
-      af[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-#pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
-      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_b[0] + j * 32 * BKP);
-      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_b[1] + j * 32 * BKP);
-      bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-      for (int j = 0; j < C::TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[i][j], 0, 0,
-                                                                    0, 0, 0, 0);
-    // own DMA of step kt+1 landed (LDS reads of this step too) before the next barrier
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    wait_steps<D, PD - 1, false>(max(min(kt + PD, KT - 1) - (kt + 1), 0));
-  }
-  bare_barrier();  // all operand reads done: the stage buffers may hold epilogue tiles
-}
-
-// Two waves per SIMD in both flavours (8 waves of one workgroup, or 4 + 4 of two).
+// Two waves per SIMD: at most 256 VGPRs.
 template <class C>
 __global__ __launch_bounds__(C::THREADS, 2) void gemm_fp8_pingpong(GemmArgs g, int tiles_m,
                                                                    int tiles_n) {
@@ -494,11 +358,6 @@ __global__ __launch_bounds__(C::THREADS, 2) void gemm_fp8_pingpong(GemmArgs g, i
   const int wm = wave / C::WGN, wn = wave % C::WGN;  // wm is also the ping-pong group
   constexpr int BKP = C::BKP;
 
-  long long dbg_t0 = 0, dbg_r0 = 0;
-  if constexpr (C::DBG & 16) {
-    dbg_t0 = clock64();
-    dbg_r0 = wall_clock64();
-  }
   int tm, tn;
   tile_of_block<C::GROUP_M>(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
   const int m0 = tm * C::BM, n0 = tn * C::BN;
@@ -538,57 +397,20 @@ __global__ __launch_bounds__(C::THREADS, 2) void gemm_fp8_pingpong(GemmArgs g, i
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   const int KT = g.K / BKP;
-  if constexpr (C::SWP) {
-    if constexpr (C::NT % C::WAVES == 0) {
-      swp_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, rd_a, rd_b);
-    } else {
-      if (wave < C::NT % C::WAVES) {
-        swp_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, rd_a, rd_b);
-      } else {
-        swp_loop<C, C::DMAX - 1>(acc, smem, A, B, off, KT, wave, rd_a, rd_b);
-      }
-    }
-  } else if constexpr (C::PINGPONG) {
-    if constexpr (C::NT % C::WAVES == 0) {
+  if constexpr (C::NT % C::WAVES == 0) {
+    pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
+  } else {
+    if (wave < C::NT % C::WAVES) {
       pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
     } else {
-      if (wave < C::NT % C::WAVES) {
-        pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
-      } else {
-        pingpong_loop<C, C::DMAX - 1>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
-      }
-    }
-  } else {
-    if constexpr (C::NT % C::WAVES == 0) {
-      inphase_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, rd_a, rd_b);
-    } else {
-      if (wave < C::NT % C::WAVES) {
-        inphase_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, rd_a, rd_b);
-      } else {
-        inphase_loop<C, C::DMAX - 1>(acc, smem, A, B, off, KT, wave, rd_a, rd_b);
-      }
+      pingpong_loop<C, C::DMAX - 1>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
     }
   }
 
   // All LDS operand reads and all DMA are complete here (the last slot barrier
   // follows group 1's last reads), so the stage buffers can hold the epilogue tiles.
   uint8_t* et = smem + wave * (32 * C::EPI_PITCH);
-  if constexpr (C::DBG & 16) {
-    long long t1 = clock64(), r1 = wall_clock64();
-    tile_epilogue<C>(acc, g, et, m0, n0, wm, wn, lane);
-    long long t2 = clock64(), r2 = wall_clock64();
-    if (tid == 0 && blockIdx.x < 1024) {
-      long long* d = reinterpret_cast<long long*>(const_cast<float*>(g.a_scale)) + blockIdx.x * 6;
-      d[0] = t1 - dbg_t0;
-      d[1] = r1 - dbg_r0;
-      d[2] = t2 - t1;
-      d[3] = r2 - r1;
-      d[4] = dbg_r0;
-      d[5] = r2;
-    }
-  } else {
-    tile_epilogue<C>(acc, g, et, m0, n0, wm, wn, lane);
-  }
+  tile_epilogue<C>(acc, g, et, m0, n0, wm, wn, lane);
 }
 
 template <class C>
@@ -731,37 +553,18 @@ bool tiled_ok(const GemmArgs& g) {
 
 }  // namespace
 
-//                 BM   BN  WGM WGN direct epiLDS groupM
-typedef Cfg<256, 256, 2, 2, false, false, 8> V0;  // register staging, direct stores
-typedef Cfg<256, 256, 2, 2, true, true, 8> V1;    // LDS-DMA staging, LDS-transposed stores
-typedef Cfg<256, 256, 2, 2, false, true, 8> V2;
-typedef Cfg<256, 256, 2, 2, true, false, 8> V3;
-typedef Cfg<256, 128, 2, 2, true, true, 8> V4;
-typedef Cfg<128, 256, 2, 2, true, true, 8> V5;
-typedef Cfg<128, 128, 2, 2, true, true, 8> V6;
-typedef Cfg<256, 256, 2, 4, true, true, 8> V7;  // 8 waves, 128x64 wave tiles
-typedef Cfg<128, 128, 2, 2, true, true, 8, 4> V19;  // small tiles, 4 stages of 128 B
-typedef Cfg<128, 64, 2, 2, true, true, 8, 4> V20;
+// Kernel variants. The entry point picks one by shape; tests and the tuning hook
+// (cdit_set_gemm_variant) can force any of them.
+//          BM   BN  WGM WGN direct epiLDS groupM stages
+typedef Cfg<256, 256, 2, 2, false, false, 8> V0;      // register staging, direct stores
+typedef Cfg<256, 256, 2, 2, true, true, 8> V1;        // LDS-DMA, 2 stages, 4 waves
+typedef Cfg<128, 128, 2, 2, true, true, 8> V6;        // two workgroups per CU
+typedef Cfg<256, 256, 2, 4, true, true, 8> V7;        // 8 waves in phase, 2 stages
+typedef Cfg<128, 64, 2, 2, true, true, 8, 4> V20;     // small tiles, 4 stages of 128 B
 typedef Cfg<64, 128, 2, 2, true, true, 8, 4> V21;
-typedef Cfg<128, 128, 2, 4, true, true, 8, 4> V22;  // 8 waves, 64x32 wave tiles
-typedef CfgPP<256, 256, 4, true, 8> V8;   // ping-pong, 4 stages of 64 B
-typedef CfgPP<256, 256, 4, false, 8> V9;
-typedef CfgPP<192, 384, 4, true, 8> V10;  // 96x96 wave tiles
-typedef CfgPP<256, 256, 3, true, 8> V12;
-typedef CfgPP<256, 128, 4, true, 8> V13;  // 128x32 wave tiles
-typedef CfgPP<128, 256, 4, true, 8> V14;  // 64x64 wave tiles
-typedef CfgPP<128, 128, 8, true, 8> V15;   // small tiles, deep prefetch
-typedef CfgPP<128, 256, 6, true, 8> V16;
-typedef CfgPP<64, 256, 6, true, 8> V17;
-typedef CfgPP<64, 128, 8, true, 8> V18;
-typedef CfgPP<192, 192, 3, true, 8, 0, 4> V23;  // 4 waves, 96x96 wave tiles, 2 WGs/CU
-typedef CfgPP<256, 128, 3, true, 8, 0, 4> V24;  // 4 waves, 128x64 wave tiles, 2 WGs/CU
-typedef CfgPP<128, 128, 4, true, 8, 0, 4> V26;  // 4 waves, 64x64 wave tiles
-typedef CfgPP<256, 256, 3, true, 8, 0, 8, true> V27;  // software-pipelined, 3 stages
-typedef CfgPP<256, 256, 4, true, 8, 0, 8, true> V28;
-typedef CfgPP<192, 384, 3, true, 8, 0, 8, true> V29;
-typedef CfgPP<256, 256, 4, true, 8, 16> D16;
-typedef CfgPP<192, 384, 4, true, 8, 16> D17;
+typedef CfgPP<256, 256, 4, true, 8> V8;               // ping-pong, 4 stages of 64 B
+typedef CfgPP<256, 256, 4, false, 8> V9;              // ... with direct 8-byte stores
+typedef CfgPP<192, 384, 4, true, 8> V10;              // ping-pong, 96x96 wave tiles
 
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {
@@ -798,34 +601,13 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   switch (variant) {
     case 0: return launch_tiled<V0>(g, stream);
     case 1: return launch_tiled<V1>(g, stream);
-    case 2: return launch_tiled<V2>(g, stream);
-    case 3: return launch_tiled<V3>(g, stream);
-    case 4: return launch_tiled<V4>(g, stream);
-    case 5: return launch_tiled<V5>(g, stream);
     case 6: return launch_tiled<V6>(g, stream);
     case 7: return launch_tiled<V7>(g, stream);
-    case 19: return launch_tiled<V19>(g, stream);
     case 20: return launch_tiled<V20>(g, stream);
     case 21: return launch_tiled<V21>(g, stream);
-    case 22: return launch_tiled<V22>(g, stream);
     case 8: return launch_pingpong<V8>(g, stream);
     case 9: return launch_pingpong<V9>(g, stream);
     case 10: return launch_pingpong<V10>(g, stream);
-    case 12: return launch_pingpong<V12>(g, stream);
-    case 13: return launch_pingpong<V13>(g, stream);
-    case 14: return launch_pingpong<V14>(g, stream);
-    case 15: return launch_pingpong<V15>(g, stream);
-    case 16: return launch_pingpong<V16>(g, stream);
-    case 17: return launch_pingpong<V17>(g, stream);
-    case 18: return launch_pingpong<V18>(g, stream);
-    case 23: return launch_pingpong<V23>(g, stream);
-    case 24: return launch_pingpong<V24>(g, stream);
-    case 26: return launch_pingpong<V26>(g, stream);
-    case 27: return launch_pingpong<V27>(g, stream);
-    case 28: return launch_pingpong<V28>(g, stream);
-    case 29: return launch_pingpong<V29>(g, stream);
-    case 30: return launch_pingpong<D16>(g, stream);
-    case 31: return launch_pingpong<D17>(g, stream);
     default:
       set_error("cdit_fp8_gemm_rowwise: unknown kernel variant %d", variant);
       return CDIT_EINVAL;
