@@ -53,9 +53,9 @@ def flux_step_linears():
       ("norm1_context.linear", 1, d, 6 * d, False),
   ]
   single = [
+      ("norm.linear", 1, d, 3 * d, False), ("proj_mlp", both, d, mlp, True),
       ("attn.to_q", both, d, d, False), ("attn.to_k", both, d, d, False),
-      ("attn.to_v", both, d, d, False), ("proj_mlp", both, d, mlp, True),
-      ("proj_out", both, d + mlp, d, False), ("norm.linear", 1, d, 3 * d, False),
+      ("attn.to_v", both, d, d, False), ("proj_out", both, d + mlp, d, False),
   ]
   out = []
   for i in range(19):
@@ -105,6 +105,21 @@ class HotPath:
     for M, K, N, w, ws, b, epi in self.layers:
       out = self.out[:M * N].view(M, N)
       ops.linear_w8a8_into(self.x[(M, K)], w, ws, b, out, self.q[(M, K)], self.s[(M, K)], 0, epi)
+
+  def step_shared_quant(self):
+    """The same pass with one quantizer launch per distinct input: q/k/v (and
+    proj_mlp in single blocks) read one activation, as share_activation_quant_
+    arranges in a real model. Outputs are bit-identical to step()."""
+    from cache_dit_amd import ops
+    names = [n for n, *_ in flux_step_linears()]
+    for name, (M, K, N, w, ws, b, epi) in zip(names, self.layers):
+      out = self.out[:M * N].view(M, N)
+      leaf = name.split(".", 2)[2]
+      reuse = leaf in ("attn.to_k", "attn.to_v", "attn.add_k_proj", "attn.add_v_proj") or (
+          name.startswith("single") and leaf == "attn.to_q")  # after proj_mlp
+      if not reuse:
+        ops.quant_rowwise_into(self.x[(M, K)], self.q[(M, K)], self.s[(M, K)], 0)
+      ops.gemm_rowwise_into(self.q[(M, K)], self.s[(M, K)], w, ws, b, out, epi)
 
 
 def _time_events(fn, iters, warmup):
@@ -251,11 +266,14 @@ def dit_forward_ms(device):
   with torch.device(device):
     model = FluxLikeTransformer().to(torch.bfloat16)
   cache_dit_amd.quantize(model, cache_dit_amd.QuantizeConfig(quant_type="float8_per_row"))
-  cache_dit_amd.testing.dit_shapes.fuse_gelu_epilogues(model)
+  from cache_dit_amd.testing import dit_shapes
+  dit_shapes.fuse_gelu_epilogues(model)
+  cache_dit_amd.share_activation_quant_(model)
   inputs = flux_like_inputs(device)
-  with torch.inference_mode():
+  with torch.no_grad():
     ms = _time_events(lambda: model(**inputs), 5, 2)
-  return ms, None
+  return ms, "float8_per_row, GELU-tanh fused into the producing Linear, shared activation " \
+             "quantization; bf16 SDPA attention, norms and RoPE in eager PyTorch"
 
 
 def main():
@@ -312,6 +330,22 @@ def main():
     dt = eager_ms * args.steps / 1e3
   ms_per_step = dt / args.steps * 1e3
   value = hot.flop / (dt / args.steps) / 1e12
+  # extra: the same step with shared activation quantization (304 quantizer launches)
+  try:
+    g2 = torch.cuda.CUDAGraph()
+    hot.step_shared_quant()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g2):
+      hot.step_shared_quant()
+    g2.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+      g2.replay()
+    torch.cuda.synchronize()
+    shared_ms = (time.perf_counter() - t0) / args.steps * 1e3
+  except Exception:
+    shared_ms = None
   n_layers = len(hot.layers)
   step_flop = hot.flop
   del hot
@@ -327,7 +361,9 @@ def main():
       "peak": FP8_PEAK_TFLOPS,
       "unit": "TFLOP/s",
       "frac": head["gemm_tflops"] / FP8_PEAK_TFLOPS,
-      "traffic": None,
+      # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain
+      # copy of known size (profiles/pmc_traffic_headline_kernels.md); algorithmic 165.2 MB
+      "traffic": 340.3e6,
   }
   roofline_quant = {
       "kernel": "quant_rowwise_regs at M=4608 K=3072",
@@ -336,7 +372,7 @@ def main():
       "peak": HBM_PEAK_GBPS,
       "unit": "GB/s",
       "frac": head["quant_gbps"] / HBM_PEAK_GBPS,
-      "traffic": None,
+      "traffic": 42.68e6,  # same source; algorithmic 3MK + 4M = 42.49 MB
   }
   dit_ms, dit_note = (None, "skipped") if args.skip_dit else dit_forward_ms(device)
   cpu = None if args.skip_cpu else cpu_baseline()
@@ -366,6 +402,7 @@ def main():
       },
       "frac_fp8_peak": value / FP8_PEAK_TFLOPS,
       "eager_ms_per_step": eager_ms,
+      "shared_quant_ms_per_step": shared_ms,
       "linear_headline": head,
       "dit_step_ms": dit_ms,
       "dit_step_note": dit_note,

@@ -18,6 +18,7 @@ from .caching import load_quantize_config
 from .nn import Fp8DynamicLinear
 from .nn import Fp8WeightOnlyLinear
 from .nn import fuse_gelu_tanh_
+from .nn import share_activation_quant_
 from .utils import check_quantized
 
 __version__ = "0.1.0"
@@ -34,4 +35,5 @@ __all__ = [
     "Fp8DynamicLinear",
     "Fp8WeightOnlyLinear",
     "fuse_gelu_tanh_",
+    "share_activation_quant_",
 ]

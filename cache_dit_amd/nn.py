@@ -48,6 +48,7 @@ class _Fp8LinearBase(nn.Linear):
   `convert_linear_` re-classes an existing nn.Linear."""
 
   weight_scale: torch.Tensor
+  share_input_quant: bool = False
   epilogue: int
   scale_mode: str
   quant_type: str
@@ -78,9 +79,13 @@ class Fp8DynamicLinear(_Fp8LinearBase):
     M = x2.shape[0]
     out = torch.empty((M, self.out_features), dtype=torch.bfloat16, device=x2.device)
     if M > 0:
-      q, s = ops.activation_workspace(M, self.in_features, x2.device)
-      ops.linear_w8a8_into(x2, self.weight, self.weight_scale, self.bias, out, q, s,
-                           self._scale_mode_id, self.epilogue)
+      if self.share_input_quant:
+        q, s = ops.shared_activation_quant(x2, self._scale_mode_id)
+        ops.gemm_rowwise_into(q, s, self.weight, self.weight_scale, self.bias, out, self.epilogue)
+      else:
+        q, s = ops.activation_workspace(M, self.in_features, x2.device)
+        ops.linear_w8a8_into(x2, self.weight, self.weight_scale, self.bias, out, q, s,
+                             self._scale_mode_id, self.epilogue)
     return out.view(*x.shape[:-1], self.out_features)
 
 
@@ -150,6 +155,22 @@ def fuse_gelu_tanh_(linear: nn.Linear, act: nn.Module) -> None:
   linear.epilogue |= _native.EPI_GELU_TANH
   act.forward = lambda x: x  # type: ignore[method-assign]
   act._cdit_fused_into_linear = True  # type: ignore[attr-defined]
+
+
+def share_activation_quant_(module: nn.Module, enable: bool = True) -> int:
+  """Lets every `float8_per_row` Linear under `module` reuse the activation codes of
+  the previous Linear on the stream when it is handed the very same, unmodified
+  input buffer (q/k/v projections, FLUX `proj_mlp` + q/k/v): one quantizer launch
+  per distinct input instead of one per Linear, with bit-identical outputs. Returns
+  the number of Linears switched."""
+  n = 0
+  for m in module.modules():
+    if isinstance(m, Fp8DynamicLinear):
+      m.share_input_quant = bool(enable)
+      n += 1
+  if not enable:
+    ops.clear_shared_activation_quant()
+  return n
 
 
 def dequantize_weight(linear: _Fp8LinearBase) -> torch.Tensor:

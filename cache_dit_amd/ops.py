@@ -130,6 +130,61 @@ def w8a16_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
         w.stride(0), out.stride(0), epilogue, _native.DT_BF16, _stream_ptr(x2)))
 
 
+class _SharedQuant:
+  """Last activation quantized on a (device, stream): the input view (kept alive, so
+  its storage cannot be freed and handed out again), its version counter, and the
+  codes / scales computed from it."""
+  __slots__ = ("x", "version", "mode", "q", "s")
+
+
+_shared_quant: dict = {}
+quant_launches = 0  # quantizer launches issued through shared_activation_quant (for tests)
+
+
+def shared_activation_quant(x2: torch.Tensor, scale_mode_id: int):
+  """Codes and scales of `x2` [M,K], reusing the previous result when the same
+  buffer (storage, offset, shape, strides), unmodified since (same `_version`), is
+  quantized again on the same stream -- sibling Linears such as to_q / to_k / to_v
+  (and proj_mlp in FLUX single blocks) all read one normalized activation
+  (reference dataflow: src/cache_dit/caching/patch_functors/functor_flux.py:60-67).
+  The results are bit-identical to quantizing again. In-place changes made through
+  PyTorch bump `_version` and miss; writes by foreign kernels into a live input
+  between two sibling calls would not be seen, which is why sharing is opt-in."""
+  global quant_launches
+  dev = x2.device
+  if x2.is_inference():
+    # inference-mode tensors carry no version counter: an in-place change could not be
+    # told from an unchanged buffer, so nothing is shared (torch.no_grad() keeps it)
+    M, K = x2.shape
+    q = torch.empty((M, K), dtype=FP8, device=dev)
+    s = torch.empty((M, ), dtype=torch.float32, device=dev)
+    quant_rowwise_into(x2, q, s, scale_mode_id)
+    quant_launches += 1
+    return q, s
+  key = (dev.index, torch._C._cuda_getCurrentRawStream(dev.index),
+         torch.cuda.is_current_stream_capturing())
+  e = _shared_quant.get(key)
+  if (e is not None and e.mode == scale_mode_id and e.version == x2._version
+      and e.x.data_ptr() == x2.data_ptr() and e.x.shape == x2.shape
+      and e.x.stride() == x2.stride()
+      and e.x.untyped_storage().data_ptr() == x2.untyped_storage().data_ptr()):
+    return e.q, e.s
+  M, K = x2.shape
+  q = torch.empty((M, K), dtype=FP8, device=dev)
+  s = torch.empty((M, ), dtype=torch.float32, device=dev)
+  quant_rowwise_into(x2, q, s, scale_mode_id)
+  quant_launches += 1
+  if e is None:
+    e = _SharedQuant()
+    _shared_quant[key] = e
+  e.x, e.version, e.mode, e.q, e.s = x2, x2._version, scale_mode_id, q, s
+  return q, s
+
+
+def clear_shared_activation_quant() -> None:
+  _shared_quant.clear()
+
+
 def linear_w8a8_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
                      bias: Optional[torch.Tensor], out: torch.Tensor, q_ws: torch.Tensor,
                      s_ws: torch.Tensor, scale_mode_id: int, epilogue: int) -> None:

@@ -179,6 +179,44 @@ def test_small_flux_like_step_cosine_vs_oracle_ops():
   assert cosine(y_fused, y_ref) >= 0.999
 
 
+def test_shared_activation_quant_is_bit_identical_and_saves_launches():
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd import ops
+  from cache_dit_amd.testing import dit_shapes as ds
+  torch.manual_seed(0)
+  kw = dict(dim=512, heads=4, mlp=2048, n_double=2, n_single=3, in_channels=64, text_dim=256,
+            pooled_dim=128)
+  model = ds.FluxLikeTransformer(**kw).to(torch.bfloat16).cuda()
+  cache_dit.quantize(model, cache_dit.QuantizeConfig())
+  inputs = ds.flux_like_inputs("cuda", n_img=320, n_txt=64, in_channels=64, text_dim=256,
+                               pooled_dim=128)
+  with torch.inference_mode():
+    y0 = model(**inputs)
+  n = cache_dit.share_activation_quant_(model)
+  assert n == 2 * 14 + 3 * 6
+  ops.quant_launches = 0
+  with torch.no_grad():
+    y1 = model(**inputs)
+    y2 = model(**inputs)
+  assert torch.equal(y0, y1) and torch.equal(y0, y2)
+  # per double block: q/k/v share (img), add_q/k/v share (txt), the other 8 do not: 10 of 14;
+  # per single block: proj_mlp + q/k/v share, proj_out and norm.linear do not: 3 of 6
+  assert ops.quant_launches == 2 * (2 * 10 + 3 * 3), ops.quant_launches
+  ops.quant_launches = 0
+  with torch.inference_mode():  # no version counters there: nothing is shared
+    y3 = model(**inputs)
+  assert torch.equal(y0, y3) and ops.quant_launches == 2 * 14 + 3 * 6
+  # an in-place change of the shared input must not reuse stale codes
+  lin = model.single_transformer_blocks[0].attn.to_q
+  x = torch.randn(64, 512, device="cuda").to(torch.bfloat16)
+  with torch.no_grad():
+    a = lin(x)
+    x.mul_(2.0)
+    b = lin(x)
+  cache_dit.share_activation_quant_(model, False)
+  assert torch.equal(b, lin(x)) and not torch.equal(a, b)
+
+
 def test_full_flux_shaped_step_cosine():
   """BASELINE config 2 at full size (19 + 38 blocks, 4096 + 512 tokens): the HIP
   path against the oracle's arithmetic in torch ops on the same GPU, and against
