@@ -264,9 +264,9 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_tiled(GemmArgs g, int til
 // The 1 KiB DMA instructions of a step (A panel first, then B) are dealt to the
 // waves round-robin; when their number is not a multiple of 8 the first waves
 // issue one more than the others, and each wave counts its own (D) for s_waitcnt.
-template <int BM_, int BN_, int STAGES_, bool EPI_LDS_, int GROUP_M_>
+template <int BM_, int BN_, int STAGES_, bool EPI_LDS_, int GROUP_M_, int WGM_ = 2>
 struct CfgPP {
-  static constexpr int BM = BM_, BN = BN_, STAGES = STAGES_, WGM = 2, WGN = 4;
+  static constexpr int BM = BM_, BN = BN_, STAGES = STAGES_, WGM = WGM_, WGN = 8 / WGM_;
   static constexpr bool EPI_LDS = EPI_LDS_;
   static constexpr int GROUP_M = GROUP_M_;
   static constexpr int WAVES = 8, THREADS = 512;
@@ -355,7 +355,8 @@ __global__ __launch_bounds__(C::THREADS, 2) void gemm_fp8_pingpong(GemmArgs g, i
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave / C::WGN, wn = wave % C::WGN;  // wm is also the ping-pong group
+  const int wm = wave / C::WGN, wn = wave % C::WGN;
+  const int group = wave >> 2;  // ping-pong group: waves 0-3 and 4-7, one of each per SIMD
   constexpr int BKP = C::BKP;
 
   int tm, tn;
@@ -398,12 +399,12 @@ __global__ __launch_bounds__(C::THREADS, 2) void gemm_fp8_pingpong(GemmArgs g, i
 
   const int KT = g.K / BKP;
   if constexpr (C::NT % C::WAVES == 0) {
-    pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
+    pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, group, rd_a, rd_b);
   } else {
     if (wave < C::NT % C::WAVES) {
-      pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
+      pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, group, rd_a, rd_b);
     } else {
-      pingpong_loop<C, C::DMAX - 1>(acc, smem, A, B, off, KT, wave, wm, rd_a, rd_b);
+      pingpong_loop<C, C::DMAX - 1>(acc, smem, A, B, off, KT, wave, group, rd_a, rd_b);
     }
   }
 
@@ -565,6 +566,7 @@ typedef Cfg<64, 128, 2, 2, true, true, 8, 4> V21;
 typedef CfgPP<256, 256, 4, true, 8> V8;               // ping-pong, 4 stages of 64 B
 typedef CfgPP<256, 256, 4, false, 8> V9;              // ... with direct 8-byte stores
 typedef CfgPP<192, 384, 4, true, 8> V10;              // ping-pong, 96x96 wave tiles
+typedef CfgPP<256, 192, 4, true, 8, 4> V11;           // ping-pong, 64x96 wave tiles (4x2 waves)
 
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {
@@ -582,16 +584,24 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   }
   if (variant < 0) {
     // Cost model: full rounds over the 256 CUs times the tile area. With enough
-    // 256x256 tiles to fill the chip, take whichever of 256x256 and 192x384 needs
-    // fewer CU-rounds of work (ties to 256x256); smaller problems take smaller
+    // 256x256 tiles to fill most of the chip, take whichever of 256x256, 192x384 and
+    // 256x192 needs the fewest CU-rounds of work (ties to the larger tile, which is
+    // the more efficient one per tile); smaller problems take smaller
     // tiles: 128x128 (two workgroups per CU) when those fill the chip, else 64x128
     // with a 4-deep DMA pipeline.
     auto tiles = [&](int bm, int bn) {
       return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
     };
     auto cost = [&](int bm, int bn) { return ((tiles(bm, bn) + 255) / 256) * bm * bn; };
-    if (tiles(256, 256) >= 200) {
-      variant = cost(192, 384) < cost(256, 256) ? 10 : 8;
+    if (tiles(256, 256) >= 160) {
+      // 256x256, or 192x384 / 256x192 when they need strictly fewer CU-rounds of work
+      variant = 8;
+      int64_t best = cost(256, 256);
+      if (cost(192, 384) < best) {
+        best = cost(192, 384);
+        variant = 10;
+      }
+      if (cost(256, 192) < best) variant = 11;
     } else if (tiles(128, 128) >= 256) {
       variant = 6;
     } else {
@@ -608,6 +618,7 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     case 8: return launch_pingpong<V8>(g, stream);
     case 9: return launch_pingpong<V9>(g, stream);
     case 10: return launch_pingpong<V10>(g, stream);
+    case 11: return launch_pingpong<V11>(g, stream);
     default:
       set_error("cdit_fp8_gemm_rowwise: unknown kernel variant %d", variant);
       return CDIT_EINVAL;

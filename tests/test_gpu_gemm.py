@@ -49,7 +49,7 @@ def _assert_close(out, ref):
   assert elementwise_ok(out, ref, REL_TOL)
 
 
-TILED_VARIANTS = [0, 1, 6, 7, 8, 9, 10, 20, 21]
+TILED_VARIANTS = [0, 1, 6, 7, 8, 9, 10, 11, 20, 21]
 
 
 @pytest.mark.parametrize("variant", TILED_VARIANTS + [100])
@@ -141,6 +141,26 @@ def test_reference_partition_shape_m512_k3072_n3072():
   # tests/kernels/test_rowwise_cudagraph_partition.py:35-37 of the reference
   p = _rand_problem(512, 3072, 3072, seed=2)
   _assert_close(_run(*p), to.scaled_mm_rowwise(*p))
+
+
+@pytest.mark.parametrize("M,N,K", [(6889, 3072, 3072), (6889, 12288, 3072), (32760, 5120, 5120),
+                                   (32760, 13824, 5120), (4608, 3072, 15360)])
+def test_qwen_and_wan_shapes_sampled_rows(M, N, K):
+  """Odd token counts of the other BASELINE models (Qwen-Image 6889 = 83 x 83, Wan
+  32760 = 8 x 4095) at full size: every 97th row plus the last rows against the oracle."""
+  from cache_dit_amd import ops
+  g = torch.Generator(device="cuda").manual_seed(M + N)
+  x = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
+  w = (torch.randn(N, K, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+  b = (torch.randn(N, generator=g, device="cuda") * 0.01).to(torch.bfloat16)
+  xq, xs = ops.fp8_rowwise_quant(x)
+  wq, ws = ops.fp8_rowwise_quant(w)
+  out = ops.float8_inference_scaled_mm(xq, xs, wq.t(), ws.t(), torch.bfloat16, bias=b)
+  rows = torch.cat([torch.arange(0, M, 97), torch.arange(M - 3, M)])
+  ref = to.scaled_mm_rowwise(xq[rows.cuda()].cpu(), xs[rows.cuda()].cpu(), wq.cpu(), ws.cpu(),
+                             b.cpu())
+  _assert_close(out[rows.cuda()], ref)
+  assert torch.isfinite(out.float()).all()
 
 
 def test_config1_full():

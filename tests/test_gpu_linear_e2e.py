@@ -217,6 +217,36 @@ def test_shared_activation_quant_is_bit_identical_and_saves_launches():
   assert torch.equal(b, lin(x)) and not torch.equal(a, b)
 
 
+def test_linear_forward_under_hip_graph_capture():
+  """A captured forward replays correctly with new input data (no allocation-order or
+  stream assumptions in the launch path); every replay is checked against eager, with
+  eager work and synchronisation between the replays."""
+  import cache_dit_amd as cache_dit
+  torch.manual_seed(0)
+  net = _Net().to(torch.bfloat16).cuda()
+  cache_dit.quantize(net, cache_dit.QuantizeConfig())
+  static_x = torch.randn(3, 70, 256, device="cuda").to(torch.bfloat16)
+  with torch.no_grad():
+    net(static_x)  # warm-up outside capture (sets kernel attributes)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+      net(static_x)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+      static_y = net(static_x)
+    for seed in range(4):
+      new_x = torch.randn(3, 70, 256, device="cuda",
+                          generator=torch.Generator(device="cuda").manual_seed(seed)).to(torch.bfloat16)
+      expect = net(new_x)  # eager, also between replays
+      torch.cuda.synchronize()
+      static_x.copy_(new_x)
+      graph.replay()
+      torch.cuda.synchronize()
+      assert torch.equal(static_y, expect), f"replay {seed} differs from eager"
+
+
 def test_full_flux_shaped_step_cosine():
   """BASELINE config 2 at full size (19 + 38 blocks, 4096 + 512 tokens): the HIP
   path against the oracle's arithmetic in torch ops on the same GPU, and against
