@@ -344,6 +344,87 @@ int launch_pingpong(const GemmArgs& g, hipStream_t stream) {
   return 0;
 }
 
+// ---------------------------------------------------------------------------
+// Skinny kernel for M <= 16 (M = 1 modulation Linears): weight streaming. A
+// workgroup of 4 waves owns 16 output channels, each wave a quarter of K. Per
+// 128-element chunk a lane (weight row l&15, K group l>>4) loads 32 e4m3 bytes
+// straight from HBM and the matching 32 bf16 activations (zero for rows >= M),
+// converts the weights to bf16 and issues four v_mfma_f32_16x16x32_bf16; the four
+// partial tiles are summed through LDS.
+__global__ __launch_bounds__(256) void gemm_w8a16_skinny(GemmArgs g) {
+  __shared__ float part[4][16][17];
+  typedef float v4f_ __attribute__((ext_vector_type(4)));
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, kg = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int nrow = min(n0 + r, g.N - 1);
+  const int KT = g.K / 128;
+  const int per = (KT + 3) / 4;
+  const int k_begin = wave * per, k_end = min(KT, k_begin + per);
+  const uint8_t* __restrict__ wp = g.b + (int64_t)nrow * g.ldb + kg * 32;
+  const uint16_t* __restrict__ ap =
+      static_cast<const uint16_t*>(g.a) + (int64_t)min(r, g.M - 1) * g.lda + kg * 32;
+  const bool a_valid = r < g.M;
+  v4f_ acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  constexpr int U = 3;  // chunks in flight
+  for (int k0 = k_begin; k0 < k_end; k0 += U) {
+    uint4 w[U][2];
+    v8bf a[U][4];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kt = min(k0 + u, k_end - 1);
+      const uint4* wq = reinterpret_cast<const uint4*>(wp + (int64_t)kt * 128);
+      w[u][0] = wq[0];
+      w[u][1] = wq[1];
+      const v8bf* aq = reinterpret_cast<const v8bf*>(ap + (int64_t)kt * 128);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) a[u][t] = aq[t];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (k0 + u < k_end) {
+        const uint32_t words[8] = {w[u][0].x, w[u][0].y, w[u][0].z, w[u][0].w,
+                                   w[u][1].x, w[u][1].y, w[u][1].z, w[u][1].w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const v2bf c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(words[2 * t], 1.0f, false);
+          const v2bf c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(words[2 * t], 1.0f, true);
+          const v2bf c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(words[2 * t + 1], 1.0f, false);
+          const v2bf c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(words[2 * t + 1], 1.0f, true);
+          const v8bf wf = {c0[0], c0[1], c1[0], c1[1], c2[0], c2[1], c3[0], c3[1]};
+          v8bf af = a[u][t];
+          if (!a_valid) af = v8bf{0, 0, 0, 0, 0, 0, 0, 0};
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af, acc, 0, 0, 0);
+        }
+      }
+    }
+  }
+  // acc[e] = partial out[m = lane&15][n0 + 4*(lane>>4) + e]
+#pragma unroll
+  for (int e = 0; e < 4; ++e) part[wave][r][4 * kg + e] = acc[e];
+  __syncthreads();
+  if (wave == 0) {
+    const int m = r, nl = 4 * kg;
+    if (m < g.M && n0 + nl < g.N) {
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float sum = (part[0][m][nl + e] + part[1][m][nl + e]) +
+                          (part[2][m][nl + e] + part[3][m][nl + e]);
+        const int n = n0 + nl + e;
+        float t = sum * g.b_scale[n];
+        if (g.bias) t += __uint_as_float((uint32_t)g.bias[n] << 16);
+        if (g.epilogue & CDIT_EPI_GELU_TANH) t = gelu_tanh(t);
+        v[e] = t;
+      }
+      uint2 pk;
+      pk.x = pack_bf16x2(v[0], v[1]);
+      pk.y = pack_bf16x2(v[2], v[3]);
+      *reinterpret_cast<uint2*>(g.out + (int64_t)m * g.ldo + n0 + nl) = pk;
+    }
+  }
+}
+
 // Any shape: one output element per thread, scalar decode + FMA.
 __global__ __launch_bounds__(256) void gemm_w8a16_generic(GemmArgs g) {
   const int n = blockIdx.x * 16 + (threadIdx.x & 15);
@@ -401,6 +482,14 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {
     dim3 grid((g.N + 15) / 16, (g.M + 15) / 16);
     hipLaunchKernelGGL(gemm_w8a16_generic, grid, dim3(256), 0, stream, g);
+    return 0;
+  }
+  if ((variant < 0 && g.M <= 16 && g.K % 128 == 0) || variant == 50) {
+    if (g.M > 16 || g.K % 128 != 0) {
+      set_error("cdit_w8a16_gemm: the skinny kernel takes M <= 16 and K %% 128 == 0");
+      return CDIT_EINVAL;
+    }
+    hipLaunchKernelGGL(gemm_w8a16_skinny, dim3((g.N + 15) / 16), dim3(256), 0, stream, g);
     return 0;
   }
   if (variant < 0) {

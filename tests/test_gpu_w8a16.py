@@ -68,6 +68,36 @@ def test_exact_small_integers(variant):
   assert torch.equal(out.cpu(), to.w8a16_linear(x, w, ws, fused=True))
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 18432, 3072), (1, 9216, 3072), (3, 264, 384), (16, 512, 128)])
+@pytest.mark.parametrize("gelu", [0, 1])
+def test_skinny_kernel(M, N, K, gelu):
+  from cache_dit_amd import _native
+  x, wq, ws, b = _problem(M, N, K, seed=M * 5 + N + K)
+  ws = ws * (8 if gelu else 1)
+  ref = to.w8a16_linear(x, wq, ws, b, gelu="fused" if gelu else None, fused=True)
+  _assert_close(_run(x, wq, ws, b, epilogue=gelu), ref)
+  _native.set_gemm_variant(50)
+  _assert_close(_run(x, wq, ws, b, epilogue=gelu), ref)
+
+
+def test_skinny_exact_and_every_code():
+  from cache_dit_amd import _native
+  g = torch.Generator().manual_seed(14)
+  M, N, K = 5, 272, 1024
+  x = torch.randint(-4, 5, (M, K), generator=g).to(torch.bfloat16)
+  w = torch.randint(-4, 5, (N, K), generator=g).float().to(FP8)
+  ws = torch.full((N, 1), 0.25)
+  _native.set_gemm_variant(50)
+  assert torch.equal(_run(x, w, ws, None).cpu(), to.w8a16_linear(x, w, ws, fused=True))
+  # K positions: one-hot activations pick single weights whose value encodes K
+  x = torch.zeros(M, K)
+  x[torch.arange(M), torch.tensor([0, 33, 130, 517, 1023])] = 1.0
+  w = ((torch.arange(K) % 15) + 1).float().repeat(N, 1).to(FP8)
+  ones = torch.ones(N, 1)
+  assert torch.equal(_run(x.to(torch.bfloat16), w, ones, None).cpu(),
+                     to.w8a16_linear(x.to(torch.bfloat16), w, ones, fused=True))
+
+
 def test_k_position_sensitivity():
   M, N, K = 256, 256, 256
   x = torch.zeros(M, K)
