@@ -26,6 +26,8 @@
 //
 // Replaces torch._scaled_mm as called at
 // src/cache_dit/quantization/torchao/_scaled_mm.py:62-91.
+#include <type_traits>
+
 #include "gemm_common.h"
 
 namespace cdit {
@@ -433,6 +435,289 @@ int launch_pingpong(const GemmArgs& g, hipStream_t stream) {
 }
 
 // ---------------------------------------------------------------------------
+// Wide kernel: 256x256 tile, 4 waves (one per SIMD, up to 512 registers each), each
+// owning a 128x128 wave tile as 8x8 blocks of v_mfma_f32_16x16x128_f8f6f4 (8 passes;
+// one wave alone keeps the matrix core busy with it, which the 16-pass 32x32x64
+// does not). K advances in 128-byte steps through two LDS stages filled by LDS-DMA.
+// A wave holds all 16 operand fragments of a step in registers (A_i: rows 16i..16i+15
+// of its half of the A panel, B_j likewise), so every panel byte is read from LDS
+// once per wave: 32 KiB per wave and step for 64 MFMAs.
+//
+// The A panel has three LDS stages and the B panel two. Step kt:
+//   rows 0..H-1, i-major:  MFMA(i, 0..TN-1); meanwhile read the remaining A
+//                          fragments of step kt, and issue the A-panel DMA of step
+//                          kt+2 (into the stage that step kt-1 read)
+//   wait (own LDS reads; own DMA of step kt+1, not the A panel just issued),
+//   workgroup barrier: the B stage of step kt is now free, step kt+1 is in LDS
+//   rows H..TM-1, j-major: MFMA(H..TM-1, j), then B_j is dead: read B_j of step
+//                          kt+1; A_0 of step kt+1 likewise; the B-panel DMA of step
+//                          kt+2 is issued in between
+// One barrier per step, in the middle of the MFMA stream. Spreading the DMA over
+// both halves matters: a CU's vector memory path moves 64 B per clock, a step
+// needs (BM + BN) * 128 B through it against TM * TN * 32 clocks of MFMA per wave,
+// and a wave that cannot issue its DMA cannot issue its MFMAs either.
+//
+// Panel rows are 128 B = 8 chunks of 16 B. An operand read takes row (lane & 15),
+// chunks 2*(lane >> 4) + {0, 1}; the LDS serves 16 lanes per pass (lane bit 5 and
+// the parity of lane bits 2..4 select the pass), and chunk c of row r stored at
+// c ^ swz(r) with swz = (bit 1 of r) | 6 * (bit 3 of r) makes every pass hit 16
+// distinct 16-byte bank groups. The B fragments take their 16 rows in a permuted
+// order, fragment j = 4t + q, operand row p:
+//     n = 64 t + 32 (q >> 1) + 8 (p >> 2) + 4 (q & 1) + (p & 3)
+// so that a lane ends with 8 consecutive output columns per pair of fragments and
+// stores 16 bytes without a transpose (4 lanes cover 64 contiguous bytes of a row);
+// for those rows lane bit 3 is row bit 4, hence swz_b.
+template <int BM_, int BN_, int GROUP_M_>
+struct CfgWide {
+  static constexpr int BM = BM_, BN = BN_, GROUP_M = GROUP_M_;
+  static constexpr int WAVES = 4, THREADS = 256;
+  static constexpr int WM = BM / 2, WN = BN / 2;      // wave tile (2 x 2 waves)
+  static constexpr int TM = WM / 16, TN = WN / 16;    // 16x16 MFMA blocks per wave
+  static constexpr int H = TM / 2;                    // rows of the first (i-major) half
+  static constexpr int BKW = 128;
+  static constexpr int A_BYTES = BM * BKW, B_BYTES = BN * BKW;
+  // A panel: 3 LDS stages (its DMA goes out in the first half of a step, into the
+  // stage read one step earlier); B panel: 2 stages (DMA in the second half)
+  static constexpr int A_STAGES = 3, B_STAGES = 2;
+  static constexpr int B_BASE = A_STAGES * A_BYTES;
+  static constexpr int LDS_BYTES = A_STAGES * A_BYTES + B_STAGES * B_BYTES;
+  // DMA instructions (1 KiB = 8 panel rows) per wave and step
+  static constexpr int NDA = BM / 8 / WAVES, NDB = BN / 8 / WAVES, ND = NDA + NDB;
+  static_assert(WM % 16 == 0 && WN % 32 == 0, "wave tile: 16-row A fragments, B fragments in pairs");
+  static_assert(BM % 32 == 0 && BN % 32 == 0, "panels are dealt 8 rows x 4 waves at a time");
+  static_assert(TM * TN <= 64, "accumulators: at most 256 registers");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+};
+
+__device__ __forceinline__ int swz_a(int row) { return ((row >> 1) & 1) | (((row >> 3) & 1) * 6); }
+__device__ __forceinline__ int swz_b(int row) { return ((row >> 1) & 1) | (((row >> 4) & 1) * 6); }
+
+// acc += B-fragment x A-fragment. Inline assembly with the accumulator tied to an
+// AGPR tuple: with the builtin the register allocator now and then gives source and
+// destination accumulators different registers and copies them through VGPRs
+// inside the loop (all 256 AGPRs hold accumulators, there is no room to shuffle).
+// The compiler does not know this is an MFMA, so the code that reads the
+// accumulators afterwards (the epilogue) waits for the matrix core itself.
+__device__ __forceinline__ void mfma_16x16x128_fp8(v4f& acc, const v8i& b, const v8i& a) {
+  asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+}
+
+template <class C>
+__global__ __launch_bounds__(C::THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void
+gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  // wave-uniform on purpose: LDS-DMA destinations (M0) then come from scalar code
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  constexpr int BKW = C::BKW, TM = C::TM, TN = C::TN, H = C::H;
+
+  int tm, tn;
+  tile_of_block<C::GROUP_M>(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
+  const int m0 = tm * C::BM, n0 = tn * C::BN;
+  const uint8_t* __restrict__ A = static_cast<const uint8_t*>(g.a) + (int64_t)m0 * g.lda;
+  const uint8_t* __restrict__ B = g.b + (int64_t)n0 * g.ldb;
+  const int rows_a = g.M - m0, rows_b = g.N - n0;
+
+  // DMA map: instruction p of this wave fills 8 panel rows (1 KiB): rows
+  // 8 (wave + 4p) of the A panel for p < NDA, of the B panel after that. Lane l
+  // lands on row l/8, position l%8 and fetches the logical chunk that the swizzle
+  // stores there.
+  uint32_t off[C::ND];
+#pragma unroll
+  for (int p = 0; p < C::ND; ++p) {
+    const bool is_a = p < C::NDA;
+    const int row = (wave + 4 * (is_a ? p : p - C::NDA)) * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ (is_a ? swz_a(row) : swz_b(row));
+    off[p] = is_a ? (uint32_t)min(row, rows_a - 1) * (uint32_t)g.lda + c * 16
+                  : (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
+  }
+  // buffer_load ... lds (MUBUF form: the compiler tracks it with vmcnt only, while
+  // the global_load form makes it wait for all LDS reads at every use). A step past
+  // the end of K gets a descriptor of zero records: every lane is then out of range,
+  // nothing is fetched and zeros land in a free stage, so the loop body needs no
+  // special cases for its last two steps.
+  const int KT = g.K / BKW;
+  auto dma_a = [&](int kt, int a_lds, int p) {
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(A), 0, kt < KT ? 0x7fffffff : 0, 0x00020000);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        rsrc, (__attribute__((address_space(3))) void*)(smem + a_lds + (wave + 4 * p) * 1024), 16,
+        (int)off[p], kt * BKW, 0, 0);
+  };
+  auto dma_b = [&](int kt, int b_lds, int p) {
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(B), 0, kt < KT ? 0x7fffffff : 0, 0x00020000);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        rsrc, (__attribute__((address_space(3))) void*)(smem + b_lds + (wave + 4 * p) * 1024), 16,
+        (int)off[C::NDA + p], kt * BKW, 0, 0);
+  };
+
+  // operand read map
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int brow = 8 * (r16 >> 2) + (r16 & 3);
+  uint32_t rd_a[2], rd_b[2];
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    rd_a[e] = (wm * C::WM + r16) * BKW + (((2 * kg + e) ^ swz_a(wm * C::WM + r16)) << 4);
+    rd_b[e] = (wn * C::WN + brow) * BKW + (((2 * kg + e) ^ swz_b(wn * C::WN + brow)) << 4);
+  }
+  auto read_a = [&](const uint8_t* st, int i) -> v8i {
+    const v4i lo = *reinterpret_cast<const v4i*>(st + rd_a[0] + i * 16 * BKW);
+    const v4i hi = *reinterpret_cast<const v4i*>(st + rd_a[1] + i * 16 * BKW);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  auto read_b = [&](const uint8_t* st, int j) -> v8i {
+    const int ro = 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
+    const v4i lo = *reinterpret_cast<const v4i*>(st + rd_b[0] + ro * BKW);
+    const v4i hi = *reinterpret_cast<const v4i*>(st + rd_b[1] + ro * BKW);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+
+  v4f acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+  v8i af[TM], bf[TN];
+
+  // LDS offsets of the stages of steps kt-1 / kt / kt+1 (A) and kt / kt+1 (B)
+  int a_prev = 2 * C::A_BYTES, a_cur = 0, a_next = C::A_BYTES;
+  int b_cur = C::B_BASE, b_next = C::B_BASE + C::B_BYTES;
+  // prologue: steps 0 and 1 in flight, step 0 landed, its B fragments and A_0 read
+#pragma unroll
+  for (int p = 0; p < C::NDA; ++p) dma_a(0, a_cur, p);
+#pragma unroll
+  for (int p = 0; p < C::NDB; ++p) dma_b(0, b_cur, p);
+#pragma unroll
+  for (int p = 0; p < C::NDA; ++p) dma_a(1, a_next, p);
+#pragma unroll
+  for (int p = 0; p < C::NDB; ++p) dma_b(1, b_next, p);
+  wait_and_barrier<C::ND>();
+#pragma unroll
+  for (int j = 0; j < TN; ++j) bf[j] = read_b(smem + b_cur, j);
+  af[0] = read_a(smem + a_cur, 0);
+
+  for (int kt = 0; kt < KT; ++kt) {
+    const uint8_t* st = smem + a_cur;
+#pragma unroll
+    for (int i = 0; i < H; ++i) {
+      // A panel of step kt+2 into the stage that step kt-1 read, spread over the rows
+#pragma unroll
+      for (int p = 0; p < C::NDA; ++p)
+        if (p * H / C::NDA == i) dma_a(kt + 2, a_prev, p);
+      if (i + 1 < H) af[i + 1] = read_a(st, i + 1);
+      // the TM-H fragments of the second half, spread over the rows of the first
+#pragma unroll
+      for (int k = 0; k < TM - H; ++k)
+        if (k * H / (TM - H) == i) af[H + k] = read_a(st, H + k);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        mfma_16x16x128_fp8(acc[i][j], bf[j], af[i]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // own LDS reads of this step done, own DMA of step kt+1 landed (the A panel of
+    // step kt+2, issued above, may still fly); then everyone's
+    wait_and_barrier<C::NDA>();
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      // B panel of step kt+2 into the B stage of step kt, spread over the columns
+#pragma unroll
+      for (int p = 0; p < C::NDB; ++p)
+        if (p * TN / C::NDB == j) dma_b(kt + 2, b_cur, p);
+#pragma unroll
+      for (int i = H; i < TM; ++i)
+        mfma_16x16x128_fp8(acc[i][j], bf[j], af[i]);
+      // fragments of step kt+1 (after the last step: zeros, never used)
+      bf[j] = read_b(smem + b_next, j);
+      if (j == 0) af[0] = read_a(smem + a_next, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // rotate the stages
+    const int a_free = a_prev;
+    a_prev = a_cur;
+    a_cur = a_next;
+    a_next = a_free;
+    const int b_free = b_cur;
+    b_cur = b_next;
+    b_next = b_free;
+  }
+  // the zero-record DMA of the last two steps must not outlive the workgroup
+  wait_vm<0>();
+  // the last MFMAs (8 passes each) must have written their accumulators
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- epilogue: acc[i][4t+q][e] is out[m][n] with
+  //   m = m0 + wm*WM + 16i + (lane&15),
+  //   n = n0 + wn*WN + 64t + 32(q>>1) + 8(lane>>4) + 4(q&1) + e
+  const bool gelu = (g.epilogue & CDIT_EPI_GELU_TANH) != 0;
+  const int nw = n0 + wn * C::WN + 8 * kg;
+  const int mw = m0 + wm * C::WM + r16;
+  v4f bs[TN], bi[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = nw + 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
+    bs[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    bi[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    if (n < g.N) {
+      bs[j] = *reinterpret_cast<const v4f*>(g.b_scale + n);
+      if (g.bias) {
+        const uint2 bb = *reinterpret_cast<const uint2*>(g.bias + n);
+        bi[j][0] = __uint_as_float(bb.x << 16);
+        bi[j][1] = __uint_as_float(bb.x & 0xffff0000u);
+        bi[j][2] = __uint_as_float(bb.y << 16);
+        bi[j][3] = __uint_as_float(bb.y & 0xffff0000u);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = mw + 16 * i;
+    const float as = m < g.M ? g.a_scale[m] : 0.0f;
+#pragma unroll
+    for (int u = 0; u < TN / 2; ++u) {  // pair of fragments 2u, 2u+1: 8 consecutive columns
+      uint32_t pk[4];
+#pragma unroll
+      for (int d = 0; d < 2; ++d) {
+        const int j = 2 * u + d;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = __fmaf_rn(acc[i][j][e] * as, bs[j][e], bi[j][e]);
+          if (gelu) v[e] = gelu_tanh(v[e]);
+        }
+        pk[2 * d] = pack_bf16x2(v[0], v[1]);
+        pk[2 * d + 1] = pack_bf16x2(v[2], v[3]);
+      }
+      const int n = nw + 64 * (u >> 1) + 32 * (u & 1);
+      if (m < g.M && n < g.N)
+        *reinterpret_cast<uint4*>(g.out + (int64_t)m * g.ldo + n) =
+            uint4{pk[0], pk[1], pk[2], pk[3]};
+    }
+  }
+}
+
+template <class C>
+int launch_wide(const GemmArgs& g, hipStream_t stream) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_fp8_wide<C>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(%d bytes LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
+      return CDIT_EHIP;
+    }
+    attr_set = true;
+  }
+  const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
+  hipLaunchKernelGGL(gemm_fp8_wide<C>, dim3(tiles_m * tiles_n), dim3(C::THREADS), C::LDS_BYTES,
+                     stream, g, tiles_m, tiles_n);
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
 // Skinny kernel for M <= 16 (the M = 1 modulation Linears `norm1.linear`,
 // `norm.linear` of every block): pure weight streaming. A workgroup of 4 waves
 // owns 16 output channels; each wave takes a quarter of K and reads its weight
@@ -567,6 +852,9 @@ typedef CfgPP<256, 256, 4, true, 8> V8;               // ping-pong, 4 stages of 
 typedef CfgPP<256, 256, 4, false, 8> V9;              // ... with direct 8-byte stores
 typedef CfgPP<192, 384, 4, true, 8> V10;              // ping-pong, 96x96 wave tiles
 typedef CfgPP<256, 192, 4, true, 8, 4> V11;           // ping-pong, 64x96 wave tiles (4x2 waves)
+typedef CfgWide<256, 256, 8> V12;                     // 4 waves, 128x128 wave tiles, 16x16x128 MFMA
+typedef CfgWide<288, 192, 8> V14;                     // ... 144x96 wave tiles
+typedef CfgWide<256, 192, 8> V15;                     // ... 128x96 wave tiles
 
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {
@@ -583,25 +871,31 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     return 0;
   }
   if (variant < 0) {
-    // Cost model: full rounds over the 256 CUs times the tile area. With enough
-    // 256x256 tiles to fill most of the chip, take whichever of 256x256, 192x384 and
-    // 256x192 needs the fewest CU-rounds of work (ties to the larger tile, which is
-    // the more efficient one per tile); smaller problems take smaller
-    // tiles: 128x128 (two workgroups per CU) when those fill the chip, else 64x128
-    // with a 4-deep DMA pipeline.
+    // Large problems take one of the wide kernels. Cost model, fitted to measured
+    // times: tile area times the number of rounds over the 256 CUs, where a last,
+    // partial round of r tiles counts 0.4 + 0.6 r/256 (the chip is power limited:
+    // with fewer CUs busy the clocks rise); ties go to the larger tile. Smaller
+    // problems take 128x128 tiles (two workgroups per CU) when those fill the
+    // chip, else 64x128 with a 4-deep DMA pipeline.
     auto tiles = [&](int bm, int bn) {
       return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
     };
-    auto cost = [&](int bm, int bn) { return ((tiles(bm, bn) + 255) / 256) * bm * bn; };
+    auto cost = [&](int bm, int bn, int pen) {
+      const int64_t t = tiles(bm, bn), full = t / 256, rem = t % 256;
+      return (full * 2560 + (rem ? 1024 + 6 * rem : 0)) * bm * bn * pen;
+    };
     if (tiles(256, 256) >= 160) {
-      // 256x256, or 192x384 / 256x192 when they need strictly fewer CU-rounds of work
-      variant = 8;
-      int64_t best = cost(256, 256);
-      if (cost(192, 384) < best) {
-        best = cost(192, 384);
-        variant = 10;
+      variant = 12;
+      int64_t best = cost(256, 256, 100);
+      const struct { int v, bm, bn, pen; } cand[] = {
+          {14, 288, 192, 101}, {15, 256, 192, 102}};
+      for (const auto& c : cand) {
+        const int64_t t = cost(c.bm, c.bn, c.pen);
+        if (t < best) {
+          best = t;
+          variant = c.v;
+        }
       }
-      if (cost(256, 192) < best) variant = 11;
     } else if (tiles(128, 128) >= 256) {
       variant = 6;
     } else {
@@ -619,6 +913,9 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     case 9: return launch_pingpong<V9>(g, stream);
     case 10: return launch_pingpong<V10>(g, stream);
     case 11: return launch_pingpong<V11>(g, stream);
+    case 12: return launch_wide<V12>(g, stream);
+    case 14: return launch_wide<V14>(g, stream);
+    case 15: return launch_wide<V15>(g, stream);
     default:
       set_error("cdit_fp8_gemm_rowwise: unknown kernel variant %d", variant);
       return CDIT_EINVAL;
