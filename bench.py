@@ -283,6 +283,10 @@ def main():
   ap.add_argument("--warmup", type=int, default=3)
   ap.add_argument("--skip-cpu", action="store_true", help="skip the cpu_baseline leg")
   ap.add_argument("--skip-dit", action="store_true", help="skip the full-transformer forward")
+  ap.add_argument("--headline-only", action="store_true",
+                  help="run only the headline-shape kernels (the roofline legs) and print their "
+                       "figures: the command to put under rocprofv3 when per-kernel averages "
+                       "must not mix shapes")
   args = ap.parse_args()
   if args.gpus != 1:
     sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
@@ -294,6 +298,10 @@ def main():
   device = torch.device("cuda", 0)
   torch.cuda.set_device(device)
   arch = _native.device_arch()
+
+  if args.headline_only:
+    print(json.dumps({"linear_headline": headline_kernels(device), "device": arch}))
+    return
 
   hot = HotPath(device)
   for _ in range(args.warmup):

@@ -512,43 +512,63 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   constexpr int BKW = C::BKW, TM = C::TM, TN = C::TN, H = C::H;
+  const int KT = g.K / BKW;  // >= 2 (checked by the launcher)
+  const int ntiles = tiles_m * tiles_n;
 
-  int tm, tn;
-  tile_of_block<C::GROUP_M>(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
-  const int m0 = tm * C::BM, n0 = tn * C::BN;
-  const uint8_t* __restrict__ A = static_cast<const uint8_t*>(g.a) + (int64_t)m0 * g.lda;
-  const uint8_t* __restrict__ B = g.b + (int64_t)n0 * g.ldb;
-  const int rows_a = g.M - m0, rows_b = g.N - n0;
-
-  // DMA map: instruction p of this wave fills 8 panel rows (1 KiB): rows
-  // 8 (wave + 4p) of the A panel for p < NDA, of the B panel after that. Lane l
-  // lands on row l/8, position l%8 and fetches the logical chunk that the swizzle
-  // stores there.
-  uint32_t off[C::ND];
-#pragma unroll
-  for (int p = 0; p < C::ND; ++p) {
-    const bool is_a = p < C::NDA;
-    const int row = (wave + 4 * (is_a ? p : p - C::NDA)) * 8 + (lane >> 3);
-    const int c = (lane & 7) ^ (is_a ? swz_a(row) : swz_b(row));
-    off[p] = is_a ? (uint32_t)min(row, rows_a - 1) * (uint32_t)g.lda + c * 16
-                  : (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
+  // The workgroup is persistent: it takes tiles blockIdx.x, blockIdx.x + gridDim.x,
+  // ... and runs their K loops as one stream: the DMA of the last two steps of a
+  // tile already fetches steps 0 and 1 of the next one, and the fragments read at
+  // the end of the last step are the next tile's first. The epilogue of a tile
+  // then runs with the next tile's panels landing in LDS, and its stores drain
+  // while the next K loop is under way.
+  int m0, n0;  // tile being computed
+  {
+    int tm, tn;
+    tile_of_block<C::GROUP_M>(blockIdx.x, ntiles, tiles_m, tiles_n, &tm, &tn);
+    m0 = tm * C::BM;
+    n0 = tn * C::BN;
   }
+
+  // DMA source: tile whose panels the DMA stream currently fetches. Instruction p
+  // of this wave fills 8 panel rows (1 KiB): rows 8 (wave + 4p) of the A panel for
+  // p < NDA, of the B panel after that. Lane l lands on row l/8, position l%8 and
+  // fetches the logical chunk that the swizzle stores there.
+  const uint8_t* A;
+  const uint8_t* B;
+  uint32_t off[C::ND];
+  int nrec = 0x7fffffff;  // 0: the stream has run past the last tile, fetch nothing
+  auto set_source = [&](int sm0, int sn0) {
+    A = static_cast<const uint8_t*>(g.a) + (int64_t)sm0 * g.lda;
+    B = g.b + (int64_t)sn0 * g.ldb;
+    const int rows_a = g.M - sm0, rows_b = g.N - sn0;
+    // recomputed from the lane id at every call: opaque to the optimizer, which
+    // would otherwise keep all the row indices in registers across the K loop
+    int lrow = lane >> 3;
+    asm volatile("" : "+v"(lrow));
+#pragma unroll
+    for (int p = 0; p < C::ND; ++p) {
+      const bool is_a = p < C::NDA;
+      const int row = (wave + 4 * (is_a ? p : p - C::NDA)) * 8 + lrow;
+      const int c = (lane & 7) ^ (is_a ? swz_a(row) : swz_b(row));
+      off[p] = is_a ? (uint32_t)min(row, rows_a - 1) * (uint32_t)g.lda + c * 16
+                    : (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
+    }
+  };
+  set_source(m0, n0);
   // buffer_load ... lds (MUBUF form: the compiler tracks it with vmcnt only, while
-  // the global_load form makes it wait for all LDS reads at every use). A step past
-  // the end of K gets a descriptor of zero records: every lane is then out of range,
-  // nothing is fetched and zeros land in a free stage, so the loop body needs no
-  // special cases for its last two steps.
-  const int KT = g.K / BKW;
+  // the global_load form makes it wait for all LDS reads at every use). With a
+  // descriptor of zero records every lane is out of range: nothing is fetched and
+  // zeros land in the (free) stage, so the loop body has no special cases.
   auto dma_a = [&](int kt, int a_lds, int p) {
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(A), 0, kt < KT ? 0x7fffffff : 0, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(A), 0, nrec, 0x00020000);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(
         rsrc, (__attribute__((address_space(3))) void*)(smem + a_lds + (wave + 4 * p) * 1024), 16,
         (int)off[p], kt * BKW, 0, 0);
   };
   auto dma_b = [&](int kt, int b_lds, int p) {
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(B), 0, kt < KT ? 0x7fffffff : 0, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(B), 0, nrec, 0x00020000);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(
         rsrc, (__attribute__((address_space(3))) void*)(smem + b_lds + (wave + 4 * p) * 1024), 16,
         (int)off[C::NDA + p], kt * BKW, 0, 0);
@@ -576,10 +596,6 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
   };
 
   v4f acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
   v8i af[TM], bf[TN];
 
   // LDS offsets of the stages of steps kt-1 / kt / kt+1 (A) and kt / kt+1 (B)
@@ -595,108 +611,155 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
 #pragma unroll
   for (int p = 0; p < C::NDB; ++p) dma_b(1, b_next, p);
   wait_and_barrier<C::ND>();
-#pragma unroll
-  for (int j = 0; j < TN; ++j) bf[j] = read_b(smem + b_cur, j);
-  af[0] = read_a(smem + a_cur, 0);
 
-  for (int kt = 0; kt < KT; ++kt) {
-    const uint8_t* st = smem + a_cur;
+  for (int tile = blockIdx.x;; tile += gridDim.x) {
+    const int next_tile = tile + gridDim.x;
+    int nm0 = 0, nn0 = 0;
+    // fragments of step 0 (in LDS since the prologue, or since the barrier of the
+    // previous tile's last step). The last step of a tile reads them too, like
+    // every step does for its successor, but keeping them across the epilogue
+    // would cost 72 registers there.
 #pragma unroll
-    for (int i = 0; i < H; ++i) {
-      // A panel of step kt+2 into the stage that step kt-1 read, spread over the rows
+    for (int j = 0; j < TN; ++j) bf[j] = read_b(smem + b_cur, j);
+    af[0] = read_a(smem + a_cur, 0);
 #pragma unroll
-      for (int p = 0; p < C::NDA; ++p)
-        if (p * H / C::NDA == i) dma_a(kt + 2, a_prev, p);
-      if (i + 1 < H) af[i + 1] = read_a(st, i + 1);
-      // the TM-H fragments of the second half, spread over the rows of the first
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int k = 0; k < TM - H; ++k)
-        if (k * H / (TM - H) == i) af[H + k] = read_a(st, H + k);
+      for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int kt = 0; kt < KT; ++kt) {
+      if (kt == KT - 2) {
+        // every DMA of this tile has been issued: the stream moves on
+        if (next_tile < ntiles) {
+          int tm, tn;
+          tile_of_block<C::GROUP_M>(next_tile, ntiles, tiles_m, tiles_n, &tm, &tn);
+          nm0 = tm * C::BM;
+          nn0 = tn * C::BN;
+          set_source(nm0, nn0);
+        } else {
+          nrec = 0;
+        }
+      }
+      const int kd = kt + 2 < KT ? kt + 2 : kt + 2 - KT;  // step (of its tile) to fetch
+      const uint8_t* st = smem + a_cur;
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        mfma_16x16x128_fp8(acc[i][j], bf[j], af[i]);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int i = 0; i < H; ++i) {
+        // A panel two steps ahead into the stage that step kt-1 read, spread over the rows
+#pragma unroll
+        for (int p = 0; p < C::NDA; ++p)
+          if (p * H / C::NDA == i) dma_a(kd, a_prev, p);
+        if (i + 1 < H) af[i + 1] = read_a(st, i + 1);
+        // the TM-H fragments of the second half, spread over the rows of the first
+#pragma unroll
+        for (int k = 0; k < TM - H; ++k)
+          if (k * H / (TM - H) == i) af[H + k] = read_a(st, H + k);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) mfma_16x16x128_fp8(acc[i][j], bf[j], af[i]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // own LDS reads of this step done, own DMA of the next step landed (the A
+      // panel issued above may still fly); then everyone's. In step 0 of a later
+      // tile the DMA in question was waited for before the previous epilogue's
+      // stores, which may keep flying.
+      if (kt == 0 && tile != (int)blockIdx.x) {
+        wait_and_barrier<63>();
+      } else {
+        wait_and_barrier<C::NDA>();
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        // B panel two steps ahead into the B stage of this step, spread over the columns
+#pragma unroll
+        for (int p = 0; p < C::NDB; ++p)
+          if (p * TN / C::NDB == j) dma_b(kd, b_cur, p);
+#pragma unroll
+        for (int i = H; i < TM; ++i) mfma_16x16x128_fp8(acc[i][j], bf[j], af[i]);
+        // fragments of the next step (after the very last one: zeros, never used)
+        bf[j] = read_b(smem + b_next, j);
+        if (j == 0) af[0] = read_a(smem + a_next, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // rotate the stages
+      const int a_free = a_prev;
+      a_prev = a_cur;
+      a_cur = a_next;
+      a_next = a_free;
+      const int b_free = b_cur;
+      b_cur = b_next;
+      b_next = b_free;
     }
-    // own LDS reads of this step done, own DMA of step kt+1 landed (the A panel of
-    // step kt+2, issued above, may still fly); then everyone's
-    wait_and_barrier<C::NDA>();
+    // the last MFMAs (8 passes each) must have written their accumulators
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- epilogue: acc[i][4t+q][e] is out[m][n] with
+    //   m = m0 + wm*WM + 16i + (lane&15),
+    //   n = n0 + wn*WN + 64t + 32(q>>1) + 8(lane>>4) + 4(q&1) + e
+    const bool gelu = (g.epilogue & CDIT_EPI_GELU_TANH) != 0;
+    const int nw = n0 + wn * C::WN + 8 * kg;
+    const int mw = m0 + wm * C::WM + r16;
+    v4f bs[TN];
+    uint2 bi[TN];  // bias stays packed (bf16 pairs) until used: registers are scarce here
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      // B panel of step kt+2 into the B stage of step kt, spread over the columns
-#pragma unroll
-      for (int p = 0; p < C::NDB; ++p)
-        if (p * TN / C::NDB == j) dma_b(kt + 2, b_cur, p);
-#pragma unroll
-      for (int i = H; i < TM; ++i)
-        mfma_16x16x128_fp8(acc[i][j], bf[j], af[i]);
-      // fragments of step kt+1 (after the last step: zeros, never used)
-      bf[j] = read_b(smem + b_next, j);
-      if (j == 0) af[0] = read_a(smem + a_next, 0);
-      __builtin_amdgcn_sched_barrier(0);
+      const int n = nw + 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
+      bs[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+      bi[j] = uint2{0u, 0u};
+      if (n < g.N) {
+        bs[j] = *reinterpret_cast<const v4f*>(g.b_scale + n);
+        if (g.bias) bi[j] = *reinterpret_cast<const uint2*>(g.bias + n);
+      }
     }
-    // rotate the stages
-    const int a_free = a_prev;
-    a_prev = a_cur;
-    a_cur = a_next;
-    a_next = a_free;
-    const int b_free = b_cur;
-    b_cur = b_next;
-    b_next = b_free;
+    float as[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) as[i] = mw + 16 * i < g.M ? g.a_scale[mw + 16 * i] : 0.0f;
+    // scales and bias are here, and so is every DMA issued before them (the next
+    // tile's first two steps): from now on only this epilogue's stores are in flight
+    wait_vm<0>();
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int m = mw + 16 * i;
+#pragma unroll
+      for (int u = 0; u < TN / 2; ++u) {  // pair of fragments 2u, 2u+1: 8 consecutive columns
+        uint32_t pk[4];
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+          const int j = 2 * u + d;
+          const float b4[4] = {__uint_as_float(bi[j].x << 16), __uint_as_float(bi[j].x & 0xffff0000u),
+                               __uint_as_float(bi[j].y << 16), __uint_as_float(bi[j].y & 0xffff0000u)};
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[e] = __fmaf_rn(acc[i][j][e] * as[i], bs[j][e], b4[e]);
+            if (gelu) v[e] = gelu_tanh(v[e]);
+          }
+          pk[2 * d] = pack_bf16x2(v[0], v[1]);
+          pk[2 * d + 1] = pack_bf16x2(v[2], v[3]);
+        }
+        const int n = nw + 64 * (u >> 1) + 32 * (u & 1);
+        if (m < g.M && n < g.N)
+          *reinterpret_cast<uint4*>(g.out + (int64_t)m * g.ldo + n) =
+              uint4{pk[0], pk[1], pk[2], pk[3]};
+      }
+    }
+    if (next_tile >= ntiles) break;
+    m0 = nm0;
+    n0 = nn0;
   }
   // the zero-record DMA of the last two steps must not outlive the workgroup
   wait_vm<0>();
-  // the last MFMAs (8 passes each) must have written their accumulators
-  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-  __builtin_amdgcn_sched_barrier(0);
+}
 
-  // ---- epilogue: acc[i][4t+q][e] is out[m][n] with
-  //   m = m0 + wm*WM + 16i + (lane&15),
-  //   n = n0 + wn*WN + 64t + 32(q>>1) + 8(lane>>4) + 4(q&1) + e
-  const bool gelu = (g.epilogue & CDIT_EPI_GELU_TANH) != 0;
-  const int nw = n0 + wn * C::WN + 8 * kg;
-  const int mw = m0 + wm * C::WM + r16;
-  v4f bs[TN], bi[TN];
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int n = nw + 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
-    bs[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-    bi[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-    if (n < g.N) {
-      bs[j] = *reinterpret_cast<const v4f*>(g.b_scale + n);
-      if (g.bias) {
-        const uint2 bb = *reinterpret_cast<const uint2*>(g.bias + n);
-        bi[j][0] = __uint_as_float(bb.x << 16);
-        bi[j][1] = __uint_as_float(bb.x & 0xffff0000u);
-        bi[j][2] = __uint_as_float(bb.y << 16);
-        bi[j][3] = __uint_as_float(bb.y & 0xffff0000u);
-      }
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int m = mw + 16 * i;
-    const float as = m < g.M ? g.a_scale[m] : 0.0f;
-#pragma unroll
-    for (int u = 0; u < TN / 2; ++u) {  // pair of fragments 2u, 2u+1: 8 consecutive columns
-      uint32_t pk[4];
-#pragma unroll
-      for (int d = 0; d < 2; ++d) {
-        const int j = 2 * u + d;
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          v[e] = __fmaf_rn(acc[i][j][e] * as, bs[j][e], bi[j][e]);
-          if (gelu) v[e] = gelu_tanh(v[e]);
-        }
-        pk[2 * d] = pack_bf16x2(v[0], v[1]);
-        pk[2 * d + 1] = pack_bf16x2(v[2], v[3]);
-      }
-      const int n = nw + 64 * (u >> 1) + 32 * (u & 1);
-      if (m < g.M && n < g.N)
-        *reinterpret_cast<uint4*>(g.out + (int64_t)m * g.ldo + n) =
-            uint4{pk[0], pk[1], pk[2], pk[3]};
-    }
-  }
+// Number of CUs of the current device (cached per device ordinal); 0 on error.
+int cu_count() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64 && cached[dev] > 0) return cached[dev];
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64) cached[dev] = n;
+  return n;
 }
 
 template <class C>
@@ -711,9 +774,16 @@ int launch_wide(const GemmArgs& g, hipStream_t stream) {
     }
     attr_set = true;
   }
+  const int cus = cu_count();
+  if (cus <= 0) {
+    set_error("cannot query the CU count of the current device");
+    return CDIT_EHIP;
+  }
   const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
-  hipLaunchKernelGGL(gemm_fp8_wide<C>, dim3(tiles_m * tiles_n), dim3(C::THREADS), C::LDS_BYTES,
-                     stream, g, tiles_m, tiles_n);
+  const int ntiles = tiles_m * tiles_n;
+  // one persistent workgroup per CU (its LDS and registers fill the CU)
+  hipLaunchKernelGGL(gemm_fp8_wide<C>, dim3(ntiles < cus ? ntiles : cus), dim3(C::THREADS),
+                     C::LDS_BYTES, stream, g, tiles_m, tiles_n);
   return 0;
 }
 
@@ -902,6 +972,8 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
       variant = 21;
     }
   }
+  // the wide kernels stream K two steps ahead: shorter K runs the 128x128 kernel
+  const bool wide_ok = g.K >= 256;
   switch (variant) {
     case 0: return launch_tiled<V0>(g, stream);
     case 1: return launch_tiled<V1>(g, stream);
@@ -913,9 +985,9 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     case 9: return launch_pingpong<V9>(g, stream);
     case 10: return launch_pingpong<V10>(g, stream);
     case 11: return launch_pingpong<V11>(g, stream);
-    case 12: return launch_wide<V12>(g, stream);
-    case 14: return launch_wide<V14>(g, stream);
-    case 15: return launch_wide<V15>(g, stream);
+    case 12: return wide_ok ? launch_wide<V12>(g, stream) : launch_tiled<V6>(g, stream);
+    case 14: return wide_ok ? launch_wide<V14>(g, stream) : launch_tiled<V6>(g, stream);
+    case 15: return wide_ok ? launch_wide<V15>(g, stream) : launch_tiled<V6>(g, stream);
     default:
       set_error("cdit_fp8_gemm_rowwise: unknown kernel variant %d", variant);
       return CDIT_EINVAL;
