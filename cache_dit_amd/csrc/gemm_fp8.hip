@@ -498,8 +498,16 @@ __device__ __forceinline__ int swz_b(int row) { return ((row >> 1) & 1) | (((row
 // inside the loop (all 256 AGPRs hold accumulators, there is no room to shuffle).
 // The compiler does not know this is an MFMA, so the code that reads the
 // accumulators afterwards (the epilogue) waits for the matrix core itself.
+// FIRST: the first K step of a tile, acc = product (C operand 0). The accumulators
+// are never initialised by other instructions: a VALU write of an AGPR right before
+// an MFMA that reads it needs wait states which the compiler cannot insert here.
+template <bool FIRST>
 __device__ __forceinline__ void mfma_16x16x128_fp8(v4f& acc, const v8i& b, const v8i& a) {
-  asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+  if constexpr (FIRST) {
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=a"(acc) : "v"(b), "v"(a));
+  } else {
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+  }
 }
 
 template <class C>
@@ -622,13 +630,32 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) bf[j] = read_b(smem + b_cur, j);
     af[0] = read_a(smem + a_cur, 0);
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    // epilogue operands of this tile, fetched two steps before they are needed:
+    // acc[i][4t+q][e] is out[m][n] with
+    //   m = m0 + wm*WM + 16i + (lane&15),
+    //   n = n0 + wn*WN + 64t + 32(q>>1) + 8(lane>>4) + 4(q&1) + e
+    const int nw = n0 + wn * C::WN + 8 * kg;
+    const int mw = m0 + wm * C::WM + r16;
+    v4f bs[TN];
+    uint2 bi[TN];  // bias stays packed (bf16 pairs) until used: registers are scarce
+    float as[TM];
 
-    for (int kt = 0; kt < KT; ++kt) {
+    // One K step; FIRST: step 0 of the tile (the accumulators start from zero).
+    auto step = [&](int kt, auto first_tag) {
+      constexpr bool FIRST = decltype(first_tag)::value;
       if (kt == KT - 2) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int n = nw + 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
+          bs[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+          bi[j] = uint2{0u, 0u};
+          if (n < g.N) {
+            bs[j] = *reinterpret_cast<const v4f*>(g.b_scale + n);
+            if (g.bias) bi[j] = *reinterpret_cast<const uint2*>(g.bias + n);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) as[i] = mw + 16 * i < g.M ? g.a_scale[mw + 16 * i] : 0.0f;
         // every DMA of this tile has been issued: the stream moves on
         if (next_tile < ntiles) {
           int tm, tn;
@@ -644,18 +671,21 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
       const uint8_t* st = smem + a_cur;
 #pragma unroll
       for (int i = 0; i < H; ++i) {
-        // A panel two steps ahead into the stage that step kt-1 read, spread over the rows
-#pragma unroll
-        for (int p = 0; p < C::NDA; ++p)
-          if (p * H / C::NDA == i) dma_a(kd, a_prev, p);
         if (i + 1 < H) af[i + 1] = read_a(st, i + 1);
         // the TM-H fragments of the second half, spread over the rows of the first
 #pragma unroll
         for (int k = 0; k < TM - H; ++k)
           if (k * H / (TM - H) == i) af[H + k] = read_a(st, H + k);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) mfma_16x16x128_fp8(acc[i][j], bf[j], af[i]);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int j = 0; j < TN; ++j) {
+          // A panel two steps ahead into the stage that step kt-1 read, one DMA
+          // instruction every few MFMAs
+#pragma unroll
+          for (int p = 0; p < C::NDA; ++p)
+            if (p * (H * TN) / C::NDA == i * TN + j) dma_a(kd, a_prev, p);
+          mfma_16x16x128_fp8<FIRST>(acc[i][j], bf[j], af[i]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
       // own LDS reads of this step done, own DMA of the next step landed (the A
       // panel issued above may still fly); then everyone's. In step 0 of a later
@@ -668,12 +698,15 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
       }
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        // B panel two steps ahead into the B stage of this step, spread over the columns
 #pragma unroll
-        for (int p = 0; p < C::NDB; ++p)
-          if (p * TN / C::NDB == j) dma_b(kd, b_cur, p);
+        for (int i = H; i < TM; ++i) {
+          // B panel two steps ahead into the B stage of this step, one DMA
+          // instruction every few MFMAs
 #pragma unroll
-        for (int i = H; i < TM; ++i) mfma_16x16x128_fp8(acc[i][j], bf[j], af[i]);
+          for (int p = 0; p < C::NDB; ++p)
+            if (p * ((TM - H) * TN) / C::NDB == j * (TM - H) + (i - H)) dma_b(kd, b_cur, p);
+          mfma_16x16x128_fp8<FIRST>(acc[i][j], bf[j], af[i]);
+        }
         // fragments of the next step (after the very last one: zeros, never used)
         bf[j] = read_b(smem + b_next, j);
         if (j == 0) af[0] = read_a(smem + a_next, 0);
@@ -687,34 +720,17 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
       const int b_free = b_cur;
       b_cur = b_next;
       b_next = b_free;
-    }
+    };
+    step(0, std::true_type{});
+    for (int kt = 1; kt < KT; ++kt) step(kt, std::false_type{});
     // the last MFMAs (8 passes each) must have written their accumulators
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 
-    // ---- epilogue: acc[i][4t+q][e] is out[m][n] with
-    //   m = m0 + wm*WM + 16i + (lane&15),
-    //   n = n0 + wn*WN + 64t + 32(q>>1) + 8(lane>>4) + 4(q&1) + e
+    // ---- epilogue
     const bool gelu = (g.epilogue & CDIT_EPI_GELU_TANH) != 0;
-    const int nw = n0 + wn * C::WN + 8 * kg;
-    const int mw = m0 + wm * C::WM + r16;
-    v4f bs[TN];
-    uint2 bi[TN];  // bias stays packed (bf16 pairs) until used: registers are scarce here
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = nw + 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
-      bs[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-      bi[j] = uint2{0u, 0u};
-      if (n < g.N) {
-        bs[j] = *reinterpret_cast<const v4f*>(g.b_scale + n);
-        if (g.bias) bi[j] = *reinterpret_cast<const uint2*>(g.bias + n);
-      }
-    }
-    float as[TM];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) as[i] = mw + 16 * i < g.M ? g.a_scale[mw + 16 * i] : 0.0f;
-    // scales and bias are here, and so is every DMA issued before them (the next
-    // tile's first two steps): from now on only this epilogue's stores are in flight
+    // Every DMA issued so far (the next tile's first two steps) must have landed
+    // before the stores go out: step 0 of the next tile then waits for nothing.
     wait_vm<0>();
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
