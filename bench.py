@@ -362,7 +362,7 @@ def main():
   head = headline_kernels(device)
   M, K, N = HEADLINE
   roofline = {
-      "kernel": "gemm_fp8_pingpong<192x384> (w8a8 GEMM + scale/bias epilogue) at M=4608 K=3072 "
+      "kernel": "gemm_fp8_wide<288x192> (w8a8 GEMM + scale/bias epilogue) at M=4608 K=3072 "
                 "N=12288",
       "bound": "mfma",
       "achieved": head["gemm_tflops"],
@@ -371,7 +371,7 @@ def main():
       "frac": head["gemm_tflops"] / FP8_PEAK_TFLOPS,
       # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain
       # copy of known size (profiles/pmc_traffic_headline_kernels.md); algorithmic 165.2 MB
-      "traffic": 340.3e6,
+      "traffic": 425.4e6,
   }
   roofline_quant = {
       "kernel": "quant_rowwise_regs at M=4608 K=3072",
