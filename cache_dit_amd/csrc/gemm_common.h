@@ -102,6 +102,18 @@ __device__ __forceinline__ void wait_steps(int later) {
 #undef CDIT_WAIT_CASE
 }
 
+// Number of CUs of the current device (cached per device ordinal); 0 on error.
+inline int cu_count() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64 && cached[dev] > 0) return cached[dev];
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64) cached[dev] = n;
+  return n;
+}
+
 // Workgroup id -> output tile. Workgroups are handed to the 8 XCDs round-robin
 // and each XCD has its own L2, so ids that land on one XCD are first made
 // consecutive, then walked in column-major order inside groups of GROUP_M tile

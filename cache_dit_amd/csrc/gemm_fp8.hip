@@ -766,18 +766,6 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
   wait_vm<0>();
 }
 
-// Number of CUs of the current device (cached per device ordinal); 0 on error.
-int cu_count() {
-  static int cached[64];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return 0;
-  if (dev >= 0 && dev < 64 && cached[dev] > 0) return cached[dev];
-  int n = 0;
-  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-  if (dev >= 0 && dev < 64) cached[dev] = n;
-  return n;
-}
-
 template <class C>
 int launch_wide(const GemmArgs& g, hipStream_t stream) {
   static bool attr_set = false;
@@ -920,6 +908,9 @@ bool tiled_ok(const GemmArgs& g) {
          reinterpret_cast<uintptr_t>(g.a) % 16 == 0 && reinterpret_cast<uintptr_t>(g.b) % 16 == 0 &&
          reinterpret_cast<uintptr_t>(g.out) % 16 == 0 &&
          // 32-bit in-tile byte offsets
+         // the epilogues load scales as float4 and bias as 8-byte packs
+         reinterpret_cast<uintptr_t>(g.b_scale) % 16 == 0 &&
+         reinterpret_cast<uintptr_t>(g.bias) % 16 == 0 &&
          (int64_t)512 * g.lda < (int64_t)1 << 31 && (int64_t)512 * g.ldb < (int64_t)1 << 31;
 }
 

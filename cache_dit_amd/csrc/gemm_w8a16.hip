@@ -24,6 +24,8 @@
 //
 // Replaces F.linear(x, W.dequantize(), bias) of the reference's
 // float8_weight_only mode (src/cache_dit/quantization/torchao/quantize_ao.py:604-610).
+#include <type_traits>
+
 #include "gemm_common.h"
 
 namespace cdit {
@@ -345,6 +347,378 @@ int launch_pingpong(const GemmArgs& g, hipStream_t stream) {
 }
 
 // ---------------------------------------------------------------------------
+// Wide kernel: the schedule of the wide w8a8 kernel (one persistent workgroup of 4
+// waves per CU, one wave per SIMD with all 256 AGPRs as accumulators, LDS-DMA by
+// buffer loads spread over the MFMA stream, A panel in 3 LDS stages and B panel in
+// 2, one barrier per K step, the DMA stream running across tiles) with bf16 MFMAs:
+// v_mfma_f32_32x32x16_bf16 (8 passes), K steps of 64 elements, wave tile
+// (BM/2) x (BN/2) as TM x TN blocks of 32x32, four MFMAs per block and step.
+//
+// Panels as in the ping-pong kernel above: A rows 128 B (bf16), chunk c of row r at
+// c ^ ((r>>1)&7); B rows 64 B (e4m3), chunk c at c ^ ((r>>2)&3). A lane reads, per
+// 32-row block, the four A chunks 4t+2h+s (h = lane>>5) and the two B chunks 2t+h:
+// the 16 B bytes of one chunk are the weights of MFMA steps 2t and 2t+1 (K order
+// permuted identically on both sides). The weights are converted to bf16 once per
+// step, when they arrive from LDS, and kept for all row blocks.
+//
+// The B fragments take their 32 rows in a permuted order, operand row p reads
+// panel row 16 ((p>>2)&1) + 4 (p>>3) + (p&3) of its block: with the operands
+// swapped (weights first) a lane then ends with 16 consecutive output columns per
+// block, n = 32j + 16h + r for accumulator register r, and stores them with two
+// 16-byte stores, no transpose.
+template <int BM_, int BN_, int GROUP_M_>
+struct CfgWW {
+  static constexpr int BM = BM_, BN = BN_, GROUP_M = GROUP_M_;
+  static constexpr int WAVES = 4, THREADS = 256;
+  static constexpr int WM = BM / 2, WN = BN / 2;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int H = TM / 2;
+  static constexpr int A_ROW = BKE * 2, B_ROW = BKE;
+  static constexpr int A_BYTES = BM * A_ROW, B_BYTES = BN * B_ROW;
+  static constexpr int A_STAGES = 3, B_STAGES = 2;
+  static constexpr int B_BASE = A_STAGES * A_BYTES;
+  static constexpr int LDS_BYTES = A_STAGES * A_BYTES + B_STAGES * B_BYTES;
+  // DMA instructions (1 KiB: 8 A rows or 16 B rows) per wave and step
+  static constexpr int NDA = BM / 8 / WAVES, NDB = BN / 16 / WAVES, ND = NDA + NDB;
+  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
+  static_assert(BM % 32 == 0 && BN % 64 == 0, "panels are dealt 1 KiB x 4 waves at a time");
+  static_assert(TM * TN <= 16, "accumulators: at most 256 registers");
+  static_assert(TM >= 2, "two halves per step");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+};
+
+struct AFrag {
+  v8bf k[4];  // operands of MFMA steps 0..3 of a K step (one 32-row block)
+};
+struct WRaw {
+  uint4 t[2];  // weights as read from LDS: 2 x 16 e4m3 bytes
+};
+
+// acc (+)= W-fragment x A-fragment, accumulator tied to an AGPR tuple (see the wide
+// w8a8 kernel for why this is inline assembly and what that obliges the code to do).
+template <bool FIRST>
+__device__ __forceinline__ void mfma_32x32x16_bf16(v16f& acc, const v8bf& w, const v8bf& a) {
+  if constexpr (FIRST) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=a"(acc) : "v"(w), "v"(a));
+  } else {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(w), "v"(a));
+  }
+}
+
+// 16 e4m3 bytes -> two bf16 MFMA operands (MFMA steps 2t and 2t+1)
+__device__ __forceinline__ void convert_w(const uint4& w, v8bf& lo, v8bf& hi) {
+  const v2bf c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.x, 1.0f, false);
+  const v2bf c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.x, 1.0f, true);
+  const v2bf c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.y, 1.0f, false);
+  const v2bf c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.y, 1.0f, true);
+  const v2bf c4 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.z, 1.0f, false);
+  const v2bf c5 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.z, 1.0f, true);
+  const v2bf c6 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.w, 1.0f, false);
+  const v2bf c7 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.w, 1.0f, true);
+  lo = v8bf{c0[0], c0[1], c1[0], c1[1], c2[0], c2[1], c3[0], c3[1]};
+  hi = v8bf{c4[0], c4[1], c5[0], c5[1], c6[0], c6[1], c7[0], c7[1]};
+}
+
+template <class C>
+__global__ __launch_bounds__(C::THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void
+gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: M0 from scalar code
+  const int wm = wave >> 1, wn = wave & 1;
+  // local copies: a template-dependent expression as a builtin argument inside a
+  // lambda makes the host pass drop the kernel stub without a diagnostic
+  constexpr int TM = C::TM, TN = C::TN, H = C::H, A_ROW = C::A_ROW, B_ROW = C::B_ROW;
+  const int KT = g.K / BKE;  // >= 2 (checked by the launcher)
+  const int ntiles = tiles_m * tiles_n;
+
+  int m0, n0;  // tile being computed
+  {
+    int tm, tn;
+    tile_of_block<C::GROUP_M>(blockIdx.x, ntiles, tiles_m, tiles_n, &tm, &tn);
+    m0 = tm * C::BM;
+    n0 = tn * C::BN;
+  }
+
+  // DMA source: the tile whose panels the DMA stream currently fetches
+  const uint8_t* A;
+  const uint8_t* B;
+  uint32_t off[C::ND];
+  int nrec = 0x7fffffff;  // 0: the stream has run past the last tile, fetch nothing
+  auto set_source = [&](int sm0, int sn0) {
+    A = static_cast<const uint8_t*>(g.a) + (int64_t)sm0 * g.lda * 2;
+    B = g.b + (int64_t)sn0 * g.ldb;
+    const int rows_a = g.M - sm0, rows_b = g.N - sn0;
+    int l = lane;  // opaque: keeps the row indices out of registers across the K loop
+    asm volatile("" : "+v"(l));
+#pragma unroll
+    for (int p = 0; p < C::NDA; ++p) {  // 8 rows of 128 B per instruction
+      const int row = (wave + 4 * p) * 8 + (l >> 3);
+      const int c = (l & 7) ^ ((row >> 1) & 7);
+      off[p] = (uint32_t)min(row, rows_a - 1) * (uint32_t)(g.lda * 2) + c * 16;
+    }
+#pragma unroll
+    for (int p = 0; p < C::NDB; ++p) {  // 16 rows of 64 B per instruction
+      const int row = (wave + 4 * p) * 16 + (l >> 2);
+      const int c = (l & 3) ^ ((row >> 2) & 3);
+      off[C::NDA + p] = (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
+    }
+  };
+  set_source(m0, n0);
+  auto dma_a = [&](int kt, int a_lds, int p) {
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(A), 0, nrec, 0x00020000);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        rsrc, (__attribute__((address_space(3))) void*)(smem + a_lds + (wave + 4 * p) * 1024), 16,
+        (int)off[p], kt * A_ROW, 0, 0);
+  };
+  auto dma_b = [&](int kt, int b_lds, int p) {
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(B), 0, nrec, 0x00020000);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        rsrc, (__attribute__((address_space(3))) void*)(smem + b_lds + (wave + 4 * p) * 1024), 16,
+        (int)off[C::NDA + p], kt * B_ROW, 0, 0);
+  };
+
+  // operand read map: A row lane&31 of its block, chunks 4t+2h+s; W operand row
+  // p = lane&31 reads panel row 16((p>>2)&1) + 4(p>>3) + (p&3), chunks 2t+h
+  const int h = lane >> 5, r32 = lane & 31;
+  const int wrow = 16 * ((r32 >> 2) & 1) + 4 * (r32 >> 3) + (r32 & 3);
+  uint32_t rd_a[4], rd_b[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+      rd_a[2 * t + e] =
+          (wm * C::WM + r32) * C::A_ROW + (((4 * t + 2 * h + e) ^ ((r32 >> 1) & 7)) << 4);
+    rd_b[t] = (wn * C::WN + wrow) * C::B_ROW + (((2 * t + h) ^ ((wrow >> 2) & 3)) << 4);
+  }
+  auto read_a = [&](const uint8_t* st, int i) -> AFrag {
+    AFrag f;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      f.k[q] = *reinterpret_cast<const v8bf*>(st + rd_a[q] + i * 32 * C::A_ROW);
+    return f;
+  };
+  auto read_w = [&](const uint8_t* st, int j) -> WRaw {
+    WRaw f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+      f.t[t] = *reinterpret_cast<const uint4*>(st + rd_b[t] + j * 32 * C::B_ROW);
+    return f;
+  };
+
+  v16f acc[TM][TN];
+  AFrag af[TM];
+  AFrag wf[TN];  // converted weights
+  WRaw wr[TN];   // weights as read from LDS (next step's, until converted)
+
+  int a_prev = 2 * C::A_BYTES, a_cur = 0, a_next = C::A_BYTES;
+  int b_cur = C::B_BASE, b_next = C::B_BASE + C::B_BYTES;
+  // prologue: steps 0 and 1 in flight, step 0 landed
+#pragma unroll
+  for (int p = 0; p < C::NDA; ++p) dma_a(0, a_cur, p);
+#pragma unroll
+  for (int p = 0; p < C::NDB; ++p) dma_b(0, b_cur, p);
+#pragma unroll
+  for (int p = 0; p < C::NDA; ++p) dma_a(1, a_next, p);
+#pragma unroll
+  for (int p = 0; p < C::NDB; ++p) dma_b(1, b_next, p);
+  wait_and_barrier<C::ND>();
+
+  for (int tile = blockIdx.x;; tile += gridDim.x) {
+    const int next_tile = tile + gridDim.x;
+    int nm0 = 0, nn0 = 0;
+    // fragments of step 0 (in LDS since the prologue, or since the barrier of the
+    // previous tile's last step)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) wr[j] = read_w(smem + b_cur, j);
+    af[0] = read_a(smem + a_cur, 0);
+
+    // One K step; FIRST: step 0 of the tile (the accumulators start from zero).
+    auto step = [&](int kt, auto first_tag) {
+      constexpr bool FIRST = decltype(first_tag)::value;
+      if (kt == KT - 2) {
+        // every DMA of this tile has been issued: the stream moves on
+        if (next_tile < ntiles) {
+          int tm, tn;
+          tile_of_block<C::GROUP_M>(next_tile, ntiles, tiles_m, tiles_n, &tm, &tn);
+          nm0 = tm * C::BM;
+          nn0 = tn * C::BN;
+          set_source(nm0, nn0);
+        } else {
+          nrec = 0;
+        }
+      }
+      const int kd = kt + 2 < KT ? kt + 2 : kt + 2 - KT;  // step (of its tile) to fetch
+      const uint8_t* st = smem + a_cur;
+      auto convert = [&](int j) {
+        convert_w(wr[j].t[0], wf[j].k[0], wf[j].k[1]);
+        convert_w(wr[j].t[1], wf[j].k[2], wf[j].k[3]);
+      };
+      auto mfma = [&](int i, int j, int q) {
+        if (FIRST && q == 0) {
+          mfma_32x32x16_bf16<true>(acc[i][j], wf[j].k[q], af[i].k[q]);
+        } else {
+          mfma_32x32x16_bf16<false>(acc[i][j], wf[j].k[q], af[i].k[q]);
+        }
+      };
+      // The weights of this step were read from LDS during the previous step. They are
+      // converted one block ahead of their first use: an MFMA operand written by a
+      // VALU instruction just before the (inline-assembly) MFMA reads stale data.
+      convert(0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < H; ++i) {
+        if (i + 1 < H) af[i + 1] = read_a(st, i + 1);
+#pragma unroll
+        for (int k = 0; k < TM - H; ++k)
+          if (k * H / (TM - H) == i) af[H + k] = read_a(st, H + k);
+        // MFMA step q of all TN blocks of the row before step q+1: consecutive MFMAs
+        // never depend on each other
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            if (i == 0 && q == 0 && j + 1 < TN) convert(j + 1);
+            // A panel two steps ahead into the stage that step kt-1 read
+#pragma unroll
+            for (int p = 0; p < C::NDA; ++p)
+              if (p * (H * TN * 4) / C::NDA == (i * 4 + q) * TN + j) dma_a(kd, a_prev, p);
+            mfma(i, j, q);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+      }
+      // own LDS reads of this step done, own DMA of the next step landed (the A
+      // panel issued above may still fly); then everyone's. In step 0 of a later
+      // tile that DMA was waited for before the previous epilogue's stores.
+      if (kt == 0 && tile != (int)blockIdx.x) {
+        wait_and_barrier<63>();
+      } else {
+        wait_and_barrier<C::NDA>();
+      }
+      // second half: pairs of columns, so that dependent MFMAs are 2 (TM-H) apart
+#pragma unroll
+      for (int j0 = 0; j0 < TN; j0 += 2) {
+        constexpr int R = TM - H;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int i = H; i < TM; ++i)
+#pragma unroll
+            for (int j = j0; j < j0 + 2 && j < TN; ++j) {
+              // B panel two steps ahead into the B stage of this step
+#pragma unroll
+              for (int p = 0; p < C::NDB; ++p)
+                if (p * (R * TN * 4) / C::NDB ==
+                    j0 * R * 4 + (q * R + (i - H)) * (TN - j0 < 2 ? TN - j0 : 2) + (j - j0))
+                  dma_b(kd, b_cur, p);
+              mfma(i, j, q);
+            }
+        // weights of the next step (after the very last one: zeros, never used)
+#pragma unroll
+        for (int j = j0; j < j0 + 2 && j < TN; ++j) wr[j] = read_w(smem + b_next, j);
+        if (j0 == 0) af[0] = read_a(smem + a_next, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      const int a_free = a_prev;
+      a_prev = a_cur;
+      a_cur = a_next;
+      a_next = a_free;
+      const int b_free = b_cur;
+      b_cur = b_next;
+      b_next = b_free;
+    };
+    step(0, std::true_type{});
+    for (int kt = 1; kt < KT; ++kt) step(kt, std::false_type{});
+    // the last MFMAs (8 passes each) must have written their accumulators
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- epilogue: acc[i][j][r] is out[m][n] with
+    //   m = m0 + wm*WM + 32i + (lane&31),  n = n0 + wn*WN + 32j + 16h + r
+    const bool gelu = (g.epilogue & CDIT_EPI_GELU_TANH) != 0;
+    const int nw = n0 + wn * C::WN + 16 * h;
+    const int mw = m0 + wm * C::WM + r32;
+    // every DMA issued so far (the next tile's first two steps) must have landed
+    // before the stores go out: step 0 of the next tile then waits for nothing
+    wait_vm<0>();
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = nw + 32 * j;
+      v4f bs[4];
+      uint4 bi[2];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) bs[q] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+      bi[0] = bi[1] = uint4{0u, 0u, 0u, 0u};
+      if (n < g.N) {  // N % 16 == 0 on this path: 16 columns are all in or all out
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bs[q] = *reinterpret_cast<const v4f*>(g.b_scale + n + 4 * q);
+        if (g.bias) {
+          bi[0] = *reinterpret_cast<const uint4*>(g.bias + n);
+          bi[1] = *reinterpret_cast<const uint4*>(g.bias + n + 8);
+        }
+      }
+      const uint32_t bw[8] = {bi[0].x, bi[0].y, bi[0].z, bi[0].w, bi[1].x, bi[1].y, bi[1].z, bi[1].w};
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int m = mw + 32 * i;
+        uint32_t pk[8];
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          const float b0 = __uint_as_float(bw[r >> 1] << 16);
+          const float b1 = __uint_as_float(bw[r >> 1] & 0xffff0000u);
+          float v0 = __fmaf_rn(acc[i][j][r], bs[r >> 2][r & 3], b0);
+          float v1 = __fmaf_rn(acc[i][j][r + 1], bs[r >> 2][(r + 1) & 3], b1);
+          if (gelu) {
+            v0 = gelu_tanh(v0);
+            v1 = gelu_tanh(v1);
+          }
+          pk[r >> 1] = pack_bf16x2(v0, v1);
+        }
+        if (m < g.M && n < g.N) {
+          uint16_t* dst = g.out + (int64_t)m * g.ldo + n;
+          *reinterpret_cast<uint4*>(dst) = uint4{pk[0], pk[1], pk[2], pk[3]};
+          *reinterpret_cast<uint4*>(dst + 8) = uint4{pk[4], pk[5], pk[6], pk[7]};
+        }
+      }
+    }
+    if (next_tile >= ntiles) break;
+    m0 = nm0;
+    n0 = nn0;
+  }
+  // the zero-record DMA of the last two steps must not outlive the workgroup
+  wait_vm<0>();
+}
+
+template <class C>
+int launch_wide(const GemmArgs& g, hipStream_t stream) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_w8a16_wide<C>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(%d bytes LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
+      return CDIT_EHIP;
+    }
+    attr_set = true;
+  }
+  const int cus = cu_count();
+  if (cus <= 0) {
+    set_error("cannot query the CU count of the current device");
+    return CDIT_EHIP;
+  }
+  const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
+  const int ntiles = tiles_m * tiles_n;
+  // one persistent workgroup per CU (its LDS and registers fill the CU)
+  hipLaunchKernelGGL(gemm_w8a16_wide<C>, dim3(ntiles < cus ? ntiles : cus), dim3(C::THREADS),
+                     C::LDS_BYTES, stream, g, tiles_m, tiles_n);
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
 // Skinny kernel for M <= 16 (M = 1 modulation Linears): weight streaming. A
 // workgroup of 4 waves owns 16 output channels, each wave a quarter of K. Per
 // 128-element chunk a lane (weight row l&15, K group l>>4) loads 32 e4m3 bytes
@@ -467,6 +841,9 @@ bool tiled_ok(const GemmArgs& g) {
          g.ldo % 8 == 0 && reinterpret_cast<uintptr_t>(g.a) % 16 == 0 &&
          reinterpret_cast<uintptr_t>(g.b) % 16 == 0 &&
          reinterpret_cast<uintptr_t>(g.out) % 16 == 0 &&
+         // the epilogues load scales as float4 and bias as 8-byte packs
+         reinterpret_cast<uintptr_t>(g.b_scale) % 16 == 0 &&
+         reinterpret_cast<uintptr_t>(g.bias) % 16 == 0 &&
          (int64_t)1024 * g.lda < (int64_t)1 << 31 && (int64_t)512 * g.ldb < (int64_t)1 << 31;
 }
 
@@ -477,6 +854,9 @@ typedef CfgW<128, 128, 2, 2, true, 8> W3;   // small tiles, two workgroups per C
 typedef CfgWP<256, 256, 3, 8> W4;           // ping-pong, 3 stages of 64 elements
 typedef CfgWP<192, 384, 3, 8> W5;           // ping-pong, 96x96 wave tiles
 typedef CfgWP<128, 256, 4, 8> W6;
+typedef CfgWW<256, 256, 8> W7;              // wide: 4 waves, 128x128 wave tiles
+typedef CfgWW<256, 192, 8> W8;              // wide: 128x96 wave tiles
+typedef CfgWW<192, 256, 8> W9;              // wide: 96x128 wave tiles
 
 int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {
@@ -492,14 +872,22 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
     hipLaunchKernelGGL(gemm_w8a16_skinny, dim3((g.N + 15) / 16), dim3(256), 0, stream, g);
     return 0;
   }
+  // the wide kernels stream K two steps ahead and store 16 columns per lane
+  const bool wide_ok = g.K >= 2 * BKE && g.N % 16 == 0;
   if (variant < 0) {
-    // same cost model as the w8a8 entry point: CU rounds times tile area
+    // Same cost model as the w8a8 entry point: tile area times rounds over the 256
+    // CUs, a last partial round of r tiles counting 0.4 + 0.6 r/256.
     auto tiles = [&](int bm, int bn) {
       return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
     };
-    auto cost = [&](int bm, int bn) { return ((tiles(bm, bn) + 255) / 256) * bm * bn; };
-    if (tiles(256, 256) >= 200) {
-      variant = cost(192, 384) < cost(256, 256) ? 5 : 4;
+    auto cost = [&](int bm, int bn, int pen) {
+      const int64_t t = tiles(bm, bn), full = t / 256, rem = t % 256;
+      return (full * 2560 + (rem ? 1024 + 6 * rem : 0)) * bm * bn * pen;
+    };
+    if (tiles(256, 256) >= 160 && wide_ok) {
+      variant = cost(256, 192, 103) < cost(256, 256, 100) ? 8 : 7;
+    } else if (tiles(256, 256) >= 200) {
+      variant = ((tiles(192, 384) + 255) / 256) * 192 * 384 < ((tiles(256, 256) + 255) / 256) * 256 * 256 ? 5 : 4;
     } else {
       variant = 3;
     }
@@ -510,6 +898,9 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
     case 4: return launch_pingpong<W4>(g, stream);
     case 5: return launch_pingpong<W5>(g, stream);
     case 6: return launch_pingpong<W6>(g, stream);
+    case 7: return wide_ok ? launch_wide<W7>(g, stream) : launch_tiled<W3>(g, stream);
+    case 8: return wide_ok ? launch_wide<W8>(g, stream) : launch_tiled<W3>(g, stream);
+    case 9: return wide_ok ? launch_wide<W9>(g, stream) : launch_tiled<W3>(g, stream);
     default:
       set_error("cdit_w8a16_gemm: unknown kernel variant %d", variant);
       return CDIT_EINVAL;

@@ -1,14 +1,16 @@
-"""The wide FP8 GEMM kernel issues its MFMAs through inline assembly (the
-accumulators are tied to AGPR tuples), so the compiler's hazard recognizer does
-not see them. This test compiles gemm_fp8.hip to gfx950 assembly (no GPU needed)
-and checks, in the code the compiler produced for every instance of that kernel,
+"""The wide GEMM kernels (w8a8 and w8a16) issue their MFMAs through inline assembly
+(the accumulators are tied to AGPR tuples), so the compiler's hazard recognizer
+does not see them. This test compiles their sources to gfx950 assembly (no GPU
+needed) and checks, in the code the compiler produced for every instance,
 the three situations in which the hardware needs software wait states:
 
-  1. no VALU instruction (v_accvgpr_write / v_accvgpr_mov) writes an AGPR that an
-     MFMA uses as accumulator: accumulators are only ever written by MFMAs;
-  2. no VALU instruction writes a VGPR within the 8 instructions before an MFMA
-     that reads it as A or B operand (operands come from LDS reads, which
-     s_waitcnt covers);
+  1. no MFMA reads (as its C operand) an AGPR that a VALU instruction
+     (v_accvgpr_write / v_accvgpr_mov) wrote: accumulators start from MFMAs with a
+     zero C operand and are otherwise only written by MFMAs;
+  2. no VALU instruction writes a VGPR in the 4 instructions before an MFMA that
+     reads it as A or B operand (the w8a16 kernel converts its weights to bf16 one
+     block ahead of their use; an operand converted right before the MFMA gave
+     wrong results on hardware);
   3. at least 18 wait states lie between an MFMA and the first v_accvgpr_read of
      an accumulator (the epilogue).
 """
@@ -20,7 +22,8 @@ import subprocess
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-SRC = os.path.join(ROOT, "cache_dit_amd", "csrc", "gemm_fp8.hip")
+CSRC = os.path.join(ROOT, "cache_dit_amd", "csrc")
+SOURCES = {"gemm_fp8.hip": "gemm_fp8_wide", "gemm_w8a16.hip": "gemm_w8a16_wide"}
 
 
 def _hipcc():
@@ -30,20 +33,21 @@ def _hipcc():
   return None
 
 
-@pytest.fixture(scope="module")
-def wide_kernels(tmp_path_factory):
+@pytest.fixture(scope="module", params=sorted(SOURCES))
+def wide_kernels(request, tmp_path_factory):
   hipcc = _hipcc()
   if hipcc is None:
     pytest.skip("hipcc not found")
-  out = tmp_path_factory.mktemp("isa") / "gemm_fp8.s"
+  src, kernel = request.param, SOURCES[request.param]
+  out = tmp_path_factory.mktemp("isa") / (src + ".s")
   from cache_dit_amd.csrc import build
-  cmd = [hipcc, *build.DEVICE_FLAGS, "-I", os.path.join(ROOT, "include"), "-I",
-         os.path.dirname(SRC), "--cuda-device-only", "-S", SRC, "-o", str(out)]
+  cmd = [hipcc, *build.DEVICE_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+         "--cuda-device-only", "-S", os.path.join(CSRC, src), "-o", str(out)]
   r = subprocess.run(cmd, capture_output=True, text=True)
   assert r.returncode == 0, r.stderr[-2000:]
   text = out.read_text()
   kernels = {}
-  for m in re.finditer(r"^(_ZN\S*gemm_fp8_wide\S*):[^\n]*\n(.*?)s_endpgm", text, re.S | re.M):
+  for m in re.finditer(r"^(_ZN\S*" + kernel + r"\S*):[^\n]*\n(.*?)s_endpgm", text, re.S | re.M):
     body = [l.strip() for l in m.group(2).split("\n")]
     kernels[m.group(1)] = [l for l in body if l and not l.startswith(";") and not l.startswith(".")]
   assert len(kernels) >= 3, "wide kernel instances not found in the assembly"
@@ -84,16 +88,23 @@ def test_inline_asm_mfma_hazards(wide_kernels):
       assert kind == "a", f"{name}: MFMA accumulator not in AGPRs: {code[i]}"
       acc |= regs
       assert ops[3] in (ops[0], "0"), f"{name}: accumulator not tied: {code[i]}"
-    # 1. accumulators written by MFMAs only
-    for l in code:
+    # 1. an MFMA never reads an accumulator that a VALU instruction wrote: after a
+    # VALU write of such an AGPR (the compiler parks VGPRs in accumulators that are
+    # dead between the epilogue and the next tile) the next MFMA on it must be one
+    # with a zero C operand, which only writes it
+    for i, l in enumerate(code):
       if l.startswith(("v_accvgpr_write", "v_accvgpr_mov")):
         kind, regs = _regs(_operands(l)[0])
-        assert not (kind == "a" and regs & acc), f"{name}: VALU write of an accumulator: {l}"
-    # 2. no VALU write of an A/B operand shortly before the MFMA that reads it
+        if not (kind == "a" and regs & acc):
+          continue
+        nxt = next((k for k in mfma if k > i and _regs(_operands(code[k])[0])[1] & regs), None)
+        assert nxt is None or _operands(code[nxt])[3] == "0", \
+            f"{name}: {code[nxt]!r} reads an accumulator written by {l!r}"
+    # 2. no VALU write of an A/B operand in the 4 instructions before the MFMA
     for i in mfma:
       ops = _operands(code[i])
       src = _regs(ops[1])[1] | _regs(ops[2])[1]
-      for l in code[max(0, i - 8):i]:
+      for l in code[max(0, i - 4):i]:
         if l.startswith("v_") and not l.startswith("v_mfma"):
           d = _regs(_operands(l)[0])
           assert not (d and d[0] == "v" and d[1] & src), \
