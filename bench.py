@@ -203,7 +203,7 @@ def headline_kernels(device):
   try:
     def w8a16():
       i = it["i"] = (it["i"] + 1) % nbuf
-      ops.w8a16_into(xs[i], ws[i], wsc, b, outs[i & 1], 1)
+      ops.w8a16_into(xs[i], ws[i], wsc, b, outs[i & 1], 0)
 
     w_ms = _time_events(w8a16, 30, 5)
     res["w8a16_ms"] = w_ms
