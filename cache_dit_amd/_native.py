@@ -28,6 +28,7 @@ EXPORTS = (
     "cdit_last_error",
     "cdit_device_arch",
     "cdit_fp8_quant_rowwise",
+    "cdit_fp8_quant_tensorwise",
     "cdit_fp8_gemm_rowwise",
     "cdit_w8a16_gemm",
     "cdit_fp8_linear_w8a8",
@@ -54,6 +55,8 @@ def _bind(L: ctypes.CDLL) -> None:
   L.cdit_set_gemm_variant.argtypes = [ci]
   L.cdit_fp8_quant_rowwise.restype = ci
   L.cdit_fp8_quant_rowwise.argtypes = [vp, i64, i64, i64, vp, i64, vp, ci, vp]
+  L.cdit_fp8_quant_tensorwise.restype = ci
+  L.cdit_fp8_quant_tensorwise.argtypes = [vp, i64, i64, i64, vp, i64, vp, vp, ci, vp]
   L.cdit_fp8_gemm_rowwise.restype = ci
   L.cdit_fp8_gemm_rowwise.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci,
                                       vp]

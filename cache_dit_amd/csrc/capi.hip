@@ -158,6 +158,40 @@ int cdit_fp8_quant_rowwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_
   return rc ? rc : after_launch(fn);
 }
 
+int cdit_fp8_quant_tensorwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_x,
+                              void* q_e4m3, int64_t ld_q, float* scale, void* amax_ws,
+                              int scale_mode, void* stream) {
+  const char* fn = "cdit_fp8_quant_tensorwise";
+  if (M < 0 || K < 0 || M > INT32_MAX || K > INT32_MAX) {
+    set_error("%s: bad shape M=%lld K=%lld", fn, (long long)M, (long long)K);
+    return CDIT_EINVAL;
+  }
+  if (scale_mode != CDIT_SCALE_BF16DIV && scale_mode != CDIT_SCALE_FP32DIV) {
+    set_error("%s: unknown scale_mode %d", fn, scale_mode);
+    return CDIT_EINVAL;
+  }
+  if (M == 0) return CDIT_OK;
+  if (ld_x < K || ld_q < K) {
+    set_error("%s: leading dimension smaller than K (ld_x=%lld ld_q=%lld K=%lld)", fn,
+              (long long)ld_x, (long long)ld_q, (long long)K);
+    return CDIT_EINVAL;
+  }
+  if (!scale || !amax_ws || (K > 0 && (!x_bf16 || !q_e4m3))) {
+    set_error("%s: null pointer argument", fn);
+    return CDIT_EINVAL;
+  }
+  if (reinterpret_cast<uintptr_t>(amax_ws) % 4 != 0) {
+    set_error("%s: amax_ws must be 4-byte aligned", fn);
+    return CDIT_EINVAL;
+  }
+  int rc = check_arch();
+  if (rc) return rc;
+  rc = launch_quant_tensorwise(x_bf16, M, K, ld_x, q_e4m3, ld_q, scale,
+                               static_cast<uint32_t*>(amax_ws), scale_mode,
+                               static_cast<hipStream_t>(stream));
+  return rc ? rc : after_launch(fn);
+}
+
 int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale, const void* b_q,
                           const float* b_scale, const void* bias_bf16, void* out, int64_t M,
                           int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldo,

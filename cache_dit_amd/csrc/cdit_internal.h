@@ -14,6 +14,10 @@ namespace cdit {
 int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void* q,
                          int64_t ld_q, float* scale, int scale_mode, hipStream_t stream);
 
+int launch_quant_tensorwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void* q,
+                            int64_t ld_q, float* scale, uint32_t* amax_ws, int scale_mode,
+                            hipStream_t stream);
+
 extern int g_quant_variant;
 
 struct GemmArgs {

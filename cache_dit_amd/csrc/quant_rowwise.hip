@@ -229,6 +229,87 @@ __global__ __launch_bounds__(64) void quant_rowwise_generic(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Per-tensor variant (one scale for the whole [M,K] tensor): three launches.
+//   zero_amax:           *amax_ws = 0 (a kernel, not a memset, so that the sequence
+//                        can be recorded into a hipGraph)
+//   tensor_amax:         amax over all elements, one wavefront per row at a time,
+//                        integer atomic max into *amax_ws (exact, order free)
+//   quant_tensorwise_*:  scale from *amax_ws, written to scale[m] for every row (the
+//                        GEMM takes per-row scales), and the same cast as above
+__global__ void zero_amax(uint32_t* amax_ws) { *amax_ws = 0u; }
+
+__global__ __launch_bounds__(64) void tensor_amax(const uint16_t* __restrict__ x, int64_t ld_x,
+                                                  int M, int K, bool vec,
+                                                  uint32_t* __restrict__ amax_ws) {
+  const int lane = threadIdx.x & 63;
+  uint32_t m = 0;
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+    const uint16_t* xr = x + row * ld_x;
+    if (vec) {
+      const uint4* xv = reinterpret_cast<const uint4*>(xr);
+      for (int idx = lane; idx < (K >> 3); idx += 64) {
+        const uint4 w = xv[idx];
+        m = absmax2(m, w.x);
+        m = absmax2(m, w.y);
+        m = absmax2(m, w.z);
+        m = absmax2(m, w.w);
+      }
+    } else {
+      for (int k = lane; k < K; k += 64) {
+        const uint32_t a = xr[k] & 0x7fffu;
+        m = m > a ? m : a;
+      }
+    }
+  }
+  m = wave_max_u32(m);
+  if (lane == 0 && m != 0u) atomicMax(amax_ws, m);
+}
+
+// vec: 16-byte aligned rows with K % 8 == 0
+__global__ __launch_bounds__(64) void quant_tensorwise_cast(
+    const uint16_t* __restrict__ x, int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q,
+    float* __restrict__ scale, int M, int K, int scale_mode, bool vec,
+    const uint32_t* __restrict__ amax_ws) {
+  const int lane = threadIdx.x & 63;
+  const float s = row_scale(*amax_ws, scale_mode);
+  const bool fast = scale_in_fast_window(s);
+  const float r = 1.0f / s;
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+    if (lane == 0) scale[row] = s;
+    const uint16_t* xr = x + row * ld_x;
+    uint8_t* qr = q + row * ld_q;
+    if (vec) {
+      const uint4* xv = reinterpret_cast<const uint4*>(xr);
+      uint2* qv = reinterpret_cast<uint2*>(qr);
+      if (fast) {
+        for (int idx = lane; idx < (K >> 3); idx += 64) {
+          const uint4 w = xv[idx];
+          uint2 o;
+          o.x = quant4<true>(w.x, w.y, s, r);
+          o.y = quant4<true>(w.z, w.w, s, r);
+          qv[idx] = o;
+        }
+      } else {
+#pragma unroll 1
+        for (int idx = lane; idx < (K >> 3); idx += 64) {
+          const uint4 w = xv[idx];
+          uint2 o;
+          o.x = quant4<false>(w.x, w.y, s, 0.0f);
+          o.y = quant4<false>(w.z, w.w, s, 0.0f);
+          qv[idx] = o;
+        }
+      }
+    } else {
+      for (int k = lane; k < K; k += 64) {
+        const float y = clamp448(__uint_as_float((uint32_t)xr[k] << 16) / s);
+        const uint32_t p = __builtin_amdgcn_cvt_pk_fp8_f32(y, y, 0u, false);
+        qr[k] = (uint8_t)(p & 0xffu);
+      }
+    }
+  }
+}
+
 }  // namespace
 
 int g_quant_variant = 0;  // 0: streaming (nontemporal) loads and stores, 1: plain
@@ -277,6 +358,25 @@ int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void
 #undef CDIT_QUANT_CASE
   hipLaunchKernelGGL(quant_rowwise_generic, grid, block, 0, stream, xp, ld_x, qp, ld_q, scale, Mi,
                      Ki, scale_mode);
+  return 0;
+}
+
+int launch_quant_tensorwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void* q,
+                            int64_t ld_q, float* scale, uint32_t* amax_ws, int scale_mode,
+                            hipStream_t stream) {
+  const uint16_t* xp = static_cast<const uint16_t*>(x);
+  uint8_t* qp = static_cast<uint8_t*>(q);
+  const bool vec = (K % 8 == 0) && (ld_x % 8 == 0) && (ld_q % 8 == 0) &&
+                   (reinterpret_cast<uintptr_t>(x) % 16 == 0) &&
+                   (reinterpret_cast<uintptr_t>(q) % 8 == 0);
+  int64_t blocks = M;
+  const int64_t kMaxBlocks = 256 * 64;  // the rest is picked up by the grid-stride loops
+  if (blocks > kMaxBlocks) blocks = kMaxBlocks;
+  hipLaunchKernelGGL(zero_amax, dim3(1), dim3(1), 0, stream, amax_ws);
+  hipLaunchKernelGGL(tensor_amax, dim3((unsigned)blocks), dim3(64), 0, stream, xp, ld_x, (int)M,
+                     (int)K, vec, amax_ws);
+  hipLaunchKernelGGL(quant_tensorwise_cast, dim3((unsigned)blocks), dim3(64), 0, stream, xp, ld_x,
+                     qp, ld_q, scale, (int)M, (int)K, scale_mode, vec, amax_ws);
   return 0;
 }
 

@@ -24,7 +24,7 @@ FP8 = torch.float8_e4m3fn
 DEFAULT_SCALE_MODE = "bf16div"
 
 
-def _quantize_weight(weight: torch.Tensor, scale_mode: str):
+def _quantize_weight(weight: torch.Tensor, scale_mode: str, per_tensor: bool = False):
   """W bf16 [N,K] -> (codes e4m3 [N,K], scale fp32 [N,1]) with the HIP quantizer.
 
   The reference quantizes the weight wherever it lives, and its CLI flow does so
@@ -39,7 +39,8 @@ def _quantize_weight(weight: torch.Tensor, scale_mode: str):
       raise RuntimeError("quantizing a CPU weight needs a GPU to run the quantizer kernel on; "
                          "there is no CPU path")
     src = src.to("cuda")
-  q, s = ops.fp8_rowwise_quant(src.contiguous(), scale_mode)
+  quant = ops.fp8_tensorwise_quant if per_tensor else ops.fp8_rowwise_quant
+  q, s = quant(src.contiguous(), scale_mode)
   return q.to(weight.device), s.to(weight.device)
 
 
@@ -89,6 +90,24 @@ class Fp8DynamicLinear(_Fp8LinearBase):
     return out.view(*x.shape[:-1], self.out_features)
 
 
+class Fp8DynamicLinearPerTensor(_Fp8LinearBase):
+  """`float8_per_tensor` (w8a8 dynamic, one scale per tensor): the activation is
+  quantized with a single scale computed from its global amax, the weight likewise
+  at conversion time; `weight_scale` [N,1] then holds N copies of the weight's scale
+  and the GEMM is the per-row one fed with constant scales."""
+
+  def forward(self, x: torch.Tensor) -> torch.Tensor:
+    x2 = self._check_input(x)
+    M = x2.shape[0]
+    out = torch.empty((M, self.out_features), dtype=torch.bfloat16, device=x2.device)
+    if M > 0:
+      q, s = ops.activation_workspace(M, self.in_features, x2.device)
+      ws = ops.amax_workspace(x2.device)
+      ops.quant_tensorwise_into(x2, q, s, ws, self._scale_mode_id)
+      ops.gemm_rowwise_into(q, s, self.weight, self.weight_scale, self.bias, out, self.epilogue)
+    return out.view(*x.shape[:-1], self.out_features)
+
+
 class Fp8WeightOnlyLinear(_Fp8LinearBase):
   """`float8_weight_only` (w8a16): bf16 activations, e4m3 weights dequantized in
   the GEMM mainloop, per-channel scale in the epilogue."""
@@ -104,6 +123,7 @@ class Fp8WeightOnlyLinear(_Fp8LinearBase):
 
 _CLASS_OF = {
     "float8_per_row": Fp8DynamicLinear,
+    "float8_per_tensor": Fp8DynamicLinearPerTensor,
     "float8_weight_only": Fp8WeightOnlyLinear,
 }
 
@@ -125,7 +145,7 @@ def convert_linear_(linear: nn.Linear,
   if linear.in_features % 16 != 0 or linear.out_features % 16 != 0:
     raise ValueError(f"FP8 matmul needs in/out features that are multiples of 16, got "
                      f"{linear.in_features}x{linear.out_features}")
-  q, s = _quantize_weight(linear.weight, scale_mode)
+  q, s = _quantize_weight(linear.weight, scale_mode, per_tensor=quant_type == "float8_per_tensor")
   bias = linear.bias
   del linear.weight
   linear.weight = nn.Parameter(q, requires_grad=False)

@@ -85,6 +85,23 @@ def activation_workspace(M: int, K: int, device: torch.device):
   return ws[0][:M * K].view(M, K), ws[1][:M]
 
 
+_amax_workspaces: dict = {}
+
+
+def amax_workspace(device: torch.device) -> torch.Tensor:
+  """4 bytes of device scratch for the per-tensor quantizer, one per (device,
+  stream) outside graph capture (uses are ordered on the stream), fresh from the
+  graph's pool during capture."""
+  if torch.cuda.is_current_stream_capturing():
+    return torch.empty((1,), dtype=torch.int32, device=device)
+  key = (device.index, torch._C._cuda_getCurrentRawStream(device.index))
+  ws = _amax_workspaces.get(key)
+  if ws is None:
+    ws = torch.empty((1,), dtype=torch.int32, device=device)
+    _amax_workspaces[key] = ws
+  return ws
+
+
 def _require_cuda(name: str, *tensors: Optional[torch.Tensor]) -> None:
   for t in tensors:
     if t is not None and not t.is_cuda:
@@ -94,6 +111,18 @@ def _require_cuda(name: str, *tensors: Optional[torch.Tensor]) -> None:
 
 # --------------------------------------------------------------------------- raw launchers
 # These take already-validated 2-D tensors and write into caller-provided outputs.
+
+
+def quant_tensorwise_into(x2: torch.Tensor, q: torch.Tensor, scale: torch.Tensor,
+                          amax_ws: torch.Tensor, scale_mode_id: int) -> None:
+  """Per-tensor quantizer: one scale for all of x2, written to every scale[m].
+  amax_ws: 4 bytes of device scratch (an int32 tensor of one element)."""
+  M, K = x2.shape
+  with _DeviceOf(x2):
+    _native.check(_native.load().cdit_fp8_quant_tensorwise(x2.data_ptr(), M, K, x2.stride(0),
+                                                           q.data_ptr(), q.stride(0),
+                                                           scale.data_ptr(), amax_ws.data_ptr(),
+                                                           scale_mode_id, _stream_ptr(x2)))
 
 
 def quant_rowwise_into(x2: torch.Tensor, q: torch.Tensor, scale: torch.Tensor,
@@ -328,6 +357,25 @@ def _fake_w8a16_mm(x, b_data, b_scale, bias, out_dtype_id, epilogue=0):
 
 
 # --------------------------------------------------------------------------- python-level API
+
+
+def fp8_tensorwise_quant(x: torch.Tensor,
+                         scale_mode: str = "bf16div") -> Tuple[torch.Tensor, torch.Tensor]:
+  """Per-tensor dynamic e4m3 quantization of a bf16 tensor -> (codes, scale[M,1]
+  with every entry equal to the tensor's scale)."""
+  _require_cuda("fp8_tensorwise_quant", x)
+  if x.dtype != torch.bfloat16:
+    raise ValueError(f"fp8_tensorwise_quant: x must be bfloat16, got {x.dtype}")
+  x2 = x.reshape(-1, x.shape[-1])
+  if x2.stride(-1) != 1:
+    x2 = x2.contiguous()
+  M, K = x2.shape
+  q = torch.empty((M, K), dtype=FP8, device=x.device)
+  s = torch.empty((M,), dtype=torch.float32, device=x.device)
+  ws = torch.empty((1,), dtype=torch.int32, device=x.device)
+  if M > 0:
+    quant_tensorwise_into(x2, q, s, ws, _native.SCALE_MODE_IDS[scale_mode])
+  return q.view(x.shape), s.view(*x.shape[:-1], 1)
 
 
 def fp8_rowwise_quant(x: torch.Tensor,

@@ -28,7 +28,7 @@ ALLOWED_QUANTIZE_TYPES = [
     "int4_weight_only",
 ]
 #: the ones with MI355X kernels behind them
-BUILT_QUANTIZE_TYPES = ["float8_per_row", "float8_weight_only"]
+BUILT_QUANTIZE_TYPES = ["float8_per_row", "float8_per_tensor", "float8_weight_only"]
 
 _DEFAULT_EXCLUDE = ("embedder", "embed", "modulation", "mod")
 

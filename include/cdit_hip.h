@@ -92,6 +92,25 @@ int cdit_fp8_quant_rowwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_
                            int scale_mode, void* stream);
 
 /*
+ * Per-tensor dynamic FP8 quantization: one scale for the whole tensor. Replaces
+ * torchao's Float8Tensor.from_hp(x, PerTensor()) as selected for the
+ * "float8_per_tensor" quant type and the per-tensor fallback pass,
+ * src/cache_dit/quantization/torchao/quantize_ao.py:559-575 and :139-148.
+ *
+ *   amax     = max_{m,k} |x[m,k]|
+ *   s        = amax/448 rounded per scale_mode; 0 -> 1
+ *   q[m,k]   = e4m3fn_rne(clamp(float(x[m,k]) / s, -448, 448))
+ *   scale[m] = s for every m (the GEMM entry point takes per-row scales)
+ *
+ * amax_ws: 4 bytes of device memory owned by the caller, used as scratch (the
+ * bf16 bit pattern of amax is left in it). Three kernels are enqueued; nothing is
+ * allocated or synchronised.
+ */
+int cdit_fp8_quant_tensorwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_x,
+                              void* q_e4m3, int64_t ld_q, float* scale, void* amax_ws,
+                              int scale_mode, void* stream);
+
+/*
  * Row-wise scaled FP8 GEMM with fused epilogue. Replaces
  * torch._scaled_mm(a, b, scale_a, scale_b, bias, out_dtype) as called by
  * _run_float8_inference_scaled_mm, src/cache_dit/quantization/torchao/_scaled_mm.py:62-91

@@ -38,6 +38,8 @@ def lib() -> ctypes.CDLL:
     i64, vp, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
     L.oracle_quant_rowwise.restype = None
     L.oracle_quant_rowwise.argtypes = [vp, i64, i64, i64, vp, i64, vp, ci]
+    L.oracle_quant_tensorwise.restype = None
+    L.oracle_quant_tensorwise.argtypes = [vp, i64, i64, i64, vp, i64, vp, ci]
     L.oracle_gemm_rowwise.restype = None
     L.oracle_gemm_rowwise.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci]
     L.oracle_w8a16.restype = None
@@ -57,6 +59,16 @@ def quant_rowwise(x_bits: np.ndarray, mode: int):
   q = np.empty((M, K), dtype=np.uint8)
   s = np.empty((M,), dtype=np.float32)
   lib().oracle_quant_rowwise(_ptr(x_bits), M, K, K, _ptr(q), K, _ptr(s), mode)
+  return q, s
+
+
+def quant_tensorwise(x_bits: np.ndarray, mode: int):
+  """Per-tensor variant: (codes uint8 [M,K], scale f32 [M], all entries equal)."""
+  x_bits = np.ascontiguousarray(x_bits, dtype=np.uint16)
+  M, K = x_bits.shape
+  q = np.empty((M, K), dtype=np.uint8)
+  s = np.empty((M,), dtype=np.float32)
+  lib().oracle_quant_tensorwise(_ptr(x_bits), M, K, K, _ptr(q), K, _ptr(s), mode)
   return q, s
 
 

@@ -143,6 +143,26 @@ void oracle_quant_rowwise(const uint16_t* x, int64_t M, int64_t K, int64_t ld_x,
   }
 }
 
+/* Per-tensor: one amax over the whole tensor, scale[m] = that scale for every m. */
+void oracle_quant_tensorwise(const uint16_t* x, int64_t M, int64_t K, int64_t ld_x, uint8_t* q,
+                             int64_t ld_q, float* scale, int mode) {
+  uint16_t amax = 0;
+  int has_nan = 0;
+  for (int64_t m = 0; m < M; ++m)
+    for (int64_t k = 0; k < K; ++k) {
+      uint16_t a = x[m * ld_x + k] & 0x7fff;
+      if (a > 0x7f80) has_nan = 1;
+      if (a > amax) amax = a;
+    }
+  if (has_nan) amax = 0x7fc0;
+  const float s = oracle_row_scale(amax, mode);
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    scale[m] = s;
+    for (int64_t k = 0; k < K; ++k) q[m * ld_q + k] = oracle_quant_one(x[m * ld_x + k], s);
+  }
+}
+
 float oracle_gelu_tanh(float v) {
   const float kAlpha = 0.7978845608028654f, kBeta = 0.044715f;
   return 0.5f * v * (1.0f + tanhf(kAlpha * (v + kBeta * v * v * v)));

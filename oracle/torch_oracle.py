@@ -58,6 +58,28 @@ def quantize_rowwise(x: torch.Tensor,
   return quantize_affine_float8(x, scale), scale
 
 
+def choose_scale_tensorwise(x: torch.Tensor, scale_mode: str = "bf16div") -> torch.Tensor:
+  """One fp32 scale (shape [1, 1]) for the whole bf16 tensor: torchao
+  `_choose_scale_float8` with `PerTensor()` granularity, the config built at
+  src/cache_dit/quantization/torchao/quantize_ao.py:559-575, under the same
+  zero-scale patch (:43-71)."""
+  assert scale_mode in SCALE_MODES, scale_mode
+  amax = x.abs().amax().reshape(1, 1)
+  if scale_mode == "bf16div":
+    scale = (amax / FP8_MAX).to(torch.float32)
+  else:
+    scale = amax.to(torch.float32) / FP8_MAX
+  return torch.where(scale == 0, torch.ones_like(scale), scale)
+
+
+def quantize_tensorwise(x: torch.Tensor,
+                        scale_mode: str = "bf16div") -> Tuple[torch.Tensor, torch.Tensor]:
+  """x bf16 [M, K] -> (codes float8_e4m3fn [M, K], scale fp32 [M, 1] with every
+  entry equal to the tensor's scale: the layout the GEMM entry point takes)."""
+  scale = choose_scale_tensorwise(x, scale_mode)
+  return quantize_affine_float8(x, scale), scale.expand(x.shape[0], 1).contiguous()
+
+
 def gelu_tanh(v: torch.Tensor) -> torch.Tensor:
   return torch.nn.functional.gelu(v, approximate="tanh")
 
