@@ -120,13 +120,19 @@ __device__ __forceinline__ uint32_t quant4(uint32_t w0, uint32_t w1, float s, fl
   return p;
 }
 
+// Running max of packed |bf16| pairs, both halves at once: m and the result hold
+// two independent 16-bit maxima (v_pk_max_u16), compared as unsigned integers
+// (monotone in magnitude; a NaN pattern wins, as in torch.amax). fold2 merges the
+// halves at the end.
 __device__ __forceinline__ uint32_t absmax2(uint32_t m, uint32_t w) {
-  // running max of two packed |bf16| values, compared as unsigned 16-bit
-  // integers (monotone in magnitude; a NaN pattern wins, as in torch.amax).
-  uint32_t a = w & 0x7fff7fffu;
-  uint32_t lo = a & 0xffffu, hi = a >> 16;
-  uint32_t mx = lo > hi ? lo : hi;
-  return m > mx ? m : mx;
+  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+  const u16x2 a = __builtin_bit_cast(u16x2, w & 0x7fff7fffu);
+  const u16x2 r = __builtin_elementwise_max(__builtin_bit_cast(u16x2, m), a);
+  return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint32_t fold2(uint32_t m) {
+  const uint32_t lo = m & 0xffffu, hi = m >> 16;
+  return lo > hi ? lo : hi;
 }
 
 // Row resident in registers: CH 16-byte chunks per lane (K <= CH*512).
@@ -165,7 +171,7 @@ __global__ __launch_bounds__(64) void quant_rowwise_regs(
       m = absmax2(m, v[c].z);
       m = absmax2(m, v[c].w);
     }
-    m = wave_max_u32(m);
+    m = wave_max_u32(fold2(m));
     const float s = row_scale(m, scale_mode);
     if (lane == 0) scale[row] = s;
     uint2* qr = reinterpret_cast<uint2*>(q + row * ld_q);
@@ -262,7 +268,7 @@ __global__ __launch_bounds__(64) void tensor_amax(const uint16_t* __restrict__ x
       }
     }
   }
-  m = wave_max_u32(m);
+  m = wave_max_u32(fold2(m));
   if (lane == 0 && m != 0u) atomicMax(amax_ws, m);
 }
 
