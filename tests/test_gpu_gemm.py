@@ -163,6 +163,33 @@ def test_qwen_and_wan_shapes_sampled_rows(M, N, K):
   assert torch.isfinite(out.float()).all()
 
 
+@pytest.mark.parametrize("variant", [12, 14, 15])
+def test_wide_kernels_random_shapes_many_tiles_per_workgroup(variant):
+  """Random shapes with edge tiles in M and N and more tiles than CUs (a persistent
+  workgroup then runs several tiles, the DMA stream crossing tile boundaries), exact
+  small-integer data: sampled rows must match the oracle bit for bit."""
+  from cache_dit_amd import _native, ops
+  rng = torch.Generator().manual_seed(100 + variant)
+  for _ in range(6):
+    M = int(torch.randint(2000, 9000, (1,), generator=rng))
+    N = int(torch.randint(250, 1200, (1,), generator=rng)) * 8
+    K = int(torch.randint(2, 13, (1,), generator=rng)) * 128
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    a = torch.randint(-3, 4, (M, K), generator=g, device="cuda").float().to(FP8)
+    w = torch.randint(-3, 4, (N, K), generator=g, device="cuda").float().to(FP8)
+    sa = torch.full((M,), 0.5, device="cuda")
+    sw = torch.full((N,), 0.25, device="cuda")
+    b = torch.randint(-8, 9, (N,), generator=g, device="cuda").to(torch.bfloat16)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    _native.set_gemm_variant(variant)
+    ops.gemm_rowwise_into(a, sa, w, sw, b, out, 0)
+    torch.cuda.synchronize()
+    rows = torch.cat([torch.arange(0, M, 61), torch.arange(M - 5, M)])
+    ref = to.scaled_mm_rowwise(a[rows.cuda()].cpu(), sa[rows.cuda()].cpu().reshape(-1, 1), w.cpu(),
+                               sw.cpu().reshape(-1, 1), b.cpu())
+    assert torch.equal(out[rows.cuda()].cpu(), ref), (M, N, K)
+
+
 def test_config1_full():
   x, w, b = config1_inputs()
   xq, xs = to.quantize_rowwise(x[0])

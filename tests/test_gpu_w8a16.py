@@ -145,3 +145,28 @@ def test_against_c_oracle_and_gelu():
     ref = torch.from_numpy(ref_bits.view(np.int16)).view(torch.bfloat16)
     _assert_close(_run(x, wq, ws * (8 if gelu else 1), b, epilogue=gelu), ref if not gelu else
                   to.w8a16_linear(x, wq, ws * 8, b, gelu="fused", fused=True))
+
+
+@pytest.mark.parametrize("variant", [7, 8, 9])
+def test_wide_kernels_random_shapes_many_tiles_per_workgroup(variant):
+  """Random shapes with edge tiles in M and N and more tiles than CUs (persistent
+  workgroups run several tiles each), exact small-integer data: sampled rows must
+  match the oracle bit for bit."""
+  from cache_dit_amd import _native, ops
+  rng = torch.Generator().manual_seed(200 + variant)
+  for _ in range(6):
+    M = int(torch.randint(2000, 9000, (1,), generator=rng))
+    N = int(torch.randint(130, 600, (1,), generator=rng)) * 16
+    K = int(torch.randint(2, 17, (1,), generator=rng)) * 64
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    x = torch.randint(-3, 4, (M, K), generator=g, device="cuda").to(torch.bfloat16)
+    w = torch.randint(-3, 4, (N, K), generator=g, device="cuda").float().to(FP8)
+    sw = torch.full((N,), 0.25, device="cuda")
+    b = torch.randint(-8, 9, (N,), generator=g, device="cuda").to(torch.bfloat16)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    _native.set_gemm_variant(variant)
+    ops.w8a16_into(x, w, sw, b, out, 0)
+    torch.cuda.synchronize()
+    rows = torch.cat([torch.arange(0, M, 61), torch.arange(M - 5, M)])
+    ref = to.w8a16_linear(x[rows.cuda()].cpu(), w.cpu(), sw.cpu().reshape(-1, 1), b.cpu(), fused=True)
+    assert torch.equal(out[rows.cuda()].cpu(), ref), (M, N, K)
