@@ -467,18 +467,23 @@ int launch_pingpong(const GemmArgs& g, hipStream_t stream) {
 // so that a lane ends with 8 consecutive output columns per pair of fragments and
 // stores 16 bytes without a transpose (4 lanes cover 64 contiguous bytes of a row);
 // for those rows lane bit 3 is row bit 4, hence swz_b.
-template <int BM_, int BN_, int GROUP_M_>
+template <int BM_, int BN_, int GROUP_M_, int DEPTH_ = 2>
 struct CfgWide {
   static constexpr int BM = BM_, BN = BN_, GROUP_M = GROUP_M_;
+  // K steps the DMA stream runs ahead of the MFMAs. 2 for the large tiles (their
+  // stages fill the LDS); small tiles have short steps and need more of them in
+  // flight to cover the memory latency.
+  static constexpr int DEPTH = DEPTH_;
   static constexpr int WAVES = 4, THREADS = 256;
   static constexpr int WM = BM / 2, WN = BN / 2;      // wave tile (2 x 2 waves)
   static constexpr int TM = WM / 16, TN = WN / 16;    // 16x16 MFMA blocks per wave
   static constexpr int H = TM / 2;                    // rows of the first (i-major) half
   static constexpr int BKW = 128;
   static constexpr int A_BYTES = BM * BKW, B_BYTES = BN * BKW;
-  // A panel: 3 LDS stages (its DMA goes out in the first half of a step, into the
-  // stage read one step earlier); B panel: 2 stages (DMA in the second half)
-  static constexpr int A_STAGES = 3, B_STAGES = 2;
+  // A panel: DEPTH + 1 LDS stages (its DMA goes out in the first half of a step,
+  // into the stage read one step earlier); B panel: DEPTH stages (DMA in the
+  // second half, into the stage just read)
+  static constexpr int A_STAGES = DEPTH + 1, B_STAGES = DEPTH;
   static constexpr int B_BASE = A_STAGES * A_BYTES;
   static constexpr int LDS_BYTES = A_STAGES * A_BYTES + B_STAGES * B_BYTES;
   // DMA instructions (1 KiB = 8 panel rows) per wave and step
@@ -487,6 +492,7 @@ struct CfgWide {
   static_assert(BM % 32 == 0 && BN % 32 == 0, "panels are dealt 8 rows x 4 waves at a time");
   static_assert(TM * TN <= 64, "accumulators: at most 256 registers");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+  static_assert(DEPTH >= 2 && (DEPTH - 2) * ND + NDA < 63, "DMA instructions in flight: vmcnt has 6 bits");
 };
 
 __device__ __forceinline__ int swz_a(int row) { return ((row >> 1) & 1) | (((row >> 3) & 1) * 6); }
@@ -520,7 +526,8 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   constexpr int BKW = C::BKW, TM = C::TM, TN = C::TN, H = C::H;
-  const int KT = g.K / BKW;  // >= 2 (checked by the launcher)
+  constexpr int D = C::DEPTH;
+  const int KT = g.K / BKW;  // >= D (checked by the launcher)
   const int ntiles = tiles_m * tiles_n;
 
   // The workgroup is persistent: it takes tiles blockIdx.x, blockIdx.x + gridDim.x,
@@ -606,19 +613,19 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
   v4f acc[TM][TN];
   v8i af[TM], bf[TN];
 
-  // LDS offsets of the stages of steps kt-1 / kt / kt+1 (A) and kt / kt+1 (B)
-  int a_prev = 2 * C::A_BYTES, a_cur = 0, a_next = C::A_BYTES;
+  // LDS offsets of the stages of steps kt-1 / kt / kt+1 (A) and kt / kt+1 (B);
+  // step s lives in A stage s mod (D+1) and B stage s mod D
+  int a_prev = D * C::A_BYTES, a_cur = 0, a_next = C::A_BYTES;
   int b_cur = C::B_BASE, b_next = C::B_BASE + C::B_BYTES;
-  // prologue: steps 0 and 1 in flight, step 0 landed, its B fragments and A_0 read
+  // prologue: steps 0 .. D-1 in flight, step 0 landed
 #pragma unroll
-  for (int p = 0; p < C::NDA; ++p) dma_a(0, a_cur, p);
+  for (int s = 0; s < D; ++s) {
 #pragma unroll
-  for (int p = 0; p < C::NDB; ++p) dma_b(0, b_cur, p);
+    for (int p = 0; p < C::NDA; ++p) dma_a(s, s * C::A_BYTES, p);
 #pragma unroll
-  for (int p = 0; p < C::NDA; ++p) dma_a(1, a_next, p);
-#pragma unroll
-  for (int p = 0; p < C::NDB; ++p) dma_b(1, b_next, p);
-  wait_and_barrier<C::ND>();
+    for (int p = 0; p < C::NDB; ++p) dma_b(s, C::B_BASE + s * C::B_BYTES, p);
+  }
+  wait_and_barrier<(D - 1) * C::ND>();
 
   for (int tile = blockIdx.x;; tile += gridDim.x) {
     const int next_tile = tile + gridDim.x;
@@ -643,6 +650,18 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     // One K step; FIRST: step 0 of the tile (the accumulators start from zero).
     auto step = [&](int kt, auto first_tag) {
       constexpr bool FIRST = decltype(first_tag)::value;
+      if (kt == KT - D) {
+        // every DMA of this tile has been issued: the stream moves on
+        if (next_tile < ntiles) {
+          int tm, tn;
+          tile_of_block<C::GROUP_M>(next_tile, ntiles, tiles_m, tiles_n, &tm, &tn);
+          nm0 = tm * C::BM;
+          nn0 = tn * C::BN;
+          set_source(nm0, nn0);
+        } else {
+          nrec = 0;
+        }
+      }
       if (kt == KT - 2) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
@@ -656,18 +675,8 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
         }
 #pragma unroll
         for (int i = 0; i < TM; ++i) as[i] = mw + 16 * i < g.M ? g.a_scale[mw + 16 * i] : 0.0f;
-        // every DMA of this tile has been issued: the stream moves on
-        if (next_tile < ntiles) {
-          int tm, tn;
-          tile_of_block<C::GROUP_M>(next_tile, ntiles, tiles_m, tiles_n, &tm, &tn);
-          nm0 = tm * C::BM;
-          nn0 = tn * C::BN;
-          set_source(nm0, nn0);
-        } else {
-          nrec = 0;
-        }
       }
-      const int kd = kt + 2 < KT ? kt + 2 : kt + 2 - KT;  // step (of its tile) to fetch
+      const int kd = kt + D < KT ? kt + D : kt + D - KT;  // step (of its tile) to fetch
       const uint8_t* st = smem + a_cur;
 #pragma unroll
       for (int i = 0; i < H; ++i) {
@@ -678,7 +687,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
           if (k * H / (TM - H) == i) af[H + k] = read_a(st, H + k);
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          // A panel two steps ahead into the stage that step kt-1 read, one DMA
+          // A panel D steps ahead into the stage that step kt-1 read, one DMA
           // instruction every few MFMAs
 #pragma unroll
           for (int p = 0; p < C::NDA; ++p)
@@ -687,20 +696,20 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
           __builtin_amdgcn_sched_barrier(0);
         }
       }
-      // own LDS reads of this step done, own DMA of the next step landed (the A
-      // panel issued above may still fly); then everyone's. In step 0 of a later
-      // tile the DMA in question was waited for before the previous epilogue's
-      // stores, which may keep flying.
-      if (kt == 0 && tile != (int)blockIdx.x) {
+      // own LDS reads of this step done, own DMA of the next step landed (the
+      // steps after it and the A panel issued above may still fly); then
+      // everyone's. In the first D-1 steps of a later tile the DMA in question was
+      // waited for before the previous epilogue's stores, which may keep flying.
+      if (kt <= D - 2 && tile != (int)blockIdx.x) {
         wait_and_barrier<63>();
       } else {
-        wait_and_barrier<C::NDA>();
+        wait_and_barrier<(D - 2) * C::ND + C::NDA>();
       }
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
 #pragma unroll
         for (int i = H; i < TM; ++i) {
-          // B panel two steps ahead into the B stage of this step, one DMA
+          // B panel D steps ahead into the B stage of this step, one DMA
           // instruction every few MFMAs
 #pragma unroll
           for (int p = 0; p < C::NDB; ++p)
@@ -713,13 +722,12 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
         __builtin_amdgcn_sched_barrier(0);
       }
       // rotate the stages
-      const int a_free = a_prev;
       a_prev = a_cur;
       a_cur = a_next;
-      a_next = a_free;
-      const int b_free = b_cur;
+      a_next = a_next + C::A_BYTES == C::A_STAGES * C::A_BYTES ? 0 : a_next + C::A_BYTES;
       b_cur = b_next;
-      b_next = b_free;
+      b_next = b_next + C::B_BYTES == C::B_BASE + C::B_STAGES * C::B_BYTES ? C::B_BASE
+                                                                           : b_next + C::B_BYTES;
     };
     step(0, std::true_type{});
     for (int kt = 1; kt < KT; ++kt) step(kt, std::false_type{});
@@ -729,7 +737,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
 
     // ---- epilogue
     const bool gelu = (g.epilogue & CDIT_EPI_GELU_TANH) != 0;
-    // Every DMA issued so far (the next tile's first two steps) must have landed
+    // Every DMA issued so far (the next tile's first D steps) must have landed
     // before the stores go out: step 0 of the next tile then waits for nothing.
     wait_vm<0>();
 #pragma unroll
@@ -762,7 +770,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     m0 = nm0;
     n0 = nn0;
   }
-  // the zero-record DMA of the last two steps must not outlive the workgroup
+  // the zero-record DMA of the last D steps must not outlive the workgroup
   wait_vm<0>();
 }
 
@@ -932,6 +940,9 @@ typedef CfgPP<256, 192, 4, true, 8, 4> V11;           // ping-pong, 64x96 wave t
 typedef CfgWide<256, 256, 8> V12;                     // 4 waves, 128x128 wave tiles, 16x16x128 MFMA
 typedef CfgWide<288, 192, 8> V14;                     // ... 144x96 wave tiles
 typedef CfgWide<256, 192, 8> V15;                     // ... 128x96 wave tiles
+typedef CfgWide<128, 192, 4, 3> V16;                  // ... 64x96 wave tiles, DMA 3 steps ahead
+typedef CfgWide<64, 128, 8, 5> V17;                   // ... 32x64 wave tiles, DMA 5 steps ahead
+typedef CfgWide<128, 128, 4, 4> V18;                  // ... 64x64 wave tiles, DMA 4 steps ahead
 
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {
@@ -947,21 +958,21 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     hipLaunchKernelGGL(gemm_fp8_skinny, dim3((g.N + 15) / 16), dim3(256), 0, stream, g);
     return 0;
   }
+  // the wide kernels stream K two or more steps ahead: shorter K runs the 128x128 kernel
+  auto wide_ok = [&](int depth) { return g.K >= 128 * depth; };
   if (variant < 0) {
-    // Large problems take one of the wide kernels. Cost model, fitted to measured
-    // times: tile area times the number of rounds over the 256 CUs, where a last,
-    // partial round of r tiles counts 0.4 + 0.6 r/256 (the chip is power limited:
-    // with fewer CUs busy the clocks rise); ties go to the larger tile. Smaller
-    // problems take 128x128 tiles (two workgroups per CU) when those fill the
-    // chip, else 64x128 with a 4-deep DMA pipeline.
     auto tiles = [&](int bm, int bn) {
       return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
     };
-    auto cost = [&](int bm, int bn, int pen) {
-      const int64_t t = tiles(bm, bn), full = t / 256, rem = t % 256;
-      return (full * 2560 + (rem ? 1024 + 6 * rem : 0)) * bm * bn * pen;
-    };
     if (tiles(256, 256) >= 160) {
+      // Large problems take one of the large-tile wide kernels. Cost model, fitted to
+      // measured times: tile area times the number of rounds over the 256 CUs, where a
+      // last, partial round of r tiles counts 0.4 + 0.6 r/256 (the chip is power
+      // limited: with fewer CUs busy the clocks rise); ties go to the larger tile.
+      auto cost = [&](int bm, int bn, int pen) {
+        const int64_t t = tiles(bm, bn), full = t / 256, rem = t % 256;
+        return (full * 2560 + (rem ? 1024 + 6 * rem : 0)) * bm * bn * pen;
+      };
       variant = 12;
       int64_t best = cost(256, 256, 100);
       const struct { int v, bm, bn, pen; } cand[] = {
@@ -973,14 +984,27 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
           variant = c.v;
         }
       }
-    } else if (tiles(128, 128) >= 256) {
-      variant = 6;
     } else {
-      variant = 21;
+      // Smaller problems (the text-stream Linears, M of a few hundred to a few
+      // thousand): whole rounds over the CUs times tile area, the small tiles
+      // penalised by their measured lower MFMA rate (per mille); ties go to the
+      // larger tile. Tiles whose prefetch depth K cannot feed are left out.
+      const struct { int v, bm, bn, pen, depth; } cand[] = {
+          {12, 256, 256, 1000, 2}, {14, 288, 192, 1000, 2}, {15, 256, 192, 1000, 2},
+          {16, 128, 192, 1124, 3}, {18, 128, 128, 1000, 4}, {17, 64, 128, 1493, 5}};
+      int64_t best = INT64_MAX;
+      // K < 256: the kernels without a K stream across tiles
+      variant = tiles(128, 128) >= 256 ? 6 : 21;
+      for (const auto& c : cand) {
+        if (!wide_ok(c.depth)) continue;
+        const int64_t t = (tiles(c.bm, c.bn) + 255) / 256 * c.bm * c.bn * c.pen;
+        if (t < best) {
+          best = t;
+          variant = c.v;
+        }
+      }
     }
   }
-  // the wide kernels stream K two steps ahead: shorter K runs the 128x128 kernel
-  const bool wide_ok = g.K >= 256;
   switch (variant) {
     case 0: return launch_tiled<V0>(g, stream);
     case 1: return launch_tiled<V1>(g, stream);
@@ -992,9 +1016,12 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     case 9: return launch_pingpong<V9>(g, stream);
     case 10: return launch_pingpong<V10>(g, stream);
     case 11: return launch_pingpong<V11>(g, stream);
-    case 12: return wide_ok ? launch_wide<V12>(g, stream) : launch_tiled<V6>(g, stream);
-    case 14: return wide_ok ? launch_wide<V14>(g, stream) : launch_tiled<V6>(g, stream);
-    case 15: return wide_ok ? launch_wide<V15>(g, stream) : launch_tiled<V6>(g, stream);
+    case 12: return wide_ok(V12::DEPTH) ? launch_wide<V12>(g, stream) : launch_tiled<V6>(g, stream);
+    case 14: return wide_ok(V14::DEPTH) ? launch_wide<V14>(g, stream) : launch_tiled<V6>(g, stream);
+    case 15: return wide_ok(V15::DEPTH) ? launch_wide<V15>(g, stream) : launch_tiled<V6>(g, stream);
+    case 16: return wide_ok(V16::DEPTH) ? launch_wide<V16>(g, stream) : launch_tiled<V6>(g, stream);
+    case 17: return wide_ok(V17::DEPTH) ? launch_wide<V17>(g, stream) : launch_tiled<V6>(g, stream);
+    case 18: return wide_ok(V18::DEPTH) ? launch_wide<V18>(g, stream) : launch_tiled<V6>(g, stream);
     default:
       set_error("cdit_fp8_gemm_rowwise: unknown kernel variant %d", variant);
       return CDIT_EINVAL;

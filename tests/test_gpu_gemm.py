@@ -49,7 +49,7 @@ def _assert_close(out, ref):
   assert elementwise_ok(out, ref, REL_TOL)
 
 
-TILED_VARIANTS = [0, 1, 6, 7, 8, 9, 10, 11, 12, 14, 15, 20, 21]
+TILED_VARIANTS = [0, 1, 6, 7, 8, 9, 10, 11, 12, 14, 15, 16, 17, 18, 20, 21]
 
 
 @pytest.mark.parametrize("variant", TILED_VARIANTS + [100])
@@ -163,7 +163,7 @@ def test_qwen_and_wan_shapes_sampled_rows(M, N, K):
   assert torch.isfinite(out.float()).all()
 
 
-@pytest.mark.parametrize("variant", [12, 14, 15])
+@pytest.mark.parametrize("variant", [12, 14, 15, 16, 17, 18])
 def test_wide_kernels_random_shapes_many_tiles_per_workgroup(variant):
   """Random shapes with edge tiles in M and N and more tiles than CUs (a persistent
   workgroup then runs several tiles, the DMA stream crossing tile boundaries), exact
