@@ -598,12 +598,17 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     rd_a[e] = (wm * C::WM + r16) * BKW + (((2 * kg + e) ^ swz_a(wm * C::WM + r16)) << 4);
     rd_b[e] = (wn * C::WN + brow) * BKW + (((2 * kg + e) ^ swz_b(wn * C::WN + brow)) << 4);
   }
-  auto read_a = [&](const uint8_t* st, int i) -> v8i {
+  // __restrict__: loads through a restrict-qualified pointer carry alias scope
+  // information. Without it the compiler assumes that an LDS read may alias any
+  // LDS-DMA write in flight and puts s_waitcnt vmcnt(0) in front of the read, which
+  // drains the DMA stream at every step. The stages read in a step are never the
+  // ones its DMA fills; the explicit waits before the barriers order the two.
+  auto read_a = [&](const uint8_t* __restrict__ st, int i) -> v8i {
     const v4i lo = *reinterpret_cast<const v4i*>(st + rd_a[0] + i * 16 * BKW);
     const v4i hi = *reinterpret_cast<const v4i*>(st + rd_a[1] + i * 16 * BKW);
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
-  auto read_b = [&](const uint8_t* st, int j) -> v8i {
+  auto read_b = [&](const uint8_t* __restrict__ st, int j) -> v8i {
     const int ro = 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
     const v4i lo = *reinterpret_cast<const v4i*>(st + rd_b[0] + ro * BKW);
     const v4i hi = *reinterpret_cast<const v4i*>(st + rd_b[1] + ro * BKW);

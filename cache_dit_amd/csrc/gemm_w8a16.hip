@@ -366,16 +366,19 @@ int launch_pingpong(const GemmArgs& g, hipStream_t stream) {
 // swapped (weights first) a lane then ends with 16 consecutive output columns per
 // block, n = 32j + 16h + r for accumulator register r, and stores them with two
 // 16-byte stores, no transpose.
-template <int BM_, int BN_, int GROUP_M_>
+template <int BM_, int BN_, int GROUP_M_, int DEPTH_ = 2>
 struct CfgWW {
   static constexpr int BM = BM_, BN = BN_, GROUP_M = GROUP_M_;
+  // K steps the DMA stream runs ahead of the MFMAs (A panel in DEPTH + 1 LDS stages,
+  // B panel in DEPTH): 2 for the large tiles, more for small tiles with short steps
+  static constexpr int DEPTH = DEPTH_;
   static constexpr int WAVES = 4, THREADS = 256;
   static constexpr int WM = BM / 2, WN = BN / 2;
   static constexpr int TM = WM / 32, TN = WN / 32;
   static constexpr int H = TM / 2;
   static constexpr int A_ROW = BKE * 2, B_ROW = BKE;
   static constexpr int A_BYTES = BM * A_ROW, B_BYTES = BN * B_ROW;
-  static constexpr int A_STAGES = 3, B_STAGES = 2;
+  static constexpr int A_STAGES = DEPTH + 1, B_STAGES = DEPTH;
   static constexpr int B_BASE = A_STAGES * A_BYTES;
   static constexpr int LDS_BYTES = A_STAGES * A_BYTES + B_STAGES * B_BYTES;
   // DMA instructions (1 KiB: 8 A rows or 16 B rows) per wave and step
@@ -385,6 +388,7 @@ struct CfgWW {
   static_assert(TM * TN <= 16, "accumulators: at most 256 registers");
   static_assert(TM >= 2, "two halves per step");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+  static_assert(DEPTH >= 2 && (DEPTH - 2) * ND + NDA < 63, "DMA instructions in flight: vmcnt has 6 bits");
 };
 
 struct AFrag {
@@ -430,7 +434,8 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
   // local copies: a template-dependent expression as a builtin argument inside a
   // lambda makes the host pass drop the kernel stub without a diagnostic
   constexpr int TM = C::TM, TN = C::TN, H = C::H, A_ROW = C::A_ROW, B_ROW = C::B_ROW;
-  const int KT = g.K / BKE;  // >= 2 (checked by the launcher)
+  constexpr int D = C::DEPTH;
+  const int KT = g.K / BKE;  // >= D (checked by the launcher)
   const int ntiles = tiles_m * tiles_n;
 
   int m0, n0;  // tile being computed
@@ -494,14 +499,19 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
           (wm * C::WM + r32) * C::A_ROW + (((4 * t + 2 * h + e) ^ ((r32 >> 1) & 7)) << 4);
     rd_b[t] = (wn * C::WN + wrow) * C::B_ROW + (((2 * t + h) ^ ((wrow >> 2) & 3)) << 4);
   }
-  auto read_a = [&](const uint8_t* st, int i) -> AFrag {
+  // __restrict__: loads through a restrict-qualified pointer carry alias scope
+  // information. Without it the compiler assumes that an LDS read may alias any
+  // LDS-DMA write in flight and puts s_waitcnt vmcnt(0) in front of the read, which
+  // drains the DMA stream at every step. The stages read in a step are never the
+  // ones its DMA fills; the explicit waits before the barriers order the two.
+  auto read_a = [&](const uint8_t* __restrict__ st, int i) -> AFrag {
     AFrag f;
 #pragma unroll
     for (int q = 0; q < 4; ++q)
       f.k[q] = *reinterpret_cast<const v8bf*>(st + rd_a[q] + i * 32 * C::A_ROW);
     return f;
   };
-  auto read_w = [&](const uint8_t* st, int j) -> WRaw {
+  auto read_w = [&](const uint8_t* __restrict__ st, int j) -> WRaw {
     WRaw f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -514,18 +524,18 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
   AFrag wf[TN];  // converted weights
   WRaw wr[TN];   // weights as read from LDS (next step's, until converted)
 
-  int a_prev = 2 * C::A_BYTES, a_cur = 0, a_next = C::A_BYTES;
+  // step s lives in A stage s mod (D+1) and B stage s mod D
+  int a_prev = D * C::A_BYTES, a_cur = 0, a_next = C::A_BYTES;
   int b_cur = C::B_BASE, b_next = C::B_BASE + C::B_BYTES;
-  // prologue: steps 0 and 1 in flight, step 0 landed
+  // prologue: steps 0 .. D-1 in flight, step 0 landed
 #pragma unroll
-  for (int p = 0; p < C::NDA; ++p) dma_a(0, a_cur, p);
+  for (int s = 0; s < D; ++s) {
 #pragma unroll
-  for (int p = 0; p < C::NDB; ++p) dma_b(0, b_cur, p);
+    for (int p = 0; p < C::NDA; ++p) dma_a(s, s * C::A_BYTES, p);
 #pragma unroll
-  for (int p = 0; p < C::NDA; ++p) dma_a(1, a_next, p);
-#pragma unroll
-  for (int p = 0; p < C::NDB; ++p) dma_b(1, b_next, p);
-  wait_and_barrier<C::ND>();
+    for (int p = 0; p < C::NDB; ++p) dma_b(s, C::B_BASE + s * C::B_BYTES, p);
+  }
+  wait_and_barrier<(D - 1) * C::ND>();
 
   for (int tile = blockIdx.x;; tile += gridDim.x) {
     const int next_tile = tile + gridDim.x;
@@ -539,7 +549,7 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
     // One K step; FIRST: step 0 of the tile (the accumulators start from zero).
     auto step = [&](int kt, auto first_tag) {
       constexpr bool FIRST = decltype(first_tag)::value;
-      if (kt == KT - 2) {
+      if (kt == KT - D) {
         // every DMA of this tile has been issued: the stream moves on
         if (next_tile < ntiles) {
           int tm, tn;
@@ -551,7 +561,7 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
           nrec = 0;
         }
       }
-      const int kd = kt + 2 < KT ? kt + 2 : kt + 2 - KT;  // step (of its tile) to fetch
+      const int kd = kt + D < KT ? kt + D : kt + D - KT;  // step (of its tile) to fetch
       const uint8_t* st = smem + a_cur;
       auto convert = [&](int j) {
         convert_w(wr[j].t[0], wf[j].k[0], wf[j].k[1]);
@@ -582,7 +592,7 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
 #pragma unroll
           for (int j = 0; j < TN; ++j) {
             if (i == 0 && q == 0 && j + 1 < TN) convert(j + 1);
-            // A panel two steps ahead into the stage that step kt-1 read
+            // A panel D steps ahead into the stage that step kt-1 read
 #pragma unroll
             for (int p = 0; p < C::NDA; ++p)
               if (p * (H * TN * 4) / C::NDA == (i * 4 + q) * TN + j) dma_a(kd, a_prev, p);
@@ -591,13 +601,14 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
           }
         }
       }
-      // own LDS reads of this step done, own DMA of the next step landed (the A
-      // panel issued above may still fly); then everyone's. In step 0 of a later
-      // tile that DMA was waited for before the previous epilogue's stores.
-      if (kt == 0 && tile != (int)blockIdx.x) {
+      // own LDS reads of this step done, own DMA of the next step landed (the steps
+      // after it and the A panel issued above may still fly); then everyone's. In the
+      // first D-1 steps of a later tile that DMA was waited for before the previous
+      // epilogue's stores.
+      if (kt <= D - 2 && tile != (int)blockIdx.x) {
         wait_and_barrier<63>();
       } else {
-        wait_and_barrier<C::NDA>();
+        wait_and_barrier<(D - 2) * C::ND + C::NDA>();
       }
       // second half: pairs of columns, so that dependent MFMAs are 2 (TM-H) apart
 #pragma unroll
@@ -609,7 +620,7 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
           for (int i = H; i < TM; ++i)
 #pragma unroll
             for (int j = j0; j < j0 + 2 && j < TN; ++j) {
-              // B panel two steps ahead into the B stage of this step
+              // B panel D steps ahead into the B stage of this step
 #pragma unroll
               for (int p = 0; p < C::NDB; ++p)
                 if (p * (R * TN * 4) / C::NDB ==
@@ -623,13 +634,12 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
         if (j0 == 0) af[0] = read_a(smem + a_next, 0);
         __builtin_amdgcn_sched_barrier(0);
       }
-      const int a_free = a_prev;
       a_prev = a_cur;
       a_cur = a_next;
-      a_next = a_free;
-      const int b_free = b_cur;
+      a_next = a_next + C::A_BYTES == C::A_STAGES * C::A_BYTES ? 0 : a_next + C::A_BYTES;
       b_cur = b_next;
-      b_next = b_free;
+      b_next = b_next + C::B_BYTES == C::B_BASE + C::B_STAGES * C::B_BYTES ? C::B_BASE
+                                                                           : b_next + C::B_BYTES;
     };
     step(0, std::true_type{});
     for (int kt = 1; kt < KT; ++kt) step(kt, std::false_type{});
@@ -642,7 +652,7 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
     const bool gelu = (g.epilogue & CDIT_EPI_GELU_TANH) != 0;
     const int nw = n0 + wn * C::WN + 16 * h;
     const int mw = m0 + wm * C::WM + r32;
-    // every DMA issued so far (the next tile's first two steps) must have landed
+    // every DMA issued so far (the next tile's first D steps) must have landed
     // before the stores go out: step 0 of the next tile then waits for nothing
     wait_vm<0>();
 #pragma unroll
@@ -689,7 +699,7 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
     m0 = nm0;
     n0 = nn0;
   }
-  // the zero-record DMA of the last two steps must not outlive the workgroup
+  // the zero-record DMA of the last D steps must not outlive the workgroup
   wait_vm<0>();
 }
 
@@ -857,6 +867,9 @@ typedef CfgWP<128, 256, 4, 8> W6;
 typedef CfgWW<256, 256, 8> W7;              // wide: 4 waves, 128x128 wave tiles
 typedef CfgWW<256, 192, 8> W8;              // wide: 128x96 wave tiles
 typedef CfgWW<192, 256, 8> W9;              // wide: 96x128 wave tiles
+typedef CfgWW<128, 192, 4, 4> W10;          // wide: 64x96 wave tiles, DMA 4 steps ahead
+typedef CfgWW<128, 128, 4, 5> W11;          // wide: 64x64 wave tiles, DMA 5 steps ahead
+typedef CfgWW<128, 64, 4, 6> W12;           // wide: 64x32 wave tiles, DMA 6 steps ahead
 
 int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {
@@ -872,8 +885,8 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
     hipLaunchKernelGGL(gemm_w8a16_skinny, dim3((g.N + 15) / 16), dim3(256), 0, stream, g);
     return 0;
   }
-  // the wide kernels stream K two steps ahead and store 16 columns per lane
-  const bool wide_ok = g.K >= 2 * BKE && g.N % 16 == 0;
+  // the wide kernels stream K two or more steps ahead and store 16 columns per lane
+  auto wide_ok = [&](int depth) { return g.K >= depth * BKE && g.N % 16 == 0; };
   if (variant < 0) {
     // Same cost model as the w8a8 entry point: tile area times rounds over the 256
     // CUs, a last partial round of r tiles counting 0.4 + 0.6 r/256.
@@ -884,12 +897,30 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
       const int64_t t = tiles(bm, bn), full = t / 256, rem = t % 256;
       return (full * 2560 + (rem ? 1024 + 6 * rem : 0)) * bm * bn * pen;
     };
-    if (tiles(256, 256) >= 160 && wide_ok) {
+    if (tiles(256, 256) >= 160 && wide_ok(2)) {
       variant = cost(256, 192, 103) < cost(256, 256, 100) ? 8 : 7;
-    } else if (tiles(256, 256) >= 200) {
-      variant = ((tiles(192, 384) + 255) / 256) * 192 * 384 < ((tiles(256, 256) + 255) / 256) * 256 * 256 ? 5 : 4;
     } else {
-      variant = 3;
+      // Smaller problems: whole rounds over the CUs times tile area, the small tiles
+      // penalised by their measured lower MFMA rate (per mille); ties go to the larger
+      // tile. Tiles whose prefetch depth K cannot feed are left out; without any wide
+      // tile (N not a multiple of 16, very short K) the older kernels run.
+      const struct { int v, bm, bn, pen, depth; } cand[] = {
+          {7, 256, 256, 1000, 2}, {8, 256, 192, 1000, 2}, {10, 128, 192, 1300, 4},
+          {11, 128, 128, 1400, 5}, {12, 128, 64, 1700, 6}};
+      int64_t best = INT64_MAX;
+      if (tiles(256, 256) >= 200) {
+        variant = ((tiles(192, 384) + 255) / 256) * 192 * 384 < ((tiles(256, 256) + 255) / 256) * 256 * 256 ? 5 : 4;
+      } else {
+        variant = 3;
+      }
+      for (const auto& c : cand) {
+        if (!wide_ok(c.depth)) continue;
+        const int64_t t = (tiles(c.bm, c.bn) + 255) / 256 * c.bm * c.bn * c.pen;
+        if (t < best) {
+          best = t;
+          variant = c.v;
+        }
+      }
     }
   }
   switch (variant) {
@@ -898,9 +929,12 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
     case 4: return launch_pingpong<W4>(g, stream);
     case 5: return launch_pingpong<W5>(g, stream);
     case 6: return launch_pingpong<W6>(g, stream);
-    case 7: return wide_ok ? launch_wide<W7>(g, stream) : launch_tiled<W3>(g, stream);
-    case 8: return wide_ok ? launch_wide<W8>(g, stream) : launch_tiled<W3>(g, stream);
-    case 9: return wide_ok ? launch_wide<W9>(g, stream) : launch_tiled<W3>(g, stream);
+    case 7: return wide_ok(W7::DEPTH) ? launch_wide<W7>(g, stream) : launch_tiled<W3>(g, stream);
+    case 8: return wide_ok(W8::DEPTH) ? launch_wide<W8>(g, stream) : launch_tiled<W3>(g, stream);
+    case 9: return wide_ok(W9::DEPTH) ? launch_wide<W9>(g, stream) : launch_tiled<W3>(g, stream);
+    case 10: return wide_ok(W10::DEPTH) ? launch_wide<W10>(g, stream) : launch_tiled<W3>(g, stream);
+    case 11: return wide_ok(W11::DEPTH) ? launch_wide<W11>(g, stream) : launch_tiled<W3>(g, stream);
+    case 12: return wide_ok(W12::DEPTH) ? launch_wide<W12>(g, stream) : launch_tiled<W3>(g, stream);
     default:
       set_error("cdit_w8a16_gemm: unknown kernel variant %d", variant);
       return CDIT_EINVAL;

@@ -2,7 +2,8 @@
 (the accumulators are tied to AGPR tuples), so the compiler's hazard recognizer
 does not see them. This test compiles their sources to gfx950 assembly (no GPU
 needed) and checks, in the code the compiler produced for every instance,
-the three situations in which the hardware needs software wait states:
+three situations in which the hardware needs software wait states, and one
+in which the compiler adds a wait that the kernels must not have:
 
   1. no MFMA reads (as its C operand) an AGPR that a VALU instruction
      (v_accvgpr_write / v_accvgpr_mov) wrote: accumulators start from MFMAs with a
@@ -12,7 +13,12 @@ the three situations in which the hardware needs software wait states:
      block ahead of their use; an operand converted right before the MFMA gave
      wrong results on hardware);
   3. at least 18 wait states lie between an MFMA and the first v_accvgpr_read of
-     an accumulator (the epilogue).
+     an accumulator (the epilogue);
+  4. no `s_waitcnt vmcnt(0)` lies between the first and the last MFMA: the K loop
+     waits for the LDS-DMA of the next step only. The compiler drains all of it
+     before an LDS read that it thinks may alias an LDS-DMA write, which exposes
+     the memory latency at every step; reads through a restrict-qualified pointer
+     carry alias scope information and are exempt.
 """
 import os
 import re
@@ -121,3 +127,7 @@ def test_inline_asm_mfma_hazards(wide_kernels):
           states += _wait_states(code[j])
           j -= 1
         assert states >= 18 or j < 0, f"{name}: accumulator read {states} wait states after an MFMA"
+    # 4. no complete drain of the DMA stream inside the K loop
+    for l in code[mfma[0]:mfma[-1]]:
+      assert not (l.startswith("s_waitcnt") and "vmcnt(0)" in l), \
+          f"{name}: {l!r} between MFMAs"
