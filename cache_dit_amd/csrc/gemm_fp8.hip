@@ -741,35 +741,50 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- epilogue
-    const bool gelu = (g.epilogue & CDIT_EPI_GELU_TANH) != 0;
     // Every DMA issued so far (the next tile's first D steps) must have landed
     // before the stores go out: step 0 of the next tile then waits for nothing.
     wait_vm<0>();
+    // The accumulators are read with inline assembly, one row of blocks at a time:
+    // left to itself the compiler copies all of them to VGPRs first, parks everything
+    // else that is live (DMA offsets, scales) in spare AGPRs and scratch, and a scratch
+    // reload waits for every output store in flight (vmcnt). The GELU decision is
+    // taken once per tile, not once per element.
+    auto epilogue = [&](auto gelu_tag) {
+      constexpr bool GELU = decltype(gelu_tag)::value;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int m = mw + 16 * i;
+      for (int i = 0; i < TM; ++i) {
+        const int m = mw + 16 * i;
 #pragma unroll
-      for (int u = 0; u < TN / 2; ++u) {  // pair of fragments 2u, 2u+1: 8 consecutive columns
-        uint32_t pk[4];
+        for (int u = 0; u < TN / 2; ++u) {  // pair of fragments 2u, 2u+1: 8 consecutive columns
+          uint32_t pk[4];
 #pragma unroll
-        for (int d = 0; d < 2; ++d) {
-          const int j = 2 * u + d;
-          const float b4[4] = {__uint_as_float(bi[j].x << 16), __uint_as_float(bi[j].x & 0xffff0000u),
-                               __uint_as_float(bi[j].y << 16), __uint_as_float(bi[j].y & 0xffff0000u)};
-          float v[4];
+          for (int d = 0; d < 2; ++d) {
+            const int j = 2 * u + d;
+            const float b4[4] = {__uint_as_float(bi[j].x << 16), __uint_as_float(bi[j].x & 0xffff0000u),
+                                 __uint_as_float(bi[j].y << 16), __uint_as_float(bi[j].y & 0xffff0000u)};
+            float v[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            v[e] = __fmaf_rn(acc[i][j][e] * as[i], bs[j][e], b4[e]);
-            if (gelu) v[e] = gelu_tanh(v[e]);
+            for (int e = 0; e < 4; ++e) {
+              float a;
+              asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a) : "a"(acc[i][j][e]));
+              v[e] = __fmaf_rn(a * as[i], bs[j][e], b4[e]);
+              if constexpr (GELU) v[e] = gelu_tanh(v[e]);
+            }
+            pk[2 * d] = pack_bf16x2(v[0], v[1]);
+            pk[2 * d + 1] = pack_bf16x2(v[2], v[3]);
           }
-          pk[2 * d] = pack_bf16x2(v[0], v[1]);
-          pk[2 * d + 1] = pack_bf16x2(v[2], v[3]);
+          const int n = nw + 64 * (u >> 1) + 32 * (u & 1);
+          if (m < g.M && n < g.N)
+            *reinterpret_cast<uint4*>(g.out + (int64_t)m * g.ldo + n) =
+                uint4{pk[0], pk[1], pk[2], pk[3]};
         }
-        const int n = nw + 64 * (u >> 1) + 32 * (u & 1);
-        if (m < g.M && n < g.N)
-          *reinterpret_cast<uint4*>(g.out + (int64_t)m * g.ldo + n) =
-              uint4{pk[0], pk[1], pk[2], pk[3]};
+        __builtin_amdgcn_sched_barrier(0);
       }
+    };
+    if (g.epilogue & CDIT_EPI_GELU_TANH) {
+      epilogue(std::true_type{});
+    } else {
+      epilogue(std::false_type{});
     }
     if (next_tile >= ntiles) break;
     m0 = nm0;

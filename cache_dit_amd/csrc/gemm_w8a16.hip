@@ -649,51 +649,72 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
 
     // ---- epilogue: acc[i][j][r] is out[m][n] with
     //   m = m0 + wm*WM + 32i + (lane&31),  n = n0 + wn*WN + 32j + 16h + r
-    const bool gelu = (g.epilogue & CDIT_EPI_GELU_TANH) != 0;
     const int nw = n0 + wn * C::WN + 16 * h;
     const int mw = m0 + wm * C::WM + r32;
-    // every DMA issued so far (the next tile's first D steps) must have landed
-    // before the stores go out: step 0 of the next tile then waits for nothing
-    wait_vm<0>();
+    // epilogue operands of all column blocks (the fragment registers are free now)
+    v4f bs[TN][4];
+    uint4 bi[TN][2];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n = nw + 32 * j;
-      v4f bs[4];
-      uint4 bi[2];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) bs[q] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-      bi[0] = bi[1] = uint4{0u, 0u, 0u, 0u};
+      for (int q = 0; q < 4; ++q) bs[j][q] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+      bi[j][0] = bi[j][1] = uint4{0u, 0u, 0u, 0u};
       if (n < g.N) {  // N % 16 == 0 on this path: 16 columns are all in or all out
 #pragma unroll
-        for (int q = 0; q < 4; ++q) bs[q] = *reinterpret_cast<const v4f*>(g.b_scale + n + 4 * q);
+        for (int q = 0; q < 4; ++q)
+          bs[j][q] = *reinterpret_cast<const v4f*>(g.b_scale + n + 4 * q);
         if (g.bias) {
-          bi[0] = *reinterpret_cast<const uint4*>(g.bias + n);
-          bi[1] = *reinterpret_cast<const uint4*>(g.bias + n + 8);
+          bi[j][0] = *reinterpret_cast<const uint4*>(g.bias + n);
+          bi[j][1] = *reinterpret_cast<const uint4*>(g.bias + n + 8);
         }
       }
-      const uint32_t bw[8] = {bi[0].x, bi[0].y, bi[0].z, bi[0].w, bi[1].x, bi[1].y, bi[1].z, bi[1].w};
+    }
+    // every DMA issued so far (the next tile's first D steps) must have landed
+    // before the stores go out: step 0 of the next tile then waits for nothing
+    wait_vm<0>();
+    // Accumulators are read with inline assembly, one block at a time (left to itself
+    // the compiler copies all of them to VGPRs first and spills what else is live);
+    // the GELU decision is taken once per tile, not once per element.
+    auto epilogue = [&](auto gelu_tag) {
+      constexpr bool GELU = decltype(gelu_tag)::value;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int m = mw + 32 * i;
-        uint32_t pk[8];
+      for (int j = 0; j < TN; ++j) {
+        const int n = nw + 32 * j;
+        const uint32_t bw[8] = {bi[j][0].x, bi[j][0].y, bi[j][0].z, bi[j][0].w,
+                                bi[j][1].x, bi[j][1].y, bi[j][1].z, bi[j][1].w};
 #pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const float b0 = __uint_as_float(bw[r >> 1] << 16);
-          const float b1 = __uint_as_float(bw[r >> 1] & 0xffff0000u);
-          float v0 = __fmaf_rn(acc[i][j][r], bs[r >> 2][r & 3], b0);
-          float v1 = __fmaf_rn(acc[i][j][r + 1], bs[r >> 2][(r + 1) & 3], b1);
-          if (gelu) {
-            v0 = gelu_tanh(v0);
-            v1 = gelu_tanh(v1);
+        for (int i = 0; i < TM; ++i) {
+          const int m = mw + 32 * i;
+          uint32_t pk[8];
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            const float b0 = __uint_as_float(bw[r >> 1] << 16);
+            const float b1 = __uint_as_float(bw[r >> 1] & 0xffff0000u);
+            float a0, a1;
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a0) : "a"(acc[i][j][r]));
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a1) : "a"(acc[i][j][r + 1]));
+            float v0 = __fmaf_rn(a0, bs[j][r >> 2][r & 3], b0);
+            float v1 = __fmaf_rn(a1, bs[j][r >> 2][(r + 1) & 3], b1);
+            if constexpr (GELU) {
+              v0 = gelu_tanh(v0);
+              v1 = gelu_tanh(v1);
+            }
+            pk[r >> 1] = pack_bf16x2(v0, v1);
           }
-          pk[r >> 1] = pack_bf16x2(v0, v1);
-        }
-        if (m < g.M && n < g.N) {
-          uint16_t* dst = g.out + (int64_t)m * g.ldo + n;
-          *reinterpret_cast<uint4*>(dst) = uint4{pk[0], pk[1], pk[2], pk[3]};
-          *reinterpret_cast<uint4*>(dst + 8) = uint4{pk[4], pk[5], pk[6], pk[7]};
+          if (m < g.M && n < g.N) {
+            uint16_t* dst = g.out + (int64_t)m * g.ldo + n;
+            *reinterpret_cast<uint4*>(dst) = uint4{pk[0], pk[1], pk[2], pk[3]};
+            *reinterpret_cast<uint4*>(dst + 8) = uint4{pk[4], pk[5], pk[6], pk[7]};
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
+    };
+    if (g.epilogue & CDIT_EPI_GELU_TANH) {
+      epilogue(std::true_type{});
+    } else {
+      epilogue(std::false_type{});
     }
     if (next_tile >= ntiles) break;
     m0 = nm0;
