@@ -50,8 +50,8 @@ int after_launch(const char* what) {
 }
 
 int check_gemm(const char* fn, const void* a, const void* b, const float* b_scale,
-               const void* out, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
-               int64_t ldo, int epilogue, int out_dtype_id) {
+               const void* bias, const void* out, int64_t M, int64_t N, int64_t K, int64_t lda,
+               int64_t ldb, int64_t ldo, int epilogue, int out_dtype_id, bool bf16_only) {
   if (M < 0 || N < 0 || K < 0) {
     set_error("%s: negative dimension (M=%lld N=%lld K=%lld)", fn, (long long)M, (long long)N,
               (long long)K);
@@ -61,8 +61,17 @@ int check_gemm(const char* fn, const void* a, const void* b, const float* b_scal
     set_error("%s: dimension exceeds int32", fn);
     return CDIT_EINVAL;
   }
-  if (out_dtype_id != CDIT_DT_BF16) {
+  if (out_dtype_id != CDIT_DT_F16 && out_dtype_id != CDIT_DT_BF16 && out_dtype_id != CDIT_DT_F32) {
+    set_error("%s: unknown out_dtype_id %d (0 = fp16, 1 = bf16, 2 = fp32)", fn, out_dtype_id);
+    return CDIT_EINVAL;
+  }
+  if (bf16_only && out_dtype_id != CDIT_DT_BF16) {
     set_error("%s: out_dtype_id %d not built (only 1 = bf16)", fn, out_dtype_id);
+    return CDIT_EINVAL;
+  }
+  if (out_dtype_id == CDIT_DT_F32 && bias) {
+    set_error("%s: an fp32 output takes no bias (add it afterwards, as the reference does around "
+              "torch._scaled_mm)", fn);
     return CDIT_EINVAL;
   }
   if (epilogue & ~CDIT_EPI_GELU_TANH) {
@@ -193,11 +202,12 @@ int cdit_fp8_quant_tensorwise(const void* x_bf16, int64_t M, int64_t K, int64_t 
 }
 
 int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale, const void* b_q,
-                          const float* b_scale, const void* bias_bf16, void* out, int64_t M,
+                          const float* b_scale, const void* bias, void* out, int64_t M,
                           int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldo,
                           int epilogue, int out_dtype_id, void* stream) {
   const char* fn = "cdit_fp8_gemm_rowwise";
-  int rc = check_gemm(fn, a_q, b_q, b_scale, out, M, N, K, lda, ldb, ldo, epilogue, out_dtype_id);
+  int rc = check_gemm(fn, a_q, b_q, b_scale, bias, out, M, N, K, lda, ldb, ldo, epilogue,
+                      out_dtype_id, false);
   if (rc) return rc;
   if (M == 0 || N == 0) return CDIT_OK;
   if (!a_scale) {
@@ -211,7 +221,7 @@ int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale, const void* b_q
   g.a_scale = a_scale;
   g.b = static_cast<const uint8_t*>(b_q);
   g.b_scale = b_scale;
-  g.bias = static_cast<const uint16_t*>(bias_bf16);
+  g.bias = static_cast<const uint16_t*>(bias);
   g.out = static_cast<uint16_t*>(out);
   g.M = (int)M;
   g.N = (int)N;
@@ -220,17 +230,18 @@ int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale, const void* b_q
   g.ldb = ldb;
   g.ldo = ldo;
   g.epilogue = epilogue;
+  g.out_dtype = out_dtype_id;
   rc = launch_gemm_fp8(g, g_gemm_variant, static_cast<hipStream_t>(stream));
   return rc ? rc : after_launch(fn);
 }
 
 int cdit_fp8_linear_w8a8(const void* x_bf16, const void* w_q, const float* w_scale,
-                         const void* bias_bf16, void* out, void* q_ws, float* scale_ws, int64_t M,
+                         const void* bias, void* out, void* q_ws, float* scale_ws, int64_t M,
                          int64_t N, int64_t K, int64_t ld_x, int64_t ldw, int64_t ldo,
                          int scale_mode, int epilogue, int out_dtype_id, void* stream) {
   int rc = cdit_fp8_quant_rowwise(x_bf16, M, K, ld_x, q_ws, K, scale_ws, scale_mode, stream);
   if (rc) return rc;
-  return cdit_fp8_gemm_rowwise(q_ws, scale_ws, w_q, w_scale, bias_bf16, out, M, N, K, K, ldw, ldo,
+  return cdit_fp8_gemm_rowwise(q_ws, scale_ws, w_q, w_scale, bias, out, M, N, K, K, ldw, ldo,
                                epilogue, out_dtype_id, stream);
 }
 
@@ -239,8 +250,8 @@ int cdit_w8a16_gemm(const void* x_bf16, const void* b_q, const float* b_scale,
                     int64_t lda, int64_t ldb, int64_t ldo, int epilogue, int out_dtype_id,
                     void* stream) {
   const char* fn = "cdit_w8a16_gemm";
-  int rc =
-      check_gemm(fn, x_bf16, b_q, b_scale, out, M, N, K, lda, ldb, ldo, epilogue, out_dtype_id);
+  int rc = check_gemm(fn, x_bf16, b_q, b_scale, bias_bf16, out, M, N, K, lda, ldb, ldo, epilogue,
+                      out_dtype_id, true);
   if (rc) return rc;
   if (M == 0 || N == 0) return CDIT_OK;
   rc = check_arch();

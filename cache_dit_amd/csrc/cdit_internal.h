@@ -25,11 +25,12 @@ struct GemmArgs {
   const float* a_scale;  // [M] (w8a8) or nullptr (w8a16)
   const uint8_t* b;      // fp8 [N,K]
   const float* b_scale;  // [N]
-  const uint16_t* bias;  // bf16 [N] or nullptr
-  uint16_t* out;         // bf16 [M,N]
+  const uint16_t* bias;  // [N] in the output's dtype (fp16 or bf16) or nullptr; fp32 output: nullptr
+  uint16_t* out;         // [M,N] of out_dtype (fp32 output: really a float*, ldo in elements)
   int M, N, K;
   int64_t lda, ldb, ldo;
   int epilogue;
+  int out_dtype = CDIT_DT_BF16;  // CDIT_DT_*; the w8a16 kernels only build bf16
 };
 
 // variant < 0: choose by shape.

@@ -31,6 +31,39 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf));
 }
 
+// two fp32 -> packed fp16 (round to nearest even, overflow to infinity).
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+  const v2f v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2h));
+}
+
+// 16 bits of a bias vector -> fp32; the bias has the output's dtype (fp16 or bf16).
+template <int OUT>
+__device__ __forceinline__ float bias_to_f32(uint32_t bits16) {
+  if constexpr (OUT == CDIT_DT_F16) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
+  } else {
+    return __uint_as_float(bits16 << 16);
+  }
+}
+
+// Element-wise forms for the kernels that are not tuned per output dtype.
+__device__ __forceinline__ float bias_at(const GemmArgs& g, int n) {
+  const uint32_t b = g.bias[n];
+  return g.out_dtype == CDIT_DT_F16 ? bias_to_f32<CDIT_DT_F16>(b) : bias_to_f32<CDIT_DT_BF16>(b);
+}
+__device__ __forceinline__ void store_out(const GemmArgs& g, int64_t idx, float v) {
+  if (g.out_dtype == CDIT_DT_F32) {
+    reinterpret_cast<float*>(g.out)[idx] = v;
+  } else if (g.out_dtype == CDIT_DT_F16) {
+    g.out[idx] = __builtin_bit_cast(uint16_t, (_Float16)v);
+  } else {
+    g.out[idx] = (uint16_t)f32_to_bf16_bits(v);
+  }
+}
+
 // tanh-approximated GELU, the formula of torch.nn.functional.gelu(approximate="tanh"):
 // 0.5 v (1 + tanh(u)), u = sqrt(2/pi) (v + 0.044715 v^3). Since
 // 0.5 (1 + tanh(u)) = 1 / (1 + exp(-2u)), it is evaluated as v * rcp(1 + exp2(c u))

@@ -516,7 +516,9 @@ __device__ __forceinline__ void mfma_16x16x128_fp8(v4f& acc, const v8i& b, const
   }
 }
 
-template <class C>
+// OUT: dtype of the output and of the bias (CDIT_DT_*), a template parameter so that
+// the bf16 instances carry no trace of the others.
+template <class C, int OUT = CDIT_DT_BF16>
 __global__ __launch_bounds__(C::THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void
 gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -756,27 +758,37 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
         const int m = mw + 16 * i;
 #pragma unroll
         for (int u = 0; u < TN / 2; ++u) {  // pair of fragments 2u, 2u+1: 8 consecutive columns
-          uint32_t pk[4];
+          float v[8];
 #pragma unroll
           for (int d = 0; d < 2; ++d) {
             const int j = 2 * u + d;
-            const float b4[4] = {__uint_as_float(bi[j].x << 16), __uint_as_float(bi[j].x & 0xffff0000u),
-                                 __uint_as_float(bi[j].y << 16), __uint_as_float(bi[j].y & 0xffff0000u)};
-            float v[4];
+            const float b4[4] = {bias_to_f32<OUT>(bi[j].x & 0xffffu), bias_to_f32<OUT>(bi[j].x >> 16),
+                                 bias_to_f32<OUT>(bi[j].y & 0xffffu), bias_to_f32<OUT>(bi[j].y >> 16)};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               float a;
               asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a) : "a"(acc[i][j][e]));
-              v[e] = __fmaf_rn(a * as[i], bs[j][e], b4[e]);
-              if constexpr (GELU) v[e] = gelu_tanh(v[e]);
+              float t = __fmaf_rn(a * as[i], bs[j][e], b4[e]);
+              if constexpr (GELU) t = gelu_tanh(t);
+              v[4 * d + e] = t;
             }
-            pk[2 * d] = pack_bf16x2(v[0], v[1]);
-            pk[2 * d + 1] = pack_bf16x2(v[2], v[3]);
           }
           const int n = nw + 64 * (u >> 1) + 32 * (u & 1);
-          if (m < g.M && n < g.N)
-            *reinterpret_cast<uint4*>(g.out + (int64_t)m * g.ldo + n) =
-                uint4{pk[0], pk[1], pk[2], pk[3]};
+          if (m < g.M && n < g.N) {
+            if constexpr (OUT == CDIT_DT_F32) {
+              float* dst = reinterpret_cast<float*>(g.out) + (int64_t)m * g.ldo + n;
+              *reinterpret_cast<v4f*>(dst) = v4f{v[0], v[1], v[2], v[3]};
+              *reinterpret_cast<v4f*>(dst + 4) = v4f{v[4], v[5], v[6], v[7]};
+            } else if constexpr (OUT == CDIT_DT_F16) {
+              *reinterpret_cast<uint4*>(g.out + (int64_t)m * g.ldo + n) =
+                  uint4{pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3]), pack_f16x2(v[4], v[5]),
+                        pack_f16x2(v[6], v[7])};
+            } else {
+              *reinterpret_cast<uint4*>(g.out + (int64_t)m * g.ldo + n) =
+                  uint4{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]),
+                        pack_bf16x2(v[6], v[7])};
+            }
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -794,11 +806,11 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
   wait_vm<0>();
 }
 
-template <class C>
+template <class C, int OUT = CDIT_DT_BF16>
 int launch_wide(const GemmArgs& g, hipStream_t stream) {
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_fp8_wide<C>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_fp8_wide<C, OUT>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
     if (e != hipSuccess) {
       set_error("hipFuncSetAttribute(%d bytes LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
@@ -814,7 +826,7 @@ int launch_wide(const GemmArgs& g, hipStream_t stream) {
   const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
   const int ntiles = tiles_m * tiles_n;
   // one persistent workgroup per CU (its LDS and registers fill the CU)
-  hipLaunchKernelGGL(gemm_fp8_wide<C>, dim3(ntiles < cus ? ntiles : cus), dim3(C::THREADS),
+  hipLaunchKernelGGL((gemm_fp8_wide<C, OUT>), dim3(ntiles < cus ? ntiles : cus), dim3(C::THREADS),
                      C::LDS_BYTES, stream, g, tiles_m, tiles_n);
   return 0;
 }
@@ -880,14 +892,19 @@ __global__ __launch_bounds__(256) void gemm_fp8_skinny(GemmArgs g) {
                           (part[2][m][nl + e] + part[3][m][nl + e]);
         const int n = n0 + nl + e;
         float t = sum * as * g.b_scale[n];
-        if (g.bias) t += __uint_as_float((uint32_t)g.bias[n] << 16);
+        if (g.bias) t += bias_at(g, n);
         if (g.epilogue & CDIT_EPI_GELU_TANH) t = gelu_tanh(t);
         v[e] = t;
       }
-      uint2 pk;
-      pk.x = pack_bf16x2(v[0], v[1]);
-      pk.y = pack_bf16x2(v[2], v[3]);
-      *reinterpret_cast<uint2*>(g.out + (int64_t)m * g.ldo + n0 + nl) = pk;
+      if (g.out_dtype == CDIT_DT_BF16) {
+        uint2 pk;
+        pk.x = pack_bf16x2(v[0], v[1]);
+        pk.y = pack_bf16x2(v[2], v[3]);
+        *reinterpret_cast<uint2*>(g.out + (int64_t)m * g.ldo + n0 + nl) = pk;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) store_out(g, (int64_t)m * g.ldo + n0 + nl + e, v[e]);
+      }
     }
   }
 }
@@ -908,9 +925,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_generic(GemmArgs g) {
     acc = fmaf(x, w, acc);
   }
   float v = acc * g.a_scale[m] * g.b_scale[n];
-  if (g.bias) v += __uint_as_float((uint32_t)g.bias[n] << 16);
+  if (g.bias) v += bias_at(g, n);
   if (g.epilogue & CDIT_EPI_GELU_TANH) v = gelu_tanh(v);
-  g.out[(int64_t)m * g.ldo + n] = (uint16_t)f32_to_bf16_bits(v);
+  store_out(g, (int64_t)m * g.ldo + n, v);
 }
 
 template <class C>
@@ -980,6 +997,28 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   }
   // the wide kernels stream K two or more steps ahead: shorter K runs the 128x128 kernel
   auto wide_ok = [&](int depth) { return g.K >= 128 * depth; };
+  if (g.out_dtype != CDIT_DT_BF16) {
+    // fp16 / fp32 outputs (the op's other two out_dtype ids): one large and one small
+    // wide tile are built for them, chosen like the small-problem case below; what
+    // those cannot take runs the generic kernel.
+    const int64_t t_large = (int64_t)((g.M + 255) / 256) * ((g.N + 191) / 192);
+    const int64_t t_small = (int64_t)((g.M + 63) / 64) * ((g.N + 127) / 128);
+    const bool large = variant == 15 ||
+                       (variant != 17 && (!wide_ok(V17::DEPTH) ||
+                                          (t_large + 255) / 256 * 256 * 192 * 1000 <=
+                                              (t_small + 255) / 256 * 64 * 128 * 1493));
+    if (large && wide_ok(V15::DEPTH)) {
+      return g.out_dtype == CDIT_DT_F16 ? launch_wide<V15, CDIT_DT_F16>(g, stream)
+                                        : launch_wide<V15, CDIT_DT_F32>(g, stream);
+    }
+    if (!large && wide_ok(V17::DEPTH)) {
+      return g.out_dtype == CDIT_DT_F16 ? launch_wide<V17, CDIT_DT_F16>(g, stream)
+                                        : launch_wide<V17, CDIT_DT_F32>(g, stream);
+    }
+    dim3 grid((g.N + 15) / 16, (g.M + 15) / 16);
+    hipLaunchKernelGGL(gemm_fp8_generic, grid, dim3(256), 0, stream, g);
+    return 0;
+  }
   if (variant < 0) {
     auto tiles = [&](int bm, int bn) {
       return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);

@@ -138,14 +138,15 @@ def quant_rowwise_into(x2: torch.Tensor, q: torch.Tensor, scale: torch.Tensor,
 def gemm_rowwise_into(a: torch.Tensor, a_scale: torch.Tensor, w: torch.Tensor,
                       w_scale: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                       epilogue: int) -> None:
-  """a [M,K] e4m3, w [N,K] e4m3 (row-major), scales fp32 contiguous, out [M,N] bf16."""
+  """a [M,K] e4m3, w [N,K] e4m3 (row-major), scales fp32 contiguous, out [M,N] fp16,
+  bf16 or fp32; bias in the output's dtype (none for an fp32 output)."""
   M, K = a.shape
   N = w.shape[0]
   with _DeviceOf(a):
     _native.check(_native.load().cdit_fp8_gemm_rowwise(
         a.data_ptr(), a_scale.data_ptr(), w.data_ptr(), w_scale.data_ptr(),
         bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, K, a.stride(0),
-        w.stride(0), out.stride(0), epilogue, _native.DT_BF16, _stream_ptr(a)))
+        w.stride(0), out.stride(0), epilogue, encode_output_dtype(out.dtype), _stream_ptr(a)))
 
 
 def w8a16_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
@@ -294,8 +295,6 @@ def _float8_inference_scaled_mm(a_data, a_scale, b_data, b_scale, bias, out_dtyp
   del use_fast_accum  # a cuBLASLt hint; fp32 accumulation is the only mode here
   name = "cdit::float8_inference_scaled_mm"
   out_dtype = decode_output_dtype(out_dtype_id)
-  if out_dtype != torch.bfloat16:
-    raise ValueError(f"{name}: only bfloat16 output is built, got {out_dtype}")
   if a_data.dtype != FP8 or b_data.dtype != FP8:
     raise ValueError(f"{name}: a_data/b_data must be float8_e4m3fn, got {a_data.dtype}/"
                      f"{b_data.dtype}")
@@ -310,12 +309,20 @@ def _float8_inference_scaled_mm(a_data, a_scale, b_data, b_scale, bias, out_dtyp
                      f"{a_scale.numel()} and {b_scale.numel()}")
   a_s = a_scale.reshape(-1).to(torch.float32).contiguous()
   b_s = b_scale.reshape(-1).to(torch.float32).contiguous()
-  if bias is not None:
-    if bias.numel() != N:
-      raise ValueError(f"{name}: bias must have {N} elements")
-    bias = bias.reshape(-1).to(torch.bfloat16).contiguous()
-  out = torch.empty((M, N), dtype=torch.bfloat16, device=a_data.device)
-  gemm_rowwise_into(a2, a_s, w, b_s, bias, out, int(epilogue))
+  if bias is not None and bias.numel() != N:
+    raise ValueError(f"{name}: bias must have {N} elements")
+  out = torch.empty((M, N), dtype=out_dtype, device=a_data.device)
+  if out_dtype == torch.float32 and bias is not None:
+    # the reference adds the bias after the matmul for an fp32 output
+    # (_scaled_mm.py:71-81); with a fused activation it has to go in before that
+    if int(epilogue) != 0:
+      raise ValueError(f"{name}: an fp32 output with bias cannot fuse an activation")
+    gemm_rowwise_into(a2, a_s, w, b_s, None, out, 0)
+    out = out + bias.reshape(-1)
+  else:
+    if bias is not None:
+      bias = bias.reshape(-1).to(out_dtype).contiguous()
+    gemm_rowwise_into(a2, a_s, w, b_s, bias, out, int(epilogue))
   return out.reshape(*a_data.shape[:-1], N)
 
 

@@ -120,14 +120,19 @@ int cdit_fp8_quant_tensorwise(const void* x_bf16, int64_t M, int64_t K, int64_t 
  *
  * a_q: e4m3 [M,K] row-major (lda); b_q: e4m3 [N,K] row-major (ldb) -- the
  * quantized nn.Linear weight as stored, i.e. the reference's column-major
- * [K,N] `qweight.t()`; a_scale fp32 [M]; b_scale fp32 [N]; bias bf16 [N] or
- * NULL; out [M,N] (ldo) of out_dtype_id (only CDIT_DT_BF16 is built).
- * Accumulation is fp32. Requires K % 16 == 0 (as the reference's FP8 matmul
- * does) and 16-byte aligned a_q/b_q rows.
+ * [K,N] `qweight.t()`; a_scale fp32 [M]; b_scale fp32 [N]; out [M,N] (ldo, in
+ * elements) of out_dtype_id: CDIT_DT_F16, CDIT_DT_BF16 or CDIT_DT_F32, the
+ * op's three out_dtype ids (_scaled_mm.py:38-59). bias [N] has the output's
+ * dtype (fp16 or bf16) or is NULL; an fp32 output takes no bias: the reference
+ * adds it after the matmul in that case (_scaled_mm.py:71-81) and so must the
+ * caller. Accumulation is fp32. Requires K % 16 == 0 (as the reference's FP8
+ * matmul does) and 16-byte aligned a_q/b_q rows. bf16 is the tuned path; the
+ * other two dtypes have two tile shapes of the same kernel and a generic
+ * fallback.
  */
 int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale,
                           const void* b_q, const float* b_scale,
-                          const void* bias_bf16, void* out,
+                          const void* bias, void* out,
                           int64_t M, int64_t N, int64_t K,
                           int64_t lda, int64_t ldb, int64_t ldo,
                           int epilogue, int out_dtype_id, void* stream);
@@ -158,12 +163,13 @@ int cdit_w8a16_gemm(const void* x_bf16, const void* b_q, const float* b_scale,
  * Float8WeightConfig(granularity=(PerRow(), PerRow())))`
  * (src/cache_dit/quantization/torchao/quantize_ao.py:166-179, :540-558).
  *
- * x_bf16 [M,K] (ld_x); w_q e4m3 [N,K] (ldw); w_scale fp32 [N]; bias bf16 [N] or
- * NULL; out bf16 [M,N] (ldo); q_ws: workspace of M*K bytes (receives the
- * activation codes, contiguous); scale_ws: workspace of M floats.
+ * x_bf16 [M,K] (ld_x); w_q e4m3 [N,K] (ldw); w_scale fp32 [N]; bias and out as
+ * for cdit_fp8_gemm_rowwise (out_dtype_id; a Linear passes CDIT_DT_BF16, the dtype
+ * of its input); q_ws: workspace of M*K bytes (receives the activation codes,
+ * contiguous); scale_ws: workspace of M floats.
  */
 int cdit_fp8_linear_w8a8(const void* x_bf16, const void* w_q, const float* w_scale,
-                         const void* bias_bf16, void* out, void* q_ws, float* scale_ws,
+                         const void* bias, void* out, void* q_ws, float* scale_ws,
                          int64_t M, int64_t N, int64_t K,
                          int64_t ld_x, int64_t ldw, int64_t ldo,
                          int scale_mode, int epilogue, int out_dtype_id, void* stream);

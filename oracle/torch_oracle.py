@@ -89,15 +89,19 @@ def scaled_mm_rowwise(a_q: torch.Tensor,
                       b_q: torch.Tensor,
                       b_scale: torch.Tensor,
                       bias: Optional[torch.Tensor] = None,
-                      gelu: Optional[str] = None) -> torch.Tensor:
-  """Row-wise scaled FP8 matmul, fp32 accumulate, bf16 out.
+                      gelu: Optional[str] = None,
+                      out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+  """Row-wise scaled FP8 matmul, fp32 accumulate, out_dtype (bf16, fp16 or fp32) out.
 
   `torch._scaled_mm(a, b.t(), scale_a[M,1], scale_b[1,N], bias, out_dtype=bf16)` as
   called at src/cache_dit/quantization/torchao/_scaled_mm.py:62-91 (the CPU backend
   of _scaled_mm only takes per-tensor scales, so the scales are applied outside).
   a_q [M,K], b_q [N,K] float8_e4m3fn; a_scale [M,1], b_scale [N,1] or [N] fp32.
-  gelu: None, "fused" (on the fp32 value) or "unfused" (on the bf16 output, as a
+  gelu: None, "fused" (on the fp32 value) or "unfused" (on the rounded output, as a
   separate nn.GELU module does).
+  An fp32 output gets its bias the way the reference adds it, after the matmul
+  (`output + bias`, _scaled_mm.py:71-81): the same value, the sum of two fp32 numbers
+  rounded once.
   """
   acc = a_q.to(torch.float32) @ b_q.to(torch.float32).t()
   y = acc * a_scale.reshape(-1, 1) * b_scale.reshape(1, -1)
@@ -105,9 +109,9 @@ def scaled_mm_rowwise(a_q: torch.Tensor,
     y = y + bias.to(torch.float32)
   if gelu == "fused":
     y = gelu_tanh(y)
-  out = y.to(torch.bfloat16)
+  out = y.to(out_dtype)
   if gelu == "unfused":
-    out = gelu_tanh(out.to(torch.float32)).to(torch.bfloat16)
+    out = gelu_tanh(out.to(torch.float32)).to(out_dtype)
   return out
 
 

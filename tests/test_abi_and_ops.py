@@ -41,8 +41,14 @@ def test_argument_validation_without_gpu():
   one = ctypes.c_void_p(16)
   assert L.cdit_fp8_gemm_rowwise(one, one, one, one, None, one, 4, 4, 24, 24, 24, 4, 0, 1, None) == 1
   assert b"multiple of 16" in L.cdit_last_error()
-  assert L.cdit_fp8_gemm_rowwise(one, one, one, one, None, one, 4, 4, 32, 32, 32, 4, 0, 2, None) == 1
+  assert L.cdit_fp8_gemm_rowwise(one, one, one, one, None, one, 4, 4, 32, 32, 32, 4, 0, 3, None) == 1
   assert b"out_dtype_id" in L.cdit_last_error()
+  # an fp32 output takes no bias (the reference adds it after the matmul)
+  assert L.cdit_fp8_gemm_rowwise(one, one, one, one, one, one, 4, 4, 32, 32, 32, 4, 0, 2, None) == 1
+  assert b"no bias" in L.cdit_last_error()
+  # the weight-only GEMM builds bf16 only
+  assert L.cdit_w8a16_gemm(one, one, one, None, one, 4, 4, 32, 32, 32, 4, 0, 0, None) == 1
+  assert b"not built" in L.cdit_last_error()
   assert L.cdit_fp8_gemm_rowwise(one, one, one, one, None, one, 4, 4, 32, 32, 32, 4, 8, 1, None) == 1
   assert L.cdit_fp8_gemm_rowwise(one, one, one, one, None, one, 4, 4, 32, 16, 32, 4, 0, 1, None) == 1
   assert b"leading dimension" in L.cdit_last_error()

@@ -256,8 +256,6 @@ def test_error_paths():
   with pytest.raises(ValueError):
     ops.float8_inference_scaled_mm(a, s_a, w.t(), s_w, torch.float64)
   with pytest.raises(ValueError):
-    ops.float8_inference_scaled_mm(a, s_a, w.t(), s_w, torch.float32)  # not built
-  with pytest.raises(ValueError):
     ops.float8_inference_scaled_mm(a, s_a[:2], w.t(), s_w, torch.bfloat16)
   from cache_dit_amd import _native
   L = _native.load()
@@ -268,3 +266,71 @@ def test_error_paths():
   rc = L.cdit_fp8_gemm_rowwise(a.data_ptr(), s_a.data_ptr(), w.data_ptr(), s_w.data_ptr(), None,
                                o.data_ptr(), 0, 32, 64, 64, 64, 32, 0, 1, None)
   assert rc == 0  # empty M is a no-op
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K,variant", [(300, 520, 1024, -1), (2100, 1800, 512, 15),
+                                           (2100, 1800, 1024, 17), (5, 264, 256, -1),
+                                           (64, 48, 64, -1), (257, 72, 384, 100)])
+def test_output_dtypes(out_dtype, M, N, K, variant):
+  """The op's three out_dtype ids (reference _scaled_mm.py:38-59): fp16 and fp32 outputs
+  through the wide kernel (both tiles built for them), the skinny and the generic kernel,
+  against the oracle; an fp32 output with bias is the matmul plus a separate add."""
+  from cache_dit_amd import _native, ops
+  g = torch.Generator().manual_seed(M + N + K)
+  x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+  w = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16)
+  b = (torch.randn(N, generator=g) * 0.1).to(out_dtype)
+  aq, a_s = to.quantize_rowwise(x)
+  wq, w_s = to.quantize_rowwise(w)
+  ref = to.scaled_mm_rowwise(aq, a_s, wq, w_s, b, out_dtype=out_dtype)
+  _native.set_gemm_variant(variant)
+  out = ops.float8_inference_scaled_mm(aq.cuda(), a_s.cuda(), wq.cuda().t(), w_s.cuda().t(),
+                                       out_dtype, bias=b.cuda())
+  torch.cuda.synchronize()
+  assert out.dtype == out_dtype and out.shape == ref.shape
+  assert max_rel_err(out, ref) <= REL_TOL
+  assert elementwise_ok(out, ref, REL_TOL)
+  # GELU in the epilogue (no bias for fp32: the separate add would come after it)
+  bias = None if out_dtype == torch.float32 else b
+  ref = to.scaled_mm_rowwise(aq, a_s * 4, wq, w_s, bias, gelu="fused", out_dtype=out_dtype)
+  out = ops.float8_inference_scaled_mm(aq.cuda(), a_s.cuda() * 4, wq.cuda().t(), w_s.cuda().t(),
+                                       out_dtype, bias=None if bias is None else bias.cuda(),
+                                       epilogue=1)
+  assert max_rel_err(out, ref) <= REL_TOL
+
+
+def test_output_dtypes_exact():
+  """Small integers: every product and sum is exact, so fp16 / fp32 outputs must equal the
+  oracle bit for bit."""
+  from cache_dit_amd import ops
+  g = torch.Generator().manual_seed(5)
+  M, N, K = 700, 392, 768
+  a = torch.randint(-4, 5, (M, K), generator=g).float().to(FP8)
+  w = torch.randint(-4, 5, (N, K), generator=g).float().to(FP8)
+  s_a = torch.full((M, 1), 0.5)
+  s_w = torch.full((N, 1), 0.25)
+  for dt in (torch.float16, torch.float32):
+    b = torch.randint(-8, 9, (N,), generator=g).to(dt)
+    ref = to.scaled_mm_rowwise(a, s_a, w, s_w, b, out_dtype=dt)
+    out = ops.float8_inference_scaled_mm(a.cuda(), s_a.cuda(), w.cuda().t(), s_w.cuda().t(), dt,
+                                         bias=b.cuda())
+    assert torch.equal(out.cpu(), ref)
+
+
+def test_output_dtypes_second_witness():
+  """torch._scaled_mm on the same codes at fp16 / fp32 output, where the vendor library
+  offers it (on ROCm its row-wise FP8 matmul may only build bf16 outputs: then skipped)."""
+  from cache_dit_amd import ops
+  g = torch.Generator(device="cuda").manual_seed(6)
+  x = torch.randn(1024, 1024, generator=g, device="cuda").to(torch.bfloat16)
+  wt = (torch.randn(768, 1024, generator=g, device="cuda") * 0.03).to(torch.bfloat16)
+  aq, a_s = ops.fp8_rowwise_quant(x)
+  wq, w_s = ops.fp8_rowwise_quant(wt)
+  for dt in (torch.float16, torch.float32):
+    out = ops.float8_inference_scaled_mm(aq, a_s, wq.t(), w_s.t(), dt)
+    try:
+      ref = torch._scaled_mm(aq, wq.t(), scale_a=a_s, scale_b=w_s.t(), out_dtype=dt)
+    except Exception as e:  # pragma: no cover - depends on the box's hipBLASLt
+      pytest.skip(f"torch._scaled_mm row-wise {dt} not available here: {e}")
+    assert max_rel_err(out, ref) <= REL_TOL

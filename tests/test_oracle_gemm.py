@@ -99,3 +99,26 @@ def test_w8a8_tracks_the_unquantized_linear():
   y = to.w8a8_linear(x, wq, ws).float().flatten()
   ref = (x.float() @ w.float().t()).flatten()
   assert float(y @ ref / (y.norm() * ref.norm())) > 0.999
+
+
+def test_output_dtypes_are_one_rounding_of_the_fp32_result():
+  """fp16 / bf16 outputs are the fp32-output result rounded once (the GEMM accumulates and
+  applies scales and bias in fp32 whatever the output dtype), and an fp32 output with bias
+  equals the reference's `matmul(out_dtype=fp32) + bias` (_scaled_mm.py:71-81)."""
+  g = torch.Generator().manual_seed(21)
+  x = torch.randn(40, 64, generator=g).to(torch.bfloat16)
+  w = (torch.randn(24, 64, generator=g) * 0.1).to(torch.bfloat16)
+  aq, a_s = to.quantize_rowwise(x)
+  wq, w_s = to.quantize_rowwise(w)
+  b = (torch.randn(24, generator=g) * 0.1).to(torch.bfloat16)
+  f32 = to.scaled_mm_rowwise(aq, a_s, wq, w_s, b, out_dtype=torch.float32)
+  assert f32.dtype == torch.float32
+  for dt in (torch.float16, torch.bfloat16):
+    out = to.scaled_mm_rowwise(aq, a_s, wq, w_s, b.to(dt), out_dtype=dt)
+    if dt == torch.bfloat16:
+      assert torch.equal(out, f32.to(dt))
+    assert out.dtype == dt
+    assert (out.float() - to.scaled_mm_rowwise(aq, a_s, wq, w_s, b.to(dt), out_dtype=torch.float32)
+            ).abs().max() <= f32.abs().max() * 2.0**-8
+  no_bias = to.scaled_mm_rowwise(aq, a_s, wq, w_s, None, out_dtype=torch.float32)
+  assert torch.equal(f32, no_bias + b)
