@@ -2,8 +2,8 @@
 (the accumulators are tied to AGPR tuples), so the compiler's hazard recognizer
 does not see them. This test compiles their sources to gfx950 assembly (no GPU
 needed) and checks, in the code the compiler produced for every instance,
-three situations in which the hardware needs software wait states, and one
-in which the compiler adds a wait that the kernels must not have:
+three situations in which the hardware needs software wait states, and two
+things the compiler may add that the kernels must not have:
 
   1. no MFMA reads (as its C operand) an AGPR that a VALU instruction
      (v_accvgpr_write / v_accvgpr_mov) wrote: accumulators start from MFMAs with a
@@ -18,7 +18,10 @@ in which the compiler adds a wait that the kernels must not have:
      waits for the LDS-DMA of the next step only. The compiler drains all of it
      before an LDS read that it thinks may alias an LDS-DMA write, which exposes
      the memory latency at every step; reads through a restrict-qualified pointer
-     carry alias scope information and are exempt.
+     carry alias scope information and are exempt;
+  5. no scratch (register spill) access anywhere: a scratch reload is a vector
+     memory load, the wait for it (vmcnt) also waits for every output store in
+     flight, which serialises the epilogue of a tile with the next tile's K loop.
 """
 import os
 import re
@@ -127,6 +130,9 @@ def test_inline_asm_mfma_hazards(wide_kernels):
           states += _wait_states(code[j])
           j -= 1
         assert states >= 18 or j < 0, f"{name}: accumulator read {states} wait states after an MFMA"
+    # 5. no register spills
+    for l in code:
+      assert not l.startswith("scratch_"), f"{name}: register spill {l!r}"
     # 4. no complete drain of the DMA stream inside the K loop
     for l in code[mfma[0]:mfma[-1]]:
       assert not (l.startswith("s_waitcnt") and "vmcnt(0)" in l), \
