@@ -135,6 +135,22 @@ __device__ __forceinline__ void wait_steps(int later) {
 #undef CDIT_WAIT_CASE
 }
 
+// Raises a kernel's dynamic LDS limit to `bytes`, once per device: the attribute belongs
+// to the function on the current device. done: one flag per device ordinal, owned by the
+// caller (a static array per kernel instance; setting the attribute twice is harmless).
+inline int allow_dynamic_lds(const void* kernel, int bytes, bool* done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+  if (dev >= 0 && done[dev]) return 0;
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) {
+    set_error("hipFuncSetAttribute(%d bytes LDS): %s", bytes, hipGetErrorString(e));
+    return CDIT_EHIP;
+  }
+  if (dev >= 0) done[dev] = true;
+  return 0;
+}
+
 // Number of CUs of the current device (cached per device ordinal); 0 on error.
 inline int cu_count() {
   static int cached[64];

@@ -418,16 +418,10 @@ __global__ __launch_bounds__(C::THREADS, 2) void gemm_fp8_pingpong(GemmArgs g, i
 
 template <class C>
 int launch_pingpong(const GemmArgs& g, hipStream_t stream) {
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_fp8_pingpong<C>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(%d bytes LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
-      return CDIT_EHIP;
-    }
-    attr_set = true;
-  }
+  static bool lds_allowed[64];
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_fp8_pingpong<C>), C::LDS_BYTES,
+                                 lds_allowed))
+    return rc;
   const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
   hipLaunchKernelGGL(gemm_fp8_pingpong<C>, dim3(tiles_m * tiles_n), dim3(C::THREADS),
                      C::LDS_BYTES, stream, g, tiles_m, tiles_n);
@@ -808,16 +802,10 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
 
 template <class C, int OUT = CDIT_DT_BF16>
 int launch_wide(const GemmArgs& g, hipStream_t stream) {
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_fp8_wide<C, OUT>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(%d bytes LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
-      return CDIT_EHIP;
-    }
-    attr_set = true;
-  }
+  static bool lds_allowed[64];
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_fp8_wide<C, OUT>), C::LDS_BYTES,
+                                 lds_allowed))
+    return rc;
   const int cus = cu_count();
   if (cus <= 0) {
     set_error("cannot query the CU count of the current device");
@@ -932,16 +920,10 @@ __global__ __launch_bounds__(256) void gemm_fp8_generic(GemmArgs g) {
 
 template <class C>
 int launch_tiled(const GemmArgs& g, hipStream_t stream) {
-  static bool attr_set = false;  // benign race: setting it twice is harmless
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_fp8_tiled<C>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(%d bytes LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
-      return CDIT_EHIP;
-    }
-    attr_set = true;
-  }
+  static bool lds_allowed[64];
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_fp8_tiled<C>), C::LDS_BYTES,
+                                 lds_allowed))
+    return rc;
   const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
   hipLaunchKernelGGL(gemm_fp8_tiled<C>, dim3(tiles_m * tiles_n), dim3(C::THREADS), C::LDS_BYTES,
                      stream, g, tiles_m, tiles_n);
