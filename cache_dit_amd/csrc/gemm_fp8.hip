@@ -487,6 +487,44 @@ struct CfgWide {
   static_assert(TM * TN <= 64, "accumulators: at most 256 registers");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
   static_assert(DEPTH >= 2 && (DEPTH - 2) * ND + NDA < 63, "DMA instructions in flight: vmcnt has 6 bits");
+
+  // Issue schedule of a K step: which LDS reads and DMA instructions go in front of
+  // which MFMA. An LDS read pair or a DMA instruction holds the wave's instruction
+  // issue for a dozen clocks or more, an MFMA gives it 32: one such item between two
+  // MFMAs is free, a cluster of them leaves the matrix core idle.
+  // First half: S1 MFMAs (slot s = i*TN + j). Items: the TM-1 fragment reads A_1 ..
+  // A_{TM-1} of this step (in that order) and the NDA DMA instructions of the A panel,
+  // merged evenly, a read first, and spread evenly over the slots.
+  static constexpr int S1 = H * TN, NR1 = TM - 1, T1 = NR1 + NDA;
+  static constexpr int item_of_read1(int q) { return q * T1 / NR1; }  // a read leads
+  static constexpr bool is_read1(int t) {
+    for (int q = 0; q < NR1; ++q)
+      if (item_of_read1(q) == t) return true;
+    return false;
+  }
+  static constexpr int read1_index(int t) {  // reads before item t
+    int n = 0;
+    for (int q = 0; q < NR1; ++q) n += item_of_read1(q) < t;
+    return n;
+  }
+  static constexpr int dma1_index(int t) { return t - read1_index(t); }  // DMAs before item t
+  static constexpr int slot1(int t) { return t * S1 / T1; }
+  // A_{i} (i < H) is used from slot i*TN on: its read must be a few MFMAs earlier
+  static constexpr bool first_half_reads_in_time() {
+    for (int t = 0; t < T1; ++t)
+      if (is_read1(t) && read1_index(t) + 1 < H && slot1(t) + 3 > (read1_index(t) + 1) * TN)
+        return false;
+    return true;
+  }
+  static_assert(first_half_reads_in_time(), "A fragment read too late for its first use");
+  // Second half: S2 MFMAs, column-major (slot s = j*R + i-H). B_j of the next step is
+  // read one MFMA after the last use of B_j (slot (j+1)*R + 1, at most S2 = after the
+  // last MFMA), A_0 of the next step in front of slot 1, the NDB DMA instructions of
+  // the B panel in the middle of their share of the slots.
+  static constexpr int R = TM - H, S2 = R * TN;
+  static constexpr int slot_b(int j) { return (j + 1) * R + 1 < S2 ? (j + 1) * R + 1 : S2; }
+  static constexpr int slot_a0 = S2 > 1 ? 1 : 0;
+  static constexpr int slot_dma2(int p) { return (2 * p + 1) * S2 / (2 * NDB); }
 };
 
 __device__ __forceinline__ int swz_a(int row) { return ((row >> 1) & 1) | (((row >> 3) & 1) * 6); }
@@ -679,23 +717,22 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
       }
       const int kd = kt + D < KT ? kt + D : kt + D - KT;  // step (of its tile) to fetch
       const uint8_t* st = smem + a_cur;
+      // first half: rows 0..H-1, row-major; meanwhile the other A fragments of this
+      // step are read and the A panel D steps ahead goes into the stage that step
+      // kt-1 read (schedule: CfgWide::slot1)
 #pragma unroll
-      for (int i = 0; i < H; ++i) {
-        if (i + 1 < H) af[i + 1] = read_a(st, i + 1);
-        // the TM-H fragments of the second half, spread over the rows of the first
+      for (int sl = 0; sl < C::S1; ++sl) {
 #pragma unroll
-        for (int k = 0; k < TM - H; ++k)
-          if (k * H / (TM - H) == i) af[H + k] = read_a(st, H + k);
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          // A panel D steps ahead into the stage that step kt-1 read, one DMA
-          // instruction every few MFMAs
-#pragma unroll
-          for (int p = 0; p < C::NDA; ++p)
-            if (p * (H * TN) / C::NDA == i * TN + j) dma_a(kd, a_prev, p);
-          mfma_16x16x128_fp8<FIRST>(acc[i][j], bf[j], af[i]);
-          __builtin_amdgcn_sched_barrier(0);
+        for (int t = 0; t < C::T1; ++t) {
+          if (C::slot1(t) != sl) continue;
+          if (C::is_read1(t)) {
+            af[C::read1_index(t) + 1] = read_a(st, C::read1_index(t) + 1);
+          } else {
+            dma_a(kd, a_prev, C::dma1_index(t));
+          }
         }
+        mfma_16x16x128_fp8<FIRST>(acc[sl / TN][sl % TN], bf[sl % TN], af[sl / TN]);
+        __builtin_amdgcn_sched_barrier(0);
       }
       // own LDS reads of this step done, own DMA of the next step landed (the
       // steps after it and the A panel issued above may still fly); then
@@ -706,22 +743,26 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
       } else {
         wait_and_barrier<(D - 2) * C::ND + C::NDA>();
       }
+      // second half: rows H..TM-1, column-major; B_j of the next step replaces B_j
+      // after its last use, the B panel D steps ahead goes into the B stage of this
+      // step (after the very last step the reads fetch zeros that are never used)
+      auto second_half_items = [&](int sl) {
+        if (sl == C::slot_a0) af[0] = read_a(smem + a_next, 0);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
+        for (int j = 0; j < TN; ++j)
+          if (C::slot_b(j) == sl) bf[j] = read_b(smem + b_next, j);
 #pragma unroll
-        for (int i = H; i < TM; ++i) {
-          // B panel D steps ahead into the B stage of this step, one DMA
-          // instruction every few MFMAs
+        for (int p = 0; p < C::NDB; ++p)
+          if (C::slot_dma2(p) == sl) dma_b(kd, b_cur, p);
+      };
 #pragma unroll
-          for (int p = 0; p < C::NDB; ++p)
-            if (p * ((TM - H) * TN) / C::NDB == j * (TM - H) + (i - H)) dma_b(kd, b_cur, p);
-          mfma_16x16x128_fp8<FIRST>(acc[i][j], bf[j], af[i]);
-        }
-        // fragments of the next step (after the very last one: zeros, never used)
-        bf[j] = read_b(smem + b_next, j);
-        if (j == 0) af[0] = read_a(smem + a_next, 0);
+      for (int sl = 0; sl < C::S2; ++sl) {
+        second_half_items(sl);
+        mfma_16x16x128_fp8<FIRST>(acc[H + sl % C::R][sl / C::R], bf[sl / C::R], af[H + sl % C::R]);
         __builtin_amdgcn_sched_barrier(0);
       }
+      second_half_items(C::S2);
+      __builtin_amdgcn_sched_barrier(0);
       // rotate the stages
       a_prev = a_cur;
       a_cur = a_next;
