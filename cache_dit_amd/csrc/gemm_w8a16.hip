@@ -383,6 +383,50 @@ struct CfgWW {
   static_assert(TM >= 2, "two halves per step");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
   static_assert(DEPTH >= 2 && (DEPTH - 2) * ND + NDA < 63, "DMA instructions in flight: vmcnt has 6 bits");
+
+  // Issue schedule of a K step (see the wide w8a8 kernel: one LDS read, DMA instruction
+  // or group of four conversions between two MFMAs is free, a cluster is not).
+  // First half: S1 MFMAs, slot s = (i*4 + q)*TN + j. Items: the 4 (TM-1) single LDS
+  // reads of the fragments A_1 .. A_{TM-1} (MFMA step q of block i: read 4 (i-1) + q)
+  // and the NDA DMA instructions of the A panel, merged evenly, a read first, and spread
+  // evenly over the slots. The weights of column j, MFMA step q (4 conversions) are
+  // converted two slots ahead of their first use at slot q*TN + j.
+  static constexpr int S1 = H * 4 * TN, NR1 = 4 * (TM - 1), T1 = NR1 + NDA;
+  static constexpr int item_of_read1(int r) { return r * T1 / NR1; }
+  static constexpr bool is_read1(int t) {
+    for (int r = 0; r < NR1; ++r)
+      if (item_of_read1(r) == t) return true;
+    return false;
+  }
+  static constexpr int read1_index(int t) {  // reads before item t
+    int n = 0;
+    for (int r = 0; r < NR1; ++r) n += item_of_read1(r) < t;
+    return n;
+  }
+  static constexpr int dma1_index(int t) { return t - read1_index(t); }
+  static constexpr int slot1(int t) { return t * S1 / T1; }
+  static constexpr bool first_half_reads_in_time() {
+    for (int t = 0; t < T1; ++t) {
+      const int r = read1_index(t), i = r / 4 + 1, q = r % 4;
+      if (is_read1(t) && i < H && slot1(t) + 3 > (i * 4 + q) * TN) return false;
+    }
+    return true;
+  }
+  static_assert(first_half_reads_in_time(), "A fragment read too late for its first use");
+  static constexpr int CONVERT_AHEAD = 2;
+  // Second half: S2 MFMAs in blocks of column pairs (the order of the loops below). The
+  // raw weights of the next step replace those of a column pair from one slot after
+  // the pair's block on (one LDS read per slot), A_0 of the next step is read in front
+  // of slots 1..4, the NDB DMA instructions of the B panel go in the middle of their
+  // share of the slots.
+  static constexpr int R = TM - H, S2 = R * 4 * TN;
+  static constexpr int pair_end(int j0) { return (j0 + 2 < TN ? j0 + 2 : TN) * R * 4; }  // slots before it
+  static constexpr int slot_w(int j, int t) {  // read t (0/1) of column j
+    const int s = pair_end(j & ~1) + 1 + 2 * (j & 1) + t;
+    return s < S2 ? s : S2;
+  }
+  static constexpr int slot_a0(int q) { return 1 + q < S2 ? 1 + q : S2; }
+  static constexpr int slot_dma2(int p) { return (2 * p + 1) * S2 / (2 * NDB); }
 };
 
 struct AFrag {
@@ -505,6 +549,12 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
       f.k[q] = *reinterpret_cast<const v8bf*>(st + rd_a[q] + i * 32 * C::A_ROW);
     return f;
   };
+  auto read_a1 = [&](const uint8_t* __restrict__ st, int i, int q) -> v8bf {
+    return *reinterpret_cast<const v8bf*>(st + rd_a[q] + i * 32 * C::A_ROW);
+  };
+  auto read_w1 = [&](const uint8_t* __restrict__ st, int j, int t) -> uint4 {
+    return *reinterpret_cast<const uint4*>(st + rd_b[t] + j * 32 * C::B_ROW);
+  };
   auto read_w = [&](const uint8_t* __restrict__ st, int j) -> WRaw {
     WRaw f;
 #pragma unroll
@@ -557,9 +607,15 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
       }
       const int kd = kt + D < KT ? kt + D : kt + D - KT;  // step (of its tile) to fetch
       const uint8_t* st = smem + a_cur;
-      auto convert = [&](int j) {
-        convert_w(wr[j].t[0], wf[j].k[0], wf[j].k[1]);
-        convert_w(wr[j].t[1], wf[j].k[2], wf[j].k[3]);
+      // weights of column j, MFMA step q: 8 e4m3 bytes -> one bf16 operand
+      auto convert = [&](int j, int q) {
+        const uint4& w = wr[j].t[q >> 1];
+        const uint32_t lo = (q & 1) ? w.z : w.x, hi = (q & 1) ? w.w : w.y;
+        const v2bf c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
+        const v2bf c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
+        const v2bf c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
+        const v2bf c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
+        wf[j].k[q] = v8bf{c0[0], c0[1], c1[0], c1[1], c2[0], c2[1], c3[0], c3[1]};
       };
       auto mfma = [&](int i, int j, int q) {
         if (FIRST && q == 0) {
@@ -568,32 +624,38 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
           mfma_32x32x16_bf16<false>(acc[i][j], wf[j].k[q], af[i].k[q]);
         }
       };
-      // The weights of this step were read from LDS during the previous step. They are
-      // converted one block ahead of their first use: an MFMA operand written by a
-      // VALU instruction just before the (inline-assembly) MFMA reads stale data.
-      convert(0);
+      // The weights of this step were read from LDS during the previous step. Each
+      // operand is converted CONVERT_AHEAD MFMAs before its first use: an MFMA operand
+      // written by a VALU instruction just before the (inline-assembly) MFMA reads
+      // stale data.
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          if (q * TN + j < C::CONVERT_AHEAD) convert(j, q);
       __builtin_amdgcn_sched_barrier(0);
+      // first half: rows 0..H-1; MFMA step q of all TN blocks of a row before step
+      // q+1, so that consecutive MFMAs never depend on each other (schedule: CfgWW::slot1)
 #pragma unroll
-      for (int i = 0; i < H; ++i) {
-        if (i + 1 < H) af[i + 1] = read_a(st, i + 1);
+      for (int sl = 0; sl < C::S1; ++sl) {
+        const int i = sl / (4 * TN), q = sl / TN % 4, j = sl % TN;
 #pragma unroll
-        for (int k = 0; k < TM - H; ++k)
-          if (k * H / (TM - H) == i) af[H + k] = read_a(st, H + k);
-        // MFMA step q of all TN blocks of the row before step q+1: consecutive MFMAs
-        // never depend on each other
+        for (int qq = 0; qq < 4; ++qq)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+          for (int jj = 0; jj < TN; ++jj)
+            if (qq * TN + jj - C::CONVERT_AHEAD == sl) convert(jj, qq);
 #pragma unroll
-          for (int j = 0; j < TN; ++j) {
-            if (i == 0 && q == 0 && j + 1 < TN) convert(j + 1);
-            // A panel D steps ahead into the stage that step kt-1 read
-#pragma unroll
-            for (int p = 0; p < C::NDA; ++p)
-              if (p * (H * TN * 4) / C::NDA == (i * 4 + q) * TN + j) dma_a(kd, a_prev, p);
-            mfma(i, j, q);
-            __builtin_amdgcn_sched_barrier(0);
+        for (int t = 0; t < C::T1; ++t) {
+          if (C::slot1(t) != sl) continue;
+          if (C::is_read1(t)) {
+            const int r = C::read1_index(t);
+            af[r / 4 + 1].k[r % 4] = read_a1(st, r / 4 + 1, r % 4);
+          } else {
+            dma_a(kd, a_prev, C::dma1_index(t));
           }
         }
+        mfma(i, j, q);
+        __builtin_amdgcn_sched_barrier(0);
       }
       // own LDS reads of this step done, own DMA of the next step landed (the steps
       // after it and the A panel issued above may still fly); then everyone's. In the
@@ -604,28 +666,40 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
       } else {
         wait_and_barrier<(D - 2) * C::ND + C::NDA>();
       }
-      // second half: pairs of columns, so that dependent MFMAs are 2 (TM-H) apart
-#pragma unroll
-      for (int j0 = 0; j0 < TN; j0 += 2) {
-        constexpr int R = TM - H;
+      // second half: rows H..TM-1 in pairs of columns, so that dependent MFMAs are
+      // 2 (TM-H) apart; the next step's raw weights and A_0 are read and the B panel D
+      // steps ahead goes into the B stage of this step (schedule: CfgWW::slot_w ...)
+      auto second_half_items = [&](int sl) {
 #pragma unroll
         for (int q = 0; q < 4; ++q)
+          if (C::slot_a0(q) == sl) af[0].k[q] = read_a1(smem + a_next, 0, q);
 #pragma unroll
-          for (int i = H; i < TM; ++i)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int j = j0; j < j0 + 2 && j < TN; ++j) {
-              // B panel D steps ahead into the B stage of this step
+          for (int t = 0; t < 2; ++t)
+            if (C::slot_w(j, t) == sl) wr[j].t[t] = read_w1(smem + b_next, j, t);
 #pragma unroll
-              for (int p = 0; p < C::NDB; ++p)
-                if (p * (R * TN * 4) / C::NDB ==
-                    j0 * R * 4 + (q * R + (i - H)) * (TN - j0 < 2 ? TN - j0 : 2) + (j - j0))
-                  dma_b(kd, b_cur, p);
-              mfma(i, j, q);
-            }
-        // weights of the next step (after the very last one: zeros, never used)
+        for (int p = 0; p < C::NDB; ++p)
+          if (C::slot_dma2(p) == sl) dma_b(kd, b_cur, p);
+      };
+      {
+        constexpr int R = C::R;
+        int sl = 0;
 #pragma unroll
-        for (int j = j0; j < j0 + 2 && j < TN; ++j) wr[j] = read_w(smem + b_next, j);
-        if (j0 == 0) af[0] = read_a(smem + a_next, 0);
+        for (int j0 = 0; j0 < TN; j0 += 2)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int i = H; i < TM; ++i)
+#pragma unroll
+              for (int j = j0; j < j0 + 2 && j < TN; ++j) {
+                second_half_items(sl);
+                mfma(i, j, q);
+                __builtin_amdgcn_sched_barrier(0);
+                ++sl;
+              }
+        static_assert(R * 4 * TN == C::S2, "slot count");
+        second_half_items(C::S2);
         __builtin_amdgcn_sched_barrier(0);
       }
       a_prev = a_cur;
