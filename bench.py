@@ -371,7 +371,7 @@ def main():
       "frac": head["gemm_tflops"] / FP8_PEAK_TFLOPS,
       # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain
       # copy of known size (profiles/pmc_traffic_headline_kernels.md); algorithmic 165.2 MB
-      "traffic": 425.4e6,
+      "traffic": 415.7e6,
   }
   roofline_quant = {
       "kernel": "quant_rowwise_regs at M=4608 K=3072",
@@ -380,7 +380,7 @@ def main():
       "peak": HBM_PEAK_GBPS,
       "unit": "GB/s",
       "frac": head["quant_gbps"] / HBM_PEAK_GBPS,
-      "traffic": 42.68e6,  # same source; algorithmic 3MK + 4M = 42.49 MB
+      "traffic": 42.66e6,  # same source; algorithmic 3MK + 4M = 42.49 MB
   }
   dit_ms, dit_note = (None, "skipped") if args.skip_dit else dit_forward_ms(device)
   cpu = None if args.skip_cpu else cpu_baseline()
