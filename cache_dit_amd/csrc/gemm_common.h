@@ -97,12 +97,6 @@ __device__ __forceinline__ void wait_vm() {
   __builtin_amdgcn_s_waitcnt((VM & 0xf) | (7 << 4) | (0xf << 8) | ((VM >> 4) << 14));
   asm volatile("" ::: "memory");
 }
-__device__ __forceinline__ void bare_barrier() {
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
-
 // Waits until at most `later` steps (of D DMA instructions each) are in flight,
 // `later` in [0, MAXL]; the count has to be an immediate, hence the switch.
 template <int D, int MAXL, bool BARRIER>

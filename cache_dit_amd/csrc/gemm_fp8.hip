@@ -249,186 +249,6 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_tiled(GemmArgs g, int til
 }
 
 // ---------------------------------------------------------------------------
-// Ping-pong kernel: 8 waves as two groups of 4 (one wave of each group per SIMD).
-// K advances in 64-byte steps through STAGES LDS buffers filled by LDS-DMA
-// STAGES-1 steps ahead. Every wave alternates a memory slot (issue the DMA for
-// step kt+STAGES-1, read its MFMA operands of step kt from LDS) and a compute
-// slot (its MFMAs of step kt); slots are separated by workgroup barriers and
-// group 1 runs one slot behind group 0, so on every SIMD one wave feeds the
-// matrix core while the other one moves data. Barriers are bare s_barrier with
-// explicit s_waitcnt: a fenced barrier would wait for all DMA in flight and
-// drain the pipeline.
-//
-// Panel rows are 64 B = 4 chunks; LDS has 64 banks x 4 B and serves a 16-byte
-// access 16 lanes per pass, so chunk c of row r sits at c ^ ((r>>2)&3)
-// (measured conflict free).
-//
-// The 1 KiB DMA instructions of a step (A panel first, then B) are dealt to the
-// waves round-robin; when their number is not a multiple of 8 the first waves
-// issue one more than the others, and each wave counts its own (D) for s_waitcnt.
-template <int BM_, int BN_, int STAGES_, bool EPI_LDS_, int GROUP_M_, int WGM_ = 2>
-struct CfgPP {
-  static constexpr int BM = BM_, BN = BN_, STAGES = STAGES_, WGM = WGM_, WGN = 8 / WGM_;
-  static constexpr bool EPI_LDS = EPI_LDS_;
-  static constexpr int GROUP_M = GROUP_M_;
-  static constexpr int WAVES = 8, THREADS = 512;
-  static constexpr int WM = BM / WGM, WN = BN / WGN;
-  static constexpr int TM = WM / 32, TN = WN / 32;
-  static constexpr int BKP = 64;
-  static constexpr int A_BYTES = BM * BKP, B_BYTES = BN * BKP;
-  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int NA = A_BYTES / 1024, NB = B_BYTES / 1024, NT = NA + NB;  // DMA per step
-  static constexpr int DMAX = (NT + WAVES - 1) / WAVES;
-  static constexpr int EPI_PITCH = WN * 2 + 16;
-  static constexpr int EPI_BYTES = EPI_LDS ? WAVES * 32 * EPI_PITCH : 0;
-  static constexpr int LDS_BYTES =
-      (STAGES * STAGE_BYTES > EPI_BYTES) ? STAGES * STAGE_BYTES : EPI_BYTES;
-  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
-  static_assert(BM % 16 == 0 && BN % 16 == 0, "panels are filled 16 rows at a time");
-  static_assert(STAGES >= 3 && STAGES <= 8, "prefetch distance 2..7");
-  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
-};
-
-// Main loop for a wave that issues D DMA instructions per step.
-template <class C, int D>
-__device__ __forceinline__ void pingpong_loop(v16f (&acc)[C::TM][C::TN], uint8_t* smem,
-                                              const uint8_t* __restrict__ A,
-                                              const uint8_t* __restrict__ B,
-                                              const uint32_t (&off)[C::DMAX], int KT, int wave,
-                                              int group, const uint32_t (&rd_a)[2],
-                                              const uint32_t (&rd_b)[2]) {
-  constexpr int BKP = C::BKP, PD = C::STAGES - 1;
-  auto fetch = [&](int kt) {
-    uint8_t* st = smem + (kt % C::STAGES) * C::STAGE_BYTES;
-#pragma unroll
-    for (int p = 0; p < D; ++p) {
-      const int id = wave + C::WAVES * p;  // A panel: ids [0, NA); B panel: [NA, NT)
-      const uint8_t* src = (id < C::NA ? A : B) + (int64_t)kt * BKP + off[p];
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(st + id * 1024),
-                                       16, 0, 0);
-    }
-  };
-  // prologue: PD steps in flight; step 0 must have landed before the first slot
-#pragma unroll
-  for (int s = 0; s < PD; ++s)
-    if (s < KT) fetch(s);
-  wait_steps<D, PD - 1, false>(min(PD, KT) - 1);  // step 0 landed; the later ones may fly
-  if (group == 1) bare_barrier();  // group 1 runs one slot behind
-
-  for (int kt = 0; kt < KT; ++kt) {
-    bare_barrier();  // ---- memory slot of this wave
-    if (kt + PD < KT) fetch(kt + PD);
-    const uint8_t* st = smem + (kt % C::STAGES) * C::STAGE_BYTES;
-    v8i af[C::TM], bf[C::TN];
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i) {
-      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_a[0] + i * 32 * BKP);
-      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_a[1] + i * 32 * BKP);
-      af[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-#pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
-      const v4i lo = *reinterpret_cast<const v4i*>(st + rd_b[0] + j * 32 * BKP);
-      const v4i hi = *reinterpret_cast<const v4i*>(st + rd_b[1] + j * 32 * BKP);
-      bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-    // step kt+1 of this wave has landed once only the later steps are in flight
-    const int later = min(kt + PD, KT - 1) - (kt + 1);  // steps issued after kt+1
-    wait_steps<D, PD - 1, true>(max(later, 0));
-    // ---- compute slot
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-      for (int j = 0; j < C::TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[i][j], 0, 0,
-                                                                    0, 0, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  if (group == 0) bare_barrier();
-}
-
-// Two waves per SIMD: at most 256 VGPRs.
-template <class C>
-__global__ __launch_bounds__(C::THREADS, 2) void gemm_fp8_pingpong(GemmArgs g, int tiles_m,
-                                                                   int tiles_n) {
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave / C::WGN, wn = wave % C::WGN;
-  const int group = wave >> 2;  // ping-pong group: waves 0-3 and 4-7, one of each per SIMD
-  constexpr int BKP = C::BKP;
-
-  int tm, tn;
-  tile_of_block<C::GROUP_M>(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
-  const int m0 = tm * C::BM, n0 = tn * C::BN;
-  const uint8_t* __restrict__ A = static_cast<const uint8_t*>(g.a) + (int64_t)m0 * g.lda;
-  const uint8_t* __restrict__ B = g.b + (int64_t)n0 * g.ldb;
-  const int rows_a = g.M - m0, rows_b = g.N - n0;
-
-  // DMA map: instruction id fills 16 panel rows (1 KiB); lane l lands on row l/4,
-  // position l%4 and fetches the logical chunk the swizzle puts there.
-  uint32_t off[C::DMAX];
-  const int drow = lane >> 2;
-#pragma unroll
-  for (int p = 0; p < C::DMAX; ++p) {
-    const int id = wave + C::WAVES * p;
-    const bool is_a = id < C::NA;
-    const int row = (is_a ? id : id - C::NA) * 16 + drow;
-    const int c = (lane & 3) ^ ((row >> 2) & 3);
-    off[p] = is_a ? (uint32_t)min(row, rows_a - 1) * (uint32_t)g.lda + c * 16
-                  : (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
-  }
-  // operand read map: row lane&31, K-half h: chunks 2h, 2h+1
-  const int h = lane >> 5;
-  uint32_t rd_a[2], rd_b[2];
-#pragma unroll
-  for (int e = 0; e < 2; ++e) {
-    const int pos = ((2 * h + e) ^ ((lane >> 2) & 3)) << 4;
-    rd_a[e] = (wm * C::WM + (lane & 31)) * BKP + pos;
-    rd_b[e] = C::A_BYTES + (wn * C::WN + (lane & 31)) * BKP + pos;
-  }
-
-  v16f acc[C::TM][C::TN];
-#pragma unroll
-  for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-    for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-  const int KT = g.K / BKP;
-  if constexpr (C::NT % C::WAVES == 0) {
-    pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, group, rd_a, rd_b);
-  } else {
-    if (wave < C::NT % C::WAVES) {
-      pingpong_loop<C, C::DMAX>(acc, smem, A, B, off, KT, wave, group, rd_a, rd_b);
-    } else {
-      pingpong_loop<C, C::DMAX - 1>(acc, smem, A, B, off, KT, wave, group, rd_a, rd_b);
-    }
-  }
-
-  // All LDS operand reads and all DMA are complete here (the last slot barrier
-  // follows group 1's last reads), so the stage buffers can hold the epilogue tiles.
-  uint8_t* et = smem + wave * (32 * C::EPI_PITCH);
-  tile_epilogue<C>(acc, g, et, m0, n0, wm, wn, lane);
-}
-
-template <class C>
-int launch_pingpong(const GemmArgs& g, hipStream_t stream) {
-  static bool lds_allowed[64];
-  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_fp8_pingpong<C>), C::LDS_BYTES,
-                                 lds_allowed))
-    return rc;
-  const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
-  hipLaunchKernelGGL(gemm_fp8_pingpong<C>, dim3(tiles_m * tiles_n), dim3(C::THREADS),
-                     C::LDS_BYTES, stream, g, tiles_m, tiles_n);
-  return 0;
-}
-
-// ---------------------------------------------------------------------------
 // Wide kernel: 256x256 tile, 4 waves (one per SIMD, up to 512 registers each), each
 // owning a 128x128 wave tile as 8x8 blocks of v_mfma_f32_16x16x128_f8f6f4 (8 passes;
 // one wave alone keeps the matrix core busy with it, which the 16-pass 32x32x64
@@ -993,10 +813,6 @@ typedef Cfg<128, 128, 2, 2, true, true, 8> V6;        // two workgroups per CU
 typedef Cfg<256, 256, 2, 4, true, true, 8> V7;        // 8 waves in phase, 2 stages
 typedef Cfg<128, 64, 2, 2, true, true, 8, 4> V20;     // small tiles, 4 stages of 128 B
 typedef Cfg<64, 128, 2, 2, true, true, 8, 4> V21;
-typedef CfgPP<256, 256, 4, true, 8> V8;               // ping-pong, 4 stages of 64 B
-typedef CfgPP<256, 256, 4, false, 8> V9;              // ... with direct 8-byte stores
-typedef CfgPP<192, 384, 4, true, 8> V10;              // ping-pong, 96x96 wave tiles
-typedef CfgPP<256, 192, 4, true, 8, 4> V11;           // ping-pong, 64x96 wave tiles (4x2 waves)
 typedef CfgWide<256, 256, 8> V12;                     // 4 waves, 128x128 wave tiles, 16x16x128 MFMA
 typedef CfgWide<288, 192, 8> V14;                     // ... 144x96 wave tiles
 typedef CfgWide<256, 192, 8> V15;                     // ... 128x96 wave tiles
@@ -1094,10 +910,6 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     case 7: return launch_tiled<V7>(g, stream);
     case 20: return launch_tiled<V20>(g, stream);
     case 21: return launch_tiled<V21>(g, stream);
-    case 8: return launch_pingpong<V8>(g, stream);
-    case 9: return launch_pingpong<V9>(g, stream);
-    case 10: return launch_pingpong<V10>(g, stream);
-    case 11: return launch_pingpong<V11>(g, stream);
     case 12: return wide_ok(V12::DEPTH) ? launch_wide<V12>(g, stream) : launch_tiled<V6>(g, stream);
     case 14: return wide_ok(V14::DEPTH) ? launch_wide<V14>(g, stream) : launch_tiled<V6>(g, stream);
     case 15: return wide_ok(V15::DEPTH) ? launch_wide<V15>(g, stream) : launch_tiled<V6>(g, stream);

@@ -177,170 +177,6 @@ __global__ __launch_bounds__(C::THREADS) void gemm_w8a16_tiled(GemmArgs g, int t
 }
 
 // ---------------------------------------------------------------------------
-// Ping-pong flavour (same schedule as the w8a8 ping-pong kernel): 8 waves in two
-// groups of 4, K in 64-element steps through STAGES LDS buffers filled by LDS-DMA
-// STAGES-1 steps ahead; a wave alternates a memory slot (DMA issue + operand
-// reads) and a compute slot (e4m3 -> bf16 conversion + MFMAs), group 1 one slot
-// behind group 0, bare barriers with explicit s_waitcnt between slots.
-template <int BM_, int BN_, int STAGES_, int GROUP_M_>
-struct CfgWP {
-  static constexpr int BM = BM_, BN = BN_, STAGES = STAGES_, WGM = 2, WGN = 4;
-  static constexpr bool EPI_LDS = true;
-  static constexpr int GROUP_M = GROUP_M_;
-  static constexpr int WAVES = 8, THREADS = 512;
-  static constexpr int WM = BM / WGM, WN = BN / WGN;
-  static constexpr int TM = WM / 32, TN = WN / 32;
-  static constexpr int A_ROW = BKE * 2, B_ROW = BKE;
-  static constexpr int A_BYTES = BM * A_ROW, B_BYTES = BN * B_ROW;
-  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int NA = A_BYTES / 1024, NB = B_BYTES / 1024, NT = NA + NB;
-  static constexpr int D = NT / WAVES;  // DMA instructions per wave and step
-  static constexpr int EPI_PITCH = WN * 2 + 16;
-  static constexpr int EPI_BYTES = WAVES * 32 * EPI_PITCH;
-  static constexpr int LDS_BYTES =
-      (STAGES * STAGE_BYTES > EPI_BYTES) ? STAGES * STAGE_BYTES : EPI_BYTES;
-  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
-  static_assert(NT % WAVES == 0, "DMA instructions must split evenly over the waves");
-  static_assert(STAGES >= 3 && STAGES <= 8, "prefetch distance 2..7");
-  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
-};
-
-template <class C>
-__global__ __launch_bounds__(C::THREADS, 2) void gemm_w8a16_pingpong(GemmArgs g, int tiles_m,
-                                                                     int tiles_n) {
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave / C::WGN, wn = wave % C::WGN;  // wm is also the ping-pong group
-  constexpr int PD = C::STAGES - 1, D = C::D;
-
-  int tm, tn;
-  tile_of_block<C::GROUP_M>(blockIdx.x, gridDim.x, tiles_m, tiles_n, &tm, &tn);
-  const int m0 = tm * C::BM, n0 = tn * C::BN;
-  const uint8_t* __restrict__ A = static_cast<const uint8_t*>(g.a) + (int64_t)m0 * g.lda * 2;
-  const uint8_t* __restrict__ B = g.b + (int64_t)n0 * g.ldb;
-  const int rows_a = g.M - m0, rows_b = g.N - n0;
-
-  // DMA map: ids [0, NA) fill 8 A rows each (128-byte rows), ids [NA, NT) 16 B rows.
-  uint32_t off[D];
-#pragma unroll
-  for (int p = 0; p < D; ++p) {
-    const int id = wave + C::WAVES * p;
-    if (id < C::NA) {
-      const int row = id * 8 + (lane >> 3);
-      const int c = (lane & 7) ^ ((row >> 1) & 7);
-      off[p] = (uint32_t)min(row, rows_a - 1) * (uint32_t)(g.lda * 2) + c * 16;
-    } else {
-      const int row = (id - C::NA) * 16 + (lane >> 2);
-      const int c = (lane & 3) ^ ((row >> 2) & 3);
-      off[p] = (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
-    }
-  }
-  const int h = lane >> 5;
-  uint32_t rd_a[2][2], rd_b[2];
-#pragma unroll
-  for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-    for (int e = 0; e < 2; ++e)
-      rd_a[kb][e] = (wm * C::WM + (lane & 31)) * C::A_ROW +
-                    (((4 * kb + 2 * h + e) ^ ((lane >> 1) & 7)) << 4);
-    rd_b[kb] = C::A_BYTES + (wn * C::WN + (lane & 31)) * C::B_ROW +
-               (((2 * kb + h) ^ ((lane >> 2) & 3)) << 4);
-  }
-
-  v16f acc[C::TM][C::TN];
-#pragma unroll
-  for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-    for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-  const int KT = g.K / BKE;
-  auto fetch = [&](int kt) {
-    uint8_t* st = smem + (kt % C::STAGES) * C::STAGE_BYTES;
-#pragma unroll
-    for (int p = 0; p < D; ++p) {
-      const int id = wave + C::WAVES * p;
-      const uint8_t* src =
-          (id < C::NA ? A + (int64_t)kt * C::A_ROW : B + (int64_t)kt * C::B_ROW) + off[p];
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(st + id * 1024),
-                                       16, 0, 0);
-    }
-  };
-#pragma unroll
-  for (int s = 0; s < PD; ++s)
-    if (s < KT) fetch(s);
-  wait_steps<D, PD - 1, false>(min(PD, KT) - 1);
-  if (wm == 1) bare_barrier();  // group 1 runs one slot behind
-
-  for (int kt = 0; kt < KT; ++kt) {
-    bare_barrier();  // ---- memory slot of this wave
-    if (kt + PD < KT) fetch(kt + PD);
-    const uint8_t* st = smem + (kt % C::STAGES) * C::STAGE_BYTES;
-    v8bf fa[C::TM][2][2];  // [i][kb][MFMA step of the block]
-    uint4 fw[C::TN][2];    // [j][kb]: 16 e4m3 bytes = two MFMA steps
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int e = 0; e < 2; ++e)
-          fa[i][kb][e] = *reinterpret_cast<const v8bf*>(st + rd_a[kb][e] + i * 32 * C::A_ROW);
-#pragma unroll
-    for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-        fw[j][kb] = *reinterpret_cast<const uint4*>(st + rd_b[kb] + j * 32 * C::B_ROW);
-    wait_steps<D, PD - 1, true>(max(min(kt + PD, KT - 1) - (kt + 1), 0));
-    // ---- compute slot
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int j = 0; j < C::TN; ++j) {
-        const uint4 w = fw[j][kb];
-        const v2bf c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.x, 1.0f, false);
-        const v2bf c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.x, 1.0f, true);
-        const v2bf c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.y, 1.0f, false);
-        const v2bf c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.y, 1.0f, true);
-        const v2bf c4 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.z, 1.0f, false);
-        const v2bf c5 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.z, 1.0f, true);
-        const v2bf c6 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.w, 1.0f, false);
-        const v2bf c7 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.w, 1.0f, true);
-        const v8bf b_lo = {c0[0], c0[1], c1[0], c1[1], c2[0], c2[1], c3[0], c3[1]};
-        const v8bf b_hi = {c4[0], c4[1], c5[0], c5[1], c6[0], c6[1], c7[0], c7[1]};
-#pragma unroll
-        for (int i = 0; i < C::TM; ++i) {
-          acc[i][j] =
-              __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_lo, fa[i][kb][0], acc[i][j], 0, 0, 0);
-          acc[i][j] =
-              __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_hi, fa[i][kb][1], acc[i][j], 0, 0, 0);
-        }
-      }
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  if (wm == 0) bare_barrier();
-
-  // all operand reads and all DMA are complete: the stage buffers hold the epilogue tiles
-  tile_epilogue<C>(acc, g, smem + wave * (32 * C::EPI_PITCH), m0, n0, wm, wn, lane);
-}
-
-template <class C>
-int launch_pingpong(const GemmArgs& g, hipStream_t stream) {
-  static bool lds_allowed[64];
-  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_w8a16_pingpong<C>), C::LDS_BYTES,
-                                 lds_allowed))
-    return rc;
-  const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
-  hipLaunchKernelGGL(gemm_w8a16_pingpong<C>, dim3(tiles_m * tiles_n), dim3(C::THREADS),
-                     C::LDS_BYTES, stream, g, tiles_m, tiles_n);
-  return 0;
-}
-
-// ---------------------------------------------------------------------------
 // Wide kernel: the schedule of the wide w8a8 kernel (one persistent workgroup of 4
 // waves per CU, one wave per SIMD with all 256 AGPRs as accumulators, LDS-DMA by
 // buffer loads spread over the MFMA stream, A panel in 3 LDS stages and B panel in
@@ -348,7 +184,7 @@ int launch_pingpong(const GemmArgs& g, hipStream_t stream) {
 // v_mfma_f32_32x32x16_bf16 (8 passes), K steps of 64 elements, wave tile
 // (BM/2) x (BN/2) as TM x TN blocks of 32x32, four MFMAs per block and step.
 //
-// Panels as in the ping-pong kernel above: A rows 128 B (bf16), chunk c of row r at
+// Panels: A rows 128 B (bf16), chunk c of row r at
 // c ^ ((r>>1)&7); B rows 64 B (e4m3), chunk c at c ^ ((r>>2)&3). A lane reads, per
 // 32-row block, the four A chunks 4t+2h+s (h = lane>>5) and the two B chunks 2t+h:
 // the 16 B bytes of one chunk are the weights of MFMA steps 2t and 2t+1 (K order
@@ -938,9 +774,6 @@ bool tiled_ok(const GemmArgs& g) {
 
 typedef CfgW<256, 256, 2, 2, true, 8> W0;   // 4 waves, 2 stages
 typedef CfgW<128, 128, 2, 2, true, 8> W3;   // small tiles, two workgroups per CU
-typedef CfgWP<256, 256, 3, 8> W4;           // ping-pong, 3 stages of 64 elements
-typedef CfgWP<192, 384, 3, 8> W5;           // ping-pong, 96x96 wave tiles
-typedef CfgWP<128, 256, 4, 8> W6;
 typedef CfgWW<256, 256, 8> W7;              // wide: 4 waves, 128x128 wave tiles
 typedef CfgWW<256, 192, 8> W8;              // wide: 128x96 wave tiles
 typedef CfgWW<192, 256, 8> W9;              // wide: 96x128 wave tiles
@@ -980,16 +813,12 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
       // Smaller problems: whole rounds over the CUs times tile area, the small tiles
       // penalised by their measured lower MFMA rate (per mille); ties go to the larger
       // tile. Tiles whose prefetch depth K cannot feed are left out; without any wide
-      // tile (N not a multiple of 16, very short K) the older kernels run.
+      // tile (N not a multiple of 16, very short K) the 128x128 kernel runs.
       const struct { int v, bm, bn, pen, depth; } cand[] = {
           {7, 256, 256, 1000, 2}, {8, 256, 192, 1000, 2}, {10, 128, 192, 1300, 4},
           {11, 128, 128, 1400, 5}, {12, 128, 64, 1700, 6}};
       int64_t best = INT64_MAX;
-      if (tiles(256, 256) >= 200) {
-        variant = ((tiles(192, 384) + 255) / 256) * 192 * 384 < ((tiles(256, 256) + 255) / 256) * 256 * 256 ? 5 : 4;
-      } else {
-        variant = 3;
-      }
+      variant = 3;  // the 128x128 kernel takes what no wide tile can
       for (const auto& c : cand) {
         if (!wide_ok(c.depth)) continue;
         const int64_t t = (tiles(c.bm, c.bn) + 255) / 256 * c.bm * c.bn * c.pen;
@@ -1003,9 +832,6 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
   switch (variant) {
     case 0: return launch_tiled<W0>(g, stream);
     case 3: return launch_tiled<W3>(g, stream);
-    case 4: return launch_pingpong<W4>(g, stream);
-    case 5: return launch_pingpong<W5>(g, stream);
-    case 6: return launch_pingpong<W6>(g, stream);
     case 7: return wide_ok(W7::DEPTH) ? launch_wide<W7>(g, stream) : launch_tiled<W3>(g, stream);
     case 8: return wide_ok(W8::DEPTH) ? launch_wide<W8>(g, stream) : launch_tiled<W3>(g, stream);
     case 9: return wide_ok(W9::DEPTH) ? launch_wide<W9>(g, stream) : launch_tiled<W3>(g, stream);

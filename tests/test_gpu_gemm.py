@@ -49,7 +49,7 @@ def _assert_close(out, ref):
   assert elementwise_ok(out, ref, REL_TOL)
 
 
-TILED_VARIANTS = [0, 1, 6, 7, 8, 9, 10, 11, 12, 14, 15, 16, 17, 18, 20, 21]
+TILED_VARIANTS = [0, 1, 6, 7, 12, 14, 15, 16, 17, 18, 20, 21]
 
 
 @pytest.mark.parametrize("variant", TILED_VARIANTS + [100])
@@ -208,7 +208,7 @@ def test_against_c_oracle(M, N, K):
   _assert_close(_run(xq, xs, wq, ws, b), ref)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 8, 10, 12, 21, 100])
+@pytest.mark.parametrize("variant", [0, 1, 12, 14, 17, 21, 100])
 def test_gelu_tanh_epilogue(variant):
   from cache_dit_amd import _native
   p = _rand_problem(384, 512, 1024, seed=9)

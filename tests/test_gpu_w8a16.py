@@ -44,7 +44,7 @@ def _assert_close(out, ref):
   assert elementwise_ok(out, ref, REL_TOL)
 
 
-@pytest.mark.parametrize("variant", [0, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 100])
+@pytest.mark.parametrize("variant", [0, 3, 7, 8, 9, 10, 11, 12, 100])
 @pytest.mark.parametrize("M,N,K", [(512, 768, 1024), (300, 520, 192), (1, 264, 64), (257, 8, 384)])
 def test_variants_with_tails(variant, M, N, K):
   from cache_dit_amd import _native
@@ -55,7 +55,7 @@ def test_variants_with_tails(variant, M, N, K):
   _assert_close(out, to.w8a16_linear(*p, fused=False))  # the reference's dequantize-first form
 
 
-@pytest.mark.parametrize("variant", [0, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 100])
+@pytest.mark.parametrize("variant", [0, 3, 7, 8, 9, 10, 11, 12, 100])
 def test_exact_small_integers(variant):
   from cache_dit_amd import _native
   g = torch.Generator().manual_seed(12)
