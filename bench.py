@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A "step" is one pass of the hot path over one batch: every quantized nn.Linear
-of one denoising step of the FLUX.1-dev-shaped MMDiT (BASELINE config 2: 19
+of one denoising step of the FLUX.1-dev-shaped MMDiT (benchmark config 2: 19
 double-stream + 38 single-stream blocks, 4096 image + 512 text tokens, hidden
 3072, MLP 12288 with GELU-tanh) run back to back at its real shape with its own
 weights -- per Linear: per-token e4m3 activation quantization, FP8 GEMM, fused
@@ -216,7 +216,7 @@ def headline_kernels(device):
 
 def cpu_baseline():
   """The CPU restatement of the reference path (oracle.torch_oracle: eager PyTorch
-  CPU ops) on BASELINE config 1 (M=4608, K=3072, N=3072): activation quantization +
+  CPU ops) on benchmark config 1 (M=4608, K=3072, N=3072): activation quantization +
   scaled matmul + bias, weights pre-quantized. 1 warm-up + 3 timed runs, median."""
   import torch
   from oracle import torch_oracle as to
@@ -246,7 +246,7 @@ def cpu_baseline():
       "unit": "TFLOP/s",
       "cores": torch.get_num_threads(),
       "kind": "port",
-      "sample": f"BASELINE config 1 linear (M={M} K={K} N={N}): per-token quant + scaled matmul "
+      "sample": f"benchmark config 1 linear (M={M} K={K} N={N}): per-token quant + scaled matmul "
                 f"+ bias in eager PyTorch CPU ops, median of 3 runs, {t*1e3:.0f} ms/linear",
       "quant_gbps": (3.0 * M * K + 4.0 * M) / tq / 1e9,
       "ms_per_linear": t * 1e3,

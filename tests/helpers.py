@@ -8,7 +8,7 @@ FP8 = torch.float8_e4m3fn
 
 
 def config1_inputs(M=4608, K=3072, N=3072, seed=0):
-  """BASELINE config 1: x ~N(0,1) with 0.1% of channels x20, W ~N(0,0.02),
+  """benchmark config 1: x ~N(0,1) with 0.1% of channels x20, W ~N(0,0.02),
   bias ~N(0,0.01), all drawn in fp32 on the CPU generator and cast to bf16."""
   g = torch.Generator().manual_seed(seed)
   x = torch.randn(1, M, K, generator=g)

@@ -9,7 +9,7 @@ from oracle import torch_oracle as to
 
 pytestmark = pytest.mark.gpu
 FP8 = torch.float8_e4m3fn
-REL_TOL = 1e-2  # BASELINE north star: max relative error 1e-2, bf16 out, fp32 accumulate
+REL_TOL = 1e-2  # target: max relative error 1e-2, bf16 out, fp32 accumulate
 
 
 @pytest.fixture(autouse=True)
@@ -146,7 +146,7 @@ def test_reference_partition_shape_m512_k3072_n3072():
 @pytest.mark.parametrize("M,N,K", [(6889, 3072, 3072), (6889, 12288, 3072), (32760, 5120, 5120),
                                    (32760, 13824, 5120), (4608, 3072, 15360)])
 def test_qwen_and_wan_shapes_sampled_rows(M, N, K):
-  """Odd token counts of the other BASELINE models (Qwen-Image 6889 = 83 x 83, Wan
+  """Odd token counts of the other benchmark models (Qwen-Image 6889 = 83 x 83, Wan
   32760 = 8 x 4095) at full size: every 97th row plus the last rows against the oracle."""
   from cache_dit_amd import ops
   g = torch.Generator(device="cuda").manual_seed(M + N)

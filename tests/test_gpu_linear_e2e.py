@@ -248,7 +248,7 @@ def test_linear_forward_under_hip_graph_capture():
 
 
 def test_full_flux_shaped_step_cosine():
-  """BASELINE config 2 at full size (19 + 38 blocks, 4096 + 512 tokens): the HIP
+  """benchmark config 2 at full size (19 + 38 blocks, 4096 + 512 tokens): the HIP
   path against the oracle's arithmetic in torch ops on the same GPU, and against
   the unquantized bf16 model."""
   import cache_dit_amd as cache_dit

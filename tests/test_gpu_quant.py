@@ -133,7 +133,7 @@ def test_c_abi_error_paths():
 
 
 def test_full_size_properties_wan_shape():
-  """At the largest BASELINE activation (Wan: 32760 x 5120) the oracle is too slow
+  """At the largest benchmark activation (Wan: 32760 x 5120) the oracle is too slow
   for every row, so: a random sample of rows is checked bit-exactly against the
   oracle, and the whole tensor through size-independent properties -- every row
   reaches code 0x7E or one below, no NaN code, exact equivariance under scaling by

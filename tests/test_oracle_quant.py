@@ -1,6 +1,6 @@
 """Pins the quantizer oracle: the plain-C restatement against the PyTorch-op
 restatement, both against closed forms, invariants, the committed golden vectors
-and the known answers of the BASELINE config-1 recipe."""
+and the known answers of the benchmark config-1 recipe."""
 import json
 import os
 
@@ -86,7 +86,7 @@ def test_invariants(mode):
 
 
 def test_config1_known_answers():
-  """Numbers of the BASELINE config-1 recipe (global seed 0): which channels are
+  """Numbers of the benchmark config-1 recipe (global seed 0): which channels are
   outliers, the amax range, how the two scale modes differ, and how many codes a
   reciprocal multiply would flip. A missing bf16 rounding of the scale, an fp32
   instead of bf16 amax or a reciprocal in place of the division changes them."""
