@@ -4,9 +4,10 @@ cache-dit's `quantize()` / `enable_cache(..., quantize_config=...)` API.
     import cache_dit_amd as cache_dit
     cache_dit.quantize(transformer, cache_dit.QuantizeConfig(quant_type="float8_per_row"))
 
-Built quant types: `float8_per_row` (w8a8, dynamic per-token activation scales)
-and `float8_weight_only` (w8a16). The kernels live in lib/libcdit_hip.so (C ABI:
-include/cdit_hip.h); there is no CPU or eager fallback.
+Built quant types: `float8_per_row` (w8a8, dynamic per-token activation scales),
+`float8_per_tensor` (w8a8, one dynamic scale per tensor; also the policy's fallback
+pass) and `float8_weight_only` (w8a16). The kernels live in lib/libcdit_hip.so
+(C ABI: include/cdit_hip.h); there is no CPU or eager fallback.
 """
 from .quantization import QuantizeBackend
 from .quantization import QuantizeConfig
@@ -16,6 +17,7 @@ from .quantization import remove_quantization_stats
 from .caching import enable_cache
 from .caching import load_quantize_config
 from .nn import Fp8DynamicLinear
+from .nn import Fp8DynamicLinearPerTensor
 from .nn import Fp8WeightOnlyLinear
 from .nn import fuse_gelu_tanh_
 from .nn import share_activation_quant_
@@ -33,6 +35,7 @@ __all__ = [
     "load_quantize_config",
     "check_quantized",
     "Fp8DynamicLinear",
+    "Fp8DynamicLinearPerTensor",
     "Fp8WeightOnlyLinear",
     "fuse_gelu_tanh_",
     "share_activation_quant_",
