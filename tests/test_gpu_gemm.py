@@ -334,3 +334,34 @@ def test_output_dtypes_second_witness():
     except Exception as e:  # pragma: no cover - depends on the box's hipBLASLt
       pytest.skip(f"torch._scaled_mm row-wise {dt} not available here: {e}")
     assert max_rel_err(out, ref) <= REL_TOL
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
+def test_fused_linear_entry_point_with_other_output_dtypes(out_dtype):
+  """cdit_fp8_linear_w8a8 (quantizer + GEMM in one call) passes out_dtype_id through:
+  same result as the two entry points called one after the other."""
+  from cache_dit_amd import _native, ops
+  M, N, K = 640, 384, 768
+  g = torch.Generator(device="cuda").manual_seed(31)
+  x = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
+  w = (torch.randn(N, K, generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+  wq, w_s = ops.fp8_rowwise_quant(w)
+  w_s = w_s.reshape(-1).contiguous()
+  bias = None if out_dtype == torch.float32 else (torch.randn(N, generator=g, device="cuda") * 0.1).to(out_dtype)
+  q_ws = torch.empty(M, K, dtype=FP8, device="cuda")
+  s_ws = torch.empty(M, dtype=torch.float32, device="cuda")
+  out = torch.empty(M, N, dtype=out_dtype, device="cuda")
+  L = _native.load()
+  rc = L.cdit_fp8_linear_w8a8(x.data_ptr(), wq.data_ptr(), w_s.data_ptr(),
+                              None if bias is None else bias.data_ptr(), out.data_ptr(),
+                              q_ws.data_ptr(), s_ws.data_ptr(), M, N, K, K, K, N, 0, 0,
+                              ops.encode_output_dtype(out_dtype), None)
+  assert rc == 0, L.cdit_last_error()
+  torch.cuda.synchronize()
+  aq, a_s = ops.fp8_rowwise_quant(x)
+  assert torch.equal(q_ws.view(torch.uint8), aq.view(torch.uint8))
+  ref = ops.float8_inference_scaled_mm(aq, a_s, wq.t(), w_s.reshape(1, -1), out_dtype, bias=bias)
+  assert torch.equal(out, ref)
+  cpu = to.scaled_mm_rowwise(aq.cpu(), a_s.cpu(), wq.cpu(), w_s.cpu(),
+                             None if bias is None else bias.cpu(), out_dtype=out_dtype)
+  assert max_rel_err(out, cpu) <= REL_TOL
