@@ -86,6 +86,30 @@ def test_zero_rows_signed_zero_and_extremes(mode):
 
 
 @pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("K", [512, 4096 + 8])
+def test_non_finite_rows_stay_in_their_row(mode, K):
+  """Rows with Inf or NaN are outside the bit-exact contract; what is checked is that they
+  neither hang the kernel nor leak into their neighbours: every other row is bit-exact, an
+  Inf row gets an infinite scale (amax/448) and a NaN row a NaN scale, as in the reference
+  arithmetic (torch.amax propagates NaN)."""
+  g = torch.Generator().manual_seed(5 + K)
+  x = torch.randn(12, K, generator=g).to(torch.bfloat16)
+  x[3, 7] = float("inf")
+  x[5, K - 1] = float("-inf")
+  x[8, 100] = float("nan")
+  from cache_dit_amd import ops
+  q, s = ops.fp8_rowwise_quant(x.cuda(), mode)
+  torch.cuda.synchronize()
+  q_ref, s_ref = to.quantize_rowwise(x, mode)
+  good = torch.tensor([r not in (3, 5, 8) for r in range(12)])
+  assert (bits_u8(q)[good] == bits_u8(q_ref)[good]).all()
+  assert (bits_u32(s).reshape(-1)[good] == bits_u32(s_ref).reshape(-1)[good]).all()
+  s = s.reshape(-1).cpu()
+  assert torch.isinf(s[3]) and torch.isinf(s[5]) and torch.isnan(s[8])
+  assert torch.isinf(s_ref.reshape(-1)[3]) and torch.isnan(s_ref.reshape(-1)[8])
+
+
+@pytest.mark.parametrize("mode", MODES)
 def test_strided_rows_and_leading_dims(mode):
   g = torch.Generator().manual_seed(4)
   base = torch.randn(6, 20, 640, generator=g).to(torch.bfloat16)
