@@ -365,3 +365,28 @@ def test_fused_linear_entry_point_with_other_output_dtypes(out_dtype):
   cpu = to.scaled_mm_rowwise(aq.cpu(), a_s.cpu(), wq.cpu(), w_s.cpu(),
                              None if bias is None else bias.cpu(), out_dtype=out_dtype)
   assert max_rel_err(out, cpu) <= REL_TOL
+
+
+def test_wide_variants_agree_bit_for_bit_on_random_data():
+  """All tiles of the wide kernel accumulate K in the same order with the same MFMA, so on the
+  same (random, non-integer) operands they must give identical outputs, edge tiles included."""
+  from cache_dit_amd import _native, ops
+  g = torch.Generator(device="cuda").manual_seed(77)
+  for (M, N, K) in [(1000, 1160, 1024), (2345, 520, 768), (333, 2056, 2048)]:
+    bits = torch.randint(0, 256, (M, K), dtype=torch.uint8, device="cuda", generator=g)
+    a = (bits & 0xBF).view(FP8)
+    bits = torch.randint(0, 256, (N, K), dtype=torch.uint8, device="cuda", generator=g)
+    w = (bits & 0xBF).view(FP8)
+    sa = torch.rand(M, device="cuda", generator=g) + 0.5
+    sw = torch.rand(N, device="cuda", generator=g) * 1e-3
+    b = torch.randn(N, device="cuda", generator=g).to(torch.bfloat16)
+    outs = []
+    for variant in (12, 14, 15, 16, 17, 18):
+      _native.set_gemm_variant(variant)
+      for epi in (0, 1):
+        out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+        ops.gemm_rowwise_into(a, sa, w, sw, b, out, epi)
+        outs.append((variant, epi, out))
+    torch.cuda.synchronize()
+    for variant, epi, out in outs[2:]:
+      assert torch.equal(out, outs[epi][2]), (M, N, K, variant, epi)
