@@ -249,27 +249,30 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_tiled(GemmArgs g, int til
 }
 
 // ---------------------------------------------------------------------------
-// Wide kernel: 256x256 tile, 4 waves (one per SIMD, up to 512 registers each), each
-// owning a 128x128 wave tile as 8x8 blocks of v_mfma_f32_16x16x128_f8f6f4 (8 passes;
-// one wave alone keeps the matrix core busy with it, which the 16-pass 32x32x64
-// does not). K advances in 128-byte steps through two LDS stages filled by LDS-DMA.
-// A wave holds all 16 operand fragments of a step in registers (A_i: rows 16i..16i+15
+// Wide kernel: a BM x BN tile (256x256 and relatives) per workgroup of 4 waves, one
+// wave per SIMD with up to 512 registers, each owning a (BM/2) x (BN/2) wave tile as
+// TM x TN blocks of v_mfma_f32_16x16x128_f8f6f4 (8 passes; one wave alone keeps the
+// matrix core busy with it, which the 16-pass 32x32x64 does not). K advances in
+// 128-byte steps through LDS stages filled by LDS-DMA, D = DEPTH steps ahead. A wave
+// holds all TM + TN operand fragments of a step in registers (A_i: rows 16i..16i+15
 // of its half of the A panel, B_j likewise), so every panel byte is read from LDS
-// once per wave: 32 KiB per wave and step for 64 MFMAs.
+// once per wave: 32 KiB per wave and step for 64 MFMAs with the 128x128 wave tile.
 //
-// The A panel has three LDS stages and the B panel two. Step kt:
+// The A panel has D+1 LDS stages and the B panel D. Step kt:
 //   rows 0..H-1, i-major:  MFMA(i, 0..TN-1); meanwhile read the remaining A
 //                          fragments of step kt, and issue the A-panel DMA of step
-//                          kt+2 (into the stage that step kt-1 read)
-//   wait (own LDS reads; own DMA of step kt+1, not the A panel just issued),
+//                          kt+D (into the stage that step kt-1 read)
+//   wait (own LDS reads; own DMA of step kt+1, not the younger ones),
 //   workgroup barrier: the B stage of step kt is now free, step kt+1 is in LDS
 //   rows H..TM-1, j-major: MFMA(H..TM-1, j), then B_j is dead: read B_j of step
 //                          kt+1; A_0 of step kt+1 likewise; the B-panel DMA of step
-//                          kt+2 is issued in between
-// One barrier per step, in the middle of the MFMA stream. Spreading the DMA over
-// both halves matters: a CU's vector memory path moves 64 B per clock, a step
-// needs (BM + BN) * 128 B through it against TM * TN * 32 clocks of MFMA per wave,
-// and a wave that cannot issue its DMA cannot issue its MFMAs either.
+//                          kt+D is issued in between
+// One barrier per step, in the middle of the MFMA stream. Which read or DMA
+// instruction goes in front of which MFMA is fixed at compile time (CfgWide::slot1
+// and relatives): a CU's vector memory path moves 64 B per clock (16 clocks per
+// DMA instruction), a step needs (BM + BN) * 128 B through it against TM * TN * 32
+// clocks of MFMA per wave, and a wave that is held at a DMA instruction or a pair
+// of LDS reads for longer than the MFMA in flight lasts leaves the matrix core idle.
 //
 // Panel rows are 128 B = 8 chunks of 16 B. An operand read takes row (lane & 15),
 // chunks 2*(lane >> 4) + {0, 1}; the LDS serves 16 lanes per pass (lane bit 5 and
