@@ -388,8 +388,8 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
   const int ntiles = tiles_m * tiles_n;
 
   // The workgroup is persistent: it takes tiles blockIdx.x, blockIdx.x + gridDim.x,
-  // ... and runs their K loops as one stream: the DMA of the last two steps of a
-  // tile already fetches steps 0 and 1 of the next one, and the fragments read at
+  // ... and runs their K loops as one stream: the DMA of the last D steps of a
+  // tile already fetches the first D steps of the next one, and the fragments read at
   // the end of the last step are the next tile's first. The epilogue of a tile
   // then runs with the next tile's panels landing in LDS, and its stores drain
   // while the next K loop is under way.

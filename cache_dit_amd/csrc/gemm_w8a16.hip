@@ -179,17 +179,18 @@ __global__ __launch_bounds__(C::THREADS) void gemm_w8a16_tiled(GemmArgs g, int t
 // ---------------------------------------------------------------------------
 // Wide kernel: the schedule of the wide w8a8 kernel (one persistent workgroup of 4
 // waves per CU, one wave per SIMD with all 256 AGPRs as accumulators, LDS-DMA by
-// buffer loads spread over the MFMA stream, A panel in 3 LDS stages and B panel in
-// 2, one barrier per K step, the DMA stream running across tiles) with bf16 MFMAs:
+// buffer loads spread over the MFMA stream DEPTH steps ahead, A panel in DEPTH + 1 LDS
+// stages and B panel in DEPTH, one barrier per K step, the DMA stream running across
+// tiles) with bf16 MFMAs:
 // v_mfma_f32_32x32x16_bf16 (8 passes), K steps of 64 elements, wave tile
 // (BM/2) x (BN/2) as TM x TN blocks of 32x32, four MFMAs per block and step.
 //
-// Panels: A rows 128 B (bf16), chunk c of row r at
-// c ^ ((r>>1)&7); B rows 64 B (e4m3), chunk c at c ^ ((r>>2)&3). A lane reads, per
-// 32-row block, the four A chunks 4t+2h+s (h = lane>>5) and the two B chunks 2t+h:
-// the 16 B bytes of one chunk are the weights of MFMA steps 2t and 2t+1 (K order
-// permuted identically on both sides). The weights are converted to bf16 once per
-// step, when they arrive from LDS, and kept for all row blocks.
+// Panels: A rows 128 B (bf16), chunk c of row r at c ^ ((r>>1)&7); B rows 64 B
+// (e4m3), chunk c at c ^ ((r>>2)&3). A lane reads, per 32-row block, the four A
+// chunks 4t+2h+s (h = lane>>5) and the two B chunks 2t+h: the 16 B bytes of one
+// chunk are the weights of MFMA steps 2t and 2t+1 (K order permuted identically on
+// both sides). The weights are converted to bf16 once per step, four conversions
+// at a time two MFMAs ahead of their first use, and kept for all row blocks.
 //
 // The B fragments take their 32 rows in a permuted order, operand row p reads
 // panel row 16 ((p>>2)&1) + 4 (p>>3) + (p&3) of its block: with the operands
