@@ -284,20 +284,6 @@ __device__ __forceinline__ void mfma_32x32x16_bf16(v16f& acc, const v8bf& w, con
   }
 }
 
-// 16 e4m3 bytes -> two bf16 MFMA operands (MFMA steps 2t and 2t+1)
-__device__ __forceinline__ void convert_w(const uint4& w, v8bf& lo, v8bf& hi) {
-  const v2bf c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.x, 1.0f, false);
-  const v2bf c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.x, 1.0f, true);
-  const v2bf c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.y, 1.0f, false);
-  const v2bf c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.y, 1.0f, true);
-  const v2bf c4 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.z, 1.0f, false);
-  const v2bf c5 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.z, 1.0f, true);
-  const v2bf c6 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.w, 1.0f, false);
-  const v2bf c7 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w.w, 1.0f, true);
-  lo = v8bf{c0[0], c0[1], c1[0], c1[1], c2[0], c2[1], c3[0], c3[1]};
-  hi = v8bf{c4[0], c4[1], c5[0], c5[1], c6[0], c6[1], c7[0], c7[1]};
-}
-
 template <class C>
 __global__ __launch_bounds__(C::THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void
 gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
