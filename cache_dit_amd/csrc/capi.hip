@@ -239,6 +239,33 @@ int cdit_fp8_linear_w8a8(const void* x_bf16, const void* w_q, const float* w_sca
                          const void* bias, void* out, void* q_ws, float* scale_ws, int64_t M,
                          int64_t N, int64_t K, int64_t ld_x, int64_t ldw, int64_t ldo,
                          int scale_mode, int epilogue, int out_dtype_id, void* stream) {
+  // M <= 16 (the M = 1 modulation Linears): one kernel that quantizes the rows itself,
+  // when every argument passes the checks of the two entry points it stands for
+  if (M >= 1 && M <= 16 && N > 0 && K > 0 && K <= INT32_MAX && N <= INT32_MAX && x_bf16 && q_ws &&
+      scale_ws && w_scale && ld_x >= K &&
+      (scale_mode == CDIT_SCALE_BF16DIV || scale_mode == CDIT_SCALE_FP32DIV) &&
+      check_gemm("cdit_fp8_linear_w8a8", q_ws, w_q, w_scale, bias, out, M, N, K, K, ldw, ldo,
+                 epilogue, out_dtype_id, false) == CDIT_OK &&
+      check_arch() == CDIT_OK) {
+    GemmArgs g;
+    g.a = x_bf16;
+    g.a_scale = nullptr;
+    g.b = static_cast<const uint8_t*>(w_q);
+    g.b_scale = w_scale;
+    g.bias = static_cast<const uint16_t*>(bias);
+    g.out = static_cast<uint16_t*>(out);
+    g.M = (int)M;
+    g.N = (int)N;
+    g.K = (int)K;
+    g.lda = ld_x;
+    g.ldb = ldw;
+    g.ldo = ldo;
+    g.epilogue = epilogue;
+    g.out_dtype = out_dtype_id;
+    if (launch_linear_fp8_skinny_fused(g, q_ws, scale_ws, scale_mode, g_gemm_variant,
+                                       static_cast<hipStream_t>(stream)) == 0)
+      return after_launch("cdit_fp8_linear_w8a8");
+  }
   int rc = cdit_fp8_quant_rowwise(x_bf16, M, K, ld_x, q_ws, K, scale_ws, scale_mode, stream);
   if (rc) return rc;
   return cdit_fp8_gemm_rowwise(q_ws, scale_ws, w_q, w_scale, bias, out, M, N, K, K, ldw, ldo,

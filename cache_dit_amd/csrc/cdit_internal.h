@@ -36,6 +36,12 @@ struct GemmArgs {
 // variant < 0: choose by shape.
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream);
 int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream);
+// One w8a8 Linear forward at M <= 16 in a single kernel (per-token quantizer + GEMM);
+// g.a is the bf16 activation, g.lda its leading dimension in elements. Returns 0 when
+// launched, 1 when the shape or alignment is not taken (the caller then runs the
+// quantizer and the GEMM one after the other).
+int launch_linear_fp8_skinny_fused(const GemmArgs& g, void* q_ws, float* scale_ws, int scale_mode,
+                                   int variant, hipStream_t stream);
 
 void set_error(const char* fmt, ...);
 

@@ -29,6 +29,7 @@
 #include <type_traits>
 
 #include "gemm_common.h"
+#include "quant_device.h"
 
 namespace cdit {
 namespace {
@@ -761,6 +762,132 @@ __global__ __launch_bounds__(256) void gemm_fp8_skinny(GemmArgs g) {
   }
 }
 
+// The skinny kernel with the per-token quantizer inside, for one whole Linear forward at
+// M <= 16 (the M = 1 modulation Linears): a separate quantizer launch for a single row
+// costs as much as this GEMM's weight stream. Every workgroup quantizes the M activation
+// rows itself (a few KiB, an L2 hit for all but the first) into LDS with the quantizer's
+// own arithmetic (quant_device.h), so the codes and scales are those of
+// cdit_fp8_quant_rowwise bit for bit; workgroup 0 also writes them to the caller's
+// workspaces. The first batch of weight loads is issued before that, so the HBM latency
+// of the weights covers it. g.a is the bf16 activation here, g.lda its leading dimension.
+constexpr int kFusedPad = 16;  // LDS row pitch K + 16 bytes: rows start 4 banks apart
+__global__ __launch_bounds__(256) void linear_fp8_skinny_fused(GemmArgs g, uint8_t* q_ws,
+                                                               float* scale_ws, int scale_mode) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t codes[];  // [M][K + kFusedPad]
+  __shared__ float part[4][16][17];
+  __shared__ uint32_t wave_amax[4];
+  __shared__ float row_s[16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, kg = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int nrow = min(n0 + r, g.N - 1);
+  const int KT = g.K / 128;
+  const int per = (KT + 3) / 4;
+  const int k_begin = wave * per, k_end = min(KT, k_begin + per);
+  const int pitch = g.K + kFusedPad;
+  const uint8_t* __restrict__ wp = g.b + (int64_t)nrow * g.ldb + kg * 32;
+  constexpr int U = 6;  // steps in flight
+  v4i w[U][2];
+  auto load_w = [&](int k0) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kt = min(k0 + u, max(k_end, 1) - 1);  // clamped duplicates are not accumulated
+      const v4i* wq = reinterpret_cast<const v4i*>(wp + (int64_t)kt * 128);
+      w[u][0] = __builtin_nontemporal_load(wq);
+      w[u][1] = __builtin_nontemporal_load(wq + 1);
+    }
+  };
+  load_w(k_begin);
+
+  // ---- quantize the activation rows into LDS
+  const uint16_t* x = static_cast<const uint16_t*>(g.a);
+  const int nchunks = g.K >> 3;  // 16-byte chunks of 8 bf16
+  for (int m = 0; m < g.M; ++m) {
+    const uint4* xr = reinterpret_cast<const uint4*>(x + (int64_t)m * g.lda);
+    uint32_t am = 0;
+    for (int c = threadIdx.x; c < nchunks; c += 256) {
+      const uint4 v = xr[c];
+      am = absmax2(absmax2(absmax2(absmax2(am, v.x), v.y), v.z), v.w);
+    }
+    am = wave_max_u32(fold2(am));
+    if (lane == 0) wave_amax[wave] = am;
+    __syncthreads();
+    const uint32_t a01 = max(wave_amax[0], wave_amax[1]), a23 = max(wave_amax[2], wave_amax[3]);
+    const float s = row_scale(max(a01, a23), scale_mode);
+    if (threadIdx.x == 0) row_s[m] = s;
+    uint2* dst = reinterpret_cast<uint2*>(codes + m * pitch);
+    if (scale_in_fast_window(s)) {  // uniform
+      const float rcp = 1.0f / s;
+      for (int c = threadIdx.x; c < nchunks; c += 256) {
+        const uint4 v = xr[c];
+        dst[c] = uint2{quant4<true>(v.x, v.y, s, rcp), quant4<true>(v.z, v.w, s, rcp)};
+      }
+    } else {
+      for (int c = threadIdx.x; c < nchunks; c += 256) {
+        const uint4 v = xr[c];
+        dst[c] = uint2{quant4<false>(v.x, v.y, s, 0.0f), quant4<false>(v.z, v.w, s, 0.0f)};
+      }
+    }
+    __syncthreads();  // codes of row m complete; wave_amax free for the next row
+  }
+  if (blockIdx.x == 0) {  // the caller's workspaces get what cdit_fp8_quant_rowwise would write
+    for (int m = 0; m < g.M; ++m) {
+      const uint2* src = reinterpret_cast<const uint2*>(codes + m * pitch);
+      uint2* dst = reinterpret_cast<uint2*>(q_ws + (int64_t)m * g.K);
+      for (int c = threadIdx.x; c < nchunks; c += 256) dst[c] = src[c];
+    }
+    if ((int)threadIdx.x < g.M) scale_ws[threadIdx.x] = row_s[threadIdx.x];
+  }
+
+  // ---- the skinny GEMM, activation fragments from LDS
+  const bool a_valid = r < g.M;
+  const uint8_t* ap = codes + min(r, g.M - 1) * pitch + kg * 32;
+  v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int k0 = k_begin; k0 < k_end; k0 += U) {
+    if (k0 != k_begin) load_w(k0);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (k0 + u < k_end) {
+        const v4i* aq = reinterpret_cast<const v4i*>(ap + (k0 + u) * 128);
+        v8i af = __builtin_shufflevector(aq[0], aq[1], 0, 1, 2, 3, 4, 5, 6, 7);
+        if (!a_valid) af = v8i{0, 0, 0, 0, 0, 0, 0, 0};
+        const v8i wf = __builtin_shufflevector(w[u][0], w[u][1], 0, 1, 2, 3, 4, 5, 6, 7);
+        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, acc, 0, 0, 0, 0, 0, 0);
+      }
+    }
+  }
+  // acc[e] = partial out[m = lane&15][n0 + 4*(lane>>4) + e]
+#pragma unroll
+  for (int e = 0; e < 4; ++e) part[wave][r][4 * kg + e] = acc[e];
+  __syncthreads();
+  if (wave == 0) {
+    const int m = r, nl = 4 * kg;
+    if (m < g.M && n0 + nl < g.N) {
+      const float as = row_s[m];
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float sum = (part[0][m][nl + e] + part[1][m][nl + e]) +
+                          (part[2][m][nl + e] + part[3][m][nl + e]);
+        const int n = n0 + nl + e;
+        float t = sum * as * g.b_scale[n];
+        if (g.bias) t += bias_at(g, n);
+        if (g.epilogue & CDIT_EPI_GELU_TANH) t = gelu_tanh(t);
+        v[e] = t;
+      }
+      if (g.out_dtype == CDIT_DT_BF16) {
+        uint2 pk;
+        pk.x = pack_bf16x2(v[0], v[1]);
+        pk.y = pack_bf16x2(v[2], v[3]);
+        *reinterpret_cast<uint2*>(g.out + (int64_t)m * g.ldo + n0 + nl) = pk;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) store_out(g, (int64_t)m * g.ldo + n0 + nl + e, v[e]);
+      }
+    }
+  }
+}
+
 // Any shape, any alignment: a 16x16 output tile per workgroup, one output
 // element per thread, scalar decode + FMA. Only for shapes the tiled kernel
 // cannot take (K not a multiple of 128, N not a multiple of 8, odd strides).
@@ -822,6 +949,22 @@ typedef CfgWide<256, 192, 8> V15;                     // ... 128x96 wave tiles
 typedef CfgWide<128, 192, 4, 3> V16;                  // ... 64x96 wave tiles, DMA 3 steps ahead
 typedef CfgWide<64, 128, 8, 5> V17;                   // ... 32x64 wave tiles, DMA 5 steps ahead
 typedef CfgWide<128, 128, 4, 4> V18;                  // ... 64x64 wave tiles, DMA 4 steps ahead
+
+int launch_linear_fp8_skinny_fused(const GemmArgs& g, void* q_ws, float* scale_ws, int scale_mode,
+                                   int variant, hipStream_t stream) {
+  const int64_t lds = (int64_t)g.M * (g.K + kFusedPad);
+  const bool ok = g.M >= 1 && g.M <= 16 && (variant < 0 || variant == 50) && g.K >= 128 &&
+                  g.K % 128 == 0 && g.N % 8 == 0 && lds <= 48 * 1024 && g.lda % 8 == 0 &&
+                  g.ldb % 16 == 0 && g.ldo % 8 == 0 &&
+                  reinterpret_cast<uintptr_t>(g.a) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(g.b) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(g.out) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(q_ws) % 8 == 0;
+  if (!ok) return 1;
+  hipLaunchKernelGGL(linear_fp8_skinny_fused, dim3((g.N + 15) / 16), dim3(256), (size_t)lds, stream,
+                     g, static_cast<uint8_t*>(q_ws), scale_ws, scale_mode);
+  return 0;
+}
 
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {

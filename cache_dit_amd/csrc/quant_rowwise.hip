@@ -24,116 +24,10 @@
 #include <stdint.h>
 
 #include "cdit_internal.h"
+#include "quant_device.h"
 
 namespace cdit {
 namespace {
-
-constexpr float kFp8Max = 448.0f;
-
-__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
-__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
-
-// fp32 -> nearest-even bf16, returned widened back to fp32 (c10::BFloat16 rule).
-__device__ __forceinline__ float round_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return __uint_as_float(0x7fc00000u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return __uint_as_float(u & 0xffff0000u);
-}
-
-// max over the wavefront of an unsigned value (order independent, exact). Four
-// DPP steps reduce each row of 16 lanes (xor 1, xor 2, half mirror, mirror), then
-// the four row results are read into scalars.
-__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-  auto step = [](uint32_t a, int ctrl_id) {
-    uint32_t o;
-    switch (ctrl_id) {
-      case 0: o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)a, 0xB1, 0xf, 0xf, false); break;
-      case 1: o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)a, 0x4E, 0xf, 0xf, false); break;
-      case 2: o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)a, 0x141, 0xf, 0xf, false); break;
-      default: o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)a, 0x140, 0xf, 0xf, false); break;
-    }
-    return a > o ? a : o;
-  };
-  v = step(v, 0);  // quad_perm [1,0,3,2]
-  v = step(v, 1);  // quad_perm [2,3,0,1]
-  v = step(v, 2);  // row_half_mirror
-  v = step(v, 3);  // row_mirror
-  const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0);
-  const uint32_t b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
-  const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32);
-  const uint32_t d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
-  const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
-  return ab > cd ? ab : cd;
-}
-
-__device__ __forceinline__ float row_scale(uint32_t amax_bits, int scale_mode) {
-  // amax_bits: bf16 bit pattern of max |x| (sign cleared).
-  float amax = __uint_as_float(amax_bits << 16);
-  float s = amax / kFp8Max;
-  if (scale_mode == CDIT_SCALE_BF16DIV) s = round_to_bf16(s);
-  return s == 0.0f ? 1.0f : s;
-}
-
-__device__ __forceinline__ float clamp448(float y) {
-  return fminf(fmaxf(y, -kFp8Max), kFp8Max);
-}
-
-// x / s with s > 0 finite. FAST: r = 1/s correctly rounded, s inside the window.
-template <bool FAST>
-__device__ __forceinline__ float div_scale(float x, float s, float r) {
-  if constexpr (FAST) {
-    const float q0 = x * r;
-    const float e = __fmaf_rn(-q0, s, x);
-    const float q = __fmaf_rn(e, r, q0);
-    return __uint_as_float((__float_as_uint(q) & 0x7fffffffu) | (__float_as_uint(x) & 0x80000000u));
-  } else {
-    return x / s;
-  }
-}
-
-// 2^-100 <= s < 2^101: the window the fast division is proven on.
-__device__ __forceinline__ bool scale_in_fast_window(float s) {
-  const uint32_t e = (__float_as_uint(s) >> 23) & 0xffu;
-  return e >= 27u && e <= 227u;
-}
-
-// two bf16 pairs (4 elements) -> 4 e4m3 bytes. On the fast path the clamp is
-// implicit: |x| <= amax and scale >= amax/448 * (1 - 2^-9), so |x/scale| < 450,
-// below the tie at 464 where the e4m3 conversion would stop rounding to 448
-// (tests/native/divcheck.c checks the unclamped quotient of every input pair).
-template <bool FAST>
-__device__ __forceinline__ uint32_t quant4(uint32_t w0, uint32_t w1, float s, float r) {
-  float a = div_scale<FAST>(bf16_lo(w0), s, r);
-  float b = div_scale<FAST>(bf16_hi(w0), s, r);
-  float c = div_scale<FAST>(bf16_lo(w1), s, r);
-  float d = div_scale<FAST>(bf16_hi(w1), s, r);
-  if constexpr (!FAST) {
-    a = clamp448(a);
-    b = clamp448(b);
-    c = clamp448(c);
-    d = clamp448(d);
-  }
-  uint32_t p = 0;
-  p = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, p, false);
-  p = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, p, true);
-  return p;
-}
-
-// Running max of packed |bf16| pairs, both halves at once: m and the result hold
-// two independent 16-bit maxima (v_pk_max_u16), compared as unsigned integers
-// (monotone in magnitude; a NaN pattern wins, as in torch.amax). fold2 merges the
-// halves at the end.
-__device__ __forceinline__ uint32_t absmax2(uint32_t m, uint32_t w) {
-  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-  const u16x2 a = __builtin_bit_cast(u16x2, w & 0x7fff7fffu);
-  const u16x2 r = __builtin_elementwise_max(__builtin_bit_cast(u16x2, m), a);
-  return __builtin_bit_cast(uint32_t, r);
-}
-__device__ __forceinline__ uint32_t fold2(uint32_t m) {
-  const uint32_t lo = m & 0xffffu, hi = m >> 16;
-  return lo > hi ? lo : hi;
-}
 
 // Row resident in registers: CH 16-byte chunks per lane (K <= CH*512).
 template <int CH, bool NT = false>

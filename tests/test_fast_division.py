@@ -28,6 +28,6 @@ def test_divcheck_exhaustive(tmp_path):
 
 def test_kernel_source_uses_the_checked_window():
   """The exponent window in the kernel and in the checker must be the same."""
-  k = open(os.path.join(ROOT, "cache_dit_amd", "csrc", "quant_rowwise.hip")).read()
+  k = open(os.path.join(ROOT, "cache_dit_amd", "csrc", "quant_device.h")).read()
   c = open(os.path.join(HERE, "native", "divcheck.c")).read()
   assert "e >= 27u && e <= 227u" in k and "e >= 27 && e <= 227" in c

@@ -390,3 +390,43 @@ def test_wide_variants_agree_bit_for_bit_on_random_data():
     torch.cuda.synchronize()
     for variant, epi, out in outs[2:]:
       assert torch.equal(out, outs[epi][2]), (M, N, K, variant, epi)
+
+
+@pytest.mark.parametrize("scale_mode", [0, 1])
+@pytest.mark.parametrize("M,N,K", [(1, 18432, 3072), (1, 9216, 3072), (3, 264, 256), (15, 520, 3072),
+                                   (16, 512, 3072), (16, 72, 128), (2, 4096, 15360)])
+def test_fused_linear_for_few_rows_matches_the_two_calls(M, N, K, scale_mode):
+  """cdit_fp8_linear_w8a8 at M <= 16 runs one kernel that quantizes the rows itself (when
+  M (K + 16) bytes of codes fit in 48 KiB of LDS; (16, ., 3072) does not and takes the two
+  kernels): codes, scales and outputs must equal those of the quantizer and the GEMM called
+  one after the other, bit for bit, including zero rows and scales outside the fast-division
+  window."""
+  from cache_dit_amd import _native, ops
+  g = torch.Generator(device="cuda").manual_seed(M * 7 + N + K + scale_mode)
+  x = (torch.randn(M, K, generator=g, device="cuda") * 2).to(torch.bfloat16)
+  if M >= 3:
+    x[0] = 0
+    x[1] = x[1] * 1e-32
+    x[2] = x[2] * 1e32
+  w = (torch.randn(N, K, generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+  wq, w_s = ops.fp8_rowwise_quant(w)
+  w_s = w_s.reshape(-1).contiguous()
+  bias = (torch.randn(N, generator=g, device="cuda") * 0.1).to(torch.bfloat16)
+  L = _native.load()
+  for epi in (0, 1):
+    q_ws = torch.full((M, K), 0x55, dtype=torch.uint8, device="cuda").view(FP8)
+    s_ws = torch.full((M,), -1.0, dtype=torch.float32, device="cuda")
+    out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    rc = L.cdit_fp8_linear_w8a8(x.data_ptr(), wq.data_ptr(), w_s.data_ptr(), bias.data_ptr(),
+                                out.data_ptr(), q_ws.data_ptr(), s_ws.data_ptr(), M, N, K, K, K, N,
+                                scale_mode, epi, 1, None)
+    assert rc == 0, L.cdit_last_error()
+    q2 = torch.empty(M, K, dtype=FP8, device="cuda")
+    s2 = torch.empty(M, dtype=torch.float32, device="cuda")
+    out2 = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    ops.quant_rowwise_into(x, q2, s2, scale_mode)
+    ops.gemm_rowwise_into(q2, s2, wq, w_s, bias, out2, epi)
+    torch.cuda.synchronize()
+    assert torch.equal(q_ws.view(torch.uint8), q2.view(torch.uint8))
+    assert torch.equal(s_ws.view(torch.int32), s2.view(torch.int32))
+    assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
