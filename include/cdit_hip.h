@@ -157,7 +157,9 @@ int cdit_w8a16_gemm(const void* x_bf16, const void* b_q, const float* b_scale,
 /*
  * One quantized nn.Linear forward in the w8a8 dynamic mode: the two calls above
  * back to back on `stream` (per-token quantization of x into the caller's
- * workspace, then the scaled GEMM), saving one trip through the caller's FFI.
+ * workspace, then the scaled GEMM), saving one trip through the caller's FFI;
+ * at M <= 16 a single kernel that quantizes the rows itself, with the same
+ * results and the same workspace contents.
  * This is what torchao's Float8Tensor `aten.linear` override does for a Linear
  * that cache-dit converted with `quantize_(..., Float8DynamicActivation
  * Float8WeightConfig(granularity=(PerRow(), PerRow())))`
