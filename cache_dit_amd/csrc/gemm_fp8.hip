@@ -610,11 +610,19 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     // else that is live (DMA offsets, scales) in spare AGPRs and scratch, and a scratch
     // reload waits for every output store in flight (vmcnt). The GELU decision is
     // taken once per tile, not once per element.
+    // Store addresses: a wave-uniform 64-bit base per row of blocks plus a 32-bit byte
+    // offset per lane (the launcher bounds 512 * ldo), instead of 64-bit arithmetic
+    // per store.
+    constexpr int OB = OUT == CDIT_DT_F32 ? 4 : 2;  // bytes per output element
+    uint8_t* const out_wave = reinterpret_cast<uint8_t*>(g.out) +
+                              ((int64_t)(m0 + wm * C::WM) * g.ldo + (n0 + wn * C::WN)) * OB;
+    const uint32_t out_lane = ((uint32_t)r16 * (uint32_t)g.ldo + 8u * kg) * OB;
     auto epilogue = [&](auto gelu_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
         const int m = mw + 16 * i;
+        uint8_t* const out_row = out_wave + (int64_t)(16 * i) * g.ldo * OB;
 #pragma unroll
         for (int u = 0; u < TN / 2; ++u) {  // pair of fragments 2u, 2u+1: 8 consecutive columns
           float v[8];
@@ -634,16 +642,16 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
           }
           const int n = nw + 64 * (u >> 1) + 32 * (u & 1);
           if (m < g.M && n < g.N) {
+            uint8_t* const dst = out_row + out_lane + (64 * (u >> 1) + 32 * (u & 1)) * OB;
             if constexpr (OUT == CDIT_DT_F32) {
-              float* dst = reinterpret_cast<float*>(g.out) + (int64_t)m * g.ldo + n;
               *reinterpret_cast<v4f*>(dst) = v4f{v[0], v[1], v[2], v[3]};
-              *reinterpret_cast<v4f*>(dst + 4) = v4f{v[4], v[5], v[6], v[7]};
+              *reinterpret_cast<v4f*>(dst + 16) = v4f{v[4], v[5], v[6], v[7]};
             } else if constexpr (OUT == CDIT_DT_F16) {
-              *reinterpret_cast<uint4*>(g.out + (int64_t)m * g.ldo + n) =
+              *reinterpret_cast<uint4*>(dst) =
                   uint4{pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3]), pack_f16x2(v[4], v[5]),
                         pack_f16x2(v[6], v[7])};
             } else {
-              *reinterpret_cast<uint4*>(g.out + (int64_t)m * g.ldo + n) =
+              *reinterpret_cast<uint4*>(dst) =
                   uint4{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]),
                         pack_bf16x2(v[6], v[7])};
             }
@@ -929,7 +937,8 @@ bool tiled_ok(const GemmArgs& g) {
          // the epilogues load scales as float4 and bias as 8-byte packs
          reinterpret_cast<uintptr_t>(g.b_scale) % 16 == 0 &&
          reinterpret_cast<uintptr_t>(g.bias) % 16 == 0 &&
-         (int64_t)512 * g.lda < (int64_t)1 << 31 && (int64_t)512 * g.ldb < (int64_t)1 << 31;
+         (int64_t)512 * g.lda < (int64_t)1 << 31 && (int64_t)512 * g.ldb < (int64_t)1 << 31 &&
+         (int64_t)512 * g.ldo < (int64_t)1 << 29;
 }
 
 }  // namespace
