@@ -385,6 +385,9 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
   const int wm = wave >> 1, wn = wave & 1;
   constexpr int BKW = C::BKW, TM = C::TM, TN = C::TN, H = C::H;
   constexpr int D = C::DEPTH;
+  // output stores per wave and tile (16 bytes per lane each); every wave issues all of them
+  constexpr int NST = TM * (TN / 2) * (OUT == CDIT_DT_F32 ? 2 : 1);
+  static_assert((D - 2) * C::ND + C::NDA + NST <= 63, "vmcnt is a 6-bit counter");
   const int KT = g.K / BKW;  // >= D (checked by the launcher)
   const int ntiles = tiles_m * tiles_n;
 
@@ -560,10 +563,11 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
       }
       // own LDS reads of this step done, own DMA of the next step landed (the
       // steps after it and the A panel issued above may still fly); then
-      // everyone's. In the first D-1 steps of a later tile the DMA in question was
-      // waited for before the previous epilogue's stores, which may keep flying.
+      // everyone's. In the first D-1 steps of a later tile the NST output stores of
+      // the previous epilogue were issued after the DMA in question (the counter
+      // retires in issue order) and may keep flying as well.
       if (kt <= D - 2 && tile != (int)blockIdx.x) {
-        wait_and_barrier<63>();
+        wait_and_barrier<(D - 2) * C::ND + C::NDA + NST>();
       } else {
         wait_and_barrier<(D - 2) * C::ND + C::NDA>();
       }
@@ -602,27 +606,39 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- epilogue
-    // Every DMA issued so far (the next tile's first D steps) must have landed
-    // before the stores go out: step 0 of the next tile then waits for nothing.
-    wait_vm<0>();
+    // Nothing is drained here: the next tile's step 0 landed before the barrier of
+    // the last step, its later steps keep flying under the epilogue.
     // The accumulators are read with inline assembly, one row of blocks at a time:
     // left to itself the compiler copies all of them to VGPRs first, parks everything
     // else that is live (DMA offsets, scales) in spare AGPRs and scratch, and a scratch
     // reload waits for every output store in flight (vmcnt). The GELU decision is
     // taken once per tile, not once per element.
-    // Store addresses: a wave-uniform 64-bit base per row of blocks plus a 32-bit byte
-    // offset per lane (the launcher bounds 512 * ldo), instead of 64-bit arithmetic
-    // per store.
+    // Stores are buffer stores that every wave always issues, NST per tile, so that
+    // the waits of the next K loop can count them: the descriptor of a row of blocks
+    // covers the rows of it that exist (the hardware drops lanes beyond), lanes whose
+    // columns do not exist get an offset beyond any descriptor. Per lane a 32-bit
+    // byte offset (the launcher bounds 512 * ldo), per row of blocks a scalar base.
     constexpr int OB = OUT == CDIT_DT_F32 ? 4 : 2;  // bytes per output element
+    constexpr uint32_t kNoColumn = 0x80000000u;
     uint8_t* const out_wave = reinterpret_cast<uint8_t*>(g.out) +
                               ((int64_t)(m0 + wm * C::WM) * g.ldo + (n0 + wn * C::WN)) * OB;
+    const int rows_wave = g.M - (m0 + wm * C::WM);  // rows of the wave tile that exist
     const uint32_t out_lane = ((uint32_t)r16 * (uint32_t)g.ldo + 8u * kg) * OB;
+    uint32_t out_off[TN / 2];
+#pragma unroll
+    for (int u = 0; u < TN / 2; ++u)
+      out_off[u] = nw + 64 * (u >> 1) + 32 * (u & 1) < g.N
+                       ? out_lane + (64 * (u >> 1) + 32 * (u & 1)) * OB
+                       : kNoColumn;
     auto epilogue = [&](auto gelu_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
-        const int m = mw + 16 * i;
-        uint8_t* const out_row = out_wave + (int64_t)(16 * i) * g.ldo * OB;
+        // (made a scalar explicitly: a descriptor the compiler takes for divergent is
+        // applied in a loop over its distinct values)
+        const int rows = __builtin_amdgcn_readfirstlane(min(max(rows_wave - 16 * i, 0), 16));
+        const __amdgpu_buffer_rsrc_t out_row = __builtin_amdgcn_make_buffer_rsrc(
+            out_wave + (int64_t)(16 * i) * g.ldo * OB, 0, rows * g.ldo * OB, 0x00020000);
 #pragma unroll
         for (int u = 0; u < TN / 2; ++u) {  // pair of fragments 2u, 2u+1: 8 consecutive columns
           float v[8];
@@ -640,21 +656,25 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
               v[4 * d + e] = t;
             }
           }
-          const int n = nw + 64 * (u >> 1) + 32 * (u & 1);
-          if (m < g.M && n < g.N) {
-            uint8_t* const dst = out_row + out_lane + (64 * (u >> 1) + 32 * (u & 1)) * OB;
-            if constexpr (OUT == CDIT_DT_F32) {
-              *reinterpret_cast<v4f*>(dst) = v4f{v[0], v[1], v[2], v[3]};
-              *reinterpret_cast<v4f*>(dst + 16) = v4f{v[4], v[5], v[6], v[7]};
-            } else if constexpr (OUT == CDIT_DT_F16) {
-              *reinterpret_cast<uint4*>(dst) =
-                  uint4{pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3]), pack_f16x2(v[4], v[5]),
-                        pack_f16x2(v[6], v[7])};
-            } else {
-              *reinterpret_cast<uint4*>(dst) =
-                  uint4{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]),
-                        pack_bf16x2(v[6], v[7])};
-            }
+          if constexpr (OUT == CDIT_DT_F32) {
+            __builtin_amdgcn_raw_buffer_store_b128(
+                v4u{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]),
+                    __float_as_uint(v[3])},
+                out_row, (int)out_off[u], 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(
+                v4u{__float_as_uint(v[4]), __float_as_uint(v[5]), __float_as_uint(v[6]),
+                    __float_as_uint(v[7])},
+                out_row, (int)(out_off[u] + 16u), 0, 0);
+          } else if constexpr (OUT == CDIT_DT_F16) {
+            __builtin_amdgcn_raw_buffer_store_b128(
+                v4u{pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3]), pack_f16x2(v[4], v[5]),
+                    pack_f16x2(v[6], v[7])},
+                out_row, (int)out_off[u], 0, 0);
+          } else {
+            __builtin_amdgcn_raw_buffer_store_b128(
+                v4u{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]),
+                    pack_bf16x2(v[6], v[7])},
+                out_row, (int)out_off[u], 0, 0);
           }
         }
         __builtin_amdgcn_sched_barrier(0);

@@ -430,3 +430,30 @@ def test_fused_linear_for_few_rows_matches_the_two_calls(M, N, K, scale_mode):
     assert torch.equal(q_ws.view(torch.uint8), q2.view(torch.uint8))
     assert torch.equal(s_ws.view(torch.int32), s2.view(torch.int32))
     assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
+
+
+@pytest.mark.parametrize("variant", [-1] + TILED_VARIANTS + [100])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float32])
+def test_nothing_is_written_outside_the_output(variant, dt):
+  """The output is a window of a larger buffer (rows below it, columns to its right, ldo > N)
+  holding a sentinel, with M and N that leave partial tiles in both directions: the window
+  must equal the result of the contiguous call and not one sentinel may change."""
+  from cache_dit_amd import _native, ops
+  for M, N, K in [(300, 528, 256), (70, 1040, 384), (5, 272, 640)]:
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randint(-4, 5, (M, K), generator=g).float().to(FP8).cuda()
+    w = torch.randint(-4, 5, (N, K), generator=g).float().to(FP8).cuda()
+    s_a = torch.full((M,), 0.5, device="cuda")
+    s_w = torch.full((N,), 0.25, device="cuda")
+    b = None if dt == torch.float32 else torch.randint(-8, 9, (N,), generator=g).to(dt).cuda()
+    _native.set_gemm_variant(variant)
+    plain = torch.empty(M, N, dtype=dt, device="cuda")
+    ops.gemm_rowwise_into(a, s_a, w, s_w, b, plain, 0)
+    buf = torch.full((M + 40, N + 24), -7.0, dtype=dt, device="cuda")
+    ops.gemm_rowwise_into(a, s_a, w, s_w, b, buf[:M, :N], 0)
+    torch.cuda.synchronize()
+    assert torch.equal(buf[:M, :N], plain), (M, N, K)
+    assert bool((buf[M:] == -7.0).all()) and bool((buf[:, N:] == -7.0).all()), (M, N, K)
+    ref = to.scaled_mm_rowwise(a.cpu(), s_a.cpu().reshape(-1, 1), w.cpu(), s_w.cpu().reshape(-1, 1),
+                               None if b is None else b.cpu(), out_dtype=dt)
+    assert torch.equal(plain.cpu(), ref), (M, N, K)

@@ -170,3 +170,26 @@ def test_wide_kernels_random_shapes_many_tiles_per_workgroup(variant):
     rows = torch.cat([torch.arange(0, M, 61), torch.arange(M - 5, M)])
     ref = to.w8a16_linear(x[rows.cuda()].cpu(), w.cpu(), sw.cpu().reshape(-1, 1), b.cpu(), fused=True)
     assert torch.equal(out[rows.cuda()].cpu(), ref), (M, N, K)
+
+
+@pytest.mark.parametrize("variant", [-1, 0, 3, 7, 8, 9, 10, 11, 12, 100])
+def test_nothing_is_written_outside_the_output(variant):
+  """The output is a window of a larger buffer holding a sentinel (ldo > N, rows below),
+  M and N leave partial tiles: the window equals the contiguous result, no sentinel changes."""
+  from cache_dit_amd import _native, ops
+  for M, N, K in [(300, 528, 256), (70, 1040, 384), (5, 272, 640)]:
+    g = torch.Generator().manual_seed(M + N)
+    x = torch.randint(-3, 4, (M, K), generator=g).to(torch.bfloat16).cuda()
+    w = torch.randint(-3, 4, (N, K), generator=g).float().to(FP8).cuda()
+    sw = torch.full((N,), 0.25, device="cuda")
+    b = torch.randint(-8, 9, (N,), generator=g).to(torch.bfloat16).cuda()
+    _native.set_gemm_variant(variant)
+    plain = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    ops.w8a16_into(x, w, sw, b, plain, 0)
+    buf = torch.full((M + 40, N + 24), -7.0, dtype=torch.bfloat16, device="cuda")
+    ops.w8a16_into(x, w, sw, b, buf[:M, :N], 0)
+    torch.cuda.synchronize()
+    assert torch.equal(buf[:M, :N], plain), (M, N, K)
+    assert bool((buf[M:] == -7.0).all()) and bool((buf[:, N:] == -7.0).all()), (M, N, K)
+    ref = to.w8a16_linear(x.cpu(), w.cpu(), sw.cpu().reshape(-1, 1), b.cpu(), fused=True)
+    assert torch.equal(plain.cpu(), ref), (M, N, K)

@@ -21,7 +21,11 @@ things the compiler may add that the kernels must not have:
      carry alias scope information and are exempt;
   5. no scratch (register spill) access anywhere: a scratch reload is a vector
      memory load, the wait for it (vmcnt) also waits for every output store in
-     flight, which serialises the epilogue of a tile with the next tile's K loop.
+     flight, which serialises the epilogue of a tile with the next tile's K loop;
+  6. (w8a8 kernel) the waits of the first K steps of a tile count the output stores
+     of the previous tile's epilogue, so every wave must issue all of them whatever
+     part of the tile exists: each copy of the epilogue is one basic block with
+     TM * TN/2 buffer stores (twice that for fp32 output) and no global stores.
 """
 import os
 import re
@@ -137,3 +141,29 @@ def test_inline_asm_mfma_hazards(wide_kernels):
     for l in code[mfma[0]:mfma[-1]]:
       assert not (l.startswith("s_waitcnt") and "vmcnt(0)" in l), \
           f"{name}: {l!r} between MFMAs"
+
+
+def test_output_stores_are_unconditional(wide_kernels):
+  counted = 0
+  for name, code in wide_kernels.items():
+    m = re.search(r"gemm_fp8_wideINS0_7CfgWideILi(\d+)ELi(\d+)ELi\d+ELi\d+EEELi(\d)E", name)
+    if not m:
+      continue
+    bm, bn, out = int(m.group(1)), int(m.group(2)), int(m.group(3))
+    expect = (bm // 32) * (bn // 32) // 2 * (2 if out == 2 else 1)
+    assert not any(l.startswith("global_store") for l in code), name
+    # basic blocks end at branches and at labels
+    blocks, cur = [], 0
+    for l in code:
+      if l.startswith("buffer_store_dwordx4"):
+        cur += 1
+      if l.startswith(("s_cbranch", "s_branch")) or re.match(r"\.?\w+:", l):
+        if cur:
+          blocks.append(cur)
+        cur = 0
+    if cur:
+      blocks.append(cur)
+    assert blocks == [expect, expect], f"{name}: stores per basic block {blocks}, expected {expect} twice"
+    counted += 1
+  if any("gemm_fp8_wide" in n for n in wide_kernels):
+    assert counted >= 3
