@@ -623,22 +623,48 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     uint8_t* const out_wave = reinterpret_cast<uint8_t*>(g.out) +
                               ((int64_t)(m0 + wm * C::WM) * g.ldo + (n0 + wn * C::WN)) * OB;
     const int rows_wave = g.M - (m0 + wm * C::WM);  // rows of the wave tile that exist
-    const uint32_t out_lane = ((uint32_t)r16 * (uint32_t)g.ldo + 8u * kg) * OB;
+    // The memory pipeline merges the lanes of a store into one request only when
+    // adjacent lanes write adjacent bytes: with lane = 16 kg + r16 holding row r16,
+    // 16-byte piece kg, every lane is a request of its own (measured: 294 clocks per
+    // store instruction with four waves storing, against 77 when lanes 4r .. 4r+3 hold
+    // the 64 contiguous bytes of row r). 16-bit outputs are therefore moved to that
+    // arrangement with ds_bpermute_b32 (the LDS crossbar, no LDS memory) before they
+    // are stored: lane L takes the packed words of lane 16 (L & 3) + (L >> 2).
+    constexpr bool PERMUTE = OUT != CDIT_DT_F32;
+    const int st_row = PERMUTE ? lane >> 2 : r16, st_piece = PERMUTE ? lane & 3 : kg;
+    const int bp_addr = 4 * (16 * (lane & 3) + (lane >> 2));
+    const uint32_t out_lane = ((uint32_t)st_row * (uint32_t)g.ldo + 8u * st_piece) * OB;
     uint32_t out_off[TN / 2];
 #pragma unroll
     for (int u = 0; u < TN / 2; ++u)
-      out_off[u] = nw + 64 * (u >> 1) + 32 * (u & 1) < g.N
+      out_off[u] = n0 + wn * C::WN + 8 * st_piece + 64 * (u >> 1) + 32 * (u & 1) < g.N
                        ? out_lane + (64 * (u >> 1) + 32 * (u & 1)) * OB
                        : kNoColumn;
+    auto out_row_of = [&](int i) {
+      // (made a scalar explicitly: a descriptor the compiler takes for divergent is
+      // applied in a loop over its distinct values)
+      const int rows = __builtin_amdgcn_readfirstlane(min(max(rows_wave - 16 * i, 0), 16));
+      return __builtin_amdgcn_make_buffer_rsrc(out_wave + (int64_t)(16 * i) * g.ldo * OB, 0,
+                                               rows * g.ldo * OB, 0x00020000);
+    };
+    // 16-bit outputs: the permuted words of a row of blocks are stored while the next
+    // row is being computed, so the latency of the permutation is not waited for; the
+    // last row's after the two copies of the epilogue have joined
+    uint32_t moved[TN / 2][4];
+    auto store_moved = [&](int i) {
+      const __amdgpu_buffer_rsrc_t row = out_row_of(i);
+#pragma unroll
+      for (int u = 0; u < TN / 2; ++u)
+        __builtin_amdgcn_raw_buffer_store_b128(
+            v4u{moved[u][0], moved[u][1], moved[u][2], moved[u][3]}, row, (int)out_off[u], 0, 0);
+    };
     auto epilogue = [&](auto gelu_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
-        // (made a scalar explicitly: a descriptor the compiler takes for divergent is
-        // applied in a loop over its distinct values)
-        const int rows = __builtin_amdgcn_readfirstlane(min(max(rows_wave - 16 * i, 0), 16));
-        const __amdgpu_buffer_rsrc_t out_row = __builtin_amdgcn_make_buffer_rsrc(
-            out_wave + (int64_t)(16 * i) * g.ldo * OB, 0, rows * g.ldo * OB, 0x00020000);
+        if (PERMUTE && i > 0) store_moved(i - 1);
+        const __amdgpu_buffer_rsrc_t out_row = out_row_of(i);
+        uint32_t pk[TN / 2][4];
 #pragma unroll
         for (int u = 0; u < TN / 2; ++u) {  // pair of fragments 2u, 2u+1: 8 consecutive columns
           float v[8];
@@ -665,17 +691,23 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
                 v4u{__float_as_uint(v[4]), __float_as_uint(v[5]), __float_as_uint(v[6]),
                     __float_as_uint(v[7])},
                 out_row, (int)(out_off[u] + 16u), 0, 0);
-          } else if constexpr (OUT == CDIT_DT_F16) {
-            __builtin_amdgcn_raw_buffer_store_b128(
-                v4u{pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3]), pack_f16x2(v[4], v[5]),
-                    pack_f16x2(v[6], v[7])},
-                out_row, (int)out_off[u], 0, 0);
           } else {
-            __builtin_amdgcn_raw_buffer_store_b128(
-                v4u{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]),
-                    pack_bf16x2(v[6], v[7])},
-                out_row, (int)out_off[u], 0, 0);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              if constexpr (OUT == CDIT_DT_F16) {
+                pk[u][k] = pack_f16x2(v[2 * k], v[2 * k + 1]);
+              } else {
+                pk[u][k] = pack_bf16x2(v[2 * k], v[2 * k + 1]);
+              }
+            }
           }
+        }
+        if constexpr (PERMUTE) {
+#pragma unroll
+          for (int u = 0; u < TN / 2; ++u)
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+              moved[u][k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_addr, (int)pk[u][k]);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -685,6 +717,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     } else {
       epilogue(std::false_type{});
     }
+    if constexpr (PERMUTE) store_moved(TM - 1);
     if (next_tile >= ntiles) break;
     m0 = nm0;
     n0 = nn0;

@@ -46,6 +46,9 @@ def _hipcc():
   return None
 
 
+labeled = {}  # the same kernels with their branch labels kept (for control-flow checks)
+
+
 @pytest.fixture(scope="module", params=sorted(SOURCES))
 def wide_kernels(request, tmp_path_factory):
   hipcc = _hipcc()
@@ -60,9 +63,13 @@ def wide_kernels(request, tmp_path_factory):
   assert r.returncode == 0, r.stderr[-2000:]
   text = out.read_text()
   kernels = {}
+  labeled.clear()
   for m in re.finditer(r"^(_ZN\S*" + kernel + r"\S*):[^\n]*\n(.*?)s_endpgm", text, re.S | re.M):
     body = [l.strip() for l in m.group(2).split("\n")]
     kernels[m.group(1)] = [l for l in body if l and not l.startswith(";") and not l.startswith(".")]
+    labeled[m.group(1)] = [l.split(";")[0].strip() for l in body
+                           if l and not l.startswith(";") and
+                           (not l.startswith(".") or re.match(r"\.\w+:", l))]
   assert len(kernels) >= 3, "wide kernel instances not found in the assembly"
   return kernels
 
@@ -144,26 +151,31 @@ def test_inline_asm_mfma_hazards(wide_kernels):
 
 
 def test_output_stores_are_unconditional(wide_kernels):
+  """Rule 6. The epilogue exists twice (with and without GELU, chosen by a scalar
+  branch); for 16-bit outputs the stores of the last row of blocks follow the join."""
   counted = 0
   for name, code in wide_kernels.items():
     m = re.search(r"gemm_fp8_wideINS0_7CfgWideILi(\d+)ELi(\d+)ELi\d+ELi\d+EEELi(\d)E", name)
     if not m:
       continue
     bm, bn, out = int(m.group(1)), int(m.group(2)), int(m.group(3))
-    expect = (bm // 32) * (bn // 32) // 2 * (2 if out == 2 else 1)
+    per_row = bn // 64 * (2 if out == 2 else 1)
+    expect = bm // 32 * per_row
+    shared = 0 if out == 2 else per_row
     assert not any(l.startswith("global_store") for l in code), name
-    # basic blocks end at branches and at labels
-    blocks, cur = [], 0
-    for l in code:
-      if l.startswith("buffer_store_dwordx4"):
-        cur += 1
-      if l.startswith(("s_cbranch", "s_branch")) or re.match(r"\.?\w+:", l):
-        if cur:
-          blocks.append(cur)
-        cur = 0
-    if cur:
-      blocks.append(cur)
-    assert blocks == [expect, expect], f"{name}: stores per basic block {blocks}, expected {expect} twice"
+    code = labeled[name]
+    stores = [i for i, l in enumerate(code) if l.startswith("buffer_store_dwordx4")]
+    assert len(stores) == 2 * (expect - shared) + shared, \
+        f"{name}: {len(stores)} output stores, expected 2 * {expect - shared} + {shared}"
+    # no store under a lane mask (a store that may be skipped) or in a loop over the
+    # values of a descriptor: none lies between an exec-conditional branch and its target
+    label_at = {m.group(1): i for i, l in enumerate(code) for m in [re.match(r"(\.\w+):", l)] if m}
+    for i, l in enumerate(code):
+      if l.startswith(("s_cbranch_execz", "s_cbranch_execnz")):
+        lo, hi = sorted((i, label_at[l.split()[-1]]))
+        if any(c.startswith("v_mfma") for c in code[lo:hi]):
+          continue  # the loop over the tiles
+        assert not any(lo <= k <= hi for k in stores), f"{name}: output store under {l!r}"
     counted += 1
   if any("gemm_fp8_wide" in n for n in wide_kernels):
     assert counted >= 3
