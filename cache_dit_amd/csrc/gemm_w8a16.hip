@@ -567,16 +567,42 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
     // Accumulators are read with inline assembly, one block at a time (left to itself
     // the compiler copies all of them to VGPRs first and spills what else is live);
     // the GELU decision is taken once per tile, not once per element.
+    // Stores: the memory pipeline merges the lanes of a store into one request only
+    // when adjacent lanes write adjacent bytes; with lane = 32 h + r32 holding 32 bytes
+    // of row r32 every lane is a request of its own, which costs four times the issue
+    // time. So the packed words of a block are rearranged first: v_permlane16_swap
+    // leaves lane r32 < 16 with the first 16 bytes of rows r32 and r32 + 16 and lane
+    // r32 + 16 with their second 16 bytes, then ds_bpermute_b32 (the LDS crossbar, no
+    // LDS memory) hands lane L the piece L & 3 of row L >> 2: two stores of 16 rows x
+    // 64 contiguous bytes, lanes 4r .. 4r+3 on row r. They are issued while the next
+    // block is computed, the last block's after the two copies of the epilogue join.
+    const int bp_addr = 4 * (16 * (lane & 3) + (lane >> 2));
+    const int st_n = n0 + wn * C::WN + 8 * (lane & 3);
+    const int st_m = m0 + wm * C::WM + (lane >> 2);
+    uint32_t moved[8];
+    auto store_moved = [&](int i, int j) {
+      const int m = st_m + 32 * i, n = st_n + 32 * j;
+      if (n < g.N) {
+        uint16_t* dst = g.out + (int64_t)m * g.ldo + n;
+        if (m < g.M) *reinterpret_cast<uint4*>(dst) = uint4{moved[0], moved[1], moved[2], moved[3]};
+        if (m + 16 < g.M)
+          *reinterpret_cast<uint4*>(dst + (int64_t)16 * g.ldo) =
+              uint4{moved[4], moved[5], moved[6], moved[7]};
+      }
+    };
     auto epilogue = [&](auto gelu_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        const int n = nw + 32 * j;
         const uint32_t bw[8] = {bi[j][0].x, bi[j][0].y, bi[j][0].z, bi[j][0].w,
                                 bi[j][1].x, bi[j][1].y, bi[j][1].z, bi[j][1].w};
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-          const int m = mw + 32 * i;
+          if (i > 0) {
+            store_moved(i - 1, j);
+          } else if (j > 0) {
+            store_moved(TM - 1, j - 1);
+          }
           uint32_t pk[8];
 #pragma unroll
           for (int r = 0; r < 16; r += 2) {
@@ -593,10 +619,11 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
             }
             pk[r >> 1] = pack_bf16x2(v0, v1);
           }
-          if (m < g.M && n < g.N) {
-            uint16_t* dst = g.out + (int64_t)m * g.ldo + n;
-            *reinterpret_cast<uint4*>(dst) = uint4{pk[0], pk[1], pk[2], pk[3]};
-            *reinterpret_cast<uint4*>(dst + 8) = uint4{pk[4], pk[5], pk[6], pk[7]};
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const auto sw = __builtin_amdgcn_permlane16_swap(pk[k], pk[4 + k], false, false);
+            moved[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_addr, (int)sw[0]);
+            moved[4 + k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_addr, (int)sw[1]);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -607,6 +634,7 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
     } else {
       epilogue(std::false_type{});
     }
+    store_moved(TM - 1, TN - 1);
     if (next_tile >= ntiles) break;
     m0 = nm0;
     n0 = nn0;
