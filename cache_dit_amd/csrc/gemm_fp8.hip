@@ -662,7 +662,6 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
       constexpr bool GELU = decltype(gelu_tag)::value;
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
-        if (PERMUTE && i > 0) store_moved(i - 1);
         const __amdgpu_buffer_rsrc_t out_row = out_row_of(i);
         uint32_t pk[TN / 2][4];
 #pragma unroll
@@ -703,6 +702,9 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
           }
         }
         if constexpr (PERMUTE) {
+          // the previous row's words have had this row's arithmetic to arrive
+          __builtin_amdgcn_sched_barrier(0);
+          if (i > 0) store_moved(i - 1);
 #pragma unroll
           for (int u = 0; u < TN / 2; ++u)
 #pragma unroll

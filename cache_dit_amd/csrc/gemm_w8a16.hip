@@ -598,11 +598,6 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
                                 bi[j][1].x, bi[j][1].y, bi[j][1].z, bi[j][1].w};
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-          if (i > 0) {
-            store_moved(i - 1, j);
-          } else if (j > 0) {
-            store_moved(TM - 1, j - 1);
-          }
           uint32_t pk[8];
 #pragma unroll
           for (int r = 0; r < 16; r += 2) {
@@ -618,6 +613,13 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
               v1 = gelu_tanh(v1);
             }
             pk[r >> 1] = pack_bf16x2(v0, v1);
+          }
+          // the previous block's words have had this block's arithmetic to arrive
+          __builtin_amdgcn_sched_barrier(0);
+          if (i > 0) {
+            store_moved(i - 1, j);
+          } else if (j > 0) {
+            store_moved(TM - 1, j - 1);
           }
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
