@@ -577,18 +577,28 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
     // 64 contiguous bytes, lanes 4r .. 4r+3 on row r. They are issued while the next
     // block is computed, the last block's after the two copies of the epilogue join.
     const int bp_addr = 4 * (16 * (lane & 3) + (lane >> 2));
-    const int st_n = n0 + wn * C::WN + 8 * (lane & 3);
-    const int st_m = m0 + wm * C::WM + (lane >> 2);
+    // Buffer stores: the descriptor of a block covers the rows of it that exist (the
+    // hardware drops lanes beyond), lanes whose columns do not exist get an offset
+    // beyond any descriptor -- no bounds branches, no 64-bit address arithmetic per store.
+    constexpr uint32_t kNoColumn = 0x80000000u;
+    uint8_t* const out_wave = reinterpret_cast<uint8_t*>(g.out) +
+                              ((int64_t)(m0 + wm * C::WM) * g.ldo + (n0 + wn * C::WN)) * 2;
+    const int rows_wave = g.M - (m0 + wm * C::WM);
+    const uint32_t out_lane = ((uint32_t)(lane >> 2) * (uint32_t)g.ldo + 8u * (lane & 3)) * 2;
+    const uint32_t half_block = 16u * (uint32_t)g.ldo * 2;
+    uint32_t out_off[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      out_off[j] = n0 + wn * C::WN + 32 * j + 8 * (lane & 3) < g.N ? out_lane + 64 * j : kNoColumn;
     uint32_t moved[8];
     auto store_moved = [&](int i, int j) {
-      const int m = st_m + 32 * i, n = st_n + 32 * j;
-      if (n < g.N) {
-        uint16_t* dst = g.out + (int64_t)m * g.ldo + n;
-        if (m < g.M) *reinterpret_cast<uint4*>(dst) = uint4{moved[0], moved[1], moved[2], moved[3]};
-        if (m + 16 < g.M)
-          *reinterpret_cast<uint4*>(dst + (int64_t)16 * g.ldo) =
-              uint4{moved[4], moved[5], moved[6], moved[7]};
-      }
+      const int rows = __builtin_amdgcn_readfirstlane(min(max(rows_wave - 32 * i, 0), 32));
+      const __amdgpu_buffer_rsrc_t block = __builtin_amdgcn_make_buffer_rsrc(
+          out_wave + (int64_t)(32 * i) * g.ldo * 2, 0, rows * g.ldo * 2, 0x00020000);
+      __builtin_amdgcn_raw_buffer_store_b128(v4u{moved[0], moved[1], moved[2], moved[3]}, block,
+                                             (int)out_off[j], 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(v4u{moved[4], moved[5], moved[6], moved[7]}, block,
+                                             (int)(out_off[j] + half_block), 0, 0);
     };
     auto epilogue = [&](auto gelu_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
@@ -784,7 +794,8 @@ bool tiled_ok(const GemmArgs& g) {
          // the epilogues load scales as float4 and bias as 8-byte packs
          reinterpret_cast<uintptr_t>(g.b_scale) % 16 == 0 &&
          reinterpret_cast<uintptr_t>(g.bias) % 16 == 0 &&
-         (int64_t)1024 * g.lda < (int64_t)1 << 31 && (int64_t)512 * g.ldb < (int64_t)1 << 31;
+         (int64_t)1024 * g.lda < (int64_t)1 << 31 && (int64_t)512 * g.ldb < (int64_t)1 << 31 &&
+         (int64_t)512 * g.ldo < (int64_t)1 << 29;  // 32-bit byte offsets within a block of rows
 }
 
 }  // namespace
