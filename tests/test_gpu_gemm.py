@@ -457,3 +457,20 @@ def test_nothing_is_written_outside_the_output(variant, dt):
     ref = to.scaled_mm_rowwise(a.cpu(), s_a.cpu().reshape(-1, 1), w.cpu(), s_w.cpu().reshape(-1, 1),
                                None if b is None else b.cpu(), out_dtype=dt)
     assert torch.equal(plain.cpu(), ref), (M, N, K)
+
+
+def test_very_large_output_stride_takes_a_kernel_with_64_bit_offsets():
+  """The wide kernels address a block of output rows with 32-bit byte offsets and are only
+  chosen when 512 * ldo fits; a window of a very wide buffer must still come out right."""
+  from cache_dit_amd import ops
+  g = torch.Generator().manual_seed(9)
+  M, N, K, ldo = 5, 272, 640, 1_100_000
+  a = torch.randint(-4, 5, (M, K), generator=g).float().to(FP8).cuda()
+  w = torch.randint(-4, 5, (N, K), generator=g).float().to(FP8).cuda()
+  s_a = torch.full((M,), 0.5, device="cuda")
+  s_w = torch.full((N,), 0.25, device="cuda")
+  buf = torch.full((M, ldo), -7.0, dtype=torch.bfloat16, device="cuda")
+  ops.gemm_rowwise_into(a, s_a, w, s_w, None, buf[:, :N], 0)
+  ref = to.scaled_mm_rowwise(a.cpu(), s_a.cpu().reshape(-1, 1), w.cpu(), s_w.cpu().reshape(-1, 1))
+  assert torch.equal(buf[:, :N].cpu(), ref)
+  assert bool((buf[:, N:] == -7.0).all())

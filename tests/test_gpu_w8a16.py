@@ -193,3 +193,21 @@ def test_nothing_is_written_outside_the_output(variant):
     assert bool((buf[M:] == -7.0).all()) and bool((buf[:, N:] == -7.0).all()), (M, N, K)
     ref = to.w8a16_linear(x.cpu(), w.cpu(), sw.cpu().reshape(-1, 1), b.cpu(), fused=True)
     assert torch.equal(plain.cpu(), ref), (M, N, K)
+
+
+def test_very_large_output_stride_takes_a_kernel_with_64_bit_offsets():
+  from cache_dit_amd import ops
+  g = torch.Generator().manual_seed(9)
+  M, N, K, ldo = 5, 272, 640, 1_100_000
+  x = torch.randint(-3, 4, (M, K), generator=g).to(torch.bfloat16).cuda()
+  w = torch.randint(-3, 4, (N, K), generator=g).float().to(FP8).cuda()
+  sw = torch.full((N,), 0.25, device="cuda")
+  buf = torch.full((M, ldo), -7.0, dtype=torch.bfloat16, device="cuda")
+  for variant in (-1, 7, 12):
+    from cache_dit_amd import _native
+    _native.set_gemm_variant(variant)
+    buf.fill_(-7.0)
+    ops.w8a16_into(x, w, sw, None, buf[:, :N], 0)
+    ref = to.w8a16_linear(x.cpu(), w.cpu(), sw.cpu().reshape(-1, 1), None, fused=True)
+    assert torch.equal(buf[:, :N].cpu(), ref)
+    assert bool((buf[:, N:] == -7.0).all())
