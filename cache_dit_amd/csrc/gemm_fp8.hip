@@ -413,10 +413,17 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
   const uint8_t* B;
   uint32_t off[C::ND];
   int nrec = 0x7fffffff;  // 0: the stream has run past the last tile, fetch nothing
+  // The lane offsets only depend on the tile through the clamps at the last rows of A
+  // and B: between two tiles without partial panels they are not recomputed (some 130
+  // VALU instructions in the middle of the MFMA stream otherwise).
+  bool off_clamped = true;  // the first call computes them
   auto set_source = [&](int sm0, int sn0) {
     A = static_cast<const uint8_t*>(g.a) + (int64_t)sm0 * g.lda;
     B = g.b + (int64_t)sn0 * g.ldb;
     const int rows_a = g.M - sm0, rows_b = g.N - sn0;
+    const bool clamped = rows_a < C::BM || rows_b < C::BN;
+    if (!clamped && !off_clamped) return;
+    off_clamped = clamped;
     // recomputed from the lane id at every call: opaque to the optimizer, which
     // would otherwise keep all the row indices in registers across the K loop
     int lrow = lane >> 3;
@@ -529,18 +536,24 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
         }
       }
       if (kt == KT - 2) {
+        // buffer loads: what lies beyond N (M) reads as zero, no bounds branches; a null
+        // bias becomes an empty buffer
+        const __amdgpu_buffer_rsrc_t bs_buf = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(g.b_scale), 0, g.N * 4, 0x00020000);
+        const __amdgpu_buffer_rsrc_t bi_buf = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint16_t*>(g.bias), 0, g.bias ? g.N * 2 : 0, 0x00020000);
+        const __amdgpu_buffer_rsrc_t as_buf = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(g.a_scale), 0, g.M * 4, 0x00020000);
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
           const int n = nw + 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
-          bs[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-          bi[j] = uint2{0u, 0u};
-          if (n < g.N) {
-            bs[j] = *reinterpret_cast<const v4f*>(g.b_scale + n);
-            if (g.bias) bi[j] = *reinterpret_cast<const uint2*>(g.bias + n);
-          }
+          bs[j] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(bs_buf, n * 4, 0, 0));
+          bi[j] = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(bi_buf, n * 2, 0, 0));
         }
 #pragma unroll
-        for (int i = 0; i < TM; ++i) as[i] = mw + 16 * i < g.M ? g.a_scale[mw + 16 * i] : 0.0f;
+        for (int i = 0; i < TM; ++i)
+          as[i] = __builtin_bit_cast(
+              float, __builtin_amdgcn_raw_buffer_load_b32(as_buf, (mw + 16 * i) * 4, 0, 0));
       }
       const int kd = kt + D < KT ? kt + D : kt + D - KT;  // step (of its tile) to fetch
       const uint8_t* st = smem + a_cur;
