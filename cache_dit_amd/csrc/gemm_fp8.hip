@@ -303,7 +303,13 @@ struct CfgWide {
   // second half, into the stage just read)
   static constexpr int A_STAGES = DEPTH + 1, B_STAGES = DEPTH;
   static constexpr int B_BASE = A_STAGES * A_BYTES;
-  static constexpr int LDS_BYTES = A_STAGES * A_BYTES + B_STAGES * B_BYTES;
+  static constexpr int PANEL_BYTES = A_STAGES * A_BYTES + B_STAGES * B_BYTES;
+  // Epilogue operands of a tile (b_scale and bias of its BN columns, a_scale of its BM
+  // rows) are staged after the panels when 4 KiB are left: LDS-DMA instructions of
+  // 1 KiB each, b_scale | a_scale (two) | bias.
+  static constexpr bool STAGE_EPI = PANEL_BYTES + 4096 <= 160 * 1024 && BN * 4 <= 1024 && BM * 4 <= 2048;
+  static constexpr int EPI_BS = PANEL_BYTES, EPI_AS = PANEL_BYTES + 1024, EPI_BI = PANEL_BYTES + 3072;
+  static constexpr int LDS_BYTES = PANEL_BYTES + (STAGE_EPI ? 4096 : 0);
   // DMA instructions (1 KiB = 8 panel rows) per wave and step
   static constexpr int NDA = BM / 8 / WAVES, NDB = BN / 8 / WAVES, ND = NDA + NDB;
   static_assert(WM % 16 == 0 && WN % 32 == 0, "wave tile: 16-row A fragments, B fragments in pairs");
@@ -536,24 +542,41 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
         }
       }
       if (kt == KT - 2) {
-        // buffer loads: what lies beyond N (M) reads as zero, no bounds branches; a null
-        // bias becomes an empty buffer
+        // buffer accesses: what lies beyond N (M) reads as zero, no bounds branches; a
+        // null bias becomes an empty buffer
         const __amdgpu_buffer_rsrc_t bs_buf = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<float*>(g.b_scale), 0, g.N * 4, 0x00020000);
         const __amdgpu_buffer_rsrc_t bi_buf = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<uint16_t*>(g.bias), 0, g.bias ? g.N * 2 : 0, 0x00020000);
         const __amdgpu_buffer_rsrc_t as_buf = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<float*>(g.a_scale), 0, g.M * 4, 0x00020000);
+        if constexpr (C::STAGE_EPI) {
+          // Four LDS-DMA instructions (every wave issues all four: the same bytes land
+          // four times, and the waves' instruction counts stay equal) instead of TM +
+          // 2 TN loads per lane, whose issue alone held the MFMAs up for 700 cycles.
+          // They are older than this step's panel DMA, so the waits of the next two
+          // steps cover them.
+          auto stage = [&](__amdgpu_buffer_rsrc_t buf, int byte0, int lds) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                buf, (__attribute__((address_space(3))) void*)(smem + lds), 16, byte0 + 16 * lane, 0,
+                0, 0);
+          };
+          stage(bs_buf, n0 * 4, C::EPI_BS);
+          stage(as_buf, m0 * 4, C::EPI_AS);
+          stage(as_buf, m0 * 4 + 1024, C::EPI_AS + 1024);
+          stage(bi_buf, n0 * 2, C::EPI_BI);
+        } else {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          const int n = nw + 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
-          bs[j] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(bs_buf, n * 4, 0, 0));
-          bi[j] = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(bi_buf, n * 2, 0, 0));
+          for (int j = 0; j < TN; ++j) {
+            const int n = nw + 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
+            bs[j] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(bs_buf, n * 4, 0, 0));
+            bi[j] = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(bi_buf, n * 2, 0, 0));
+          }
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            as[i] = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(as_buf, (mw + 16 * i) * 4, 0, 0));
         }
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-          as[i] = __builtin_bit_cast(
-              float, __builtin_amdgcn_raw_buffer_load_b32(as_buf, (mw + 16 * i) * 4, 0, 0));
       }
       const int kd = kt + D < KT ? kt + D : kt + D - KT;  // step (of its tile) to fetch
       const uint8_t* st = smem + a_cur;
@@ -631,6 +654,24 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     // covers the rows of it that exist (the hardware drops lanes beyond), lanes whose
     // columns do not exist get an offset beyond any descriptor. Per lane a 32-bit
     // byte offset (the launcher bounds 512 * ldo), per row of blocks a scalar base.
+    if constexpr (C::STAGE_EPI) {
+      // staged two steps ago; landed before the barrier of the last step. (The
+      // compiler still puts a wait for all DMA in front of some of these reads: it
+      // cannot tell them from the panels in flight. Measured: no cost, the next tile's
+      // first steps are in the LDS by then.)
+      auto read_staged = [&](const uint8_t* __restrict__ ep) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int c = wn * C::WN + 8 * kg + 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
+          bs[j] = *reinterpret_cast<const v4f*>(ep + C::EPI_BS + c * 4);
+          bi[j] = *reinterpret_cast<const uint2*>(ep + C::EPI_BI + c * 2);
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          as[i] = *reinterpret_cast<const float*>(ep + C::EPI_AS + (wm * C::WM + r16 + 16 * i) * 4);
+      };
+      read_staged(smem);
+    }
     constexpr int OB = OUT == CDIT_DT_F32 ? 4 : 2;  // bytes per output element
     constexpr uint32_t kNoColumn = 0x80000000u;
     uint8_t* const out_wave = reinterpret_cast<uint8_t*>(g.out) +
