@@ -371,7 +371,7 @@ def main():
       "frac": head["gemm_tflops"] / FP8_PEAK_TFLOPS,
       # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain
       # copy of known size (profiles/pmc_traffic_headline_kernels.md); algorithmic 165.2 MB
-      "traffic": 415.7e6,
+      "traffic": 378.0e6,
   }
   roofline_quant = {
       "kernel": "quant_rowwise_regs at M=4608 K=3072",

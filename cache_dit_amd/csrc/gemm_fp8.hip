@@ -1061,9 +1061,9 @@ typedef Cfg<128, 128, 2, 2, true, true, 8> V6;        // two workgroups per CU
 typedef Cfg<256, 256, 2, 4, true, true, 8> V7;        // 8 waves in phase, 2 stages
 typedef Cfg<128, 64, 2, 2, true, true, 8, 4> V20;     // small tiles, 4 stages of 128 B
 typedef Cfg<64, 128, 2, 2, true, true, 8, 4> V21;
-typedef CfgWide<256, 256, 8> V12;                     // 4 waves, 128x128 wave tiles, 16x16x128 MFMA
-typedef CfgWide<288, 192, 8> V14;                     // ... 144x96 wave tiles
-typedef CfgWide<256, 192, 8> V15;                     // ... 128x96 wave tiles
+typedef CfgWide<256, 256, 4> V12;                     // 4 waves, 128x128 wave tiles, 16x16x128 MFMA
+typedef CfgWide<288, 192, 4> V14;                     // ... 144x96 wave tiles
+typedef CfgWide<256, 192, 4> V15;                     // ... 128x96 wave tiles
 typedef CfgWide<128, 192, 4, 3> V16;                  // ... 64x96 wave tiles, DMA 3 steps ahead
 typedef CfgWide<64, 128, 8, 5> V17;                   // ... 32x64 wave tiles, DMA 5 steps ahead
 typedef CfgWide<128, 128, 4, 4> V18;                  // ... 64x64 wave tiles, DMA 4 steps ahead

@@ -802,9 +802,9 @@ bool tiled_ok(const GemmArgs& g) {
 
 typedef CfgW<256, 256, 2, 2, true, 8> W0;   // 4 waves, 2 stages
 typedef CfgW<128, 128, 2, 2, true, 8> W3;   // small tiles, two workgroups per CU
-typedef CfgWW<256, 256, 8> W7;              // wide: 4 waves, 128x128 wave tiles
-typedef CfgWW<256, 192, 8> W8;              // wide: 128x96 wave tiles
-typedef CfgWW<192, 256, 8> W9;              // wide: 96x128 wave tiles
+typedef CfgWW<256, 256, 4> W7;              // wide: 4 waves, 128x128 wave tiles
+typedef CfgWW<256, 192, 4> W8;              // wide: 128x96 wave tiles
+typedef CfgWW<192, 256, 4> W9;              // wide: 96x128 wave tiles
 typedef CfgWW<128, 192, 4, 4> W10;          // wide: 64x96 wave tiles, DMA 4 steps ahead
 typedef CfgWW<128, 128, 4, 5> W11;          // wide: 64x64 wave tiles, DMA 5 steps ahead
 typedef CfgWW<128, 64, 4, 6> W12;           // wide: 64x32 wave tiles, DMA 6 steps ahead
