@@ -674,6 +674,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     }
     constexpr int OB = OUT == CDIT_DT_F32 ? 4 : 2;  // bytes per output element
     constexpr uint32_t kNoColumn = 0x80000000u;
+    constexpr int kStoreOnce = 2;  // cache policy of the output stores: non-temporal (written once)
     uint8_t* const out_wave = reinterpret_cast<uint8_t*>(g.out) +
                               ((int64_t)(m0 + wm * C::WM) * g.ldo + (n0 + wn * C::WN)) * OB;
     const int rows_wave = g.M - (m0 + wm * C::WM);  // rows of the wave tile that exist
@@ -710,7 +711,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
 #pragma unroll
       for (int u = 0; u < TN / 2; ++u)
         __builtin_amdgcn_raw_buffer_store_b128(
-            v4u{moved[u][0], moved[u][1], moved[u][2], moved[u][3]}, row, (int)out_off[u], 0, 0);
+            v4u{moved[u][0], moved[u][1], moved[u][2], moved[u][3]}, row, (int)out_off[u], 0, kStoreOnce);
     };
     auto epilogue = [&](auto gelu_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
@@ -739,11 +740,11 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
             __builtin_amdgcn_raw_buffer_store_b128(
                 v4u{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]),
                     __float_as_uint(v[3])},
-                out_row, (int)out_off[u], 0, 0);
+                out_row, (int)out_off[u], 0, kStoreOnce);
             __builtin_amdgcn_raw_buffer_store_b128(
                 v4u{__float_as_uint(v[4]), __float_as_uint(v[5]), __float_as_uint(v[6]),
                     __float_as_uint(v[7])},
-                out_row, (int)(out_off[u] + 16u), 0, 0);
+                out_row, (int)(out_off[u] + 16u), 0, kStoreOnce);
           } else {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {

@@ -596,9 +596,9 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
       const __amdgpu_buffer_rsrc_t block = __builtin_amdgcn_make_buffer_rsrc(
           out_wave + (int64_t)(32 * i) * g.ldo * 2, 0, rows * g.ldo * 2, 0x00020000);
       __builtin_amdgcn_raw_buffer_store_b128(v4u{moved[0], moved[1], moved[2], moved[3]}, block,
-                                             (int)out_off[j], 0, 0);
+                                             (int)out_off[j], 0, 2);
       __builtin_amdgcn_raw_buffer_store_b128(v4u{moved[4], moved[5], moved[6], moved[7]}, block,
-                                             (int)(out_off[j] + half_block), 0, 0);
+                                             (int)(out_off[j] + half_block), 0, 2);
     };
     auto epilogue = [&](auto gelu_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
