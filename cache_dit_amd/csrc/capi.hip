@@ -130,8 +130,8 @@ int cdit_device_arch(char* buf, int buf_len) {
 }
 
 int cdit_set_gemm_variant(int variant) {
-  if (variant >= 1000) {  // 1000 + v selects the quantizer kernel variant instead
-    cdit::g_quant_variant = variant - 1000;
+  if (variant >= 1000) {  // 1000 + v: cache hints of the quantizer instead, 1999: automatic
+    cdit::g_quant_variant = variant == 1999 ? -1 : variant - 1000;
     return g_gemm_variant;
   }
   int prev = g_gemm_variant;
@@ -139,9 +139,11 @@ int cdit_set_gemm_variant(int variant) {
   return prev;
 }
 
-int cdit_fp8_quant_rowwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_x, void* q_e4m3,
-                           int64_t ld_q, float* scale, int scale_mode, void* stream) {
-  const char* fn = "cdit_fp8_quant_rowwise";
+// consumer_follows: the codes are read by a GEMM launched right behind (the fused
+// Linear entry point): the quantizer then keeps its loads and stores cacheable.
+static int quant_rowwise_impl(const char* fn, const void* x_bf16, int64_t M, int64_t K,
+                             int64_t ld_x, void* q_e4m3, int64_t ld_q, float* scale,
+                             int scale_mode, void* stream, bool consumer_follows) {
   if (M < 0 || K < 0 || M > INT32_MAX || K > INT32_MAX) {
     set_error("%s: bad shape M=%lld K=%lld", fn, (long long)M, (long long)K);
     return CDIT_EINVAL;
@@ -163,8 +165,14 @@ int cdit_fp8_quant_rowwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_
   int rc = check_arch();
   if (rc) return rc;
   rc = launch_quant_rowwise(x_bf16, M, K, ld_x, q_e4m3, ld_q, scale, scale_mode,
-                            static_cast<hipStream_t>(stream));
+                            consumer_follows, static_cast<hipStream_t>(stream));
   return rc ? rc : after_launch(fn);
+}
+
+int cdit_fp8_quant_rowwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_x, void* q_e4m3,
+                           int64_t ld_q, float* scale, int scale_mode, void* stream) {
+  return quant_rowwise_impl("cdit_fp8_quant_rowwise", x_bf16, M, K, ld_x, q_e4m3, ld_q, scale,
+                           scale_mode, stream, false);
 }
 
 int cdit_fp8_quant_tensorwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_x,
@@ -266,7 +274,8 @@ int cdit_fp8_linear_w8a8(const void* x_bf16, const void* w_q, const float* w_sca
                                        static_cast<hipStream_t>(stream)) == 0)
       return after_launch("cdit_fp8_linear_w8a8");
   }
-  int rc = cdit_fp8_quant_rowwise(x_bf16, M, K, ld_x, q_ws, K, scale_ws, scale_mode, stream);
+  int rc = quant_rowwise_impl("cdit_fp8_linear_w8a8", x_bf16, M, K, ld_x, q_ws, K, scale_ws,
+                              scale_mode, stream, true);
   if (rc) return rc;
   return cdit_fp8_gemm_rowwise(q_ws, scale_ws, w_q, w_scale, bias, out, M, N, K, K, ldw, ldo,
                                epilogue, out_dtype_id, stream);

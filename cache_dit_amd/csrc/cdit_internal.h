@@ -12,7 +12,8 @@ namespace cdit {
 // Each launcher validates nothing: capi.hip checks shapes, strides, alignment
 // and the device before calling. They return 0 or a CDIT_E* code.
 int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void* q,
-                         int64_t ld_q, float* scale, int scale_mode, hipStream_t stream);
+                         int64_t ld_q, float* scale, int scale_mode, bool consumer_follows,
+                         hipStream_t stream);
 
 int launch_quant_tensorwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void* q,
                             int64_t ld_q, float* scale, uint32_t* amax_ws, int scale_mode,

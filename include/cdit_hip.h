@@ -180,6 +180,8 @@ int cdit_fp8_linear_w8a8(const void* x_bf16, const void* w_q, const float* w_sca
  * Tuning hook used by the benchmark and the tests: forces the kernel variant
  * the two GEMM entry points pick (-1 = automatic choice by shape). Returns
  * the previous value. Process-global; not meant for concurrent use.
+ * Values 1000..1003 set the cache hints of the per-row quantizer instead (0: loads and
+ * stores non-temporal, 1: neither, 2: loads, 3: stores), 1999 its automatic choice by size.
  */
 int cdit_set_gemm_variant(int variant);
 
