@@ -1043,10 +1043,11 @@ bool tiled_ok(const GemmArgs& g) {
   return g.K >= BK && g.K % BK == 0 && g.N % 8 == 0 && g.lda % 16 == 0 && g.ldb % 16 == 0 && g.ldo % 8 == 0 &&
          reinterpret_cast<uintptr_t>(g.a) % 16 == 0 && reinterpret_cast<uintptr_t>(g.b) % 16 == 0 &&
          reinterpret_cast<uintptr_t>(g.out) % 16 == 0 &&
-         // 32-bit in-tile byte offsets
-         // the epilogues load scales as float4 and bias as 8-byte packs
+         // the epilogues fetch scales and bias in 16-byte pieces
+         reinterpret_cast<uintptr_t>(g.a_scale) % 16 == 0 &&
          reinterpret_cast<uintptr_t>(g.b_scale) % 16 == 0 &&
          reinterpret_cast<uintptr_t>(g.bias) % 16 == 0 &&
+         // 32-bit byte offsets inside a tile
          (int64_t)512 * g.lda < (int64_t)1 << 31 && (int64_t)512 * g.ldb < (int64_t)1 << 31 &&
          (int64_t)512 * g.ldo < (int64_t)1 << 29;
 }

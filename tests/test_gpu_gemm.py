@@ -474,3 +474,25 @@ def test_very_large_output_stride_takes_a_kernel_with_64_bit_offsets():
   ref = to.scaled_mm_rowwise(a.cpu(), s_a.cpu().reshape(-1, 1), w.cpu(), s_w.cpu().reshape(-1, 1))
   assert torch.equal(buf[:, :N].cpu(), ref)
   assert bool((buf[:, N:] == -7.0).all())
+
+
+def test_scales_and_bias_at_odd_offsets():
+  """a_scale, b_scale and bias that are only 4-byte (2-byte) aligned: the kernels that fetch
+  them in 16-byte pieces must not be chosen; the result is the same."""
+  from cache_dit_amd import ops
+  g = torch.Generator().manual_seed(10)
+  M, N, K = 600, 400, 512
+  a = torch.randint(-4, 5, (M, K), generator=g).float().to(FP8).cuda()
+  w = torch.randint(-4, 5, (N, K), generator=g).float().to(FP8).cuda()
+  s_a = (torch.rand(M + 1, generator=g) + 0.5).cuda()
+  s_w = (torch.rand(N + 1, generator=g) * 0.01).cuda()
+  b = torch.randint(-8, 9, (N + 1,), generator=g).to(torch.bfloat16).cuda()
+  ref = to.scaled_mm_rowwise(a.cpu(), s_a[1:].cpu().reshape(-1, 1), w.cpu(), s_w[1:].cpu().reshape(-1, 1),
+                             b[1:].cpu())
+  out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+  ops.gemm_rowwise_into(a, s_a[1:], w, s_w[1:], b[1:], out, 0)
+  torch.cuda.synchronize()
+  _assert_close(out, ref)
+  aligned = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+  ops.gemm_rowwise_into(a, s_a[1:].clone(), w, s_w[1:].clone(), b[1:].clone(), aligned, 0)
+  assert torch.equal(out, aligned) or max_rel_err(out, aligned.cpu()) <= REL_TOL
