@@ -1101,7 +1101,10 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     return 0;
   }
   // the wide kernels stream K two or more steps ahead: shorter K runs the 128x128 kernel
-  auto wide_ok = [&](int depth) { return g.K >= 128 * depth; };
+  // at least `depth` K steps to prefetch, and at least 3: the epilogue operands of a tile are
+  // staged in LDS two steps before its end, which must be behind the first barrier of the
+  // tile (before it, slower waves may still be reading the previous tile's)
+  auto wide_ok = [&](int depth) { return g.K >= 128 * (depth > 3 ? depth : 3); };
   if (g.out_dtype != CDIT_DT_BF16) {
     // fp16 / fp32 outputs (the op's other two out_dtype ids): one large and one small
     // wide tile are built for them, chosen like the small-problem case below; what

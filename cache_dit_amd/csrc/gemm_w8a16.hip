@@ -211,7 +211,11 @@ struct CfgWW {
   static constexpr int A_BYTES = BM * A_ROW, B_BYTES = BN * B_ROW;
   static constexpr int A_STAGES = DEPTH + 1, B_STAGES = DEPTH;
   static constexpr int B_BASE = A_STAGES * A_BYTES;
-  static constexpr int LDS_BYTES = A_STAGES * A_BYTES + B_STAGES * B_BYTES;
+  static constexpr int PANEL_BYTES = A_STAGES * A_BYTES + B_STAGES * B_BYTES;
+  // b_scale and bias of a tile's BN columns are staged behind the panels (1 KiB each)
+  static constexpr int EPI_BS = PANEL_BYTES, EPI_BI = PANEL_BYTES + 1024;
+  static constexpr int LDS_BYTES = PANEL_BYTES + 2048;
+  static_assert(BN * 4 <= 1024, "one LDS-DMA instruction per staged operand");
   // DMA instructions (1 KiB: 8 A rows or 16 B rows) per wave and step
   static constexpr int NDA = BM / 8 / WAVES, NDB = BN / 16 / WAVES, ND = NDA + NDB;
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
@@ -312,10 +316,16 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
   const uint8_t* B;
   uint32_t off[C::ND];
   int nrec = 0x7fffffff;  // 0: the stream has run past the last tile, fetch nothing
+  // The lane offsets only depend on the tile through the clamps at the last rows of A
+  // and B: between two tiles without partial panels they are not recomputed.
+  bool off_clamped = true;  // the first call computes them
   auto set_source = [&](int sm0, int sn0) {
     A = static_cast<const uint8_t*>(g.a) + (int64_t)sm0 * g.lda * 2;
     B = g.b + (int64_t)sn0 * g.ldb;
     const int rows_a = g.M - sm0, rows_b = g.N - sn0;
+    const bool clamped = rows_a < C::BM || rows_b < C::BN;
+    if (!clamped && !off_clamped) return;
+    off_clamped = clamped;
     int l = lane;  // opaque: keeps the row indices out of registers across the K loop
     asm volatile("" : "+v"(l));
 #pragma unroll
@@ -427,6 +437,22 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
         } else {
           nrec = 0;
         }
+      }
+      if (kt == KT - 2) {
+        // b_scale and bias of this tile's columns go to the LDS with two DMA instructions
+        // (every wave issues both: equal instruction counts; the same bytes land four
+        // times) instead of 6 TN loads per lane at the start of the epilogue. What lies
+        // beyond N reads as zero, a null bias is an empty buffer.
+        const __amdgpu_buffer_rsrc_t bs_buf = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(g.b_scale), 0, g.N * 4, 0x00020000);
+        const __amdgpu_buffer_rsrc_t bi_buf = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint16_t*>(g.bias), 0, g.bias ? g.N * 2 : 0, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            bs_buf, (__attribute__((address_space(3))) void*)(smem + C::EPI_BS), 16,
+            n0 * 4 + 16 * lane, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            bi_buf, (__attribute__((address_space(3))) void*)(smem + C::EPI_BI), 16,
+            n0 * 2 + 16 * lane, 0, 0, 0);
       }
       const int kd = kt + D < KT ? kt + D : kt + D - KT;  // step (of its tile) to fetch
       const uint8_t* st = smem + a_cur;
@@ -542,28 +568,22 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
     //   m = m0 + wm*WM + 32i + (lane&31),  n = n0 + wn*WN + 32j + 16h + r
     const int nw = n0 + wn * C::WN + 16 * h;
     const int mw = m0 + wm * C::WM + r32;
-    // epilogue operands of all column blocks (the fragment registers are free now)
+    // epilogue operands of all column blocks (the fragment registers are free now):
+    // staged in LDS two steps ago, read after the wait below
     v4f bs[TN][4];
     uint4 bi[TN][2];
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = nw + 32 * j;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) bs[j][q] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-      bi[j][0] = bi[j][1] = uint4{0u, 0u, 0u, 0u};
-      if (n < g.N) {  // N % 16 == 0 on this path: 16 columns are all in or all out
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          bs[j][q] = *reinterpret_cast<const v4f*>(g.b_scale + n + 4 * q);
-        if (g.bias) {
-          bi[j][0] = *reinterpret_cast<const uint4*>(g.bias + n);
-          bi[j][1] = *reinterpret_cast<const uint4*>(g.bias + n + 8);
-        }
-      }
-    }
     // every DMA issued so far (the next tile's first D steps) must have landed
     // before the stores go out: step 0 of the next tile then waits for nothing
     wait_vm<0>();
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int c = wn * C::WN + 16 * h + 32 * j;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        bs[j][q] = *reinterpret_cast<const v4f*>(smem + C::EPI_BS + (c + 4 * q) * 4);
+      bi[j][0] = *reinterpret_cast<const uint4*>(smem + C::EPI_BI + c * 2);
+      bi[j][1] = *reinterpret_cast<const uint4*>(smem + C::EPI_BI + c * 2 + 16);
+    }
     // Accumulators are read with inline assembly, one block at a time (left to itself
     // the compiler copies all of them to VGPRs first and spills what else is live);
     // the GELU decision is taken once per tile, not once per element.
@@ -824,7 +844,10 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
     return 0;
   }
   // the wide kernels stream K two or more steps ahead and store 16 columns per lane
-  auto wide_ok = [&](int depth) { return g.K >= depth * BKE && g.N % 16 == 0; };
+  // at least `depth` K steps to prefetch, and at least 3: the epilogue operands of a tile are
+  // staged in LDS two steps before its end, which must be behind the first barrier of the
+  // tile (before it, slower waves may still be reading the previous tile's)
+  auto wide_ok = [&](int depth) { return g.K >= (depth > 3 ? depth : 3) * BKE && g.N % 16 == 0; };
   if (variant < 0) {
     // Same cost model as the w8a8 entry point: tile area times rounds over the 256
     // CUs, a last partial round of r tiles counting 0.4 + 0.6 r/256.
