@@ -7,6 +7,11 @@
 // registers want: v_mfma_f32_32x32x64_f8f6f4 takes, per lane, 32 consecutive
 // K bytes of one row (lane&31) in K-half (lane>>5).
 //
+// Kernels in this file: gemm_fp8_wide (persistent, one wave per SIMD, the one every
+// large or medium problem runs; described in front of CfgWide), gemm_fp8_tiled (the
+// older kernel described next, kept for very short K), gemm_fp8_skinny and
+// linear_fp8_skinny_fused (M <= 16), gemm_fp8_generic (any shape and alignment).
+//
 // Tiled kernel: a workgroup of WGM x WGN wavefronts owns a BM x BN output
 // tile and walks K in steps of BK = 128 bytes. A and B panels are staged in
 // LDS, double buffered; rows are 128 B = 8 chunks of 16 B and chunk c of row r
@@ -282,9 +287,11 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_tiled(GemmArgs g, int til
 // distinct 16-byte bank groups. The B fragments take their 16 rows in a permuted
 // order, fragment j = 4t + q, operand row p:
 //     n = 64 t + 32 (q >> 1) + 8 (p >> 2) + 4 (q & 1) + (p & 3)
-// so that a lane ends with 8 consecutive output columns per pair of fragments and
-// stores 16 bytes without a transpose (4 lanes cover 64 contiguous bytes of a row);
-// for those rows lane bit 3 is row bit 4, hence swz_b.
+// so that a lane ends with 8 consecutive output columns per pair of fragments (16
+// bytes of a 16-bit output; 4 lanes cover 64 contiguous bytes of a row); for those
+// rows lane bit 3 is row bit 4, hence swz_b. Before they are stored the packed words
+// change lanes once more (ds_bpermute_b32) so that adjacent lanes hold adjacent
+// bytes: the memory pipeline only merges those into one request (see the epilogue).
 template <int BM_, int BN_, int GROUP_M_, int DEPTH_ = 2>
 struct CfgWide {
   static constexpr int BM = BM_, BN = BN_, GROUP_M = GROUP_M_;
