@@ -24,8 +24,8 @@ things the compiler may add that the kernels must not have:
      flight, which serialises the epilogue of a tile with the next tile's K loop;
   6. (w8a8 kernel) the waits of the first K steps of a tile count the output stores
      of the previous tile's epilogue, so every wave must issue all of them whatever
-     part of the tile exists: each copy of the epilogue is one basic block with
-     TM * TN/2 buffer stores (twice that for fp32 output) and no global stores.
+     part of the tile exists: the expected number of buffer stores, no global stores,
+     none under a lane mask or inside a loop over descriptor values.
 """
 import os
 import re
