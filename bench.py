@@ -118,7 +118,7 @@ class HotPath:
       reuse = leaf in ("attn.to_k", "attn.to_v", "attn.add_k_proj", "attn.add_v_proj") or (
           name.startswith("single") and leaf == "attn.to_q")  # after proj_mlp
       if not reuse:
-        ops.quant_rowwise_into(self.x[(M, K)], self.q[(M, K)], self.s[(M, K)], 0)
+        ops.quant_rowwise_into(self.x[(M, K)], self.q[(M, K)], self.s[(M, K)], 0, gemm_follows=True)
       ops.gemm_rowwise_into(self.q[(M, K)], self.s[(M, K)], w, ws, b, out, epi)
 
 

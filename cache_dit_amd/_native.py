@@ -18,6 +18,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libcdit_hip.so")
 ABI_VERSION = 1
 
 SCALE_MODE_IDS = {"bf16div": 0, "fp32div": 1}
+QUANT_GEMM_FOLLOWS = 0x100  # cache hint, OR-ed into the scale mode of the per-row quantizer
 EPI_NONE = 0
 EPI_GELU_TANH = 1
 DT_F16, DT_BF16, DT_F32 = 0, 1, 2

@@ -144,6 +144,10 @@ int cdit_set_gemm_variant(int variant) {
 static int quant_rowwise_impl(const char* fn, const void* x_bf16, int64_t M, int64_t K,
                              int64_t ld_x, void* q_e4m3, int64_t ld_q, float* scale,
                              int scale_mode, void* stream, bool consumer_follows) {
+  if (scale_mode >= 0 && (scale_mode & CDIT_QUANT_GEMM_FOLLOWS)) {
+    consumer_follows = true;
+    scale_mode &= ~CDIT_QUANT_GEMM_FOLLOWS;
+  }
   if (M < 0 || K < 0 || M > INT32_MAX || K > INT32_MAX) {
     set_error("%s: bad shape M=%lld K=%lld", fn, (long long)M, (long long)K);
     return CDIT_EINVAL;

@@ -126,12 +126,15 @@ def quant_tensorwise_into(x2: torch.Tensor, q: torch.Tensor, scale: torch.Tensor
 
 
 def quant_rowwise_into(x2: torch.Tensor, q: torch.Tensor, scale: torch.Tensor,
-                       scale_mode_id: int) -> None:
+                       scale_mode_id: int, gemm_follows: bool = False) -> None:
+  """gemm_follows: the codes are read by a GEMM launched next on this stream (a cache
+  hint for the quantizer; the results are the same)."""
   M, K = x2.shape
+  mode = scale_mode_id | (_native.QUANT_GEMM_FOLLOWS if gemm_follows else 0)
   with _DeviceOf(x2):
     _native.check(_native.load().cdit_fp8_quant_rowwise(x2.data_ptr(), M, K, x2.stride(0),
                                                         q.data_ptr(), q.stride(0),
-                                                        scale.data_ptr(), scale_mode_id,
+                                                        scale.data_ptr(), mode,
                                                         _stream_ptr(x2)))
 
 
@@ -188,7 +191,7 @@ def shared_activation_quant(x2: torch.Tensor, scale_mode_id: int):
     M, K = x2.shape
     q = torch.empty((M, K), dtype=FP8, device=dev)
     s = torch.empty((M, ), dtype=torch.float32, device=dev)
-    quant_rowwise_into(x2, q, s, scale_mode_id)
+    quant_rowwise_into(x2, q, s, scale_mode_id, gemm_follows=True)
     quant_launches += 1
     return q, s
   key = (dev.index, torch._C._cuda_getCurrentRawStream(dev.index),
@@ -202,7 +205,7 @@ def shared_activation_quant(x2: torch.Tensor, scale_mode_id: int):
   M, K = x2.shape
   q = torch.empty((M, K), dtype=FP8, device=dev)
   s = torch.empty((M, ), dtype=torch.float32, device=dev)
-  quant_rowwise_into(x2, q, s, scale_mode_id)
+  quant_rowwise_into(x2, q, s, scale_mode_id, gemm_follows=True)
   quant_launches += 1
   if e is None:
     e = _SharedQuant()

@@ -180,3 +180,25 @@ def test_full_size_properties_wan_shape():
     assert bool((q2.view(torch.uint8) == qb).all()) and bool((s2 == s * 2.0**-7).all())
     q3, s3 = ops.fp8_rowwise_quant(-x, mode)
     assert bool((q3.view(torch.uint8) == (qb ^ 0x80)).all()) and bool((s3 == s).all())
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_gemm_follows_hint_changes_nothing(mode):
+  """CDIT_QUANT_GEMM_FOLLOWS is a cache hint: codes and scales are the same bits."""
+  from cache_dit_amd import _native, ops
+  g = torch.Generator().manual_seed(21)
+  x = (torch.randn(300, 3072, generator=g) * 2).to(torch.bfloat16).cuda()
+  m = _native.SCALE_MODE_IDS[mode]
+  q0 = torch.empty(300, 3072, dtype=torch.float8_e4m3fn, device="cuda")
+  q1 = torch.empty_like(q0)
+  s0 = torch.empty(300, dtype=torch.float32, device="cuda")
+  s1 = torch.empty_like(s0)
+  ops.quant_rowwise_into(x, q0, s0, m)
+  ops.quant_rowwise_into(x, q1, s1, m, gemm_follows=True)
+  torch.cuda.synchronize()
+  assert (bits_u8(q0) == bits_u8(q1)).all() and (bits_u32(s0) == bits_u32(s1)).all()
+  q_ref, s_ref = to.quantize_rowwise(x.cpu(), mode)
+  assert (bits_u8(q1) == bits_u8(q_ref)).all() and (bits_u32(s1) == bits_u32(s_ref.reshape(-1))).all()
+  L = _native.load()  # an unknown mode stays an error with the flag set
+  assert L.cdit_fp8_quant_rowwise(x.data_ptr(), 4, 64, 64, q0.data_ptr(), 64, s0.data_ptr(),
+                                  0x100 | 5, None) == 1
