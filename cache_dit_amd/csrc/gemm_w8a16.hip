@@ -255,6 +255,7 @@ struct CfgWW {
   }
   static_assert(first_half_reads_in_time(), "A fragment read too late for its first use");
   static constexpr int CONVERT_AHEAD = 2;
+  static constexpr bool PIN_CONVERT = TM * TN >= 12;  // see convert() in the kernel
   // Second half: S2 MFMAs in blocks of column pairs (the order of the loops below). The
   // raw weights of the next step replace those of a column pair from one slot after
   // the pair's block on (one LDS read per slot), A_0 of the next step is read in front
@@ -460,11 +461,25 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
       auto convert = [&](int j, int q) {
         const uint4& w = wr[j].t[q >> 1];
         const uint32_t lo = (q & 1) ? w.z : w.x, hi = (q & 1) ? w.w : w.y;
-        const v2bf c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
-        const v2bf c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
-        const v2bf c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
-        const v2bf c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
-        wf[j].k[q] = v8bf{c0[0], c0[1], c1[0], c1[1], c2[0], c2[1], c3[0], c3[1]};
+        if constexpr (C::PIN_CONVERT) {
+          // Inline assembly (volatile): the conversions stay in the MFMA slot they are
+          // written in. As builtins they are pure functions of loaded values, and with the
+          // large wave tiles the compiler gathered most of a step's conversions at the top
+          // of the loop, where the matrix core then waited for them (a tenth of a step;
+          // with the small wave tiles its own placement is the better one).
+          uint32_t c0, c1, c2, c3;
+          asm volatile("v_cvt_scalef32_pk_bf16_fp8 %0, %1, 1.0" : "=v"(c0) : "v"(lo));
+          asm volatile("v_cvt_scalef32_pk_bf16_fp8 %0, %1, 1.0 op_sel:[1,0,0]" : "=v"(c1) : "v"(lo));
+          asm volatile("v_cvt_scalef32_pk_bf16_fp8 %0, %1, 1.0" : "=v"(c2) : "v"(hi));
+          asm volatile("v_cvt_scalef32_pk_bf16_fp8 %0, %1, 1.0 op_sel:[1,0,0]" : "=v"(c3) : "v"(hi));
+          wf[j].k[q] = __builtin_bit_cast(v8bf, uint4{c0, c1, c2, c3});
+        } else {
+          const v2bf c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
+          const v2bf c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
+          const v2bf c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
+          const v2bf c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
+          wf[j].k[q] = v8bf{c0[0], c0[1], c1[0], c1[1], c2[0], c2[1], c3[0], c3[1]};
+        }
       };
       auto mfma = [&](int i, int j, int q) {
         if (FIRST && q == 0) {
