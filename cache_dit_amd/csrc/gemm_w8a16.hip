@@ -225,14 +225,32 @@ struct CfgWW {
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
   static_assert(DEPTH >= 2 && (DEPTH - 2) * ND + NDA < 63, "DMA instructions in flight: vmcnt has 6 bits");
 
-  // Issue schedule of a K step (see the wide w8a8 kernel: one LDS read, DMA instruction
-  // or group of four conversions between two MFMAs is free, a cluster is not).
-  // First half: S1 MFMAs, slot s = (i*4 + q)*TN + j. Items: the 4 (TM-1) single LDS
-  // reads of the fragments A_1 .. A_{TM-1} (MFMA step q of block i: read 4 (i-1) + q)
-  // and the NDA DMA instructions of the A panel, merged evenly, a read first, and spread
-  // evenly over the slots. The weights of column j, MFMA step q (4 conversions) are
-  // converted two slots ahead of their first use at slot q*TN + j.
+  // Issue schedule of a K step. Between two MFMAs (8 passes, 32 cycles) the wave issues
+  // in order; one LDS read or DMA instruction and two conversions (8 cycles each) fit,
+  // more delays the next MFMA, and the matrix core never makes that up. So everything is
+  // spread: all slot numbers below are compile-time constants.
+  //
+  // First half: S1 MFMAs over the rows 0..H-1, MFMA step q of all their blocks before step
+  // q+1: slot s = (q*H + i)*TN + j. A new weight operand (j, q) is then needed every
+  // H*TN/TN slots only, which leaves room to convert it in pieces (below). Items: the
+  // 4 (TM-1) single LDS reads of the fragments A_1 .. A_{TM-1} in the order of their first
+  // use, and the NDA DMA instructions of the A panel, merged evenly, a read first, and
+  // spread evenly over the slots.
   static constexpr int S1 = H * 4 * TN, NR1 = 4 * (TM - 1), T1 = NR1 + NDA;
+  static constexpr int R = TM - H, S2 = R * 4 * TN, NR2 = 4 + 2 * TN;
+  static constexpr int i_of_slot1(int s) { return s / TN % H; }
+  static constexpr int q_of_slot1(int s) { return s / (H * TN); }
+  // first use of A_i, MFMA step q, counted in slots from the start of the step
+  static constexpr int use_a(int i, int q) {
+    return i < H ? (q * H + i) * TN : S1 + (q * R + i - H) * TN;
+  }
+  static constexpr int H1 = H > 1 ? H - 1 : 1;
+  static constexpr int read1_row(int r) {  // read r of the first half: fragment A_i ...
+    return r < 4 * (H - 1) ? 1 + r % H1 : H + (r - 4 * (H - 1)) % R;
+  }
+  static constexpr int read1_step(int r) {  // ... MFMA step q
+    return r < 4 * (H - 1) ? r / H1 : (r - 4 * (H - 1)) / R;
+  }
   static constexpr int item_of_read1(int r) { return r * T1 / NR1; }
   static constexpr bool is_read1(int t) {
     for (int r = 0; r < NR1; ++r)
@@ -247,27 +265,86 @@ struct CfgWW {
   static constexpr int dma1_index(int t) { return t - read1_index(t); }
   static constexpr int slot1(int t) { return t * S1 / T1; }
   static constexpr bool first_half_reads_in_time() {
-    for (int t = 0; t < T1; ++t) {
-      const int r = read1_index(t), i = r / 4 + 1, q = r % 4;
-      if (is_read1(t) && i < H && slot1(t) + 3 > (i * 4 + q) * TN) return false;
-    }
+    for (int r = 0; r < NR1; ++r)
+      if (slot1(item_of_read1(r)) + 3 > use_a(read1_row(r), read1_step(r))) return false;
     return true;
   }
   static_assert(first_half_reads_in_time(), "A fragment read too late for its first use");
-  static constexpr int CONVERT_AHEAD = 2;
-  static constexpr bool PIN_CONVERT = TM * TN >= 12;  // see convert() in the kernel
-  // Second half: S2 MFMAs in blocks of column pairs (the order of the loops below). The
-  // raw weights of the next step replace those of a column pair from one slot after
-  // the pair's block on (one LDS read per slot), A_0 of the next step is read in front
-  // of slots 1..4, the NDB DMA instructions of the B panel go in the middle of their
-  // share of the slots.
-  static constexpr int R = TM - H, S2 = R * 4 * TN;
-  static constexpr int pair_end(int j0) { return (j0 + 2 < TN ? j0 + 2 : TN) * R * 4; }  // slots before it
-  static constexpr int slot_w(int j, int t) {  // read t (0/1) of column j
-    const int s = pair_end(j & ~1) + 1 + 2 * (j & 1) + t;
-    return s < S2 ? s : S2;
+  // Second half: S2 MFMAs over the rows H..TM-1 in the same order, slot s =
+  // (q*R + i-H)*TN + j. The LDS reads of the next step (its raw weights, 2 per column, and
+  // A_0, 4) are spread evenly over the slots from 1 on: first halves of the weights, A_0 of
+  // MFMA step 0, second halves, rest of A_0. The NDB DMA instructions of the B panel go in
+  // the middle of their share of the slots.
+  static constexpr int key_w(int j, int t) { return t == 0 ? j : TN + 1 + j; }
+  static constexpr int key_a0(int q) { return q == 0 ? TN : 2 * TN + 1 + q; }
+  static constexpr int rank2(int key) {  // reads of the second half with a smaller key
+    int n = 0;
+    for (int j = 0; j < TN; ++j)
+      for (int t = 0; t < 2; ++t) n += key_w(j, t) < key;
+    for (int q = 0; q < 4; ++q) n += key_a0(q) < key;
+    return n;
   }
-  static constexpr int slot_a0(int q) { return 1 + q < S2 ? 1 + q : S2; }
+  static constexpr int slot2(int key) { return 1 + rank2(key) * (S2 - 1) / NR2; }
+  static constexpr int slot_w(int j, int t) { return slot2(key_w(j, t)); }  // read t (0/1) of column j
+  static constexpr int slot_a0(int q) { return slot2(key_a0(q)); }
+  // Conversions. Weight operand (j, q) (8 e4m3 bytes -> 8 bf16, four conversion
+  // instructions) is converted as two half operands. Time t counts first-half slots of the
+  // step the operand belongs to; t < 0 is second-half slot S2 + t of the step before (the
+  // raw weights of a step are read during the step before it). A half operand must be
+  // converted in front of slot use - CONVERT_AHEAD at the latest (an MFMA operand written
+  // by a VALU instruction just before the inline-assembly MFMA reads stale data), and not
+  // before the registers it goes to have been read for the last time (plus one MFMA) and
+  // the LDS read it comes from has had three slots to land. Operands are placed latest
+  // deadline first, each half in the latest slot with room for it; the smallest number of
+  // half operands per slot that works is taken. Tiles too small for any of that convert
+  // each operand whole in front of slot use - CONVERT_AHEAD, the first ones at the top of
+  // the step (kConvTop).
+  static constexpr int CONVERT_AHEAD = 2;
+  static constexpr int kConvTop = -1000;
+  static constexpr bool PIN_CONVERT = TM * TN >= 12;  // see convert_half() in the kernel
+  static constexpr int last_use2(int j, int q) { return (q * R + R - 1) * TN + j; }
+  static constexpr int conv_deadline(int j, int q) { return q * H * TN + j - CONVERT_AHEAD; }
+  static constexpr int conv_release(int j, int q) {
+    const int a = last_use2(j, q) + 2, b = slot_w(j, q >> 1) + 3;
+    return (a > b ? a : b) - S2;
+  }
+  struct ConvSched {
+    int t[TN][4][2];
+    bool ok;
+  };
+  static constexpr ConvSched conv_sched_with(int cap) {
+    ConvSched c{};
+    c.ok = true;
+    int load[S1 + S2] = {};  // half operands in slot t, at index t + S2
+    for (int o = 4 * TN - 1; o >= 0; --o) {
+      const int q = o / TN, j = o % TN;
+      for (int h = 1; h >= 0; --h) {
+        int t = conv_deadline(j, q);
+        while (t >= conv_release(j, q) && load[t + S2] >= cap) --t;
+        if (t < conv_release(j, q)) {
+          c.ok = false;
+          return c;
+        }
+        ++load[t + S2];
+        c.t[j][q][h] = t;
+      }
+    }
+    return c;
+  }
+  static constexpr ConvSched conv_sched() {
+    for (int cap = 1; cap <= 2; ++cap) {
+      const ConvSched c = conv_sched_with(cap);
+      if (c.ok) return c;
+    }
+    ConvSched c{};
+    c.ok = true;
+    for (int j = 0; j < TN; ++j)
+      for (int q = 0; q < 4; ++q)
+        for (int h = 0; h < 2; ++h)
+          c.t[j][q][h] = conv_deadline(j, q) < 0 ? kConvTop : conv_deadline(j, q);
+    return c;
+  }
+  static constexpr ConvSched CONV = conv_sched();
   static constexpr int slot_dma2(int p) { return (2 * p + 1) * S2 / (2 * NDB); }
 };
 
@@ -425,9 +502,15 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
     af[0] = read_a(smem + a_cur, 0);
 
     // One K step; FIRST: step 0 of the tile (the accumulators start from zero).
-    auto step = [&](int kt, auto first_tag) {
+    // EVENTS: the step may be one of the last max(D, 2) of the tile, where the DMA stream
+    // moves on to the next tile and the epilogue operands are staged. The steps before
+    // them run in a loop of their own without these tests: what stands between the last
+    // MFMA of a step and the first of the next (tests, taken branches) is time the matrix
+    // core waits.
+    auto step = [&](int kt, auto first_tag, auto events_tag) {
       constexpr bool FIRST = decltype(first_tag)::value;
-      if (kt == KT - D) {
+      constexpr bool EVENTS = decltype(events_tag)::value;
+      if (EVENTS && kt == KT - D) {
         // every DMA of this tile has been issued: the stream moves on
         if (next_tile < ntiles) {
           int tm, tn;
@@ -439,7 +522,7 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
           nrec = 0;
         }
       }
-      if (kt == KT - 2) {
+      if (EVENTS && kt == KT - 2) {
         // b_scale and bias of this tile's columns go to the LDS with two DMA instructions
         // (every wave issues both: equal instruction counts; the same bytes land four
         // times) instead of 6 TN loads per lane at the start of the epilogue. What lies
@@ -455,31 +538,45 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
             bi_buf, (__attribute__((address_space(3))) void*)(smem + C::EPI_BI), 16,
             n0 * 2 + 16 * lane, 0, 0, 0);
       }
-      const int kd = kt + D < KT ? kt + D : kt + D - KT;  // step (of its tile) to fetch
+      // step (of its tile) to fetch
+      const int kd = !EVENTS || kt + D < KT ? kt + D : kt + D - KT;
       const uint8_t* st = smem + a_cur;
-      // weights of column j, MFMA step q: 8 e4m3 bytes -> one bf16 operand
-      auto convert = [&](int j, int q) {
+      // half h of the weight operand of column j, MFMA step q: 4 e4m3 bytes -> 4 bf16
+      auto convert_half = [&](int j, int q, int h) {
         const uint4& w = wr[j].t[q >> 1];
-        const uint32_t lo = (q & 1) ? w.z : w.x, hi = (q & 1) ? w.w : w.y;
+        const uint32_t src = (q & 1) ? (h ? w.w : w.z) : (h ? w.y : w.x);
+        uint4 o = __builtin_bit_cast(uint4, wf[j].k[q]);
+        uint32_t c0, c1;
         if constexpr (C::PIN_CONVERT) {
           // Inline assembly (volatile): the conversions stay in the MFMA slot they are
           // written in. As builtins they are pure functions of loaded values, and with the
           // large wave tiles the compiler gathered most of a step's conversions at the top
-          // of the loop, where the matrix core then waited for them (a tenth of a step;
-          // with the small wave tiles its own placement is the better one).
-          uint32_t c0, c1, c2, c3;
-          asm volatile("v_cvt_scalef32_pk_bf16_fp8 %0, %1, 1.0" : "=v"(c0) : "v"(lo));
-          asm volatile("v_cvt_scalef32_pk_bf16_fp8 %0, %1, 1.0 op_sel:[1,0,0]" : "=v"(c1) : "v"(lo));
-          asm volatile("v_cvt_scalef32_pk_bf16_fp8 %0, %1, 1.0" : "=v"(c2) : "v"(hi));
-          asm volatile("v_cvt_scalef32_pk_bf16_fp8 %0, %1, 1.0 op_sel:[1,0,0]" : "=v"(c3) : "v"(hi));
-          wf[j].k[q] = __builtin_bit_cast(v8bf, uint4{c0, c1, c2, c3});
+          // of the loop, where the matrix core then waited for them (with the small wave
+          // tiles its own placement is the better one).
+          asm volatile("v_cvt_scalef32_pk_bf16_fp8 %0, %1, 1.0" : "=v"(c0) : "v"(src));
+          asm volatile("v_cvt_scalef32_pk_bf16_fp8 %0, %1, 1.0 op_sel:[1,0,0]" : "=v"(c1) : "v"(src));
         } else {
-          const v2bf c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
-          const v2bf c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
-          const v2bf c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
-          const v2bf c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
-          wf[j].k[q] = v8bf{c0[0], c0[1], c1[0], c1[1], c2[0], c2[1], c3[0], c3[1]};
+          c0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(src, 1.0f, false));
+          c1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(src, 1.0f, true));
         }
+        if (h) {
+          o.z = c0;
+          o.w = c1;
+        } else {
+          o.x = c0;
+          o.y = c1;
+        }
+        wf[j].k[q] = __builtin_bit_cast(v8bf, o);
+      };
+      // the half operands the schedule puts at time t (CfgWW::CONV)
+      auto conversions_at = [&](int t) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+              if (C::CONV.t[j][q][h] == t) convert_half(j, q, h);
       };
       auto mfma = [&](int i, int j, int q) {
         if (FIRST && q == 0) {
@@ -488,32 +585,27 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
           mfma_32x32x16_bf16<false>(acc[i][j], wf[j].k[q], af[i].k[q]);
         }
       };
-      // The weights of this step were read from LDS during the previous step. Each
-      // operand is converted CONVERT_AHEAD MFMAs before its first use: an MFMA operand
-      // written by a VALU instruction just before the (inline-assembly) MFMA reads
-      // stale data.
+      // The weights of this step were read from LDS during the previous step, which has
+      // also converted the operands the schedule puts there; step 0 of a tile converts
+      // those itself.
+      if constexpr (FIRST) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          if (q * TN + j < C::CONVERT_AHEAD) convert(j, q);
+        for (int t = -C::S2; t < 0; ++t) conversions_at(t);
+      }
+      conversions_at(C::kConvTop);
       __builtin_amdgcn_sched_barrier(0);
-      // first half: rows 0..H-1; MFMA step q of all TN blocks of a row before step
-      // q+1, so that consecutive MFMAs never depend on each other (schedule: CfgWW::slot1)
+      // first half: rows 0..H-1, MFMA step q of all their blocks before step q+1
+      // (schedule: CfgWW::slot1 ...)
 #pragma unroll
       for (int sl = 0; sl < C::S1; ++sl) {
-        const int i = sl / (4 * TN), q = sl / TN % 4, j = sl % TN;
-#pragma unroll
-        for (int qq = 0; qq < 4; ++qq)
-#pragma unroll
-          for (int jj = 0; jj < TN; ++jj)
-            if (qq * TN + jj - C::CONVERT_AHEAD == sl) convert(jj, qq);
+        const int i = C::i_of_slot1(sl), q = C::q_of_slot1(sl), j = sl % TN;
+        conversions_at(sl);
 #pragma unroll
         for (int t = 0; t < C::T1; ++t) {
           if (C::slot1(t) != sl) continue;
           if (C::is_read1(t)) {
             const int r = C::read1_index(t);
-            af[r / 4 + 1].k[r % 4] = read_a1(st, r / 4 + 1, r % 4);
+            af[C::read1_row(r)].k[C::read1_step(r)] = read_a1(st, C::read1_row(r), C::read1_step(r));
           } else {
             dma_a(kd, a_prev, C::dma1_index(t));
           }
@@ -525,56 +617,51 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
       // after it and the A panel issued above may still fly); then everyone's. In the
       // first D-1 steps of a later tile that DMA was waited for before the previous
       // epilogue's stores.
-      if (kt <= D - 2 && tile != (int)blockIdx.x) {
+      if ((FIRST || D > 2) && kt <= D - 2 && tile != (int)blockIdx.x) {
         wait_and_barrier<63>();
       } else {
         wait_and_barrier<(D - 2) * C::ND + C::NDA>();
       }
-      // second half: rows H..TM-1 in pairs of columns, so that dependent MFMAs are
-      // 2 (TM-H) apart; the next step's raw weights and A_0 are read and the B panel D
-      // steps ahead goes into the B stage of this step (schedule: CfgWW::slot_w ...)
-      auto second_half_items = [&](int sl) {
+      // second half: rows H..TM-1 in the same order; the next step's raw weights and A_0
+      // are read, its first operands converted (in the last step of a tile: of no use,
+      // step 0 of the next tile reads and converts its own) and the B panel D steps ahead
+      // goes into the B stage of this step (schedule: CfgWW::slot_w ...)
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          if (C::slot_a0(q) == sl) af[0].k[q] = read_a1(smem + a_next, 0, q);
+      for (int sl = 0; sl < C::S2; ++sl) {
+        const int q = sl / (C::R * TN), i = H + sl / TN % C::R, j = sl % TN;
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int qq = 0; qq < 4; ++qq)
+          if (C::slot_a0(qq) == sl) af[0].k[qq] = read_a1(smem + a_next, 0, qq);
+#pragma unroll
+        for (int jj = 0; jj < TN; ++jj)
 #pragma unroll
           for (int t = 0; t < 2; ++t)
-            if (C::slot_w(j, t) == sl) wr[j].t[t] = read_w1(smem + b_next, j, t);
+            if (C::slot_w(jj, t) == sl) wr[jj].t[t] = read_w1(smem + b_next, jj, t);
 #pragma unroll
         for (int p = 0; p < C::NDB; ++p)
           if (C::slot_dma2(p) == sl) dma_b(kd, b_cur, p);
-      };
-      {
-        constexpr int R = C::R;
-        int sl = 0;
-#pragma unroll
-        for (int j0 = 0; j0 < TN; j0 += 2)
-#pragma unroll
-          for (int q = 0; q < 4; ++q)
-#pragma unroll
-            for (int i = H; i < TM; ++i)
-#pragma unroll
-              for (int j = j0; j < j0 + 2 && j < TN; ++j) {
-                second_half_items(sl);
-                mfma(i, j, q);
-                __builtin_amdgcn_sched_barrier(0);
-                ++sl;
-              }
-        static_assert(R * 4 * TN == C::S2, "slot count");
-        second_half_items(C::S2);
+        conversions_at(sl - C::S2);
+        if (sl == C::S2 - 1) {
+          // the stages move on in front of the last MFMA, not behind it
+          a_prev = a_cur;
+          a_cur = a_next;
+          a_next = a_next + C::A_BYTES == C::A_STAGES * C::A_BYTES ? 0 : a_next + C::A_BYTES;
+          b_cur = b_next;
+          b_next = b_next + C::B_BYTES == C::B_BASE + C::B_STAGES * C::B_BYTES
+                       ? C::B_BASE
+                       : b_next + C::B_BYTES;
+        }
+        mfma(i, j, q);
         __builtin_amdgcn_sched_barrier(0);
       }
-      a_prev = a_cur;
-      a_cur = a_next;
-      a_next = a_next + C::A_BYTES == C::A_STAGES * C::A_BYTES ? 0 : a_next + C::A_BYTES;
-      b_cur = b_next;
-      b_next = b_next + C::B_BYTES == C::B_BASE + C::B_STAGES * C::B_BYTES ? C::B_BASE
-                                                                           : b_next + C::B_BYTES;
     };
-    step(0, std::true_type{});
-    for (int kt = 1; kt < KT; ++kt) step(kt, std::false_type{});
+    step(0, std::true_type{}, std::true_type{});
+    {
+      const int events_from = KT - (D > 2 ? D : 2);  // first step that may have an event
+      int kt = 1;
+      for (; kt < events_from; ++kt) step(kt, std::false_type{}, std::false_type{});
+      for (; kt < KT; ++kt) step(kt, std::false_type{}, std::true_type{});
+    }
     // the last MFMAs (8 passes each) must have written their accumulators
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
