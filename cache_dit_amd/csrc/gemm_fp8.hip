@@ -534,9 +534,15 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     float as[TM];
 
     // One K step; FIRST: step 0 of the tile (the accumulators start from zero).
-    auto step = [&](int kt, auto first_tag) {
+    // EVENTS: the step may be one of the last max(D, 2) of the tile, where the DMA stream
+    // moves on to the next tile and the epilogue operands are fetched. The steps before
+    // them run in a loop of their own without these tests: what stands between the last
+    // MFMA of a step and the first of the next (tests, taken branches, stage arithmetic)
+    // is time the matrix core waits.
+    auto step = [&](int kt, auto first_tag, auto events_tag) {
       constexpr bool FIRST = decltype(first_tag)::value;
-      if (kt == KT - D) {
+      constexpr bool EVENTS = decltype(events_tag)::value;
+      if (EVENTS && kt == KT - D) {
         // every DMA of this tile has been issued: the stream moves on
         if (next_tile < ntiles) {
           int tm, tn;
@@ -548,7 +554,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
           nrec = 0;
         }
       }
-      if (kt == KT - 2) {
+      if (EVENTS && kt == KT - 2) {
         // buffer accesses: what lies beyond N (M) reads as zero, no bounds branches; a
         // null bias becomes an empty buffer
         const __amdgpu_buffer_rsrc_t bs_buf = __builtin_amdgcn_make_buffer_rsrc(
@@ -585,7 +591,8 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
                 float, __builtin_amdgcn_raw_buffer_load_b32(as_buf, (mw + 16 * i) * 4, 0, 0));
         }
       }
-      const int kd = kt + D < KT ? kt + D : kt + D - KT;  // step (of its tile) to fetch
+      // step (of its tile) to fetch
+      const int kd = !EVENTS || kt + D < KT ? kt + D : kt + D - KT;
       const uint8_t* st = smem + a_cur;
       // first half: rows 0..H-1, row-major; meanwhile the other A fragments of this
       // step are read and the A panel D steps ahead goes into the stage that step
@@ -609,7 +616,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
       // everyone's. In the first D-1 steps of a later tile the NST output stores of
       // the previous epilogue were issued after the DMA in question (the counter
       // retires in issue order) and may keep flying as well.
-      if (kt <= D - 2 && tile != (int)blockIdx.x) {
+      if ((FIRST || D > 2) && kt <= D - 2 && tile != (int)blockIdx.x) {
         wait_and_barrier<(D - 2) * C::ND + C::NDA + NST>();
       } else {
         wait_and_barrier<(D - 2) * C::ND + C::NDA>();
@@ -626,9 +633,17 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
         for (int p = 0; p < C::NDB; ++p)
           if (C::slot_dma2(p) == sl) dma_b(kd, b_cur, p);
       };
+      int a_after = 0, b_after = 0;  // stages of the step after the next
 #pragma unroll
       for (int sl = 0; sl < C::S2; ++sl) {
         second_half_items(sl);
+        if (sl == C::S2 - 1) {
+          // worked out in front of the last MFMA, not behind it
+          a_after = a_next + C::A_BYTES == C::A_STAGES * C::A_BYTES ? 0 : a_next + C::A_BYTES;
+          b_after = b_next + C::B_BYTES == C::B_BASE + C::B_STAGES * C::B_BYTES
+                        ? C::B_BASE
+                        : b_next + C::B_BYTES;
+        }
         mfma_16x16x128_fp8<FIRST>(acc[H + sl % C::R][sl / C::R], bf[sl / C::R], af[H + sl % C::R]);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -637,13 +652,17 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
       // rotate the stages
       a_prev = a_cur;
       a_cur = a_next;
-      a_next = a_next + C::A_BYTES == C::A_STAGES * C::A_BYTES ? 0 : a_next + C::A_BYTES;
+      a_next = a_after;
       b_cur = b_next;
-      b_next = b_next + C::B_BYTES == C::B_BASE + C::B_STAGES * C::B_BYTES ? C::B_BASE
-                                                                           : b_next + C::B_BYTES;
+      b_next = b_after;
     };
-    step(0, std::true_type{});
-    for (int kt = 1; kt < KT; ++kt) step(kt, std::false_type{});
+    step(0, std::true_type{}, std::true_type{});
+    {
+      const int events_from = KT - (D > 2 ? D : 2);  // first step that may have an event
+      int kt = 1;
+      for (; kt < events_from; ++kt) step(kt, std::false_type{}, std::false_type{});
+      for (; kt < KT; ++kt) step(kt, std::false_type{}, std::true_type{});
+    }
     // the last MFMAs (8 passes each) must have written their accumulators
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
