@@ -297,6 +297,10 @@ def main():
                   help="run only the headline-shape kernels (the roofline legs) and print their "
                        "figures: the command to put under rocprofv3 when per-kernel averages "
                        "must not mix shapes")
+  ap.add_argument("--step-only", action="store_true",
+                  help="run only the hot-path step legs (eager, hipGraph replay, shared "
+                       "quantization) and print their figures: the command to put under "
+                       "rocprofv3 for the kernel mix of one step")
   args = ap.parse_args()
   if args.gpus != 1:
     sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
@@ -368,6 +372,12 @@ def main():
   step_flop = hot.flop
   del hot
   torch.cuda.empty_cache()
+  if args.step_only:
+    print(json.dumps({"value": value, "unit": "TFLOP/s", "ms_per_step": ms_per_step,
+                      "launch": launch_mode, "eager_ms_per_step": eager_ms,
+                      "shared_quant_ms_per_step": shared_ms, "steps": args.steps,
+                      "warmup": args.warmup, "device": arch}))
+    return
 
   head = headline_kernels(device)
   M, K, N = HEADLINE
