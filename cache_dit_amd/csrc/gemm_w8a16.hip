@@ -189,8 +189,9 @@ __global__ __launch_bounds__(C::THREADS) void gemm_w8a16_tiled(GemmArgs g, int t
 // (e4m3), chunk c at c ^ ((r>>2)&3). A lane reads, per 32-row block, the four A
 // chunks 4t+2h+s (h = lane>>5) and the two B chunks 2t+h: the 16 B bytes of one
 // chunk are the weights of MFMA steps 2t and 2t+1 (K order permuted identically on
-// both sides). The weights are converted to bf16 once per step, four conversions
-// at a time two MFMAs ahead of their first use, and kept for all row blocks.
+// both sides). The weights are converted to bf16 once per step, two conversion
+// instructions (half an operand) at a time on a compile-time schedule that ends two
+// MFMAs ahead of the first use, and kept for all row blocks.
 //
 // The B fragments take their 32 rows in a permuted order, operand row p reads
 // panel row 16 ((p>>2)&1) + 4 (p>>3) + (p&3) of its block: with the operands
@@ -232,7 +233,7 @@ struct CfgWW {
   //
   // First half: S1 MFMAs over the rows 0..H-1, MFMA step q of all their blocks before step
   // q+1: slot s = (q*H + i)*TN + j. A new weight operand (j, q) is then needed every
-  // H*TN/TN slots only, which leaves room to convert it in pieces (below). Items: the
+  // H slots only, which leaves room to convert it in pieces (below). Items: the
   // 4 (TM-1) single LDS reads of the fragments A_1 .. A_{TM-1} in the order of their first
   // use, and the NDA DMA instructions of the A panel, merged evenly, a read first, and
   // spread evenly over the slots.
