@@ -164,6 +164,33 @@ def test_qwen_and_wan_shapes_sampled_rows(M, N, K):
 
 
 @pytest.mark.parametrize("variant", [12, 14, 15, 16, 17, 18])
+def test_wide_kernels_every_short_k_loop(variant):
+  """K loops of 3 to 9 steps, more tiles than CUs: the K loop runs its steps in two
+  loops (the last steps of a tile, where the DMA stream moves on to the next tile, apart
+  from those before them), so every split of a short loop between the two is covered,
+  and the steps a tile needs before it may use the kernel at all. Exact small-integer
+  data, sampled rows bit for bit."""
+  from cache_dit_amd import _native, ops
+  M, N = 5000, 3080
+  for steps in range(3, 10):
+    K = 128 * steps
+    g = torch.Generator(device="cuda").manual_seed(steps)
+    a = torch.randint(-3, 4, (M, K), generator=g, device="cuda").float().to(FP8)
+    w = torch.randint(-3, 4, (N, K), generator=g, device="cuda").float().to(FP8)
+    sa = torch.full((M,), 0.5, device="cuda")
+    sw = torch.full((N,), 0.25, device="cuda")
+    b = torch.randint(-8, 9, (N,), generator=g, device="cuda").to(torch.bfloat16)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    _native.set_gemm_variant(variant)
+    ops.gemm_rowwise_into(a, sa, w, sw, b, out, 0)
+    torch.cuda.synchronize()
+    rows = torch.cat([torch.arange(0, M, 53), torch.arange(M - 5, M)])
+    ref = to.scaled_mm_rowwise(a[rows.cuda()].cpu(), sa[rows.cuda()].cpu().reshape(-1, 1), w.cpu(),
+                               sw.cpu().reshape(-1, 1), b.cpu())
+    assert torch.equal(out[rows.cuda()].cpu(), ref), (variant, K)
+
+
+@pytest.mark.parametrize("variant", [12, 14, 15, 16, 17, 18])
 def test_wide_kernels_random_shapes_many_tiles_per_workgroup(variant):
   """Random shapes with edge tiles in M and N and more tiles than CUs (a persistent
   workgroup then runs several tiles, the DMA stream crossing tile boundaries), exact

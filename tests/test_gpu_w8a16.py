@@ -148,6 +148,30 @@ def test_against_c_oracle_and_gelu():
 
 
 @pytest.mark.parametrize("variant", [7, 8, 9, 10, 11, 12])
+def test_wide_kernels_every_short_k_loop(variant):
+  """K loops of 3 to 9 steps of 64, more tiles than CUs: every split of a short K loop
+  between the steps before a tile's last ones and those last ones, where the DMA stream
+  moves on to the next tile and the conversions that a step does for the next one are
+  of no use. Exact small-integer data, sampled rows bit for bit."""
+  from cache_dit_amd import _native, ops
+  M, N = 5000, 3088
+  for steps in range(3, 10):
+    K = 64 * steps
+    g = torch.Generator(device="cuda").manual_seed(steps)
+    x = torch.randint(-3, 4, (M, K), generator=g, device="cuda").to(torch.bfloat16)
+    w = torch.randint(-3, 4, (N, K), generator=g, device="cuda").float().to(FP8)
+    sw = torch.full((N,), 0.25, device="cuda")
+    b = torch.randint(-8, 9, (N,), generator=g, device="cuda").to(torch.bfloat16)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    _native.set_gemm_variant(variant)
+    ops.w8a16_into(x, w, sw, b, out, 0)
+    torch.cuda.synchronize()
+    rows = torch.cat([torch.arange(0, M, 53), torch.arange(M - 5, M)])
+    ref = to.w8a16_linear(x[rows.cuda()].cpu(), w.cpu(), sw.cpu().reshape(-1, 1), b.cpu(), fused=True)
+    assert torch.equal(out[rows.cuda()].cpu(), ref), (variant, K)
+
+
+@pytest.mark.parametrize("variant", [7, 8, 9, 10, 11, 12])
 def test_wide_kernels_random_shapes_many_tiles_per_workgroup(variant):
   """Random shapes with edge tiles in M and N and more tiles than CUs (persistent
   workgroups run several tiles each), exact small-integer data: sampled rows must
