@@ -836,7 +836,9 @@ int launch_wide(const GemmArgs& g, hipStream_t stream) {
 // group l>>4; 16 x 128-byte segments per pair of loads), multiplies by the (zero
 // padded) activation rows with v_mfma_f32_16x16x128_f8f6f4, and the four partial
 // 16x16 tiles are summed through LDS before the epilogue. No LDS staging of the
-// weights: every weight byte is used exactly once.
+// weights: every weight byte is used exactly once. The weight loads carry no
+// non-temporal hint: with this access pattern (16 rows x 64 bytes per instruction)
+// the hinted loads measured 17 % slower in a read-only loop and 10 % in the kernel.
 __global__ __launch_bounds__(256) void gemm_fp8_skinny(GemmArgs g) {
   __shared__ float part[4][16][17];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -858,8 +860,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_skinny(GemmArgs g) {
     for (int u = 0; u < U; ++u) {
       const int kt = min(k0 + u, k_end - 1);  // clamped duplicates are not accumulated
       const v4i* wq = reinterpret_cast<const v4i*>(wp + (int64_t)kt * 128);
-      w[u][0] = __builtin_nontemporal_load(wq);
-      w[u][1] = __builtin_nontemporal_load(wq + 1);
+      w[u][0] = wq[0];
+      w[u][1] = wq[1];
       const v4i* aq = reinterpret_cast<const v4i*>(ap + (int64_t)kt * 128);
       a[u][0] = aq[0];
       a[u][1] = aq[1];
@@ -937,8 +939,8 @@ __global__ __launch_bounds__(256) void linear_fp8_skinny_fused(GemmArgs g, uint8
     for (int u = 0; u < U; ++u) {
       const int kt = min(k0 + u, max(k_end, 1) - 1);  // clamped duplicates are not accumulated
       const v4i* wq = reinterpret_cast<const v4i*>(wp + (int64_t)kt * 128);
-      w[u][0] = __builtin_nontemporal_load(wq);
-      w[u][1] = __builtin_nontemporal_load(wq + 1);
+      w[u][0] = wq[0];
+      w[u][1] = wq[1];
     }
   };
   load_w(k_begin);
