@@ -213,12 +213,15 @@ __global__ __launch_bounds__(64) void quant_tensorwise_cast(
 }  // namespace
 
 // Cache hints of the row-in-registers kernel. 0: non-temporal loads and stores; 1: both plain;
-// 2: non-temporal loads only; 3: non-temporal stores only; -1 (default): 1 when the GEMM that
-// reads the codes follows in the same call (the fused Linear entry point), else 3 for
-// activations of up to 64 MB and 0 above. Measured on activations that come from HBM:
-// 4608 x 3072 (28 MB) 9.2 / 10.9 / 9.8 / 8.4 us for 0 / 1 / 2 / 3, 4608 x 15360 (142 MB)
-// 40.8 / 47.6 / 40.5 / 43.3, 32760 x 5120 (335 MB) 81 / 92 / 88 / 87; inside a step of 494
-// fused Linears 1 is the fastest, 3 is 1.1 % and 0 2.3 % behind.
+// 2: non-temporal loads only; 3: non-temporal stores only; -1 (default): when the GEMM that
+// reads the codes follows in the same call (the fused Linear entry point) 1 for activations
+// of up to 64 MB and 2 above, else 3 up to 64 MB and 0 above. Measured on activations that
+// come from HBM: 4608 x 3072 (28 MB) 9.2 / 10.9 / 9.8 / 8.4 us for 0 / 1 / 2 / 3, 4608 x
+// 15360 (142 MB) 40.8 / 47.6 / 40.5 / 43.3, 32760 x 5120 (335 MB) 81 / 92 / 88 / 87; inside
+// a step of 494 fused Linears with one hint for all of them 1 is the fastest, 3 is 1.1 % and
+// 0 2.3 % behind; quantizer + GEMM of one Linear, 0 / 1 / 2 / 3: 4608 x 15360 x 3072 186.9 /
+// 187.0 / 183.8 / 190.6 us, K = 12288 150.9 / 150.7 / 148.1 / 154.1, 4608 x 3072 x 12288
+// 144.4 / 143.4 / 144.9 / 145.5, N = 3072 47.1 / 46.1 / 48.2 / 45.8.
 int g_quant_variant = -1;
 
 int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void* q,
@@ -240,7 +243,7 @@ int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void
   const int Mi = (int)M, Ki = (int)K;
   const int need = (int)((K + 511) / 512);  // 16-byte chunks per lane
   const int hints = g_quant_variant >= 0 ? g_quant_variant
-                    : consumer_follows   ? 1
+                    : consumer_follows   ? (M * K * 2 > ((int64_t)64 << 20) ? 2 : 1)
                     : M * K * 2 > ((int64_t)64 << 20) ? 0 : 3;
 #define CDIT_QUANT_LAUNCH(CH, NL, NS)                                                        \
   hipLaunchKernelGGL((quant_rowwise_regs<CH, NL, NS>), grid, block, 0, stream, xp, ld_x, qp,   \

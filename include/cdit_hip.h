@@ -47,8 +47,8 @@ enum cdit_status {
  *   FP32DIV: fp32 true divide, kept in fp32. */
 enum cdit_scale_mode { CDIT_SCALE_BF16DIV = 0, CDIT_SCALE_FP32DIV = 1 };
 /* May be OR-ed into the scale_mode of cdit_fp8_quant_rowwise: the codes are read by a GEMM
- * launched next on the same stream. A cache hint only (the quantizer then keeps its loads and
- * stores cacheable, as the fused cdit_fp8_linear_w8a8 does); results do not depend on it. */
+ * launched next on the same stream. A cache hint only (the quantizer then keeps its stores
+ * cacheable, as the fused cdit_fp8_linear_w8a8 does); results do not depend on it. */
 #define CDIT_QUANT_GEMM_FOLLOWS 0x100
 
 /* Epilogue flags of the GEMM entry points (bit mask). */
