@@ -41,15 +41,18 @@ def _find_transformers(obj: Any) -> List[tuple]:
 def enable_cache(pipe_or_adapter: Any,
                  cache_config: Optional[Any] = None,
                  calibrator_config: Optional[Any] = None,
+                 params_modifiers: Optional[Any] = None,
                  parallelism_config: Optional[Any] = None,
                  attention_backend: Optional[str] = None,
                  quantize_config: Optional[QuantizeConfig] = None,
                  **kwargs) -> Any:
   """Applies `quantize_config` to a pipeline, a block adapter or a bare
-  transformer module and returns the same object."""
+  transformer module and returns the same object. The parameter list is the
+  reference's (src/cache_dit/caching/cache_interface.py:26-47), positions included."""
   refused = {
       "cache_config": cache_config,
       "calibrator_config": calibrator_config,
+      "params_modifiers": params_modifiers,
       "parallelism_config": parallelism_config,
       "attention_backend": attention_backend,
   }

@@ -316,11 +316,9 @@ def basic_filter(m: nn.Module, name: str, ctx: QuantizeContext,
   if qt in ("float8_per_row", "float8_per_tensor", "float8_per_block") and not _bias_ok(m):
     return skip("_scaled_mm: DTensor + bias NOT supported")
 
-  if qt in ("float8_per_row", "float8_weight_only"):
-    # the FP8 matmul needs both weight dimensions to be multiples of 16
-    shape = tuple(m.weight.shape)
-    if shape[-2] % 16 != 0 or shape[-1] % 16 != 0:
-      return skip(f"weight_shape{shape}%16!=0")
+  incompatible = _kernel_incompatibility(m, qt)
+  if incompatible is not None:
+    return skip(incompatible)
 
   m._is_inner_quantized = True
   ctx.quantized_map[qt] += 1
@@ -342,9 +340,34 @@ def fallback_filter(m: nn.Module, name: str, ctx: QuantizeContext) -> bool:
     ctx.skipped_map[FALLBACK_QUANT_TYPE].append(reason)
     logger.debug(reason)
     return False
+  incompatible = _kernel_incompatibility(m, FALLBACK_QUANT_TYPE)
+  if incompatible is not None:
+    reason = f"fallback: {name} -> pattern<{incompatible}>"
+    ctx.skipped_map[FALLBACK_QUANT_TYPE].append(reason)
+    logger.debug(reason)
+    return False
   m._is_inner_quantized = True
   ctx.quantized_map[FALLBACK_QUANT_TYPE] += 1
   return True
+
+
+def _kernel_incompatibility(m: nn.Linear, qt: str) -> Optional[str]:
+  """Why the FP8 kernels cannot take Linear `m` under quant type `qt` (None if they
+  can). The reference hands every layer to torchao, whose FP8 configs leave a layer
+  they cannot run unquantized without raising; here such a layer is skipped with a
+  reason before anything about it is recorded, for every quant type that has a
+  kernel: both weight dimensions multiples of 16, bf16 weight and bias."""
+  if qt not in BUILT_QUANTIZE_TYPES:
+    return None
+  shape = tuple(m.weight.shape)
+  if shape[-2] % 16 != 0 or shape[-1] % 16 != 0:
+    return f"weight_shape{shape}%16!=0"
+  if m.weight.dtype != torch.bfloat16:
+    return f"dtype({m.weight.dtype})!=bfloat16"
+  bias = getattr(m, "bias", None)
+  if bias is not None and bias.dtype != torch.bfloat16:
+    return f"bias_dtype({bias.dtype})!=bfloat16"
+  return None
 
 
 def _bias_ok(m: nn.Linear) -> bool:
@@ -401,6 +424,20 @@ def _check_platform(ctx: QuantizeContext) -> None:
     _native.device_arch()  # raises unless the device is a gfx950
 
 
+def _check_dtype_overrides(kwargs: dict) -> None:
+  """`weight_dtype` / `activation_dtype` reach torchao's FP8 configs in the reference
+  (quantize_ao.py:548-555, :565-572, :604-607; default float8_e4m3fn). The kernels
+  here encode OCP e4m3fn only, so any other request is refused instead of being
+  quietly served as e4m3fn."""
+  for key in ("weight_dtype", "activation_dtype"):
+    dt = kwargs.get(key, torch.float8_e4m3fn)
+    if dt is None or dt == torch.float8_e4m3fn or dt == "float8_e4m3fn":
+      continue
+    raise NotImplementedError(
+        f"{key}={dt} is not built in this MI355X implementation: the quantizer and the GEMMs "
+        "encode torch.float8_e4m3fn only")
+
+
 def quantize_ao(module: nn.Module, quantize_config: QuantizeConfig,
                 _convert_fn: Optional[ConvertFn] = None, **kwargs) -> nn.Module:
   """Applies `quantize_config` to `module` in place.
@@ -411,16 +448,28 @@ def quantize_ao(module: nn.Module, quantize_config: QuantizeConfig,
   if not _check_can_quantize(module):
     return module
   ctx = QuantizeContext.from_config(quantize_config, module, **kwargs)
-  convert = _convert_fn
-  if convert is None:
+  _check_dtype_overrides(ctx.kwargs)
+  convert_impl = _convert_fn
+  if convert_impl is None:
     _check_platform(ctx)
 
-    def convert(linear: nn.Linear, qt: str) -> None:
+    def convert_impl(linear: nn.Linear, qt: str) -> None:
       if qt not in BUILT_QUANTIZE_TYPES:
         raise NotImplementedError(
             f"quant_type {qt!r} has no MI355X kernel in this build (built: "
             f"{BUILT_QUANTIZE_TYPES})")
       _default_convert(linear, qt)
+
+  def convert(linear: nn.Linear, qt: str) -> None:
+    # the filter has already booked the layer as quantized: take that back when the
+    # conversion fails, so that a caller who catches the error sees true bookkeeping
+    try:
+      convert_impl(linear, qt)
+    except BaseException:
+      if getattr(linear, "_is_inner_quantized", False):
+        del linear._is_inner_quantized
+      ctx.quantized_map[qt] -= 1
+      raise
 
   def basic(qt_override: Optional[str] = None):
     return lambda m, name: basic_filter(m, name, ctx, qt_override)

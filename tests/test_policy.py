@@ -178,10 +178,13 @@ def test_dtype_rules():
   m = nn.Sequential(lin(dtype=torch.float32))
   with pytest.raises(AssertionError, match="weight dtype of bfloat16"):
     run(m, QuantizeConfig(exclude_layers=[]))
-  # weight-only has no dtype assertion
-  ctx, calls = run(nn.Sequential(lin(dtype=torch.float32)),
-                   QuantizeConfig(quant_type="float8_weight_only", exclude_layers=[]))
-  assert calls == ["float8_weight_only"]
+  # weight-only and per-tensor have no dtype assertion: a layer the kernels cannot take
+  # is left unquantized with a reason (torchao leaves such a layer alone without raising)
+  for qt in ("float8_weight_only", "float8_per_tensor"):
+    ctx, calls = run(nn.Sequential(lin(dtype=torch.float32)),
+                     QuantizeConfig(quant_type=qt, exclude_layers=[]))
+    assert calls == [] and ctx.quantized_map[qt] == 0
+    assert ctx.skipped_map[qt] == ["skip: 0 -> pattern<dtype(torch.float32)!=bfloat16>"]
 
 
 def test_dimensions_not_multiple_of_16_are_skipped():
@@ -189,6 +192,72 @@ def test_dimensions_not_multiple_of_16_are_skipped():
   ctx, calls = run(m, QuantizeConfig(exclude_layers=[]))
   assert len(calls) == 1
   assert ctx.skipped_map["float8_per_row"] == ["skip: 0 -> pattern<weight_shape(32, 30)%16!=0>"]
+
+
+def test_per_tensor_plan_and_fallback_skip_what_the_kernels_cannot_take():
+  """A 100x64 Linear under a float8_per_tensor plan entry, and one reached by the
+  per-tensor fallback pass, are skipped with a reason instead of raising in the
+  middle of the walk."""
+
+  class Blk(nn.Module):
+
+    def __init__(self):
+      super().__init__()
+      self.odd, self.even, self.row_parallel = lin(64, 100), lin(64, 64), lin(100, 64)
+
+  class Net(nn.Module):
+    _repeated_blocks = ["Blk"]
+
+    def __init__(self):
+      super().__init__()
+      self.blocks = nn.ModuleList([Blk(), Blk()])
+
+  ctx, calls = run(Net(), QuantizeConfig(precision_plan={"odd": "float8_per_tensor"},
+                                         per_tensor_fallback=False))
+  assert calls == ["float8_per_row"] * 2  # `even`; `row_parallel` has K = 100
+  assert ctx.quantized_map["float8_per_tensor"] == 0
+  assert ctx.skipped_map["float8_per_tensor"] == ["skip: odd -> pattern<weight_shape(100, 64)%16!=0>"] * 2
+  # the default pass meets `odd` again (still unquantized) and skips it once more
+  assert ctx.skipped_map["float8_per_row"] == [
+      "skip: odd -> pattern<weight_shape(100, 64)%16!=0>",
+      "skip: row_parallel -> pattern<weight_shape(64, 100)%16!=0>"] * 2
+  net = Net()
+  net._rowwise_layers = ["row_parallel"]
+  ctx, calls = run(net, QuantizeConfig())
+  assert calls == ["float8_per_row"] * 2 and ctx.quantized_map["float8_per_tensor"] == 0
+  assert "fallback: row_parallel -> pattern<weight_shape(64, 100)%16!=0>" in ctx.skipped_map[
+      "float8_per_tensor"]
+  for blk in net.blocks:
+    assert not getattr(blk.row_parallel, "_is_inner_quantized", False)
+    assert not getattr(blk.odd, "_is_inner_quantized", False)
+
+
+def test_failed_conversion_rolls_the_bookkeeping_back():
+  m = nn.Sequential(lin(), lin())
+  seen = []
+
+  def convert(linear, qt):
+    seen.append(linear)
+    if len(seen) == 2:
+      raise RuntimeError("boom")
+
+  with pytest.raises(RuntimeError, match="boom"):
+    quantize_ao(m, QuantizeConfig(exclude_layers=[]), _convert_fn=convert)
+  assert getattr(m[0], "_is_inner_quantized", False) and not getattr(m[1], "_is_inner_quantized", False)
+  assert not getattr(m, "_is_quantized", False)
+
+
+def test_dtype_overrides_other_than_e4m3fn_are_refused():
+  """The reference forwards weight_dtype / activation_dtype to torchao
+  (quantize_ao.py:548-555); only e4m3fn is built here."""
+  for key in ("weight_dtype", "activation_dtype"):
+    with pytest.raises(NotImplementedError, match=key):
+      quantize_ao(nn.Sequential(lin()), QuantizeConfig(exclude_layers=[]),
+                  _convert_fn=lambda l, qt: None, **{key: torch.float8_e5m2})
+  calls = []
+  quantize_ao(nn.Sequential(lin()), QuantizeConfig(exclude_layers=[]),
+              _convert_fn=lambda l, qt: calls.append(qt), weight_dtype=torch.float8_e4m3fn)
+  assert calls == ["float8_per_row"]
 
 
 def test_bad_quant_types():
