@@ -65,6 +65,38 @@ def flux_step_linears():
   return out
 
 
+def qwen_step_linears():
+  """The 720 quantized Linears of one Qwen-Image-shaped step (benchmark config 4: 60
+  blocks, 83 x 83 = 6889 image + 256 text tokens, hidden 3072, MLP 12288); layer names as
+  in diffusers' QwenImageTransformer2DModel. `img_mod.1` / `txt_mod.1` stay bf16 (the
+  default exclude pattern "mod")."""
+  img, txt, d, mlp = 6889, 256, 3072, 12288
+  block = [
+      ("attn.to_q", img, d, d, False), ("attn.to_k", img, d, d, False),
+      ("attn.to_v", img, d, d, False), ("attn.to_out.0", img, d, d, False),
+      ("img_mlp.net.0.proj", img, d, mlp, True), ("img_mlp.net.2", img, mlp, d, False),
+      ("attn.add_q_proj", txt, d, d, False), ("attn.add_k_proj", txt, d, d, False),
+      ("attn.add_v_proj", txt, d, d, False), ("attn.to_add_out", txt, d, d, False),
+      ("txt_mlp.net.0.proj", txt, d, mlp, True), ("txt_mlp.net.2", txt, mlp, d, False),
+  ]
+  return [(f"transformer_blocks.{i}.{n}", M, K, N, g) for i in range(60) for n, M, K, N, g in block]
+
+
+def wan_step_linears():
+  """The 400 quantized Linears of one Wan2.1-14B-shaped step (benchmark config 5: 40
+  layers, 21 x 30 x 52 = 32760 video tokens, 512 text tokens, hidden 5120, FFN 13824);
+  layer names as in diffusers' WanTransformer3DModel."""
+  vid, txt, d, ffn = 32760, 512, 5120, 13824
+  block = [
+      ("attn1.to_q", vid, d, d, False), ("attn1.to_k", vid, d, d, False),
+      ("attn1.to_v", vid, d, d, False), ("attn1.to_out.0", vid, d, d, False),
+      ("attn2.to_q", vid, d, d, False), ("attn2.to_k", txt, d, d, False),
+      ("attn2.to_v", txt, d, d, False), ("attn2.to_out.0", vid, d, d, False),
+      ("ffn.net.0.proj", vid, d, ffn, True), ("ffn.net.2", vid, ffn, d, False),
+  ]
+  return [(f"blocks.{i}.{n}", M, K, N, g) for i in range(40) for n, M, K, N, g in block]
+
+
 def _rand_fp8(shape, gen, device):
   import torch
   # random e4m3 codes with |value| <= 1.75 (exponent field <= 7): no NaN codes
@@ -75,16 +107,18 @@ def _rand_fp8(shape, gen, device):
 class HotPath:
   """All quantized Linears of one step, each with its own weight."""
 
-  def __init__(self, device):
+  def __init__(self, device, linears=None, mode="w8a8"):
     import torch
     from cache_dit_amd import _native
     self.torch = torch
     self.native = _native
+    self.mode = mode
+    self.linears = flux_step_linears() if linears is None else linears
     g = torch.Generator(device=device).manual_seed(0)
     self.layers = []
     self.flop = 0
     max_mk, max_mn = {}, 0
-    for name, M, K, N, gelu in flux_step_linears():
+    for name, M, K, N, gelu in self.linears:
       w = _rand_fp8((N, K), g, device)
       ws = torch.rand(N, device=device, generator=g) * 1e-3 + 1e-4
       b = (torch.randn(N, device=device, generator=g) * 0.01).to(torch.bfloat16)
@@ -102,6 +136,10 @@ class HotPath:
     """One pass: for every Linear the same library call its module forward makes
     (quantizer + GEMM enqueued by cdit_fp8_linear_w8a8)."""
     from cache_dit_amd import ops
+    if self.mode == "w8a16":  # weight-only: bf16 activations straight into the GEMM
+      for M, K, N, w, ws, b, epi in self.layers:
+        ops.w8a16_into(self.x[(M, K)], w, ws, b, self.out[:M * N].view(M, N), epi)
+      return
     for M, K, N, w, ws, b, epi in self.layers:
       out = self.out[:M * N].view(M, N)
       ops.linear_w8a8_into(self.x[(M, K)], w, ws, b, out, self.q[(M, K)], self.s[(M, K)], 0, epi)
@@ -111,7 +149,7 @@ class HotPath:
     proj_mlp in single blocks) read one activation, as share_activation_quant_
     arranges in a real model. Outputs are bit-identical to step()."""
     from cache_dit_amd import ops
-    names = [n for n, *_ in flux_step_linears()]
+    names = [n for n, *_ in self.linears]
     for name, (M, K, N, w, ws, b, epi) in zip(names, self.layers):
       out = self.out[:M * N].view(M, N)
       leaf = name.split(".", 2)[2]
@@ -120,6 +158,32 @@ class HotPath:
       if not reuse:
         ops.quant_rowwise_into(self.x[(M, K)], self.q[(M, K)], self.s[(M, K)], 0, gemm_follows=True)
       ops.gemm_rowwise_into(self.q[(M, K)], self.s[(M, K)], w, ws, b, out, epi)
+
+
+def step_leg(device, linears, mode, steps, warmup):
+  """A step of another benchmark configuration (every quantized Linear of the model at
+  its real shape with its own weights), captured into a hipGraph and replayed like the
+  headline step. Returns ms per step, TFLOP/s and the Linear count."""
+  import torch
+  hot = HotPath(device, linears, mode)
+  hot.step()
+  torch.cuda.synchronize()
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    hot.step()
+  for _ in range(warmup):
+    graph.replay()
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(steps):
+    graph.replay()
+  torch.cuda.synchronize()
+  ms = (time.perf_counter() - t0) / steps * 1e3
+  res = {"ms_per_step": ms, "tflops": hot.flop / ms / 1e9, "linears": len(hot.layers),
+         "linear_flop_per_step": hot.flop}
+  del graph, hot
+  torch.cuda.empty_cache()
+  return res
 
 
 def _time_events(fn, iters, warmup):
@@ -304,6 +368,9 @@ def main():
   ap.add_argument("--warmup", type=int, default=3)
   ap.add_argument("--skip-cpu", action="store_true", help="skip the cpu_baseline leg")
   ap.add_argument("--skip-dit", action="store_true", help="skip the full-transformer forward")
+  ap.add_argument("--skip-other-configs", action="store_true",
+                  help="skip the step legs of the other benchmark configurations (FLUX-shaped "
+                       "w8a16, Qwen-Image-shaped and Wan-shaped w8a8)")
   ap.add_argument("--headline-only", action="store_true",
                   help="run only the headline-shape kernels (the roofline legs) and print their "
                        "figures: the command to put under rocprofv3 when per-kernel averages "
@@ -413,6 +480,15 @@ def main():
       "frac": head["quant_gbps"] / HBM_PEAK_GBPS,
       "traffic": 42.66e6,  # same source; algorithmic 3MK + 4M = 42.49 MB
   }
+  other = {}
+  if not args.skip_other_configs:
+    few = max(2, args.steps // 3)  # these steps are long; a few replays settle them
+    other["w8a16_step"] = step_leg(device, flux_step_linears(), "w8a16", args.steps, args.warmup)
+    other["w8a16_step"]["frac_bf16_peak"] = other["w8a16_step"]["tflops"] / BF16_PEAK_TFLOPS
+    other["qwen_step"] = step_leg(device, qwen_step_linears(), "w8a8", few, 1)
+    other["wan_step"] = step_leg(device, wan_step_linears(), "w8a8", few, 1)
+    for k in ("qwen_step", "wan_step"):
+      other[k]["frac_fp8_peak"] = other[k]["tflops"] / FP8_PEAK_TFLOPS
   dit_ms, dit_note = (None, "skipped") if args.skip_dit else dit_forward_ms(device)
   cpu = None if args.skip_cpu else cpu_baseline()
 
@@ -443,6 +519,17 @@ def main():
       "eager_ms_per_step": eager_ms,
       "shared_quant_ms_per_step": shared_ms,
       "linear_headline": head,
+      # the other benchmark configurations as steps of their own (same construction as the
+      # headline step): config 3 = FLUX-shaped w8a16, config 4 = Qwen-Image-shaped w8a8,
+      # config 5 = Wan2.1-14B-shaped w8a8
+      "w8a16_step_ms": other.get("w8a16_step", {}).get("ms_per_step"),
+      "w8a16_step_tflops": other.get("w8a16_step", {}).get("tflops"),
+      "w8a16_step_frac_bf16_peak": other.get("w8a16_step", {}).get("frac_bf16_peak"),
+      "qwen_step_ms": other.get("qwen_step", {}).get("ms_per_step"),
+      "qwen_step_tflops": other.get("qwen_step", {}).get("tflops"),
+      "wan_step_ms": other.get("wan_step", {}).get("ms_per_step"),
+      "wan_step_tflops": other.get("wan_step", {}).get("tflops"),
+      "other_configs": other,
       "dit_step_ms": dit_ms,
       "dit_step_note": dit_note,
       "roofline": roofline,

@@ -143,11 +143,17 @@ def test_reference_partition_shape_m512_k3072_n3072():
   _assert_close(_run(*p), to.scaled_mm_rowwise(*p))
 
 
-@pytest.mark.parametrize("M,N,K", [(6889, 3072, 3072), (6889, 12288, 3072), (32760, 5120, 5120),
-                                   (32760, 13824, 5120), (4608, 3072, 15360)])
+@pytest.mark.parametrize("M,N,K", [
+    (6889, 3072, 3072), (6889, 12288, 3072), (6889, 3072, 12288),  # Qwen-Image image stream
+    (256, 3072, 3072), (256, 12288, 3072), (256, 3072, 12288),  # Qwen-Image text stream
+    (32760, 5120, 5120), (32760, 13824, 5120), (32760, 5120, 13824),  # Wan2.1-14B
+    (512, 5120, 5120),  # Wan cross-attention to_k / to_v (text tokens)
+    (4608, 3072, 15360), (4608, 12288, 3072),  # FLUX proj_out and the headline shape
+])
 def test_qwen_and_wan_shapes_sampled_rows(M, N, K):
-  """Odd token counts of the other benchmark models (Qwen-Image 6889 = 83 x 83, Wan
-  32760 = 8 x 4095) at full size: every 97th row plus the last rows against the oracle."""
+  """Every (M, N, K) of the Qwen-Image and Wan2.1-14B blocks (odd token counts: 6889 =
+  83 x 83, 32760 = 8 x 4095) and the FLUX headline shape, at full size: every 97th row
+  plus the last rows against the CPU oracle."""
   from cache_dit_amd import ops
   g = torch.Generator(device="cuda").manual_seed(M + N)
   x = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)

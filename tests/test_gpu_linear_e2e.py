@@ -270,3 +270,58 @@ def test_full_flux_shaped_step_cosine():
   assert torch.isfinite(y.float()).all()
   assert c_ref >= 0.999, c_ref
   assert c_bf16 >= 0.99, c_bf16
+
+
+def _full_size_step(model_cls, inputs_fn, n_quantized, n_skipped):
+  """One full-size step of a benchmark model: the HIP path against the oracle's
+  arithmetic in torch ops on the same GPU, and against the unquantized bf16 model."""
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd.testing import dit_shapes as ds
+  torch.manual_seed(0)
+  with torch.device("cuda"):
+    model = model_cls().to(torch.bfloat16)
+  inputs = inputs_fn("cuda")
+  with torch.inference_mode():
+    y_bf16 = model(**inputs)
+  cache_dit.quantize(model, cache_dit.QuantizeConfig(verbose=True))
+  ctx = model._quantize_context
+  total, quantized = ds.count_linears(model)
+  assert quantized == n_quantized == ctx.quantized_map["float8_per_row"]
+  assert sum(len(v) for v in ctx.skipped_map.values()) == n_skipped
+  with torch.inference_mode():
+    y = model(**inputs)
+  y_ref = _oracle_ops_forward(model, inputs, "cuda")
+  c_ref, c_bf16 = cosine(y, y_ref), cosine(y, y_bf16)
+  print(f"{model_cls.__name__} full-size step: cosine vs oracle ops {c_ref:.6f}, vs bf16 "
+        f"{c_bf16:.6f}", flush=True)
+  assert torch.isfinite(y.float()).all()
+  assert c_ref >= 0.999, c_ref
+  assert c_bf16 >= 0.99, c_bf16
+  # with GELU-tanh folded into the producing Linear and shared activation quantization,
+  # as the benchmark runs the model
+  ds.fuse_gelu_epilogues(model)
+  cache_dit.share_activation_quant_(model)
+  with torch.no_grad():
+    y_fast = model(**inputs)
+  cache_dit.share_activation_quant_(model, False)
+  assert cosine(y_fast, y_ref) >= 0.999
+  return model
+
+
+def test_full_qwen_image_shaped_step_cosine():
+  """benchmark config 4 at full size: 60 blocks, 6889 image + 256 text tokens, hidden
+  3072, MLP 12288; 12 quantized Linears per block, `img_mod.1` / `txt_mod.1` skipped by
+  the default "mod" pattern (layer inventory:
+  src/cache_dit/distributed/transformers/qwen_image.py:119-134)."""
+  from cache_dit_amd.testing import dit_shapes as ds
+  model = _full_size_step(ds.QwenImageLikeTransformer, ds.qwen_image_like_inputs, 720, 120)
+  blk = model.transformer_blocks[0]
+  assert type(blk.img_mod[1]) is nn.Linear and blk.img_mod[1].weight.dtype == torch.bfloat16
+
+
+def test_full_wan_shaped_step_cosine():
+  """benchmark config 5 at full size: 40 layers, 32760 video + 512 text tokens, hidden
+  5120, FFN 13824; 10 quantized Linears per block (layer inventory:
+  src/cache_dit/distributed/transformers/wan.py:284-293)."""
+  from cache_dit_amd.testing import dit_shapes as ds
+  _full_size_step(ds.WanLikeTransformer, ds.wan_like_inputs, 400, 0)
