@@ -22,6 +22,7 @@ QUANT_GEMM_FOLLOWS = 0x100  # cache hint, OR-ed into the scale mode of the per-r
 EPI_NONE = 0
 EPI_GELU_TANH = 1
 DT_F16, DT_BF16, DT_F32 = 0, 1, 2
+STATIC_WS_CODE_BYTES, STATIC_WS_ROWS = 96 << 20, 65536  # cdit_fp8_linear_w8a8_static
 
 #: every symbol include/cdit_hip.h declares
 EXPORTS = (
@@ -33,6 +34,7 @@ EXPORTS = (
     "cdit_fp8_gemm_rowwise",
     "cdit_w8a16_gemm",
     "cdit_fp8_linear_w8a8",
+    "cdit_fp8_linear_w8a8_static",
     "cdit_set_gemm_variant",
 )
 
@@ -64,6 +66,9 @@ def _bind(L: ctypes.CDLL) -> None:
   L.cdit_fp8_linear_w8a8.restype = ci
   L.cdit_fp8_linear_w8a8.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci,
                                      ci, vp]
+  L.cdit_fp8_linear_w8a8_static.restype = ci
+  L.cdit_fp8_linear_w8a8_static.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci,
+                                            ci, vp]
   L.cdit_w8a16_gemm.restype = ci
   L.cdit_w8a16_gemm.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, vp]
 

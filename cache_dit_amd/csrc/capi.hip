@@ -6,6 +6,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "cdit_internal.h"
 
 namespace cdit {
@@ -283,6 +285,73 @@ int cdit_fp8_linear_w8a8(const void* x_bf16, const void* w_q, const float* w_sca
   if (rc) return rc;
   return cdit_fp8_gemm_rowwise(q_ws, scale_ws, w_q, w_scale, bias, out, M, N, K, K, ldw, ldo,
                                epilogue, out_dtype_id, stream);
+}
+
+// ---- allocation-free Linear: activation codes and scales in a library-owned array
+// One copy of the array lives on every GPU the library runs on, for the life of the
+// process. Host code never uses the array's name as an address (it is a host-side
+// stand-in): the device address is looked up once per device and kept.
+static __device__ __align__(256) uint8_t scratch[CDIT_STATIC_WS_CODE_BYTES +
+                                                 CDIT_STATIC_WS_ROWS * sizeof(float)];
+
+// Device address of `scratch` on the current device (looked up on the first call on that
+// device, with the device current), or nullptr with the error set.
+static uint8_t* static_scratch_of_current_device() {
+  static std::mutex mu;
+  static uint8_t* ptr[64];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    set_error("hipGetDevice: %s", hipGetErrorString(e));
+    return nullptr;
+  }
+  if (dev < 0 || dev >= 64) {
+    set_error("device ordinal %d out of range", dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      set_error("hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    ptr[dev] = static_cast<uint8_t*>(p);
+  }
+  return ptr[dev];
+}
+
+int cdit_fp8_linear_w8a8_static(const void* x_bf16, const void* w_q, const float* w_scale,
+                                const void* bias, void* out, int64_t M, int64_t N, int64_t K,
+                                int64_t ld_x, int64_t ldw, int64_t ldo, int scale_mode,
+                                int epilogue, int out_dtype_id, void* stream) {
+  const char* fn = "cdit_fp8_linear_w8a8_static";
+  if (M < 0 || K < 0 || N < 0) {
+    set_error("%s: negative dimension (M=%lld N=%lld K=%lld)", fn, (long long)M, (long long)N,
+              (long long)K);
+    return CDIT_EINVAL;
+  }
+  if (M > CDIT_STATIC_WS_ROWS || (K > 0 && M > CDIT_STATIC_WS_CODE_BYTES / K)) {
+    set_error("%s: M=%lld K=%lld exceeds the built-in workspace (M*K <= %lld bytes of codes, M <= "
+              "%lld rows); use cdit_fp8_linear_w8a8 with workspaces of your own",
+              fn, (long long)M, (long long)K, (long long)CDIT_STATIC_WS_CODE_BYTES,
+              (long long)CDIT_STATIC_WS_ROWS);
+    return CDIT_EINVAL;
+  }
+  if (M == 0 || N == 0) {
+    // nothing to compute; the arguments still get the checks of the full entry point
+    return check_gemm(fn, x_bf16, w_q, w_scale, bias, out, M, N, K, K, ldw, ldo, epilogue,
+                      out_dtype_id, false);
+  }
+  int rc = check_arch();
+  if (rc) return rc;
+  uint8_t* ws = static_scratch_of_current_device();
+  if (!ws) return CDIT_EHIP;
+  // codes first (contiguous rows of K bytes), scales behind them at a fixed, aligned offset
+  return cdit_fp8_linear_w8a8(x_bf16, w_q, w_scale, bias, out, ws,
+                              reinterpret_cast<float*>(ws + CDIT_STATIC_WS_CODE_BYTES), M, N, K,
+                              ld_x, ldw, ldo, scale_mode, epilogue, out_dtype_id, stream);
 }
 
 int cdit_w8a16_gemm(const void* x_bf16, const void* b_q, const float* b_scale,

@@ -181,6 +181,31 @@ int cdit_fp8_linear_w8a8(const void* x_bf16, const void* w_q, const float* w_sca
                          int scale_mode, int epilogue, int out_dtype_id, void* stream);
 
 /*
+ * cdit_fp8_linear_w8a8 without the two workspace arguments: the activation codes and
+ * scales go to an array inside the library (device memory that every GPU the library
+ * runs on holds from the first call on it until the process ends:
+ * CDIT_STATIC_WS_CODE_BYTES + 4 * CDIT_STATIC_WS_ROWS bytes). The call allocates and
+ * frees nothing, neither on the host nor on the device.
+ * This entry point has no counterpart in the reference. It is for callers that cannot
+ * allocate: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.
+ * Limits: M * K <= CDIT_STATIC_WS_CODE_BYTES and M <= CDIT_STATIC_WS_ROWS, else
+ * CDIT_EINVAL with a message and nothing is launched. All calls on one GPU share that
+ * GPU's array: calls that overlap in time on one GPU (different streams, different
+ * threads) race on it, so keep them on one stream or order them yourself. Nothing in
+ * the array has to be cleared between calls: every call overwrites the M rows of codes
+ * and the M scales it reads afterwards. Results are those of cdit_fp8_linear_w8a8, bit
+ * for bit (the same kernels run).
+ */
+#define CDIT_STATIC_WS_CODE_BYTES ((int64_t)96 << 20) /* 96 MiB: 6889 x 12288 and smaller */
+#define CDIT_STATIC_WS_ROWS ((int64_t)65536)
+int cdit_fp8_linear_w8a8_static(const void* x_bf16, const void* w_q, const float* w_scale,
+                                const void* bias, void* out,
+                                int64_t M, int64_t N, int64_t K,
+                                int64_t ld_x, int64_t ldw, int64_t ldo,
+                                int scale_mode, int epilogue, int out_dtype_id, void* stream);
+
+/*
  * Tuning hook used by the benchmark and the tests: forces the kernel variant
  * the two GEMM entry points pick (-1 = automatic choice by shape). Returns
  * the previous value. Process-global; not meant for concurrent use.
