@@ -36,6 +36,7 @@ EXPORTS = (
     "cdit_fp8_linear_w8a8",
     "cdit_fp8_linear_w8a8_static",
     "cdit_set_gemm_variant",
+    "cdit_stream_capture_id",
 )
 
 _lib = None
@@ -54,6 +55,8 @@ def _bind(L: ctypes.CDLL) -> None:
   L.cdit_last_error.argtypes = []
   L.cdit_device_arch.restype = ci
   L.cdit_device_arch.argtypes = [ctypes.c_char_p, ci]
+  L.cdit_stream_capture_id.restype = ci
+  L.cdit_stream_capture_id.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64)]
   L.cdit_set_gemm_variant.restype = ci
   L.cdit_set_gemm_variant.argtypes = [ci]
   L.cdit_fp8_quant_rowwise.restype = ci
@@ -118,3 +121,10 @@ def device_arch() -> str:
 
 def set_gemm_variant(variant: int) -> int:
   return load().cdit_set_gemm_variant(int(variant))
+
+
+def stream_capture_id(stream: int) -> int:
+  """Id of the graph capture `stream` is recording into, 0 when it is not capturing."""
+  out = ctypes.c_uint64(0)
+  check(load().cdit_stream_capture_id(stream, ctypes.byref(out)))
+  return int(out.value)

@@ -131,6 +131,23 @@ int cdit_device_arch(char* buf, int buf_len) {
   return check_arch();
 }
 
+int cdit_stream_capture_id(void* stream, uint64_t* id) {
+  if (!id) {
+    set_error("cdit_stream_capture_id: id is null");
+    return CDIT_EINVAL;
+  }
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  unsigned long long cid = 0;
+  hipError_t e = hipStreamGetCaptureInfo(static_cast<hipStream_t>(stream), &status, &cid);
+  if (e != hipSuccess) {
+    set_error("hipStreamGetCaptureInfo: %s", hipGetErrorString(e));
+    return CDIT_EHIP;
+  }
+  // ids start at 1 in the runtime; make sure an active capture never reads as "none"
+  *id = status == hipStreamCaptureStatusActive ? (uint64_t)cid + 1 : 0;
+  return CDIT_OK;
+}
+
 int cdit_set_gemm_variant(int variant) {
   if (variant >= 1000) {  // 1000 + v: cache hints of the quantizer instead, 1999: automatic
     cdit::g_quant_variant = variant == 1999 ? -1 : variant - 1000;

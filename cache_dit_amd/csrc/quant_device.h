@@ -58,8 +58,11 @@ __device__ __forceinline__ float row_scale(uint32_t amax_bits, int scale_mode) {
   return s == 0.0f ? 1.0f : s;
 }
 
+// torch.clamp keeps NaN (fminf / fmaxf would drop it): a NaN quotient -- Inf / Inf in a
+// row that holds an infinity, anything in a row that holds a NaN -- must reach the
+// converter as NaN. Only the cold paths clamp.
 __device__ __forceinline__ float clamp448(float y) {
-  return fminf(fmaxf(y, -kFp8Max), kFp8Max);
+  return y != y ? y : fminf(fmaxf(y, -kFp8Max), kFp8Max);
 }
 
 // x / s with s > 0 finite. FAST: r = 1/s correctly rounded, s inside the window.

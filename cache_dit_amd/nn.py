@@ -59,35 +59,30 @@ class _Fp8LinearBase(nn.Linear):
             f"bias={self.bias is not None}, quant_type={self.quant_type}, "
             f"epilogue={'gelu_tanh' if self.epilogue & _native.EPI_GELU_TANH else 'none'}")
 
-  def _check_input(self, x: torch.Tensor) -> torch.Tensor:
+  def _check_input(self, x: torch.Tensor) -> None:
     if x.dtype != torch.bfloat16:
       raise ValueError(f"{type(self).__name__} takes bfloat16 activations, got {x.dtype}")
     if not x.is_cuda:
       raise RuntimeError(f"{type(self).__name__}: input is on {x.device}; there is no CPU path")
-    x2 = x.reshape(-1, self.in_features)
-    if x2.stride(-1) != 1:
-      x2 = x2.contiguous()
-    return x2
 
 
 class Fp8DynamicLinear(_Fp8LinearBase):
   """`float8_per_row` (w8a8 dynamic): per-token e4m3 activation quantization,
   e4m3 x e4m3 GEMM with fp32 accumulate, per-token x per-channel scales, bias,
-  optional fused GELU-tanh, bf16 out."""
+  optional fused GELU-tanh, bf16 out.
+
+  Every forward is one `torch.ops.cdit.*` call, so Dynamo and Inductor see a single
+  opaque node with a fake implementation, the way the reference keeps this path
+  traceable (src/cache_dit/quantization/torchao/_scaled_mm.py:94-137, :338-357)."""
 
   def forward(self, x: torch.Tensor) -> torch.Tensor:
-    x2 = self._check_input(x)
-    M = x2.shape[0]
-    out = torch.empty((M, self.out_features), dtype=torch.bfloat16, device=x2.device)
-    if M > 0:
-      if self.share_input_quant:
-        q, s = ops.shared_activation_quant(x2, self._scale_mode_id)
-        ops.gemm_rowwise_into(q, s, self.weight, self.weight_scale, self.bias, out, self.epilogue)
-      else:
-        q, s = ops.activation_workspace(M, self.in_features, x2.device)
-        ops.linear_w8a8_into(x2, self.weight, self.weight_scale, self.bias, out, q, s,
-                             self._scale_mode_id, self.epilogue)
-    return out.view(*x.shape[:-1], self.out_features)
+    self._check_input(x)
+    # sharing keeps the last activation's codes alive between calls; a compiled graph gets
+    # the stateless form (its front end owns the memory its graphs are captured into)
+    share = self.share_input_quant and not torch.compiler.is_compiling()
+    return torch.ops.cdit.linear_w8a8(x, self.weight, self.weight_scale, self.bias,
+                                      self._scale_mode_id, self.epilogue,
+                                      ops.GRANULARITY_PER_ROW, share)
 
 
 class Fp8DynamicLinearPerTensor(_Fp8LinearBase):
@@ -97,15 +92,10 @@ class Fp8DynamicLinearPerTensor(_Fp8LinearBase):
   and the GEMM is the per-row one fed with constant scales."""
 
   def forward(self, x: torch.Tensor) -> torch.Tensor:
-    x2 = self._check_input(x)
-    M = x2.shape[0]
-    out = torch.empty((M, self.out_features), dtype=torch.bfloat16, device=x2.device)
-    if M > 0:
-      q, s = ops.activation_workspace(M, self.in_features, x2.device)
-      ws = ops.amax_workspace(x2.device)
-      ops.quant_tensorwise_into(x2, q, s, ws, self._scale_mode_id)
-      ops.gemm_rowwise_into(q, s, self.weight, self.weight_scale, self.bias, out, self.epilogue)
-    return out.view(*x.shape[:-1], self.out_features)
+    self._check_input(x)
+    return torch.ops.cdit.linear_w8a8(x, self.weight, self.weight_scale, self.bias,
+                                      self._scale_mode_id, self.epilogue,
+                                      ops.GRANULARITY_PER_TENSOR, False)
 
 
 class Fp8WeightOnlyLinear(_Fp8LinearBase):
@@ -113,12 +103,9 @@ class Fp8WeightOnlyLinear(_Fp8LinearBase):
   the GEMM mainloop, per-channel scale in the epilogue."""
 
   def forward(self, x: torch.Tensor) -> torch.Tensor:
-    x2 = self._check_input(x)
-    M = x2.shape[0]
-    out = torch.empty((M, self.out_features), dtype=torch.bfloat16, device=x2.device)
-    if M > 0:
-      ops.w8a16_into(x2, self.weight, self.weight_scale, self.bias, out, self.epilogue)
-    return out.view(*x.shape[:-1], self.out_features)
+    self._check_input(x)
+    return torch.ops.cdit.w8a16_mm(x, self.weight.t(), self.weight_scale, self.bias,
+                                   _native.DT_BF16, self.epilogue)
 
 
 _CLASS_OF = {

@@ -62,44 +62,19 @@ class _DeviceOf:
       self.guard.__exit__(*exc)
 
 
-_workspaces: dict = {}
-
-
 def activation_workspace(M: int, K: int, device: torch.device):
-  """(codes [M,K] e4m3, scales [M] fp32) scratch for one Linear forward. Outside
-  graph capture one growable buffer per (device, stream) is reused: every use is
-  ordered on that stream, so the GEMM that consumes it has been enqueued before
-  the next quantizer overwrites it. During capture fresh tensors come from the
-  graph's own pool."""
-  if torch.cuda.is_current_stream_capturing():
-    return (torch.empty((M, K), dtype=FP8, device=device),
-            torch.empty((M, ), dtype=torch.float32, device=device))
-  key = (device.index, torch._C._cuda_getCurrentRawStream(device.index))
-  ws = _workspaces.get(key)
-  if ws is None or ws[0].numel() < M * K or ws[1].numel() < M:
-    nq = max(M * K, ws[0].numel() if ws else 0)
-    ns = max(M, ws[1].numel() if ws else 0)
-    ws = (torch.empty(nq, dtype=FP8, device=device), torch.empty(ns, dtype=torch.float32,
-                                                                device=device))
-    _workspaces[key] = ws
-  return ws[0][:M * K].view(M, K), ws[1][:M]
-
-
-_amax_workspaces: dict = {}
+  """(codes [M,K] e4m3, scales [M] fp32) scratch for one Linear forward, fresh from
+  PyTorch's caching allocator: a block freed on a stream is handed out again on that
+  stream, so consecutive Linears reuse the same memory without this module keeping any
+  buffer alive (a module-level buffer created while a graph-capturing front end warms up
+  inside its private pool would be an allocation that pool never sees released)."""
+  return (torch.empty((M, K), dtype=FP8, device=device),
+          torch.empty((M, ), dtype=torch.float32, device=device))
 
 
 def amax_workspace(device: torch.device) -> torch.Tensor:
-  """4 bytes of device scratch for the per-tensor quantizer, one per (device,
-  stream) outside graph capture (uses are ordered on the stream), fresh from the
-  graph's pool during capture."""
-  if torch.cuda.is_current_stream_capturing():
-    return torch.empty((1,), dtype=torch.int32, device=device)
-  key = (device.index, torch._C._cuda_getCurrentRawStream(device.index))
-  ws = _amax_workspaces.get(key)
-  if ws is None:
-    ws = torch.empty((1,), dtype=torch.int32, device=device)
-    _amax_workspaces[key] = ws
-  return ws
+  """4 bytes of device scratch for the per-tensor quantizer."""
+  return torch.empty((1,), dtype=torch.int32, device=device)
 
 
 def _require_cuda(name: str, *tensors: Optional[torch.Tensor]) -> None:
@@ -165,9 +140,9 @@ def w8a16_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
 
 class _SharedQuant:
   """Last activation quantized on a (device, stream): the input view (kept alive, so
-  its storage cannot be freed and handed out again), its version counter, and the
-  codes / scales computed from it."""
-  __slots__ = ("x", "version", "mode", "q", "s")
+  its storage cannot be freed and handed out again), its version counter, the codes /
+  scales computed from it, and the id of the graph capture it was made in (0: none)."""
+  __slots__ = ("x", "version", "mode", "q", "s", "capture_id")
 
 
 _shared_quant: dict = {}
@@ -194,9 +169,15 @@ def shared_activation_quant(x2: torch.Tensor, scale_mode_id: int):
     quant_rowwise_into(x2, q, s, scale_mode_id, gemm_follows=True)
     quant_launches += 1
     return q, s
-  key = (dev.index, torch._C._cuda_getCurrentRawStream(dev.index),
-         torch.cuda.is_current_stream_capturing())
+  capturing = torch.cuda.is_current_stream_capturing()
+  # an entry made during a graph capture belongs to that capture alone: its codes live in
+  # that graph's pool and are only valid inside replays of that graph
+  capture_id = _native.stream_capture_id(_stream_ptr(x2)) if capturing else 0
+  key = (dev.index, torch._C._cuda_getCurrentRawStream(dev.index))
   e = _shared_quant.get(key)
+  if e is not None and e.capture_id != capture_id:
+    e = None  # made in another capture, or on the other side of a capture boundary
+    del _shared_quant[key]
   if (e is not None and e.mode == scale_mode_id and e.version == x2._version
       and e.x.data_ptr() == x2.data_ptr() and e.x.shape == x2.shape
       and e.x.stride() == x2.stride()
@@ -211,6 +192,7 @@ def shared_activation_quant(x2: torch.Tensor, scale_mode_id: int):
     e = _SharedQuant()
     _shared_quant[key] = e
   e.x, e.version, e.mode, e.q, e.s = x2, x2._version, scale_mode_id, q, s
+  e.capture_id = capture_id
   return q, s
 
 
@@ -244,6 +226,11 @@ torch.library.define(
     "cdit::float8_inference_scaled_mm",
     "(Tensor a_data, Tensor a_scale, Tensor b_data, Tensor b_scale, Tensor? bias, "
     "int out_dtype_id, bool use_fast_accum, int epilogue=0) -> Tensor",
+)
+torch.library.define(
+    "cdit::linear_w8a8",
+    "(Tensor x, Tensor weight, Tensor weight_scale, Tensor? bias, int scale_mode=0, "
+    "int epilogue=0, int granularity=0, bool share_input_quant=False) -> Tensor",
 )
 torch.library.define(
     "cdit::w8a16_mm",
@@ -292,6 +279,19 @@ def _weight_rows(b_data: torch.Tensor, name: str) -> torch.Tensor:
   return w
 
 
+def _aligned16(t: torch.Tensor) -> torch.Tensor:
+  """The tuned kernels fetch scales and bias in 16-byte pieces; a slice that starts
+  elsewhere is copied once rather than sent to the element-wise kernel."""
+  return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
+def _scale_vector(scale: torch.Tensor, n: int) -> torch.Tensor:
+  s = scale.reshape(-1).to(torch.float32)
+  if s.numel() == 1 and n != 1:
+    s = s.expand(n)
+  return _aligned16(s.contiguous())
+
+
 @torch.library.impl("cdit::float8_inference_scaled_mm", "CUDA")
 def _float8_inference_scaled_mm(a_data, a_scale, b_data, b_scale, bias, out_dtype_id,
                                 use_fast_accum, epilogue=0):
@@ -307,11 +307,13 @@ def _float8_inference_scaled_mm(a_data, a_scale, b_data, b_scale, bias, out_dtyp
   N = w.shape[0]
   if w.shape[1] != K:
     raise ValueError(f"{name}: shape mismatch a {tuple(a_data.shape)} x b {tuple(b_data.shape)}")
-  if a_scale.numel() != M or b_scale.numel() != N:
-    raise ValueError(f"{name}: expected a_scale with {M} and b_scale with {N} elements, got "
-                     f"{a_scale.numel()} and {b_scale.numel()}")
-  a_s = a_scale.reshape(-1).to(torch.float32).contiguous()
-  b_s = b_scale.reshape(-1).to(torch.float32).contiguous()
+  if a_scale.numel() not in (1, M) or b_scale.numel() not in (1, N):
+    raise ValueError(f"{name}: expected a_scale with {M} (or 1) and b_scale with {N} (or 1) "
+                     f"elements, got {a_scale.numel()} and {b_scale.numel()}")
+  # a scalar scale is a tensor-wise one (how float8_per_tensor reaches the reference's op,
+  # which hands it to torch._scaled_mm as is): the kernel takes it as a constant vector
+  a_s = _scale_vector(a_scale, M)
+  b_s = _scale_vector(b_scale, N)
   if bias is not None and bias.numel() != N:
     raise ValueError(f"{name}: bias must have {N} elements")
   out = torch.empty((M, N), dtype=out_dtype, device=a_data.device)
@@ -324,7 +326,7 @@ def _float8_inference_scaled_mm(a_data, a_scale, b_data, b_scale, bias, out_dtyp
     out = out + bias.reshape(-1)
   else:
     if bias is not None:
-      bias = bias.reshape(-1).to(out_dtype).contiguous()
+      bias = _aligned16(bias.reshape(-1).to(out_dtype).contiguous())
     gemm_rowwise_into(a2, a_s, w, b_s, bias, out, int(epilogue))
   return out.reshape(*a_data.shape[:-1], N)
 
@@ -334,6 +336,61 @@ def _fake_float8_inference_scaled_mm(a_data, a_scale, b_data, b_scale, bias, out
                                      use_fast_accum, epilogue=0):
   return a_data.new_empty((*a_data.shape[:-1], b_data.shape[-1]),
                           dtype=decode_output_dtype(out_dtype_id))
+
+
+GRANULARITY_PER_ROW, GRANULARITY_PER_TENSOR = 0, 1
+
+
+@torch.library.impl("cdit::linear_w8a8", "CUDA")
+def _linear_w8a8(x, weight, weight_scale, bias, scale_mode=0, epilogue=0, granularity=0,
+                 share_input_quant=False):
+  """One quantized nn.Linear forward in the w8a8 dynamic modes as a single opaque op, what
+  the reference gets by keeping torchao's Float8Tensor `aten.linear` behind one
+  `torch.library` op (src/cache_dit/quantization/torchao/_scaled_mm.py:94-137, patched in
+  at :338-357): x bf16 [..., K], weight e4m3 [N, K] (the nn.Linear layout), weight_scale
+  fp32 with N elements, bias bf16 [N] or None -> bf16 [..., N]. granularity 0: per-token
+  activation scales, 1: one scale for the whole activation. Workspaces are taken inside
+  the op, so a traced graph only sees tensors in and a tensor out."""
+  name = "cdit::linear_w8a8"
+  if x.dtype != torch.bfloat16:
+    raise ValueError(f"{name}: x must be bfloat16, got {x.dtype}")
+  if weight.dtype != FP8 or weight.dim() != 2:
+    raise ValueError(f"{name}: weight must be float8_e4m3fn [N,K], got {weight.dtype} "
+                     f"{tuple(weight.shape)}")
+  N, K = weight.shape
+  if x.shape[-1] != K:
+    raise ValueError(f"{name}: shape mismatch x {tuple(x.shape)} x weight {tuple(weight.shape)}")
+  if scale_mode not in (0, 1) or granularity not in (0, 1):
+    raise ValueError(f"{name}: scale_mode and granularity must be 0 or 1")
+  if weight_scale.numel() != N or weight_scale.dtype != torch.float32:
+    raise ValueError(f"{name}: weight_scale must hold {N} float32 values")
+  if bias is not None and (bias.numel() != N or bias.dtype != torch.bfloat16):
+    raise ValueError(f"{name}: bias must hold {N} bfloat16 values")
+  x2 = _as_rows(x)
+  w = weight if weight.stride(-1) == 1 else weight.contiguous()
+  w_s = weight_scale if weight_scale.is_contiguous() else weight_scale.contiguous()
+  if bias is not None and not bias.is_contiguous():
+    bias = bias.contiguous()
+  M = x2.shape[0]
+  out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+  if M > 0:
+    if granularity == GRANULARITY_PER_TENSOR:
+      q, s = activation_workspace(M, K, x2.device)
+      quant_tensorwise_into(x2, q, s, amax_workspace(x2.device), int(scale_mode))
+      gemm_rowwise_into(q, s, w, w_s, bias, out, int(epilogue))
+    elif share_input_quant:
+      q, s = shared_activation_quant(x2, int(scale_mode))
+      gemm_rowwise_into(q, s, w, w_s, bias, out, int(epilogue))
+    else:
+      q, s = activation_workspace(M, K, x2.device)
+      linear_w8a8_into(x2, w, w_s, bias, out, q, s, int(scale_mode), int(epilogue))
+  return out.view(*x.shape[:-1], N)
+
+
+@torch.library.register_fake("cdit::linear_w8a8")
+def _fake_linear_w8a8(x, weight, weight_scale, bias, scale_mode=0, epilogue=0, granularity=0,
+                      share_input_quant=False):
+  return x.new_empty((*x.shape[:-1], weight.shape[0]), dtype=torch.bfloat16)
 
 
 @torch.library.impl("cdit::w8a16_mm", "CUDA")

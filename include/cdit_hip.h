@@ -206,6 +206,15 @@ int cdit_fp8_linear_w8a8_static(const void* x_bf16, const void* w_q, const float
                                 int scale_mode, int epilogue, int out_dtype_id, void* stream);
 
 /*
+ * Writes to *id the id of the graph capture that `stream` is recording into, 0 when it is
+ * not capturing. For bindings that keep per-stream state between calls (the Python
+ * binding reuses activation codes across sibling Linears): state made inside one capture
+ * is only valid inside that capture. No counterpart in the reference, whose op holds no
+ * state.
+ */
+int cdit_stream_capture_id(void* stream, uint64_t* id);
+
+/*
  * Tuning hook used by the benchmark and the tests: forces the kernel variant
  * the two GEMM entry points pick (-1 = automatic choice by shape). Returns
  * the previous value. Process-global; not meant for concurrent use.

@@ -84,6 +84,49 @@ def test_fake_impls_shapes_and_dtypes():
       assert y.shape == (154, 12288) and y.dtype == dt
     y = torch.ops.cdit.w8a16_mm(x, b, torch.empty(12288, device="cuda"), None, 1, 1)
     assert y.shape == (2, 77, 12288) and y.dtype == torch.bfloat16
+    w = torch.empty(12288, 3072, dtype=FP8, device="cuda")
+    y = torch.ops.cdit.linear_w8a8(x, w, torch.empty(12288, 1, device="cuda"), None)
+    assert y.shape == (2, 77, 12288) and y.dtype == torch.bfloat16 and y.device.type == "cuda"
+
+
+def _meta_quantized_linear(cls_name, in_f, out_f):
+  """A quantized Linear as convert_linear_ leaves it, built without a GPU (fake
+  tensors stand in for the codes)."""
+  from cache_dit_amd import _native, nn as cnn
+  lin = torch.nn.Linear(in_f, out_f, dtype=torch.bfloat16, device="cuda")
+  lin.weight = torch.nn.Parameter(torch.empty(out_f, in_f, dtype=torch.float8_e4m3fn,
+                                              device="cuda"), requires_grad=False)
+  lin.register_buffer("weight_scale", torch.empty(out_f, 1, device="cuda"))
+  lin.bias.requires_grad_(False)
+  lin.epilogue, lin.scale_mode, lin._scale_mode_id = _native.EPI_NONE, "bf16div", 0
+  lin.quant_type = "test"
+  lin.__class__ = getattr(cnn, cls_name)
+  return lin
+
+
+@pytest.mark.parametrize("cls_name", ["Fp8DynamicLinear", "Fp8DynamicLinearPerTensor",
+                                      "Fp8WeightOnlyLinear"])
+def test_quantized_linear_forward_traces_to_one_opaque_op(cls_name):
+  """The module forward is one torch.ops.cdit call: under FakeTensorMode (what Dynamo
+  and Inductor trace with) it needs no data pointer, no ctypes call and no library, and
+  make_fx records exactly one cdit node. Shapes of the reference's opaque-op test
+  (tests/kernels/test_opaque_scaled_mm.py:46-94): W[32,64], x[4,64]."""
+  import cache_dit_amd.ops  # noqa: F401
+  from torch._subclasses.fake_tensor import FakeTensorMode
+  from torch.fx.experimental.proxy_tensor import make_fx
+  with FakeTensorMode(allow_non_fake_inputs=False) as mode:
+    lin = _meta_quantized_linear(cls_name, 64, 32)
+    x = torch.empty(4, 64, dtype=torch.bfloat16, device="cuda")
+    y = lin(x)
+    assert y.shape == (4, 32) and y.dtype == torch.bfloat16
+    y3 = lin(torch.empty(2, 5, 64, dtype=torch.bfloat16, device="cuda"))
+    assert y3.shape == (2, 5, 32)
+    gm = make_fx(lambda t: lin(t), tracing_mode="fake")(x)
+  targets = [str(n.target) for n in gm.graph.nodes if n.op == "call_function"]
+  cdit = [t for t in targets if t.startswith("cdit.")]
+  assert len(cdit) == 1, targets
+  assert cdit[0] == ("cdit.w8a16_mm.default" if cls_name == "Fp8WeightOnlyLinear" else
+                     "cdit.linear_w8a8.default")
 
 
 def test_dtype_id_codec():

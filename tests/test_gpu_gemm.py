@@ -279,6 +279,26 @@ def test_against_torch_scaled_mm_on_gpu():
   assert torch.equal(out2, out)
 
 
+def test_scalar_scales_and_misaligned_scale_slices():
+  """Tensor-wise (one-element) scales are taken as the reference's op takes them, and a
+  scale vector that is a slice starting off a 16-byte boundary gives the same bits as an
+  aligned copy."""
+  from cache_dit_amd import ops
+  xq, xs, wq, ws, b = (t.cuda() if t is not None else None for t in _rand_problem(300, 520, 512, 11))
+  sa, sb = torch.tensor([[0.03125]], device="cuda"), torch.tensor([[0.5]], device="cuda")
+  out = ops.float8_inference_scaled_mm(xq, sa, wq.t(), sb, torch.bfloat16, bias=b)
+  ref = to.scaled_mm_rowwise(xq.cpu(), sa.cpu().expand(300, 1), wq.cpu(), sb.cpu().expand(520, 1),
+                             b.cpu())
+  _assert_close(out, ref)
+  pad_a = torch.cat([torch.zeros(1, device="cuda"), xs.reshape(-1)])
+  pad_b = torch.cat([torch.zeros(3, device="cuda"), ws.reshape(-1)])
+  assert pad_a[1:].data_ptr() % 16 != 0 and pad_b[3:].data_ptr() % 16 != 0
+  want = ops.float8_inference_scaled_mm(xq, xs, wq.t(), ws.t(), torch.bfloat16, bias=b)
+  got = ops.float8_inference_scaled_mm(xq, pad_a[1:].reshape(-1, 1), wq.t(), pad_b[3:].reshape(1, -1),
+                                       torch.bfloat16, bias=b)
+  assert torch.equal(got, want)
+
+
 def test_error_paths():
   from cache_dit_amd import ops
   a = torch.zeros(4, 64, device="cuda").to(FP8)

@@ -325,3 +325,186 @@ def test_full_wan_shaped_step_cosine():
   src/cache_dit/distributed/transformers/wan.py:284-293)."""
   from cache_dit_amd.testing import dit_shapes as ds
   _full_size_step(ds.WanLikeTransformer, ds.wan_like_inputs, 400, 0)
+
+
+class _OneLinear(nn.Module):
+
+  def __init__(self, k, n):
+    super().__init__()
+    self.proj = nn.Linear(k, n)
+
+  def forward(self, x):
+    return self.proj(x)
+
+
+@pytest.mark.parametrize("quant_type", ["float8_per_row", "float8_per_tensor", "float8_weight_only"])
+@pytest.mark.parametrize("M,K,N", [(4, 64, 32), (512, 3072, 3072)])
+def test_torch_compile_fullgraph_equals_eager(quant_type, M, K, N):
+  """torch.compile(fullgraph=True) of a quantized Linear: Dynamo traces the module
+  forward into the one opaque cdit op (fake implementation), Inductor calls it; the
+  output equals eager bit for bit. Shapes: the reference's opaque-op test W[32,64] /
+  x[4,64] (tests/kernels/test_opaque_scaled_mm.py:46-94) and its CUDA-graph partition
+  test M=512, K=N=3072; like the former, also with Inductor's own graph capture."""
+  import cache_dit_amd as cache_dit
+  torch.manual_seed(0)
+  net = _OneLinear(K, N).to(torch.bfloat16).cuda()
+  cache_dit.quantize(net, cache_dit.QuantizeConfig(quant_type=quant_type, exclude_layers=[]))
+  assert net.proj._is_inner_quantized
+  x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+  with torch.no_grad():
+    eager = net(x)
+    torch._dynamo.reset()
+    compiled = torch.compile(net, fullgraph=True)
+    assert torch.equal(compiled(x), eager)
+    x3 = torch.randn(2, M, K, device="cuda").to(torch.bfloat16)  # another rank: recompiles
+    assert torch.equal(compiled(x3), net(x3))
+    graphed = torch.compile(net, fullgraph=True, options={"triton.cudagraphs": True})
+    graphed(x)
+    out = graphed(x)
+    torch.cuda.synchronize()
+    assert torch.equal(out, eager)
+  torch._dynamo.reset()
+
+
+def test_torch_compile_of_a_block_with_glue_ops():
+  """A block with element-wise glue around three quantized Linears (one with GELU-tanh
+  folded into its epilogue) compiles without graph breaks: Dynamo records three cdit
+  nodes."""
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd.nn import fuse_gelu_tanh_
+  torch.manual_seed(0)
+  net = _Net().to(torch.bfloat16).cuda()
+  cache_dit.quantize(net, cache_dit.QuantizeConfig())
+  for blk in net.blocks:
+    fuse_gelu_tanh_(blk.proj_mlp, blk.act_mlp)
+  x = torch.randn(3, 70, 256, device="cuda").to(torch.bfloat16)
+  seen = []
+
+  def backend(gm, example_inputs):
+    seen.extend(str(n.target) for n in gm.graph.nodes if n.op == "call_function")
+    return gm.forward
+
+  with torch.no_grad():
+    eager = net(x)
+    torch._dynamo.reset()
+    out = torch.compile(net, fullgraph=True, backend=backend)(x)
+  torch._dynamo.reset()
+  assert torch.equal(out, eager)
+  assert sum(t.startswith("cdit.linear_w8a8") for t in seen) == 2 * 3, seen
+
+
+def test_shared_activation_quant_across_two_graph_captures():
+  """Codes cached inside one graph capture must not be handed to another capture: two
+  graphs of a share-enabled model, captured one after the other from the same static
+  input, both replay correctly with new data."""
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd.testing import dit_shapes as ds
+  torch.manual_seed(0)
+  kw = dict(dim=256, heads=2, mlp=512, n_double=1, n_single=1, in_channels=64, text_dim=128,
+            pooled_dim=64)
+  model = ds.FluxLikeTransformer(**kw).to(torch.bfloat16).cuda()
+  cache_dit.quantize(model, cache_dit.QuantizeConfig())
+  cache_dit.share_activation_quant_(model)
+  lin_q, lin_k = model.single_transformer_blocks[0].attn.to_q, model.single_transformer_blocks[0].attn.to_k
+  static_x = torch.randn(96, 256, device="cuda").to(torch.bfloat16)
+
+  def pair():
+    return lin_q(static_x), lin_k(static_x)
+
+  with torch.no_grad():
+    pair()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+      pair()
+    torch.cuda.current_stream().wait_stream(side)
+    graphs = []
+    for _ in range(2):  # same capture stream, same static input, unchanged _version
+      g = torch.cuda.CUDAGraph()
+      with torch.cuda.graph(g):
+        outs = pair()
+      graphs.append((g, outs))
+    for seed in range(3):
+      new_x = torch.randn(96, 256, device="cuda",
+                          generator=torch.Generator(device="cuda").manual_seed(seed)).to(torch.bfloat16)
+      cache_dit.share_activation_quant_(model, False)
+      want = (lin_q(new_x), lin_k(new_x))
+      cache_dit.share_activation_quant_(model)
+      torch.cuda.synchronize()
+      static_x.copy_(new_x)
+      for g, outs in reversed(graphs):  # the second graph must carry its own quantizer node
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0], want[0]) and torch.equal(outs[1], want[1]), seed
+        outs[0].zero_(), outs[1].zero_()
+  cache_dit.share_activation_quant_(model, False)
+
+
+class _PlanBlk(nn.Module):
+
+  def __init__(self, d):
+    super().__init__()
+    self.to_q, self.to_k, self.to_v = nn.Linear(d, d), nn.Linear(d, d), nn.Linear(d, d)
+    self.to_out = nn.ModuleList([nn.Linear(d, d), nn.Dropout(0.0)])
+    self.ff_in, self.ff_out = nn.Linear(d, 2 * d), nn.Linear(2 * d, d, bias=False)
+
+
+class _PlanNet(nn.Module):
+  _repeated_blocks = ["_PlanBlk"]
+
+  def __init__(self, d=128):
+    super().__init__()
+    self.blocks = nn.ModuleList([_PlanBlk(d), _PlanBlk(d)])
+
+
+def _oracle_linear(kind, x, weight, bias):
+  """x, weight bf16 on the CPU -> the oracle's output for a Linear of quant type `kind`."""
+  if kind == "float8_per_row":
+    return to.w8a8_linear(x, *to.quantize_rowwise(weight), bias)
+  if kind == "float8_weight_only":
+    return to.w8a16_linear(x, *to.quantize_rowwise(weight), bias)
+  assert kind == "float8_per_tensor"
+  wq, ws = to.quantize_tensorwise(weight)
+  xq, xs = to.quantize_tensorwise(x.reshape(-1, x.shape[-1]))
+  return to.scaled_mm_rowwise(xq, xs, wq, ws, bias).reshape(*x.shape[:-1], weight.shape[0])
+
+
+@pytest.mark.parametrize("with_plan", [True, False])
+def test_mixed_precision_plan_and_fallback_on_device(with_plan):
+  """A precision plan mixing per-row, per-tensor and weight-only Linears, with a
+  row-parallel layer that falls back to per-tensor (merged into the plan when there is
+  one, taken by the second pass when there is none), converted for real on the GPU:
+  every layer has the class its quant type asks for, its weight codes are the oracle's
+  and its forward agrees with the oracle's arithmetic for that type
+  (reference passes: src/cache_dit/quantization/torchao/quantize_ao.py:100-148)."""
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd import nn as cnn
+  torch.manual_seed(0)
+  net = _PlanNet().to(torch.bfloat16)
+  ref = copy.deepcopy(net)
+  net = net.cuda()
+  net._rowwise_layers = ["ff_out"]
+  plan = {"to_k": "float8_per_tensor", "to_v": "float8_weight_only"} if with_plan else None
+  cache_dit.quantize(net, cache_dit.QuantizeConfig(precision_plan=plan))
+  want = {"to_q": "float8_per_row", "to_out.0": "float8_per_row", "ff_in": "float8_per_row",
+          "to_k": "float8_per_tensor" if with_plan else "float8_per_row",
+          "to_v": "float8_weight_only" if with_plan else "float8_per_row",
+          "ff_out": "float8_per_tensor"}
+  classes = {"float8_per_row": cnn.Fp8DynamicLinear, "float8_per_tensor": cnn.Fp8DynamicLinearPerTensor,
+             "float8_weight_only": cnn.Fp8WeightOnlyLinear}
+  ctx = net._quantize_context
+  for kind in classes:
+    assert ctx.quantized_map[kind] == 2 * sum(v == kind for v in want.values()), (kind, ctx.quantized_map)
+  g = torch.Generator().manual_seed(1)
+  for blk, rblk in zip(net.blocks, ref.blocks):
+    for name, kind in want.items():
+      lin, rlin = blk.get_submodule(name), rblk.get_submodule(name)
+      assert type(lin) is classes[kind] and lin.quant_type == kind, (name, type(lin))
+      w = rlin.weight.detach()
+      wq, ws = (to.quantize_tensorwise if kind == "float8_per_tensor" else to.quantize_rowwise)(w)
+      assert (bits_u8(lin.weight) == bits_u8(wq)).all(), name
+      assert torch.equal(lin.weight_scale.cpu().reshape(-1), ws.reshape(-1)), name
+      x = torch.randn(3, 37, lin.in_features, generator=g).to(torch.bfloat16)
+      y = lin(x.cuda())
+      y_ref = _oracle_linear(kind, x, w, None if rlin.bias is None else rlin.bias.detach())
+      assert max_rel_err(y, y_ref) <= 1e-2, (name, kind, max_rel_err(y, y_ref))

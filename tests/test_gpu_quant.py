@@ -107,6 +107,15 @@ def test_non_finite_rows_stay_in_their_row(mode, K):
   s = s.reshape(-1).cpu()
   assert torch.isinf(s[3]) and torch.isinf(s[5]) and torch.isnan(s[8])
   assert torch.isinf(s_ref.reshape(-1)[3]) and torch.isnan(s_ref.reshape(-1)[8])
+  # the codes of those rows follow the reference arithmetic too: finite / Inf = +-0,
+  # Inf / Inf = NaN, anything / NaN = NaN, and torch.clamp keeps NaN
+  qb, qr = bits_u8(q), bits_u8(q_ref)
+  is_nan = lambda c: (c & 0x7f) == 0x7f  # noqa: E731  (0x7f / 0xff are e4m3fn's NaNs)
+  for row, col in ((3, 7), (5, K - 1)):
+    others = np.arange(K) != col
+    assert (qb[row][others] == qr[row][others]).all() and (qb[row][others] & 0x7f == 0).all()
+    assert is_nan(qb[row][col]) and is_nan(qr[row][col])
+  assert is_nan(qb[8]).all() and is_nan(qr[8]).all()
 
 
 @pytest.mark.parametrize("mode", MODES)
