@@ -186,6 +186,49 @@ def step_leg(device, linears, mode, steps, warmup):
   return res
 
 
+def pmc_sequence(device):
+  """Launch sequence for counter collection: run under `rocprofv3 --pmc FETCH_SIZE`, then
+  under `--pmc WRITE_SIZE`, each in a run of its own. Four times over: a 512 MiB fill (to
+  push earlier data out of the caches), a plain device copy of the bf16 activation (known
+  size: the scale of the counters), the quantizer on that activation, another fill, the
+  FP8 GEMM on the codes; all at the headline shape."""
+  import torch
+  from cache_dit_amd import ops
+  M, K, N = HEADLINE
+  g = torch.Generator(device=device).manual_seed(0)
+  x = [torch.randn(M, K, device=device, generator=g).to(torch.bfloat16) for _ in range(4)]
+  q = [torch.empty(M, K, dtype=torch.float8_e4m3fn, device=device) for _ in range(4)]
+  s = torch.empty(M, dtype=torch.float32, device=device)
+  w = [_rand_fp8((N, K), g, device) for _ in range(4)]
+  ws = torch.rand(N, device=device, generator=g) * 1e-3
+  b = torch.randn(N, device=device, generator=g).to(torch.bfloat16)
+  out = torch.empty(M, N, dtype=torch.bfloat16, device=device)
+  y = torch.empty(M, K, dtype=torch.bfloat16, device=device)
+  flush = torch.empty(1 << 29, dtype=torch.uint8, device=device)
+  for i in range(4):
+    flush.zero_()
+    y.copy_(x[i])  # plain copy: reads 2MK, writes 2MK bytes
+    flush.zero_()
+    ops.quant_rowwise_into(x[i], q[i], s, 0)
+    flush.zero_()
+    ops.gemm_rowwise_into(q[i], s, w[i], ws, b, out, 0)
+  torch.cuda.synchronize()
+
+
+def measured_traffic(kernel_key):
+  """HBM-side bytes per launch of a headline kernel from the committed counter summary
+  (profiles/traffic.json): FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by
+  the factor that makes the same counter read the known size for a plain copy. None when
+  the file or the entry is missing."""
+  try:
+    with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+      t = json.load(f)
+    k, c, known = t[kernel_key], t["copy"], float(t["copy_known_kib"])
+    return (k["fetch_kib"] * known / c["fetch_kib"] + k["write_kib"] * known / c["write_kib"]) * 1024.0
+  except (OSError, KeyError, ValueError, ZeroDivisionError):
+    return None
+
+
 def _time_events(fn, iters, warmup):
   """Average duration in ms of fn() over `iters` calls, HIP events on the current
   stream (the stream the kernels are launched on)."""
@@ -375,6 +418,9 @@ def main():
                   help="run only the headline-shape kernels (the roofline legs) and print their "
                        "figures: the command to put under rocprofv3 when per-kernel averages "
                        "must not mix shapes")
+  ap.add_argument("--pmc-sequence", action="store_true",
+                  help="run only the launch sequence for rocprofv3 --pmc counter collection "
+                       "(fill, plain copy, quantizer, fill, GEMM at the headline shape, 4 times)")
   ap.add_argument("--step-only", action="store_true",
                   help="run only the hot-path step legs (eager, hipGraph replay, shared "
                        "quantization) and print their figures: the command to put under "
@@ -391,6 +437,10 @@ def main():
   torch.cuda.set_device(device)
   arch = _native.device_arch()
 
+  if args.pmc_sequence:
+    pmc_sequence(device)
+    print(json.dumps({"pmc_sequence": "done", "device": arch}))
+    return
   if args.headline_only:
     print(json.dumps({"linear_headline": headline_kernels(device), "device": arch}))
     return
@@ -468,8 +518,8 @@ def main():
       "unit": "TFLOP/s",
       "frac": head["gemm_tflops"] / FP8_PEAK_TFLOPS,
       # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain
-      # copy of known size (profiles/pmc_traffic_headline_kernels.md); algorithmic 165.2 MB
-      "traffic": 378.0e6,
+      # copy of known size (read from profiles/traffic.json); algorithmic 165.2 MB
+      "traffic": measured_traffic("gemm_fp8_wide_headline"),
   }
   roofline_quant = {
       "kernel": "quant_rowwise_regs at M=4608 K=3072",
@@ -478,7 +528,7 @@ def main():
       "peak": HBM_PEAK_GBPS,
       "unit": "GB/s",
       "frac": head["quant_gbps"] / HBM_PEAK_GBPS,
-      "traffic": 42.66e6,  # same source; algorithmic 3MK + 4M = 42.49 MB
+      "traffic": measured_traffic("quant_rowwise_headline"),  # algorithmic 3MK + 4M = 42.49 MB
   }
   other = {}
   if not args.skip_other_configs:

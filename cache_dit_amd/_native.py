@@ -36,6 +36,7 @@ EXPORTS = (
     "cdit_fp8_linear_w8a8",
     "cdit_fp8_linear_w8a8_static",
     "cdit_set_gemm_variant",
+    "cdit_debug_set_quant_hints",
     "cdit_stream_capture_id",
 )
 
@@ -59,6 +60,8 @@ def _bind(L: ctypes.CDLL) -> None:
   L.cdit_stream_capture_id.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64)]
   L.cdit_set_gemm_variant.restype = ci
   L.cdit_set_gemm_variant.argtypes = [ci]
+  L.cdit_debug_set_quant_hints.restype = ci
+  L.cdit_debug_set_quant_hints.argtypes = [ci]
   L.cdit_fp8_quant_rowwise.restype = ci
   L.cdit_fp8_quant_rowwise.argtypes = [vp, i64, i64, i64, vp, i64, vp, ci, vp]
   L.cdit_fp8_quant_tensorwise.restype = ci

@@ -149,12 +149,14 @@ int cdit_stream_capture_id(void* stream, uint64_t* id) {
 }
 
 int cdit_set_gemm_variant(int variant) {
-  if (variant >= 1000) {  // 1000 + v: cache hints of the quantizer instead, 1999: automatic
-    cdit::g_quant_variant = variant == 1999 ? -1 : variant - 1000;
-    return g_gemm_variant;
-  }
   int prev = g_gemm_variant;
   g_gemm_variant = variant;
+  return prev;
+}
+
+int cdit_debug_set_quant_hints(int hints) {
+  int prev = cdit::g_quant_variant;
+  cdit::g_quant_variant = hints >= 0 && hints <= 3 ? hints : -1;
   return prev;
 }
 

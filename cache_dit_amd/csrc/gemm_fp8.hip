@@ -4,8 +4,10 @@
 //   out[m,n] = epi((sum_k a[m,k] b[n,k]) * a_scale[m] * b_scale[n] + bias[n])
 //
 // Both operands are K-contiguous ("NT" GEMM), which is what the MFMA operand
-// registers want: v_mfma_f32_32x32x64_f8f6f4 takes, per lane, 32 consecutive
-// K bytes of one row (lane&31) in K-half (lane>>5).
+// registers want: per lane, 32 consecutive K bytes of one row. The production kernel
+// (gemm_fp8_wide) issues v_mfma_f32_16x16x128_f8f6f4: row lane&15, 32-byte K group
+// lane>>4 of a 128-byte K step; the older tiled kernel v_mfma_f32_32x32x64_f8f6f4: row
+// lane&31, K half lane>>5 of a 64-byte step.
 //
 // Kernels in this file: gemm_fp8_wide (persistent, one wave per SIMD, the one every
 // large or medium problem runs; described in front of CfgWide), gemm_fp8_tiled (the
@@ -1139,10 +1141,11 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     // those cannot take runs the generic kernel.
     const int64_t t_large = (int64_t)((g.M + 255) / 256) * ((g.N + 191) / 192);
     const int64_t t_small = (int64_t)((g.M + 63) / 64) * ((g.N + 127) / 128);
+    const int64_t ncu = cu_count() > 0 ? cu_count() : 256;
     const bool large = variant == 15 ||
                        (variant != 17 && (!wide_ok(V17::DEPTH) ||
-                                          (t_large + 255) / 256 * 256 * 192 * 1000 <=
-                                              (t_small + 255) / 256 * 64 * 128 * 1493));
+                                          (t_large + ncu - 1) / ncu * 256 * 192 * 1000 <=
+                                              (t_small + ncu - 1) / ncu * 64 * 128 * 1493));
     if (large && wide_ok(V15::DEPTH)) {
       return g.out_dtype == CDIT_DT_F16 ? launch_wide<V15, CDIT_DT_F16>(g, stream)
                                         : launch_wide<V15, CDIT_DT_F32>(g, stream);
@@ -1159,14 +1162,16 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     auto tiles = [&](int bm, int bn) {
       return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
     };
-    if (tiles(256, 256) >= 160) {
+    // workgroups a round holds: one per CU (what launch_wide starts)
+    const int64_t cus = cu_count() > 0 ? cu_count() : 256;
+    if (tiles(256, 256) * 256 >= 160 * cus) {
       // Large problems take one of the large-tile wide kernels. Cost model, fitted to
-      // measured times: tile area times the number of rounds over the 256 CUs, where a
-      // last, partial round of r tiles counts 0.4 + 0.6 r/256 (the chip is power
+      // measured times: tile area times the number of rounds over the CUs, where a
+      // last, partial round of r tiles counts 0.4 + 0.6 r/CUs (the chip is power
       // limited: with fewer CUs busy the clocks rise); ties go to the larger tile.
       auto cost = [&](int bm, int bn, int pen) {
-        const int64_t t = tiles(bm, bn), full = t / 256, rem = t % 256;
-        return (full * 2560 + (rem ? 1024 + 6 * rem : 0)) * bm * bn * pen;
+        const int64_t t = tiles(bm, bn), full = t / cus, rem = t % cus;
+        return (full * 10 * cus + (rem ? 4 * cus + 6 * rem : 0)) * bm * bn * pen;
       };
       variant = 12;
       int64_t best = cost(256, 256, 100);
@@ -1189,10 +1194,10 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
           {16, 128, 192, 1124, 3}, {18, 128, 128, 1000, 4}, {17, 64, 128, 1493, 5}};
       int64_t best = INT64_MAX;
       // K < 256: the kernels without a K stream across tiles
-      variant = tiles(128, 128) >= 256 ? 6 : 21;
+      variant = tiles(128, 128) >= cus ? 6 : 21;
       for (const auto& c : cand) {
         if (!wide_ok(c.depth)) continue;
-        const int64_t t = (tiles(c.bm, c.bn) + 255) / 256 * c.bm * c.bn * c.pen;
+        const int64_t t = (tiles(c.bm, c.bn) + cus - 1) / cus * c.bm * c.bn * c.pen;
         if (t < best) {
           best = t;
           variant = c.v;

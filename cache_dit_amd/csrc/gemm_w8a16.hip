@@ -952,16 +952,17 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
   // tile (before it, slower waves may still be reading the previous tile's)
   auto wide_ok = [&](int depth) { return g.K >= (depth > 3 ? depth : 3) * BKE && g.N % 16 == 0; };
   if (variant < 0) {
-    // Same cost model as the w8a8 entry point: tile area times rounds over the 256
-    // CUs, a last partial round of r tiles counting 0.4 + 0.6 r/256.
+    // Same cost model as the w8a8 entry point: tile area times rounds over the CUs (one
+    // persistent workgroup each), a last partial round of r tiles counting 0.4 + 0.6 r/CUs.
     auto tiles = [&](int bm, int bn) {
       return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
     };
+    const int64_t cus = cu_count() > 0 ? cu_count() : 256;
     auto cost = [&](int bm, int bn, int pen) {
-      const int64_t t = tiles(bm, bn), full = t / 256, rem = t % 256;
-      return (full * 2560 + (rem ? 1024 + 6 * rem : 0)) * bm * bn * pen;
+      const int64_t t = tiles(bm, bn), full = t / cus, rem = t % cus;
+      return (full * 10 * cus + (rem ? 4 * cus + 6 * rem : 0)) * bm * bn * pen;
     };
-    if (tiles(256, 256) >= 160 && wide_ok(2)) {
+    if (tiles(256, 256) * 256 >= 160 * cus && wide_ok(2)) {
       variant = cost(256, 192, 103) < cost(256, 256, 100) ? 8 : 7;
     } else {
       // Smaller problems: whole rounds over the CUs times tile area, the small tiles
@@ -975,7 +976,7 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
       variant = 3;  // the 128x128 kernel takes what no wide tile can
       for (const auto& c : cand) {
         if (!wide_ok(c.depth)) continue;
-        const int64_t t = (tiles(c.bm, c.bn) + 255) / 256 * c.bm * c.bn * c.pen;
+        const int64_t t = (tiles(c.bm, c.bn) + cus - 1) / cus * c.bm * c.bn * c.pen;
         if (t < best) {
           best = t;
           variant = c.v;

@@ -215,13 +215,19 @@ int cdit_fp8_linear_w8a8_static(const void* x_bf16, const void* w_q, const float
 int cdit_stream_capture_id(void* stream, uint64_t* id);
 
 /*
- * Tuning hook used by the benchmark and the tests: forces the kernel variant
- * the two GEMM entry points pick (-1 = automatic choice by shape). Returns
- * the previous value. Process-global; not meant for concurrent use.
- * Values 1000..1003 set the cache hints of the per-row quantizer instead (0: loads and
- * stores non-temporal, 1: neither, 2: loads, 3: stores), 1999 its automatic choice by size.
+ * Debug and measurement hooks, not part of the operator interface. Both set a
+ * process-global value that every later call on any thread reads; they are not thread
+ * safe and must not be called while another thread is inside the library. A production
+ * caller never needs them (the default, -1, is the automatic choice).
+ *
+ * cdit_set_gemm_variant: forces the kernel variant the GEMM entry points pick (-1 = by
+ * shape). Returns the previous value. The tests use it to run every variant on one shape.
+ * cdit_debug_set_quant_hints: forces the cache hints of the per-row quantizer (0: loads
+ * and stores non-temporal, 1: neither, 2: loads, 3: stores; anything else = -1 = by
+ * size). Returns the previous value. Results never depend on it.
  */
 int cdit_set_gemm_variant(int variant);
+int cdit_debug_set_quant_hints(int hints);
 
 #ifdef __cplusplus
 }
