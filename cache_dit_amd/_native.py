@@ -35,6 +35,10 @@ EXPORTS = (
     "cdit_w8a16_gemm",
     "cdit_fp8_linear_w8a8",
     "cdit_fp8_linear_w8a8_static",
+    "cdit_fp8_comm_per_token_quant",
+    "cdit_fp8_comm_per_token_dequant",
+    "cdit_fp8_comm_qkv_permute_quant",
+    "cdit_fp8_comm_qkv_permute_dequant",
     "cdit_set_gemm_variant",
     "cdit_debug_set_quant_hints",
     "cdit_stream_capture_id",
@@ -75,6 +79,14 @@ def _bind(L: ctypes.CDLL) -> None:
   L.cdit_fp8_linear_w8a8_static.restype = ci
   L.cdit_fp8_linear_w8a8_static.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci,
                                             ci, vp]
+  L.cdit_fp8_comm_per_token_quant.restype = ci
+  L.cdit_fp8_comm_per_token_quant.argtypes = [vp, i64, i64, vp, vp]
+  L.cdit_fp8_comm_per_token_dequant.restype = ci
+  L.cdit_fp8_comm_per_token_dequant.argtypes = [vp, i64, i64, vp, vp]
+  L.cdit_fp8_comm_qkv_permute_quant.restype = ci
+  L.cdit_fp8_comm_qkv_permute_quant.argtypes = [vp, i64, i64, i64, i64, i64, i64, i64, i64, vp, vp]
+  L.cdit_fp8_comm_qkv_permute_dequant.restype = ci
+  L.cdit_fp8_comm_qkv_permute_dequant.argtypes = [vp, i64, i64, i64, i64, i64, i64, i64, vp, vp]
   L.cdit_w8a16_gemm.restype = ci
   L.cdit_w8a16_gemm.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, vp]
 

@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 LIB_DIR = os.path.join(os.path.dirname(HERE), "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libcdit_hip.so")
-SOURCES = ["capi.hip", "quant_rowwise.hip", "gemm_fp8.hip", "gemm_w8a16.hip"]
+SOURCES = ["capi.hip", "quant_rowwise.hip", "comm_quant.hip", "gemm_fp8.hip", "gemm_w8a16.hip"]
 
 # -ffp-contract=off: the quantizer's arithmetic is specified operation by
 # operation (explicit FMAs only). The packed-fp32 feature is switched off on

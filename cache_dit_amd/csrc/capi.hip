@@ -306,6 +306,96 @@ int cdit_fp8_linear_w8a8(const void* x_bf16, const void* w_q, const float* w_sca
                                epilogue, out_dtype_id, stream);
 }
 
+// ---- FP8 quantizers with packed trailing scales (activations that cross GPUs)
+static int check_comm(const char* fn, const void* in, const void* out, int64_t rows, int64_t width,
+                      int64_t min_width) {
+  if (rows < 0 || width < min_width || rows > INT32_MAX * (int64_t)64 || width > INT32_MAX) {
+    set_error("%s: bad shape rows=%lld width=%lld", fn, (long long)rows, (long long)width);
+    return CDIT_EINVAL;
+  }
+  if (rows > 0 && (!in || !out)) {
+    set_error("%s: null pointer argument", fn);
+    return CDIT_EINVAL;
+  }
+  return CDIT_OK;
+}
+
+int cdit_fp8_comm_per_token_quant(const void* x_bf16, int64_t M, int64_t H, void* y_e4m3,
+                                  void* stream) {
+  const char* fn = "cdit_fp8_comm_per_token_quant";
+  int rc = check_comm(fn, x_bf16, y_e4m3, M, H, 0);
+  if (rc || M == 0) return rc;
+  if ((rc = check_arch())) return rc;
+  rc = launch_comm_per_token_quant(x_bf16, M, H, y_e4m3, static_cast<hipStream_t>(stream));
+  return rc ? rc : after_launch(fn);
+}
+
+int cdit_fp8_comm_per_token_dequant(const void* x_e4m3, int64_t M, int64_t H, void* y_bf16,
+                                    void* stream) {
+  const char* fn = "cdit_fp8_comm_per_token_dequant";
+  int rc = check_comm(fn, x_e4m3, y_bf16, M, H, 0);
+  if (rc || M == 0) return rc;
+  if ((rc = check_arch())) return rc;
+  rc = launch_comm_per_token_dequant(x_e4m3, M, H, y_bf16, static_cast<hipStream_t>(stream));
+  return rc ? rc : after_launch(fn);
+}
+
+int cdit_fp8_comm_qkv_permute_quant(const void* x_bf16, int64_t B, int64_t S, int64_t P, int64_t N,
+                                    int64_t D, int64_t stride_b, int64_t stride_s, int64_t stride_p,
+                                    void* quant_x, void* stream) {
+  const char* fn = "cdit_fp8_comm_qkv_permute_quant";
+  if (B < 0 || S < 0 || P < 0 || N < 0 || D < 0 || B > INT32_MAX || S > INT32_MAX || P > INT32_MAX ||
+      N > INT32_MAX || D > INT32_MAX) {
+    set_error("%s: bad shape B=%lld S=%lld P=%lld N=%lld D=%lld", fn, (long long)B, (long long)S,
+              (long long)P, (long long)N, (long long)D);
+    return CDIT_EINVAL;
+  }
+  if (D % 4 != 0) {  // the fp32 scale sits at byte D of a row that starts on a 4-byte boundary
+    set_error("%s: D=%lld is not a multiple of 4", fn, (long long)D);
+    return CDIT_EINVAL;
+  }
+  if (B * S * P * N == 0) return CDIT_OK;
+  if (!x_bf16 || !quant_x) {
+    set_error("%s: null pointer argument", fn);
+    return CDIT_EINVAL;
+  }
+  int rc = check_arch();
+  if (rc) return rc;
+  rc = launch_comm_qkv_permute_quant(x_bf16, (int)B, (int)S, (int)P, (int)N, (int)D, stride_b,
+                                     stride_s, stride_p, quant_x, static_cast<hipStream_t>(stream));
+  return rc ? rc : after_launch(fn);
+}
+
+int cdit_fp8_comm_qkv_permute_dequant(const void* quant_x, int64_t S, int64_t B, int64_t N, int64_t D,
+                                      int64_t stride_s, int64_t stride_b, int64_t stride_n,
+                                      void* x_bf16, void* stream) {
+  const char* fn = "cdit_fp8_comm_qkv_permute_dequant";
+  if (B < 0 || S < 0 || N < 0 || D < 0 || B > INT32_MAX || S > INT32_MAX || N > INT32_MAX ||
+      D > INT32_MAX) {
+    set_error("%s: bad shape S=%lld B=%lld N=%lld D=%lld", fn, (long long)S, (long long)B,
+              (long long)N, (long long)D);
+    return CDIT_EINVAL;
+  }
+  if (D % 4 != 0) {
+    set_error("%s: D=%lld is not a multiple of 4", fn, (long long)D);
+    return CDIT_EINVAL;
+  }
+  if (B * S * N == 0) return CDIT_OK;
+  if (!x_bf16 || !quant_x) {
+    set_error("%s: null pointer argument", fn);
+    return CDIT_EINVAL;
+  }
+  if (stride_n < D + 4) {
+    set_error("%s: stride_n=%lld is smaller than a row of D + 4 bytes", fn, (long long)stride_n);
+    return CDIT_EINVAL;
+  }
+  int rc = check_arch();
+  if (rc) return rc;
+  rc = launch_comm_qkv_permute_dequant(quant_x, (int)S, (int)B, (int)N, (int)D, stride_s, stride_b,
+                                       stride_n, x_bf16, static_cast<hipStream_t>(stream));
+  return rc ? rc : after_launch(fn);
+}
+
 // ---- allocation-free Linear: activation codes and scales in a library-owned array
 // One copy of the array lives on every GPU the library runs on, for the life of the
 // process. Host code never uses the array's name as an address (it is a host-side

@@ -44,6 +44,14 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream);
 int launch_linear_fp8_skinny_fused(const GemmArgs& g, void* q_ws, float* scale_ws, int scale_mode,
                                    int variant, hipStream_t stream);
 
+// FP8 quantizers with the scale packed behind each row (comm_quant.hip).
+int launch_comm_per_token_quant(const void* x, int64_t M, int64_t H, void* y, hipStream_t stream);
+int launch_comm_per_token_dequant(const void* x, int64_t M, int64_t H, void* y, hipStream_t stream);
+int launch_comm_qkv_permute_quant(const void* x, int B, int S, int P, int N, int D, int64_t sb,
+                                  int64_t ss, int64_t sp, void* y, hipStream_t stream);
+int launch_comm_qkv_permute_dequant(const void* qx, int S, int B, int N, int D, int64_t qs, int64_t qb,
+                                    int64_t qn, void* x, hipStream_t stream);
+
 void set_error(const char* fmt, ...);
 
 }  // namespace cdit

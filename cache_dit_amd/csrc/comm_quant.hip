@@ -1,0 +1,391 @@
+// FP8 (OCP e4m3fn) quantizers for activations that cross GPUs, with the scale packed
+// behind the codes of each row so that one buffer travels. Counterparts of the
+// reference's Triton kernels, src/cache_dit/kernels/triton/_float8_comm.py:
+//   per-token quant / dequant  (:5-40, :43-62; wrappers _ops_registery.py:52-112)
+//     row of H bf16 -> H codes + the scale as bf16 in 2 trailing bytes (pitch H + 2);
+//     amax floored at 1e-4, codes = cast(clamp(x * (1 / (amax / 448)), +-448)); the
+//     scale that travels is amax / 448 rounded to bf16, dequant multiplies by it.
+//   qkv permute quant / dequant (:66-113, :116-148; wrappers :115-185)
+//     x [B,S,P,N,D] -> [P,S,B,N,D+4]: per head row of D values the codes followed by the
+//     fp32 scale max(amax / 448, 1e-6) in 4 trailing bytes; codes = cast(clamp(x / scale,
+//     +-448)) with a true division; dequant [S,B,N,D+4] -> [B,S,N,D] bf16.
+// This arithmetic differs from the GEMM path's quantizer (reciprocal multiply, eps
+// floors, where the scale is rounded) and shares none of its contract.
+//
+// All four are pure HBM streaming: one 64-lane wavefront per row, the row read once
+// and kept in registers between the amax and the cast. Rows with a pitch of H + 2 (or
+// D + 4) bytes start on 2- (4-) byte boundaries, so code rows are moved in the widest
+// pieces their alignment allows.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "cdit_internal.h"
+#include "quant_device.h"
+
+namespace cdit {
+namespace {
+
+constexpr int kMaxChunks = 32;  // 16-byte chunks of bf16 per lane: rows of up to 16384 values
+
+__device__ __forceinline__ float wave_max_f32_nonneg(float v) {
+  // non-negative floats order like their bit patterns
+  return __uint_as_float(wave_max_u32(__float_as_uint(v)));
+}
+
+// fp32 -> bf16 bits, round to nearest even; NaN stays NaN.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits_rne(float f) {
+  return __float_as_uint(round_to_bf16(f)) >> 16;
+}
+
+__device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d) {
+  uint32_t p = 0;
+  p = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, p, false);
+  p = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, p, true);
+  return p;
+}
+
+// 8 code bytes to dst, which is 2-byte aligned at least (wave-uniform alignment).
+__device__ __forceinline__ void store8(uint8_t* dst, uint32_t lo, uint32_t hi, int align) {
+  if (align >= 8) {
+    *reinterpret_cast<uint2*>(dst) = uint2{lo, hi};
+  } else if (align >= 4) {
+    reinterpret_cast<uint32_t*>(dst)[0] = lo;
+    reinterpret_cast<uint32_t*>(dst)[1] = hi;
+  } else {
+    uint16_t* d = reinterpret_cast<uint16_t*>(dst);
+    d[0] = (uint16_t)lo;
+    d[1] = (uint16_t)(lo >> 16);
+    d[2] = (uint16_t)hi;
+    d[3] = (uint16_t)(hi >> 16);
+  }
+}
+
+__device__ __forceinline__ uint2 load8(const uint8_t* src, int align) {
+  if (align >= 8) return *reinterpret_cast<const uint2*>(src);
+  if (align >= 4) {
+    return uint2{reinterpret_cast<const uint32_t*>(src)[0], reinterpret_cast<const uint32_t*>(src)[1]};
+  }
+  const uint16_t* s = reinterpret_cast<const uint16_t*>(src);
+  return uint2{(uint32_t)s[0] | ((uint32_t)s[1] << 16), (uint32_t)s[2] | ((uint32_t)s[3] << 16)};
+}
+
+__device__ __forceinline__ int align_of(const void* p) {
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+  return (a & 7) == 0 ? 8 : (a & 3) == 0 ? 4 : (a & 1) == 0 ? 2 : 1;
+}
+
+// SCALE: 0 = per-token form (bf16 scale, eps on amax, reciprocal multiply),
+//        1 = qkv form (fp32 scale, eps on the scale, true division).
+// Row r of `rows` rows: source x + src_off(r) (H bf16, 16-byte aligned when VEC), codes at
+// y + r * (H + tail) followed by the scale.
+template <int SCALE>
+__device__ __forceinline__ void quant_row(const uint16_t* __restrict__ xr, uint8_t* __restrict__ yr,
+                                          int H, bool vec, int lane) {
+  const int nchunks = H >> 3;
+  uint4 v[kMaxChunks];
+  float amax = 0.0f;
+  if (vec) {
+    const uint4* xv = reinterpret_cast<const uint4*>(xr);
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) {
+      const int idx = c * 64 + lane;
+      if (c * 64 < nchunks) {  // wave-uniform: whole groups of 64 chunks
+        v[c] = idx < nchunks ? xv[idx] : make_uint4(0, 0, 0, 0);
+        uint32_t m = 0;
+        m = absmax2(m, v[c].x);
+        m = absmax2(m, v[c].y);
+        m = absmax2(m, v[c].z);
+        m = absmax2(m, v[c].w);
+        amax = fmaxf(amax, __uint_as_float(fold2(m) << 16));
+      }
+    }
+  } else {
+    for (int k = lane; k < H; k += 64) amax = fmaxf(amax, __uint_as_float((uint32_t)(xr[k] & 0x7fffu) << 16));
+  }
+  amax = wave_max_f32_nonneg(amax);
+  float scale, inv = 0.0f;
+  if constexpr (SCALE == 0) {
+    amax = fmaxf(amax, 1e-4f);
+    scale = amax / kFp8Max;
+    inv = 1.0f / scale;
+  } else {
+    scale = fmaxf(amax / kFp8Max, 1e-6f);
+  }
+  auto q = [&](float x) {
+    const float y = SCALE == 0 ? x * inv : x / scale;
+    return y != y ? y : fminf(fmaxf(y, -kFp8Max), kFp8Max);
+  };
+  if (vec) {
+    const int al = align_of(yr);
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) {
+      const int idx = c * 64 + lane;
+      if (c * 64 < nchunks && idx < nchunks) {
+        const uint32_t lo = cvt4_fp8(q(bf16_lo(v[c].x)), q(bf16_hi(v[c].x)), q(bf16_lo(v[c].y)),
+                                     q(bf16_hi(v[c].y)));
+        const uint32_t hi = cvt4_fp8(q(bf16_lo(v[c].z)), q(bf16_hi(v[c].z)), q(bf16_lo(v[c].w)),
+                                     q(bf16_hi(v[c].w)));
+        store8(yr + 8 * idx, lo, hi, al);
+      }
+    }
+  } else {
+    for (int k = lane; k < H; k += 64) {
+      const float y = q(__uint_as_float((uint32_t)xr[k] << 16));
+      yr[k] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(y, y, 0u, false) & 0xffu);
+    }
+  }
+  if (lane == 0) {
+    if constexpr (SCALE == 0) {
+      const uint16_t s16 = (uint16_t)(__float_as_uint(round_to_bf16(scale)) >> 16);
+      yr[H] = (uint8_t)s16;  // byte stores: the row end is only 1-byte aligned for odd H
+      yr[H + 1] = (uint8_t)(s16 >> 8);
+    } else {
+      const uint32_t s32 = __float_as_uint(scale);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) yr[H + b] = (uint8_t)(s32 >> (8 * b));
+    }
+  }
+}
+
+// codes (+ trailing scale) -> bf16 row. SCALE as above (only the scale's format differs).
+template <int SCALE>
+__device__ __forceinline__ void dequant_row(const uint8_t* __restrict__ xr, uint16_t* __restrict__ yr,
+                                            int H, bool vec, int lane) {
+  float scale;
+  if constexpr (SCALE == 0) {
+    scale = __uint_as_float(((uint32_t)xr[H] | ((uint32_t)xr[H + 1] << 8)) << 16);
+  } else {
+    scale = __uint_as_float((uint32_t)xr[H] | ((uint32_t)xr[H + 1] << 8) | ((uint32_t)xr[H + 2] << 16) |
+                            ((uint32_t)xr[H + 3] << 24));
+  }
+  auto de = [&](uint32_t w, int byte) {  // one code -> scaled fp32
+    float f;
+    switch (byte) {
+      case 0: f = __builtin_amdgcn_cvt_f32_fp8((int)w, 0); break;
+      case 1: f = __builtin_amdgcn_cvt_f32_fp8((int)w, 1); break;
+      case 2: f = __builtin_amdgcn_cvt_f32_fp8((int)w, 2); break;
+      default: f = __builtin_amdgcn_cvt_f32_fp8((int)w, 3); break;
+    }
+    return f * scale;
+  };
+  if (vec) {
+    const int al = align_of(xr);
+    uint4* yv = reinterpret_cast<uint4*>(yr);
+    for (int idx = lane; idx < (H >> 3); idx += 64) {
+      const uint2 w = load8(xr + 8 * idx, al);
+      uint4 o;
+      o.x = (f32_to_bf16_bits_rne(de(w.x, 0))) | (f32_to_bf16_bits_rne(de(w.x, 1)) << 16);
+      o.y = (f32_to_bf16_bits_rne(de(w.x, 2))) | (f32_to_bf16_bits_rne(de(w.x, 3)) << 16);
+      o.z = (f32_to_bf16_bits_rne(de(w.y, 0))) | (f32_to_bf16_bits_rne(de(w.y, 1)) << 16);
+      o.w = (f32_to_bf16_bits_rne(de(w.y, 2))) | (f32_to_bf16_bits_rne(de(w.y, 3)) << 16);
+      yv[idx] = o;
+    }
+  } else {
+    for (int k = lane; k < H; k += 64) {
+      const float f = __builtin_amdgcn_cvt_f32_fp8((int)xr[k], 0) * scale;
+      yr[k] = (uint16_t)f32_to_bf16_bits_rne(f);
+    }
+  }
+}
+
+__global__ __launch_bounds__(64) void comm_per_token_quant(const uint16_t* __restrict__ x,
+                                                           uint8_t* __restrict__ y, int64_t M, int H,
+                                                           bool vec) {
+  const int lane = threadIdx.x;
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x)
+    quant_row<0>(x + row * H, y + row * (H + 2), H, vec, lane);
+}
+
+__global__ __launch_bounds__(64) void comm_per_token_dequant(const uint8_t* __restrict__ x,
+                                                             uint16_t* __restrict__ y, int64_t M,
+                                                             int H, bool vec) {
+  const int lane = threadIdx.x;
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x)
+    dequant_row<0>(x + row * (H + 2), y + row * H, H, vec, lane);
+}
+
+// One wavefront per head row. Output row index r = ((p * S + s) * B + b) * N + n of
+// [P,S,B,N,D+4]; the source row is x[b,s,p,n,:] (element strides for b, s, p; heads and
+// channels contiguous, as the reference kernel assumes).
+__global__ __launch_bounds__(64) void comm_qkv_permute_quant(
+    const uint16_t* __restrict__ x, uint8_t* __restrict__ y, int B, int S, int P, int N, int D,
+    int64_t sb, int64_t ss, int64_t sp, bool vec) {
+  const int lane = threadIdx.x;
+  const int64_t rows = (int64_t)P * S * B * N;
+  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    const int n = (int)(r % N);
+    const int64_t t = r / N;
+    const int b = (int)(t % B);
+    const int s = (int)((t / B) % S);
+    const int p = (int)(t / ((int64_t)B * S));
+    quant_row<1>(x + b * sb + s * ss + p * sp + (int64_t)n * D, y + r * (D + 4), D, vec, lane);
+  }
+}
+
+// quant_x [S,B,N,D+4] (byte strides for s, b, n) -> x [B,S,N,D] contiguous bf16.
+__global__ __launch_bounds__(64) void comm_qkv_permute_dequant(
+    const uint8_t* __restrict__ qx, uint16_t* __restrict__ x, int S, int B, int N, int D, int64_t qs,
+    int64_t qb, int64_t qn, bool vec) {
+  const int lane = threadIdx.x;
+  const int64_t rows = (int64_t)B * S * N;
+  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {  // r = (b * S + s) * N + n
+    const int n = (int)(r % N);
+    const int64_t t = r / N;
+    const int s = (int)(t % S);
+    const int b = (int)(t / S);
+    dequant_row<1>(qx + s * qs + b * qb + n * qn, x + r * D, D, vec, lane);
+  }
+}
+
+// Head rows are short (D = 64 .. 256): with one lane per 16-byte chunk a row only needs
+// G = D / 8 lanes (rounded up to a power of two), so a wavefront takes 64 / G rows at a
+// time and the amax is reduced inside each group of G lanes.
+template <int G>
+__device__ __forceinline__ float group_max_nonneg(float v) {
+#pragma unroll
+  for (int o = 1; o < G; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+template <int G>
+__global__ __launch_bounds__(64) void comm_qkv_permute_quant_grouped(
+    const uint16_t* __restrict__ x, uint8_t* __restrict__ y, int B, int S, int P, int N, int D,
+    int64_t sb, int64_t ss, int64_t sp) {
+  constexpr int RPW = 64 / G;  // rows per wavefront
+  const int lane = threadIdx.x, j = lane % G, sub = lane / G;
+  const int nchunks = D >> 3;
+  const int64_t rows = (int64_t)P * S * B * N;
+  for (int64_t r0 = (int64_t)blockIdx.x * RPW; r0 < rows; r0 += (int64_t)gridDim.x * RPW) {
+    const int64_t r = r0 + sub;
+    const bool row_ok = r < rows, active = row_ok && j < nchunks;
+    const int64_t rc = row_ok ? r : rows - 1;
+    const int n = (int)(rc % N);
+    const int64_t t = rc / N;
+    const int b = (int)(t % B);
+    const int s = (int)((t / B) % S);
+    const int p = (int)(t / ((int64_t)B * S));
+    const uint16_t* xr = x + b * sb + s * ss + p * sp + (int64_t)n * D;
+    const uint4 v = active ? reinterpret_cast<const uint4*>(xr)[j] : make_uint4(0, 0, 0, 0);
+    uint32_t m = 0;
+    m = absmax2(m, v.x);
+    m = absmax2(m, v.y);
+    m = absmax2(m, v.z);
+    m = absmax2(m, v.w);
+    const float amax = group_max_nonneg<G>(__uint_as_float(fold2(m) << 16));
+    const float scale = fmaxf(amax / kFp8Max, 1e-6f);
+    auto q = [&](float f) {
+      const float yv = f / scale;
+      return yv != yv ? yv : fminf(fmaxf(yv, -kFp8Max), kFp8Max);
+    };
+    if (active) {
+      uint8_t* yr = y + rc * (D + 4);  // 4-byte aligned: D % 8 == 0 and y is
+      const uint32_t lo = cvt4_fp8(q(bf16_lo(v.x)), q(bf16_hi(v.x)), q(bf16_lo(v.y)), q(bf16_hi(v.y)));
+      const uint32_t hi = cvt4_fp8(q(bf16_lo(v.z)), q(bf16_hi(v.z)), q(bf16_lo(v.w)), q(bf16_hi(v.w)));
+      reinterpret_cast<uint32_t*>(yr + 8 * j)[0] = lo;
+      reinterpret_cast<uint32_t*>(yr + 8 * j)[1] = hi;
+      if (j == 0) *reinterpret_cast<float*>(yr + D) = scale;
+    }
+  }
+}
+
+template <int G>
+__global__ __launch_bounds__(64) void comm_qkv_permute_dequant_grouped(
+    const uint8_t* __restrict__ qx, uint16_t* __restrict__ x, int S, int B, int N, int D, int64_t qs,
+    int64_t qb, int64_t qn) {
+  constexpr int RPW = 64 / G;
+  const int lane = threadIdx.x, j = lane % G, sub = lane / G;
+  const int nchunks = D >> 3;
+  const int64_t rows = (int64_t)B * S * N;
+  for (int64_t r0 = (int64_t)blockIdx.x * RPW; r0 < rows; r0 += (int64_t)gridDim.x * RPW) {
+    const int64_t r = r0 + sub;  // (b * S + s) * N + n
+    if (r >= rows || j >= nchunks) continue;
+    const int n = (int)(r % N);
+    const int64_t t = r / N;
+    const int s = (int)(t % S);
+    const int b = (int)(t / S);
+    const uint8_t* xr = qx + s * qs + b * qb + n * qn;
+    const float scale = *reinterpret_cast<const float*>(xr + D);
+    const uint32_t w0 = reinterpret_cast<const uint32_t*>(xr + 8 * j)[0];
+    const uint32_t w1 = reinterpret_cast<const uint32_t*>(xr + 8 * j)[1];
+    auto pair = [&](float a, float c) {
+      return f32_to_bf16_bits_rne(a * scale) | (f32_to_bf16_bits_rne(c * scale) << 16);
+    };
+    uint4 o;
+    o.x = pair(__builtin_amdgcn_cvt_f32_fp8((int)w0, 0), __builtin_amdgcn_cvt_f32_fp8((int)w0, 1));
+    o.y = pair(__builtin_amdgcn_cvt_f32_fp8((int)w0, 2), __builtin_amdgcn_cvt_f32_fp8((int)w0, 3));
+    o.z = pair(__builtin_amdgcn_cvt_f32_fp8((int)w1, 0), __builtin_amdgcn_cvt_f32_fp8((int)w1, 1));
+    o.w = pair(__builtin_amdgcn_cvt_f32_fp8((int)w1, 2), __builtin_amdgcn_cvt_f32_fp8((int)w1, 3));
+    reinterpret_cast<uint4*>(x + r * D)[j] = o;
+  }
+}
+
+unsigned grid_for(int64_t rows) {
+  const int64_t cap = 256 * 256;  // the grid-stride loops take the rest
+  return (unsigned)(rows < cap ? rows : cap);
+}
+
+}  // namespace
+
+int launch_comm_per_token_quant(const void* x, int64_t M, int64_t H, void* y, hipStream_t stream) {
+  const bool vec = H % 8 == 0 && H <= kMaxChunks * 512 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(y) % 2 == 0;
+  hipLaunchKernelGGL(comm_per_token_quant, dim3(grid_for(M)), dim3(64), 0, stream,
+                     static_cast<const uint16_t*>(x), static_cast<uint8_t*>(y), M, (int)H, vec);
+  return 0;
+}
+
+int launch_comm_per_token_dequant(const void* x, int64_t M, int64_t H, void* y, hipStream_t stream) {
+  const bool vec = H % 8 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(x) % 2 == 0;
+  hipLaunchKernelGGL(comm_per_token_dequant, dim3(grid_for(M)), dim3(64), 0, stream,
+                     static_cast<const uint8_t*>(x), static_cast<uint16_t*>(y), M, (int)H, vec);
+  return 0;
+}
+
+int launch_comm_qkv_permute_quant(const void* x, int B, int S, int P, int N, int D, int64_t sb,
+                                  int64_t ss, int64_t sp, void* y, hipStream_t stream) {
+  const bool vec = D % 8 == 0 && D <= kMaxChunks * 512 && sb % 8 == 0 && ss % 8 == 0 && sp % 8 == 0 &&
+                   reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 4 == 0;
+  const int64_t rows = (int64_t)P * S * B * N;
+  if (vec && D <= 256) {
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    uint8_t* yp = static_cast<uint8_t*>(y);
+#define CDIT_QKV_Q(G)                                                                            \
+  hipLaunchKernelGGL(comm_qkv_permute_quant_grouped<G>, dim3(grid_for((rows + 64 / G - 1) / (64 / G))), \
+                     dim3(64), 0, stream, xp, yp, B, S, P, N, D, sb, ss, sp)
+    if (D <= 64) CDIT_QKV_Q(8);
+    else if (D <= 128) CDIT_QKV_Q(16);
+    else CDIT_QKV_Q(32);
+#undef CDIT_QKV_Q
+    return 0;
+  }
+  hipLaunchKernelGGL(comm_qkv_permute_quant, dim3(grid_for(rows)), dim3(64), 0,
+                     stream, static_cast<const uint16_t*>(x), static_cast<uint8_t*>(y), B, S, P, N, D, sb,
+                     ss, sp, vec);
+  return 0;
+}
+
+int launch_comm_qkv_permute_dequant(const void* qx, int S, int B, int N, int D, int64_t qs, int64_t qb,
+                                    int64_t qn, void* x, hipStream_t stream) {
+  const bool vec = D % 8 == 0 && qs % 4 == 0 && qb % 4 == 0 && qn % 4 == 0 &&
+                   reinterpret_cast<uintptr_t>(qx) % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+  const int64_t rows = (int64_t)B * S * N;
+  if (vec && D <= 256) {
+    const uint8_t* qp = static_cast<const uint8_t*>(qx);
+    uint16_t* xp = static_cast<uint16_t*>(x);
+#define CDIT_QKV_D(G)                                                                              \
+  hipLaunchKernelGGL(comm_qkv_permute_dequant_grouped<G>, dim3(grid_for((rows + 64 / G - 1) / (64 / G))), \
+                     dim3(64), 0, stream, qp, xp, S, B, N, D, qs, qb, qn)
+    if (D <= 64) CDIT_QKV_D(8);
+    else if (D <= 128) CDIT_QKV_D(16);
+    else CDIT_QKV_D(32);
+#undef CDIT_QKV_D
+    return 0;
+  }
+  hipLaunchKernelGGL(comm_qkv_permute_dequant, dim3(grid_for(rows)), dim3(64), 0, stream,
+                     static_cast<const uint8_t*>(qx), static_cast<uint16_t*>(x), S, B, N, D, qs, qb, qn,
+                     vec);
+  return 0;
+}
+
+}  // namespace cdit

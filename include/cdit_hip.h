@@ -181,6 +181,36 @@ int cdit_fp8_linear_w8a8(const void* x_bf16, const void* w_q, const float* w_sca
                          int scale_mode, int epilogue, int out_dtype_id, void* stream);
 
 /*
+ * FP8 quantizers for activations that cross GPUs: the scale is packed behind the codes
+ * of each row, so that one buffer travels. They replace the reference's Triton kernels
+ * src/cache_dit/kernels/triton/_float8_comm.py:5-148 (op wrappers
+ * src/cache_dit/kernels/triton/_ops_registery.py:52-185). Their arithmetic is NOT the
+ * GEMM path's quantizer: eps floors, a reciprocal multiply in the per-token form, and
+ * their own scale formats. All buffers are contiguous unless a stride is passed.
+ *
+ * per_token_quant (_float8_comm.py:5-40): x bf16 [M,H] -> y e4m3 [M,H+2]
+ *     amax = max(1e-4, max_h |x|);  s = amax / 448;  r = 1 / s           (fp32)
+ *     y[m,:H] = e4m3fn_rne(clamp(x * r, -448, 448));  y[m,H:H+2] = bf16_rne(s)
+ * per_token_dequant (:43-62): x e4m3 [M,H+2] -> y bf16 [M,H] = bf16_rne(float(code) * s)
+ * qkv_permute_quant (:66-113): x bf16 [B,S,P,N,D] (element strides for B, S, P; the last
+ *   two dimensions contiguous) -> quant_x e4m3 [P,S,B,N,D+4] contiguous; per head row
+ *     s = max(max_d |x| / 448, 1e-6);  codes = e4m3fn_rne(clamp(x / s, -448, 448));
+ *     the fp32 s in the 4 trailing bytes. D must be a multiple of 4.
+ * qkv_permute_dequant (:116-148): quant_x e4m3 [S,B,N,D+4] (BYTE strides for S, B, N: a
+ *   slice quant_x[p] of the above is not contiguous) -> x bf16 [B,S,N,D] contiguous.
+ */
+int cdit_fp8_comm_per_token_quant(const void* x_bf16, int64_t M, int64_t H, void* y_e4m3,
+                                  void* stream);
+int cdit_fp8_comm_per_token_dequant(const void* x_e4m3, int64_t M, int64_t H, void* y_bf16,
+                                    void* stream);
+int cdit_fp8_comm_qkv_permute_quant(const void* x_bf16, int64_t B, int64_t S, int64_t P, int64_t N,
+                                    int64_t D, int64_t stride_b, int64_t stride_s, int64_t stride_p,
+                                    void* quant_x, void* stream);
+int cdit_fp8_comm_qkv_permute_dequant(const void* quant_x, int64_t S, int64_t B, int64_t N, int64_t D,
+                                      int64_t stride_s, int64_t stride_b, int64_t stride_n,
+                                      void* x_bf16, void* stream);
+
+/*
  * cdit_fp8_linear_w8a8 without the two workspace arguments: the activation codes and
  * scales go to an array inside the library (device memory that every GPU the library
  * runs on holds from the first call on it until the process ends:

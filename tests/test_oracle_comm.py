@@ -1,0 +1,104 @@
+"""Pins the CPU restatement of the FP8 comm quantizers (oracle/comm_oracle.py): closed
+forms, the eps floors, the packed layouts read back with plain views, brute force over
+all e4m3 codes, and the round-trip bounds the reference's own tests hold
+(tests/kernels/test_triton_ops.py:111-160 of the reference)."""
+import numpy as np
+import torch
+
+from oracle import comm_oracle as co
+
+FP8 = torch.float8_e4m3fn
+
+
+def _finite_codes():
+  c = torch.arange(256, dtype=torch.uint8)
+  return c[(c & 0x7f) != 0x7f]
+
+
+def test_per_token_closed_form_amax_448_times_power_of_two():
+  """Row = every finite e4m3 value times 2^k: amax = 448 * 2^k, scale 2^k exactly, the
+  reciprocal exact, so the codes are the values' own codes and the bf16 tail is 2^k."""
+  codes = _finite_codes()
+  vals = codes.view(FP8).to(torch.float32)
+  for k in (-3, 0, 5):
+    x = (vals * 2.0**k).to(torch.bfloat16).reshape(1, -1)
+    assert torch.equal(x.to(torch.float32), (vals * 2.0**k).reshape(1, -1))  # exact in bf16
+    y = co.per_token_quant(x)
+    H = x.shape[1]
+    assert y.shape == (1, H + 2) and y.dtype == FP8
+    got = y.view(torch.uint8)[0, :H]
+    # +0 and -0 both stay as they are
+    assert torch.equal(got, codes)
+    tail = y.view(torch.uint8)[0, H:].contiguous().view(torch.bfloat16)
+    assert float(tail) == 2.0**k
+    back = co.per_token_dequant(y)
+    assert torch.equal(back, x)
+
+
+def test_per_token_eps_floor_and_layout():
+  x = torch.zeros(2, 3, 16, dtype=torch.bfloat16)
+  x[1, 2, 5] = 1e-6  # below the 1e-4 floor
+  y = co.per_token_quant(x)
+  assert y.shape == (2, 3, 18)
+  tail = y.view(torch.uint8)[..., 16:].contiguous().view(torch.bfloat16).to(torch.float32)
+  want = torch.tensor(1e-4, dtype=torch.float32) / 448.0
+  assert torch.equal(tail, want.to(torch.bfloat16).to(torch.float32).expand(2, 3, 1))
+  codes = y.view(torch.uint8)[..., :16]
+  assert int(codes[0].max()) == 0
+  # 1e-6 * (448 / 1e-4) = 4.48 -> e4m3 4.5 (code 0x49): reciprocal multiply in fp32
+  assert int(codes[1, 2, 5]) == 0x49
+
+
+def test_per_token_scale_is_rounded_for_travel_only():
+  """The codes come from the unrounded fp32 reciprocal; only the stored scale is bf16."""
+  g = torch.Generator().manual_seed(0)
+  x = torch.randn(64, 256, generator=g).to(torch.bfloat16)
+  y = co.per_token_quant(x)
+  xf = x.to(torch.float32)
+  s = xf.abs().amax(1, keepdim=True) / 448.0
+  want = (xf * (1.0 / s)).clamp(-448, 448).to(FP8)
+  assert torch.equal(y.view(torch.uint8)[:, :256], want.view(torch.uint8))
+  tail = y.view(torch.uint8)[:, 256:].contiguous().view(torch.bfloat16)
+  assert torch.equal(tail, s.to(torch.bfloat16))
+  assert not torch.equal(tail.to(torch.float32), s)  # really rounded for some rows
+
+
+def test_reference_round_trip_bounds_per_token():
+  torch.manual_seed(0)
+  x = torch.randn((2, 3, 128)).to(torch.bfloat16)
+  q = co.per_token_quant(x)
+  d = co.per_token_dequant(q)
+  diff = (d.float() - x.float()).abs()
+  assert q.shape == (2, 3, 130) and d.shape == x.shape and d.dtype == torch.bfloat16
+  assert torch.isfinite(q.float()).all() and torch.isfinite(d).all()
+  assert diff.mean().item() < 0.05 and diff.max().item() < 0.2
+
+
+def test_qkv_permute_layout_closed_form_and_eps():
+  B, S, P, N, D = 2, 3, 3, 2, 8
+  x = torch.zeros(B, S, P, N, D, dtype=torch.bfloat16)
+  x[1, 2, 0, 1] = torch.tensor([448., -224., 2., 0., 0.5, -0.25, 1., 3.]) * 4  # amax 1792 -> scale 4
+  q = co.qkv_permute_quant(x)
+  assert q.shape == (P, S, B, N, D + 4) and q.dtype == FP8
+  row = q.view(torch.uint8)[0, 2, 1, 1]
+  assert float(row[D:].contiguous().view(torch.float32)) == 4.0
+  assert torch.equal(row[:D].view(FP8).to(torch.float32),
+                     torch.tensor([448., -224., 2., 0., 0.5, -0.25, 1., 3.]))
+  zero_row = q.view(torch.uint8)[1, 0, 0, 0]
+  assert float(zero_row[D:].contiguous().view(torch.float32)) == np.float32(1e-6)
+  assert int(zero_row[:D].max()) == 0
+  d = co.qkv_permute_dequant(q[0])
+  assert d.shape == (B, S, N, D) and torch.equal(d, x[:, :, 0])
+
+
+def test_reference_round_trip_qkv_tracks_selected_slice():
+  torch.manual_seed(0)
+  x = torch.randn((2, 4, 3, 5, 64)).to(torch.bfloat16)
+  q = co.qkv_permute_quant(x)
+  assert q.shape == (3, 4, 2, 5, 68) and torch.isfinite(q[..., :64].float()).all()
+  for p in range(3):
+    d = co.qkv_permute_dequant(q[p])
+    dist = [(d.float() - x[:, :, r].float()).abs().mean().item() for r in range(3)]
+    assert d.shape == (2, 4, 5, 64) and d.dtype == torch.bfloat16
+    assert min(range(3), key=lambda i: dist[i]) == p
+    assert dist[p] < 0.05
