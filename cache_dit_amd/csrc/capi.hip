@@ -200,6 +200,48 @@ int cdit_fp8_quant_rowwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_
                            scale_mode, stream, false);
 }
 
+int cdit_fp8_ln_modulate_quant(const void* x_bf16, int64_t M, int64_t K, int64_t ld_x,
+                               const void* shift_bf16, const void* scale_bf16, int64_t ld_mod,
+                               int64_t rows_per_mod, float eps, void* y_bf16, int64_t ld_y,
+                               void* q_e4m3, int64_t ld_q, float* scale, int scale_mode,
+                               void* stream) {
+  const char* fn = "cdit_fp8_ln_modulate_quant";
+  if (M < 0 || K < 0 || M > INT32_MAX || K > INT32_MAX) {
+    set_error("%s: bad shape M=%lld K=%lld", fn, (long long)M, (long long)K);
+    return CDIT_EINVAL;
+  }
+  if (scale_mode != CDIT_SCALE_BF16DIV && scale_mode != CDIT_SCALE_FP32DIV) {
+    set_error("%s: unknown scale_mode %d", fn, scale_mode);
+    return CDIT_EINVAL;
+  }
+  if (M == 0) return CDIT_OK;
+  if (K == 0) {
+    set_error("%s: K = 0 has no mean to normalise by", fn);
+    return CDIT_EINVAL;
+  }
+  if (ld_x < K || ld_q < K || (y_bf16 && ld_y < K) || rows_per_mod < 1 ||
+      (ld_mod < K && rows_per_mod < M)) {
+    set_error("%s: bad leading dimension or rows_per_mod (ld_x=%lld ld_q=%lld ld_y=%lld "
+              "ld_mod=%lld rows_per_mod=%lld K=%lld)", fn, (long long)ld_x, (long long)ld_q,
+              (long long)ld_y, (long long)ld_mod, (long long)rows_per_mod, (long long)K);
+    return CDIT_EINVAL;
+  }
+  if (!(eps >= 0.0f)) {
+    set_error("%s: eps must be >= 0", fn);
+    return CDIT_EINVAL;
+  }
+  if (!x_bf16 || !shift_bf16 || !scale_bf16 || !q_e4m3 || !scale) {
+    set_error("%s: null pointer argument", fn);
+    return CDIT_EINVAL;
+  }
+  int rc = check_arch();
+  if (rc) return rc;
+  rc = launch_ln_modulate_quant(x_bf16, M, K, ld_x, shift_bf16, scale_bf16, ld_mod, rows_per_mod,
+                                eps, y_bf16, ld_y, q_e4m3, ld_q, scale, scale_mode,
+                                static_cast<hipStream_t>(stream));
+  return rc ? rc : after_launch(fn);
+}
+
 int cdit_fp8_quant_tensorwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_x,
                               void* q_e4m3, int64_t ld_q, float* scale, void* amax_ws,
                               int scale_mode, void* stream) {

@@ -19,6 +19,13 @@ int launch_quant_tensorwise(const void* x, int64_t M, int64_t K, int64_t ld_x, v
                             int64_t ld_q, float* scale, uint32_t* amax_ws, int scale_mode,
                             hipStream_t stream);
 
+// LayerNorm (no affine) + `* (1 + scale) + shift` + per-row quantization in one pass; y may be
+// null (then only codes and scales are written).
+int launch_ln_modulate_quant(const void* x, int64_t M, int64_t K, int64_t ld_x, const void* shift,
+                             const void* scale_mod, int64_t ld_mod, int64_t rows_per_mod, float eps,
+                             void* y, int64_t ld_y, void* q, int64_t ld_q, float* scale,
+                             int scale_mode, hipStream_t stream);
+
 extern int g_quant_variant;
 
 struct GemmArgs {

@@ -210,6 +210,168 @@ __global__ __launch_bounds__(64) void quant_tensorwise_cast(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Producer-fused quantizer: LayerNorm (no affine) + AdaLN modulation + per-row FP8
+// quantization of one activation row in one pass over it. The modulated activation
+// of a DiT block, `norm(x) * (1 + scale) + shift`, is read by quantized Linears only
+// (q/k/v, proj_mlp, ff.net.0.proj; reference dataflow
+// src/cache_dit/caching/patch_functors/functor_flux.py:48-80), so the codes can be
+// produced where the activation is: 2 B read + 1 B written per element instead of the
+// producer's bf16 write and the quantizer's read of it on top. y is written as well on
+// request (WRITE_Y), for consumers that read the bf16 tensor.
+//
+// Arithmetic, element k of a row (every step rounds to bf16 where the unfused sequence of
+// bf16 tensor ops does, so that the codes are those the stand-alone quantizer gives on y):
+//   mean = sum(x) / K,  var = sum((x - mean)^2) / K,  rstd = 1 / sqrt(var + eps)   (fp32)
+//   n = bf16((x - mean) * rstd);  t = bf16(1 + scale[k]);  u = bf16(n * t);
+//   y = bf16(u + shift[k]);  then amax / scale / e4m3 cast of y as in quant_rowwise_regs.
+// shift and scale are bf16 [*, K]; row m uses their row m / rows_per_mod (one modulation
+// vector per batch element, broadcast over its tokens).
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+__device__ __forceinline__ uint32_t bf16_bits(float f) {
+  return __float_as_uint(round_to_bf16(f)) >> 16;
+}
+
+// y bits of one element: x, scale, shift as fp32 (exact widenings of bf16 values)
+__device__ __forceinline__ uint32_t modulate1(float x, float mean, float rstd, float sc, float sh) {
+  const float n = round_to_bf16((x - mean) * rstd);
+  const float t = round_to_bf16(1.0f + sc);
+  const float u = round_to_bf16(n * t);
+  return bf16_bits(u + sh);
+}
+
+__device__ __forceinline__ uint32_t modulate2(uint32_t xw, float mean, float rstd, uint32_t scw,
+                                              uint32_t shw) {
+  return modulate1(bf16_lo(xw), mean, rstd, bf16_lo(scw), bf16_lo(shw)) |
+         (modulate1(bf16_hi(xw), mean, rstd, bf16_hi(scw), bf16_hi(shw)) << 16);
+}
+
+template <int CH, bool WRITE_Y>
+__global__ __launch_bounds__(64) void ln_modulate_quant_regs(
+    const uint16_t* __restrict__ x, int64_t ld_x, const uint16_t* __restrict__ shift,
+    const uint16_t* __restrict__ scale_mod, int64_t ld_mod, int rows_per_mod, float eps,
+    uint16_t* __restrict__ y, int64_t ld_y, uint8_t* __restrict__ q, int64_t ld_q,
+    float* __restrict__ scale, int M, int K, int scale_mode) {
+  const int lane = threadIdx.x & 63;
+  const int nchunks = K >> 3;
+  const float inv_k = 1.0f / (float)K;
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+    const uint4* xr = reinterpret_cast<const uint4*>(x + row * ld_x);
+    const int64_t mod_row = (row / rows_per_mod) * ld_mod;
+    const uint4* shr = reinterpret_cast<const uint4*>(shift + mod_row);
+    const uint4* scr = reinterpret_cast<const uint4*>(scale_mod + mod_row);
+    uint4 v[CH];
+    float sum = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int idx = c * 64 + lane;
+      v[c] = idx < nchunks ? xr[idx] : make_uint4(0, 0, 0, 0);
+      sum += (bf16_lo(v[c].x) + bf16_hi(v[c].x)) + (bf16_lo(v[c].y) + bf16_hi(v[c].y)) +
+             (bf16_lo(v[c].z) + bf16_hi(v[c].z)) + (bf16_lo(v[c].w) + bf16_hi(v[c].w));
+    }
+    const float mean = wave_sum_f32(sum) * inv_k;
+    float ss = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      if (c * 64 + lane < nchunks) {
+        const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float a = bf16_lo(w[e]) - mean, b = bf16_hi(w[e]) - mean;
+          ss = __fmaf_rn(a, a, ss);
+          ss = __fmaf_rn(b, b, ss);
+        }
+      }
+    }
+    const float var = wave_sum_f32(ss) * inv_k;
+    const float rstd = 1.0f / sqrtf(var + eps);
+    uint32_t m = 0;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int idx = c * 64 + lane;
+      if (idx < nchunks) {
+        const uint4 sh = shr[idx], sc = scr[idx];
+        v[c].x = modulate2(v[c].x, mean, rstd, sc.x, sh.x);
+        v[c].y = modulate2(v[c].y, mean, rstd, sc.y, sh.y);
+        v[c].z = modulate2(v[c].z, mean, rstd, sc.z, sh.z);
+        v[c].w = modulate2(v[c].w, mean, rstd, sc.w, sh.w);
+        if constexpr (WRITE_Y) reinterpret_cast<uint4*>(y + row * ld_y)[idx] = v[c];
+        m = absmax2(m, v[c].x);
+        m = absmax2(m, v[c].y);
+        m = absmax2(m, v[c].z);
+        m = absmax2(m, v[c].w);
+      }
+    }
+    m = wave_max_u32(fold2(m));
+    const float s = row_scale(m, scale_mode);
+    if (lane == 0) scale[row] = s;
+    uint2* qr = reinterpret_cast<uint2*>(q + row * ld_q);
+    const bool fast = scale_in_fast_window(s);  // wave-uniform
+    const float r = fast ? 1.0f / s : 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int idx = c * 64 + lane;
+      if (idx < nchunks) {
+        uint2 o;
+        if (fast) {
+          o.x = quant4<true>(v[c].x, v[c].y, s, r);
+          o.y = quant4<true>(v[c].z, v[c].w, s, r);
+        } else {
+          o.x = quant4<false>(v[c].x, v[c].y, s, 0.0f);
+          o.y = quant4<false>(v[c].z, v[c].w, s, 0.0f);
+        }
+        qr[idx] = o;
+      }
+    }
+  }
+}
+
+// Any K and alignment: the same arithmetic element by element; y is recomputed in the
+// cast pass (the row is an L2 hit by then).
+__global__ __launch_bounds__(64) void ln_modulate_quant_generic(
+    const uint16_t* __restrict__ x, int64_t ld_x, const uint16_t* __restrict__ shift,
+    const uint16_t* __restrict__ scale_mod, int64_t ld_mod, int rows_per_mod, float eps,
+    uint16_t* __restrict__ y, int64_t ld_y, uint8_t* __restrict__ q, int64_t ld_q,
+    float* __restrict__ scale, int M, int K, int scale_mode) {
+  const int lane = threadIdx.x & 63;
+  const float inv_k = 1.0f / (float)K;
+  auto f = [](uint16_t b) { return __uint_as_float((uint32_t)b << 16); };
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+    const uint16_t* xr = x + row * ld_x;
+    const uint16_t* shr = shift + (row / rows_per_mod) * ld_mod;
+    const uint16_t* scr = scale_mod + (row / rows_per_mod) * ld_mod;
+    float sum = 0.0f;
+    for (int k = lane; k < K; k += 64) sum += f(xr[k]);
+    const float mean = wave_sum_f32(sum) * inv_k;
+    float ss = 0.0f;
+    for (int k = lane; k < K; k += 64) {
+      const float a = f(xr[k]) - mean;
+      ss = __fmaf_rn(a, a, ss);
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum_f32(ss) * inv_k + eps);
+    uint32_t m = 0;
+    for (int k = lane; k < K; k += 64) {
+      const uint32_t yb = modulate1(f(xr[k]), mean, rstd, f(scr[k]), f(shr[k]));
+      if (y) y[row * ld_y + k] = (uint16_t)yb;
+      const uint32_t a = yb & 0x7fffu;
+      m = m > a ? m : a;
+    }
+    m = wave_max_u32(m);
+    const float s = row_scale(m, scale_mode);
+    if (lane == 0) scale[row] = s;
+    for (int k = lane; k < K; k += 64) {
+      const uint32_t yb = modulate1(f(xr[k]), mean, rstd, f(scr[k]), f(shr[k]));
+      const float v = clamp448(__uint_as_float(yb << 16) / s);
+      q[row * ld_q + k] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(v, v, 0u, false) & 0xffu);
+    }
+  }
+}
+
 }  // namespace
 
 // Cache hints of the row-in-registers kernel. 0: non-temporal loads and stores; 1: both plain;
@@ -275,6 +437,50 @@ int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void
 #undef CDIT_QUANT_LAUNCH
   hipLaunchKernelGGL(quant_rowwise_generic, grid, block, 0, stream, xp, ld_x, qp, ld_q, scale, Mi,
                      Ki, scale_mode);
+  return 0;
+}
+
+int launch_ln_modulate_quant(const void* x, int64_t M, int64_t K, int64_t ld_x, const void* shift,
+                             const void* scale_mod, int64_t ld_mod, int64_t rows_per_mod, float eps,
+                             void* y, int64_t ld_y, void* q, int64_t ld_q, float* scale,
+                             int scale_mode, hipStream_t stream) {
+  const uint16_t* xp = static_cast<const uint16_t*>(x);
+  const uint16_t* shp = static_cast<const uint16_t*>(shift);
+  const uint16_t* scp = static_cast<const uint16_t*>(scale_mod);
+  uint16_t* yp = static_cast<uint16_t*>(y);
+  uint8_t* qp = static_cast<uint8_t*>(q);
+  auto a16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool aligned = K % 8 == 0 && ld_x % 8 == 0 && ld_q % 8 == 0 && ld_mod % 8 == 0 &&
+                       (!y || (ld_y % 8 == 0 && a16(y))) && a16(x) && a16(shift) &&
+                       a16(scale_mod) && reinterpret_cast<uintptr_t>(q) % 8 == 0;
+  int64_t blocks = M;
+  const int64_t kMaxBlocks = 256 * 256;
+  if (blocks > kMaxBlocks) blocks = kMaxBlocks;
+  dim3 grid((unsigned)blocks), block(64);
+  const int need = (int)((K + 511) / 512);
+#define CDIT_LNQ_CASE(CH)                                                                       \
+  if (aligned && need <= CH) {                                                                  \
+    if (y)                                                                                      \
+      hipLaunchKernelGGL((ln_modulate_quant_regs<CH, true>), grid, block, 0, stream, xp, ld_x,   \
+                         shp, scp, ld_mod, (int)rows_per_mod, eps, yp, ld_y, qp, ld_q, scale,    \
+                         (int)M, (int)K, scale_mode);                                           \
+    else                                                                                        \
+      hipLaunchKernelGGL((ln_modulate_quant_regs<CH, false>), grid, block, 0, stream, xp, ld_x,  \
+                         shp, scp, ld_mod, (int)rows_per_mod, eps, yp, ld_y, qp, ld_q, scale,    \
+                         (int)M, (int)K, scale_mode);                                           \
+    return 0;                                                                                   \
+  }
+  CDIT_LNQ_CASE(1)
+  CDIT_LNQ_CASE(2)
+  CDIT_LNQ_CASE(4)
+  CDIT_LNQ_CASE(6)
+  CDIT_LNQ_CASE(8)
+  CDIT_LNQ_CASE(10)
+  CDIT_LNQ_CASE(12)
+  CDIT_LNQ_CASE(16)
+#undef CDIT_LNQ_CASE
+  hipLaunchKernelGGL(ln_modulate_quant_generic, grid, block, 0, stream, xp, ld_x, shp, scp, ld_mod,
+                     (int)rows_per_mod, eps, yp, ld_y, qp, ld_q, scale, (int)M, (int)K, scale_mode);
   return 0;
 }
 

@@ -139,60 +139,78 @@ def w8a16_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
 
 
 class _SharedQuant:
-  """Last activation quantized on a (device, stream): the input view (kept alive, so
-  its storage cannot be freed and handed out again), its version counter, the codes /
-  scales computed from it, and the id of the graph capture it was made in (0: none)."""
+  """An activation quantized on a (device, stream): the input view (kept alive, so its
+  storage cannot be freed and handed out again), its version counter, the codes / scales
+  computed from it, and the id of the graph capture it was made in (0: none)."""
   __slots__ = ("x", "version", "mode", "q", "s", "capture_id")
 
+  def matches(self, x2: torch.Tensor, scale_mode_id: int) -> bool:
+    return (self.mode == scale_mode_id and self.version == x2._version
+            and self.x.data_ptr() == x2.data_ptr() and self.x.shape == x2.shape
+            and self.x.stride() == x2.stride()
+            and self.x.untyped_storage().data_ptr() == x2.untyped_storage().data_ptr())
 
+
+#: (device, stream) -> most recent entries first. A DiT block keeps at most a few
+#: quantized activations in use at a time (image and text stream normed inputs, then the
+#: MLP input), so a handful of entries is enough.
 _shared_quant: dict = {}
+_SHARED_QUANT_ENTRIES = 4
 quant_launches = 0  # quantizer launches issued through shared_activation_quant (for tests)
 
 
+def _shared_entries(x2: torch.Tensor):
+  """The live entries of x2's (device, stream), and the current capture id. Entries made
+  inside a graph capture belong to that capture alone (their codes live in that graph's
+  pool and are only valid inside its replays): a list made under another capture id, or
+  on the other side of a capture boundary, is dropped."""
+  dev = x2.device
+  capture_id = (_native.stream_capture_id(_stream_ptr(x2))
+                if torch.cuda.is_current_stream_capturing() else 0)
+  key = (dev.index, torch._C._cuda_getCurrentRawStream(dev.index))
+  entries = _shared_quant.get(key)
+  if entries is None or (entries and entries[0].capture_id != capture_id):
+    entries = _shared_quant[key] = []
+  return entries, capture_id
+
+
+def _remember_quant(entries, capture_id, x2, scale_mode_id, q, s) -> None:
+  e = _SharedQuant()
+  e.x, e.version, e.mode, e.q, e.s, e.capture_id = x2, x2._version, scale_mode_id, q, s, capture_id
+  entries.insert(0, e)
+  del entries[_SHARED_QUANT_ENTRIES:]
+
+
 def shared_activation_quant(x2: torch.Tensor, scale_mode_id: int):
-  """Codes and scales of `x2` [M,K], reusing the previous result when the same
-  buffer (storage, offset, shape, strides), unmodified since (same `_version`), is
-  quantized again on the same stream -- sibling Linears such as to_q / to_k / to_v
-  (and proj_mlp in FLUX single blocks) all read one normalized activation
-  (reference dataflow: src/cache_dit/caching/patch_functors/functor_flux.py:60-67).
-  The results are bit-identical to quantizing again. In-place changes made through
-  PyTorch bump `_version` and miss; writes by foreign kernels into a live input
-  between two sibling calls would not be seen, which is why sharing is opt-in."""
+  """Codes and scales of `x2` [M,K], reusing an earlier result when the same buffer
+  (storage, offset, shape, strides), unmodified since (same `_version`), is quantized
+  again on the same stream -- sibling Linears such as to_q / to_k / to_v (and proj_mlp
+  in FLUX single blocks) all read one normalized activation (reference dataflow:
+  src/cache_dit/caching/patch_functors/functor_flux.py:60-67) -- or when its producer
+  already delivered them (ln_modulate_quant). The results are bit-identical to
+  quantizing again. In-place changes made through PyTorch bump `_version` and miss;
+  writes by foreign kernels into a live input between two sibling calls would not be
+  seen, which is why sharing is opt-in."""
   global quant_launches
   dev = x2.device
+  M, K = x2.shape
   if x2.is_inference():
     # inference-mode tensors carry no version counter: an in-place change could not be
     # told from an unchanged buffer, so nothing is shared (torch.no_grad() keeps it)
-    M, K = x2.shape
     q = torch.empty((M, K), dtype=FP8, device=dev)
     s = torch.empty((M, ), dtype=torch.float32, device=dev)
     quant_rowwise_into(x2, q, s, scale_mode_id, gemm_follows=True)
     quant_launches += 1
     return q, s
-  capturing = torch.cuda.is_current_stream_capturing()
-  # an entry made during a graph capture belongs to that capture alone: its codes live in
-  # that graph's pool and are only valid inside replays of that graph
-  capture_id = _native.stream_capture_id(_stream_ptr(x2)) if capturing else 0
-  key = (dev.index, torch._C._cuda_getCurrentRawStream(dev.index))
-  e = _shared_quant.get(key)
-  if e is not None and e.capture_id != capture_id:
-    e = None  # made in another capture, or on the other side of a capture boundary
-    del _shared_quant[key]
-  if (e is not None and e.mode == scale_mode_id and e.version == x2._version
-      and e.x.data_ptr() == x2.data_ptr() and e.x.shape == x2.shape
-      and e.x.stride() == x2.stride()
-      and e.x.untyped_storage().data_ptr() == x2.untyped_storage().data_ptr()):
-    return e.q, e.s
-  M, K = x2.shape
+  entries, capture_id = _shared_entries(x2)
+  for e in entries:
+    if e.matches(x2, scale_mode_id):
+      return e.q, e.s
   q = torch.empty((M, K), dtype=FP8, device=dev)
   s = torch.empty((M, ), dtype=torch.float32, device=dev)
   quant_rowwise_into(x2, q, s, scale_mode_id, gemm_follows=True)
   quant_launches += 1
-  if e is None:
-    e = _SharedQuant()
-    _shared_quant[key] = e
-  e.x, e.version, e.mode, e.q, e.s = x2, x2._version, scale_mode_id, q, s
-  e.capture_id = capture_id
+  _remember_quant(entries, capture_id, x2, scale_mode_id, q, s)
   return q, s
 
 
@@ -336,6 +354,79 @@ def _fake_float8_inference_scaled_mm(a_data, a_scale, b_data, b_scale, bias, out
                                      use_fast_accum, epilogue=0):
   return a_data.new_empty((*a_data.shape[:-1], b_data.shape[-1]),
                           dtype=decode_output_dtype(out_dtype_id))
+
+
+torch.library.define(
+    "cdit::ln_modulate_quant",
+    "(Tensor x, Tensor shift, Tensor scale, float eps=1e-6, int scale_mode=0, "
+    "bool write_y=True) -> (Tensor, Tensor, Tensor)",
+)
+
+
+@torch.library.impl("cdit::ln_modulate_quant", "CUDA")
+def _ln_modulate_quant(x, shift, scale, eps=1e-6, scale_mode=0, write_y=True):
+  """LayerNorm (no affine) over the last dimension, `* (1 + scale) + shift`, and the
+  per-row FP8 quantization of the result, in one kernel. x bf16 [..., K]; shift, scale
+  bf16 with K elements per modulation vector, either one vector for everything or one per
+  leading index of x (AdaLN: [B, 1, K] for x [B, S, K]). Returns (y bf16 like x -- left
+  unwritten when write_y is False --, codes e4m3 like x, scales fp32 [..., 1])."""
+  name = "cdit::ln_modulate_quant"
+  if x.dtype != torch.bfloat16 or shift.dtype != torch.bfloat16 or scale.dtype != torch.bfloat16:
+    raise ValueError(f"{name}: x, shift and scale must be bfloat16, got {x.dtype}, {shift.dtype}, "
+                     f"{scale.dtype}")
+  if x.dim() < 1 or x.shape[-1] == 0:
+    raise ValueError(f"{name}: x needs a non-empty last dimension")
+  if scale_mode not in (0, 1):
+    raise ValueError(f"{name}: scale_mode must be 0 or 1, got {scale_mode}")
+  K = x.shape[-1]
+  x2 = _as_rows(x)
+  M = x2.shape[0]
+  if shift.shape != scale.shape or shift.shape[-1] != K or shift.numel() % K != 0:
+    raise ValueError(f"{name}: shift {tuple(shift.shape)} / scale {tuple(scale.shape)} do not "
+                     f"hold vectors of K={K} elements")
+  nb = shift.numel() // K
+  if nb != 1 and not (x.dim() >= 2 and nb == x.shape[0] and M % nb == 0):
+    raise ValueError(f"{name}: {nb} modulation vectors for x of shape {tuple(x.shape)}: expected "
+                     "one, or one per index of x's first dimension")
+  sh2, sc2 = shift.reshape(nb, K).contiguous(), scale.reshape(nb, K).contiguous()
+  y = torch.empty((M, K), dtype=torch.bfloat16, device=x.device)
+  q = torch.empty((M, K), dtype=FP8, device=x.device)
+  s = torch.empty((M, ), dtype=torch.float32, device=x.device)
+  if M > 0:
+    with _DeviceOf(x2):
+      _native.check(_native.load().cdit_fp8_ln_modulate_quant(
+          x2.data_ptr(), M, K, x2.stride(0), sh2.data_ptr(), sc2.data_ptr(), K,
+          M if nb == 1 else M // nb, float(eps), y.data_ptr() if write_y else None, K,
+          q.data_ptr(), K, s.data_ptr(), int(scale_mode), _stream_ptr(x2)))
+  return y.view(x.shape), q.view(x.shape), s.view(*x.shape[:-1], 1)
+
+
+@torch.library.register_fake("cdit::ln_modulate_quant")
+def _fake_ln_modulate_quant(x, shift, scale, eps=1e-6, scale_mode=0, write_y=True):
+  return (x.new_empty(x.shape), x.new_empty(x.shape, dtype=FP8),
+          x.new_empty((*x.shape[:-1], 1), dtype=torch.float32))
+
+
+def ln_modulate_quant(x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor, eps: float = 1e-6,
+                      scale_mode: str = "bf16div", materialize: bool = True) -> torch.Tensor:
+  """`layer_norm(x) * (1 + scale) + shift` whose FP8 codes are produced in the same pass
+  and handed to the quantized Linears that consume the result: they find them under the
+  returned tensor's identity (the lookup `share_activation_quant_` switches on) and skip
+  their own quantizer launch. The returned tensor is a drop-in for the unfused
+  expression. With materialize=False its bf16 values are NOT written (the kernel then
+  only writes codes and scales): only for a caller that knows every consumer is such a
+  Linear. Inside torch.inference_mode() tensors carry no version counter to key the
+  lookup on; the bf16 tensor is then always written and nothing is handed over."""
+  _require_cuda("ln_modulate_quant", x, shift, scale)
+  mode_id = _native.SCALE_MODE_IDS[scale_mode]
+  no_handover = x.is_inference() or torch.is_inference_mode_enabled()
+  y, q, s = torch.ops.cdit.ln_modulate_quant(x, shift, scale, float(eps), mode_id,
+                                             bool(materialize or no_handover))
+  if not no_handover and y.numel() > 0:
+    y2 = y.view(-1, y.shape[-1])
+    entries, capture_id = _shared_entries(y2)
+    _remember_quant(entries, capture_id, y2, mode_id, q.view(y2.shape), s.view(-1))
+  return y
 
 
 GRANULARITY_PER_ROW, GRANULARITY_PER_TENSOR = 0, 1

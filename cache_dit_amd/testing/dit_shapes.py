@@ -97,6 +97,21 @@ def _ln(x, eps=1e-6):
   return F.layer_norm(x.float(), (x.shape[-1], ), eps=eps).to(x.dtype)
 
 
+class _ModulatedNorm:
+  """Mixin of the modules that compute `layer_norm(x) * (1 + scale) + shift` for quantized
+  Linears. With `fused_norm_quant` set (see fuse_norm_quant) the expression runs as one
+  HIP kernel that also delivers the FP8 codes to those Linears."""
+  fused_norm_quant = False
+  fused_norm_materialize = True
+
+  def _modulated(self, x, shift, scale):
+    if self.fused_norm_quant and x.is_cuda:
+      from .. import ops
+      return ops.ln_modulate_quant(x, shift, scale, eps=1e-6,
+                                   materialize=self.fused_norm_materialize)
+    return _ln(x) * (1 + scale) + shift
+
+
 class TimeEmbed(nn.Module):
   """timestep (+ pooled text) -> conditioning vector; names contain `embed`, so the
   default exclude list leaves these Linears alone when quantizing the whole model."""
@@ -121,7 +136,7 @@ class TimeEmbed(nn.Module):
 # ------------------------------------------------------------------------------- FLUX
 
 
-class AdaLayerNormZero(nn.Module):
+class AdaLayerNormZero(_ModulatedNorm, nn.Module):
 
   def __init__(self, dim: int, chunks: int):
     super().__init__()
@@ -131,7 +146,7 @@ class AdaLayerNormZero(nn.Module):
   def forward(self, x, temb):
     mods = self.linear(F.silu(temb)).unsqueeze(1).chunk(self.chunks, dim=-1)
     shift, scale = mods[0], mods[1]
-    return _ln(x) * (1 + scale) + shift, mods[2:]
+    return self._modulated(x, shift, scale), mods[2:]
 
 
 class FluxAttention(nn.Module):
@@ -168,7 +183,7 @@ class FluxAttention(nn.Module):
     return self.to_out[1](self.to_out[0](o[:, n_txt:])), self.to_add_out(o[:, :n_txt])
 
 
-class FluxTransformerBlock(nn.Module):
+class FluxTransformerBlock(_ModulatedNorm, nn.Module):
   """Double-stream block: 14 Linears (7 per stream)."""
 
   def __init__(self, dim: int, heads: int, mlp: int):
@@ -182,9 +197,9 @@ class FluxTransformerBlock(nn.Module):
     ne, (c_gate_msa, c_shift_mlp, c_scale_mlp, c_gate_mlp) = self.norm1_context(encoder, temb)
     a, ca = self.attn(nh, ne, rope)
     hidden = hidden + gate_msa * a
-    hidden = hidden + gate_mlp * self.ff(_ln(hidden) * (1 + scale_mlp) + shift_mlp)
+    hidden = hidden + gate_mlp * self.ff(self._modulated(hidden, shift_mlp, scale_mlp))
     encoder = encoder + c_gate_msa * ca
-    encoder = encoder + c_gate_mlp * self.ff_context(_ln(encoder) * (1 + c_scale_mlp) + c_shift_mlp)
+    encoder = encoder + c_gate_mlp * self.ff_context(self._modulated(encoder, c_shift_mlp, c_scale_mlp))
     return encoder, hidden
 
 
@@ -253,7 +268,7 @@ def flux_like_inputs(device, n_img=4096, n_txt=512, in_channels=64, text_dim=409
 # ------------------------------------------------------------------------------- Qwen-Image
 
 
-class QwenImageTransformerBlock(nn.Module):
+class QwenImageTransformerBlock(_ModulatedNorm, nn.Module):
   """12 quantized Linears + `img_mod.1` / `txt_mod.1`, which the default exclude
   pattern "mod" skips."""
 
@@ -264,9 +279,8 @@ class QwenImageTransformerBlock(nn.Module):
     self.attn = FluxAttention(dim, heads, joint=True)
     self.img_mlp, self.txt_mlp = FeedForward(dim, mlp), FeedForward(dim, mlp)
 
-  @staticmethod
-  def _modulate(x, shift, scale):
-    return _ln(x) * (1 + scale) + shift
+  def _modulate(self, x, shift, scale):
+    return self._modulated(x, shift, scale)
 
   def forward(self, hidden, encoder, temb, rope):
     i1, i2 = self.img_mod(temb).unsqueeze(1).chunk(2, dim=-1)
@@ -340,7 +354,7 @@ class WanAttention(nn.Module):
     return self.to_out[1](self.to_out[0](o))
 
 
-class WanTransformerBlock(nn.Module):
+class WanTransformerBlock(_ModulatedNorm, nn.Module):
   """10 Linears: self-attention, cross-attention to the text, GELU-tanh FFN."""
 
   def __init__(self, dim: int, heads: int, ffn: int):
@@ -352,9 +366,9 @@ class WanTransformerBlock(nn.Module):
 
   def forward(self, hidden, context, temb6, rope):
     sh1, sc1, g1, sh2, sc2, g2 = (self.scale_shift_table + temb6).chunk(6, dim=1)
-    hidden = hidden + g1 * self.attn1(_ln(hidden) * (1 + sc1) + sh1, rope=rope)
+    hidden = hidden + g1 * self.attn1(self._modulated(hidden, sh1, sc1), rope=rope)
     hidden = hidden + self.attn2(self.norm2(hidden), context)
-    return hidden + g2 * self.ffn(_ln(hidden) * (1 + sc2) + sh2)
+    return hidden + g2 * self.ffn(self._modulated(hidden, sh2, sc2))
 
 
 class WanLikeTransformer(nn.Module):
@@ -413,6 +427,25 @@ def fuse_gelu_epilogues(model: nn.Module) -> int:
     for lin, act in pairs:
       if isinstance(lin, _Fp8LinearBase) and not getattr(act, "_cdit_fused_into_linear", False):
         fuse_gelu_tanh_(lin, act)
+        n += 1
+  return n
+
+
+def fuse_norm_quant(model: nn.Module, enable: bool = True, materialize: bool = True) -> int:
+  """Switches every modulated LayerNorm of `model` to the kernel that also quantizes
+  (ops.ln_modulate_quant). Pair it with share_activation_quant_ on the Linears so that
+  they pick the delivered codes up. materialize=False also drops the bf16 write of the
+  modulated activation: valid here because only quantized Linears read it. Returns the
+  number of modules switched."""
+  n = 0
+  blocks = getattr(model, "_repeated_blocks", [])
+  for blk in model.modules():
+    if type(blk).__name__ not in blocks:
+      continue  # outside the repeated blocks (norm_out) the consumer is an unquantized Linear
+    for m in blk.modules():
+      if isinstance(m, _ModulatedNorm):
+        m.fused_norm_quant = bool(enable)
+        m.fused_norm_materialize = bool(materialize)
         n += 1
   return n
 

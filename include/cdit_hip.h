@@ -115,6 +115,31 @@ int cdit_fp8_quant_tensorwise(const void* x_bf16, int64_t M, int64_t K, int64_t 
                               int scale_mode, void* stream);
 
 /*
+ * The per-row quantizer fused into its producer: LayerNorm without affine parameters,
+ * AdaLN modulation and per-row FP8 quantization in one pass over the activation. In a DiT
+ * block the modulated activation `norm(x) * (1 + scale) + shift` is read by quantized
+ * Linears only (reference dataflow src/cache_dit/caching/patch_functors/functor_flux.py:48-80:
+ * `self.norm(...)` feeds proj_mlp and attn.to_q/k/v), so the codes are produced where the
+ * activation is. Per row m, with mod = m / rows_per_mod (one modulation vector per batch
+ * element, broadcast over its tokens):
+ *
+ *   mean = sum_k x / K;  var = sum_k (x - mean)^2 / K;  rstd = 1 / sqrt(var + eps)   (fp32)
+ *   y[m,k] = bf16(bf16(bf16((x - mean) * rstd) * bf16(1 + scale[mod,k])) + shift[mod,k])
+ *   (q[m,:], out_scale[m]) = the per-row quantization of y[m,:], exactly as
+ *                            cdit_fp8_quant_rowwise computes it
+ *
+ * Every step rounds to bf16 where the unfused sequence of bf16 tensor ops does. x bf16
+ * [M,K] (ld_x); shift, scale bf16 [ceil(M / rows_per_mod), K] (ld_mod); y bf16 [M,K]
+ * (ld_y) or NULL when no consumer reads the bf16 tensor; q e4m3 [M,K] (ld_q); out_scale
+ * fp32 [M]. Algorithmic bytes per row: 3 K + 4 (5 K + 4 with y).
+ */
+int cdit_fp8_ln_modulate_quant(const void* x_bf16, int64_t M, int64_t K, int64_t ld_x,
+                               const void* shift_bf16, const void* scale_bf16, int64_t ld_mod,
+                               int64_t rows_per_mod, float eps, void* y_bf16, int64_t ld_y,
+                               void* q_e4m3, int64_t ld_q, float* out_scale, int scale_mode,
+                               void* stream);
+
+/*
  * Row-wise scaled FP8 GEMM with fused epilogue. Replaces
  * torch._scaled_mm(a, b, scale_a, scale_b, bias, out_dtype) as called by
  * _run_float8_inference_scaled_mm, src/cache_dit/quantization/torchao/_scaled_mm.py:62-91

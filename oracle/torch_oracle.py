@@ -80,6 +80,27 @@ def quantize_tensorwise(x: torch.Tensor,
   return quantize_affine_float8(x, scale), scale.expand(x.shape[0], 1).contiguous()
 
 
+def ln_modulate(x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor,
+                eps: float = 1e-6) -> torch.Tensor:
+  """The modulated activation of a DiT block as eager bf16 tensor ops compute it:
+  LayerNorm without affine parameters (fp32 statistics, bf16 result), then
+  `* (1 + scale) + shift` with every bf16 op rounding its result -- diffusers'
+  AdaLayerNormZeroSingle / AdaLayerNormZero, whose output feeds proj_mlp and
+  attn.to_q/k/v (src/cache_dit/caching/patch_functors/functor_flux.py:60-67).
+  x bf16 [..., K]; shift, scale bf16 broadcastable to x."""
+  K = x.shape[-1]
+  n = torch.nn.functional.layer_norm(x.to(torch.float32), (K, ), eps=eps).to(x.dtype)
+  return n * (1 + scale) + shift
+
+
+def ln_modulate_quant(x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor, eps: float = 1e-6,
+                      scale_mode: str = "bf16div"):
+  """(y, codes, scales): the modulated activation and its per-row quantization."""
+  y = ln_modulate(x, shift, scale, eps)
+  q, s = quantize_rowwise(y, scale_mode)
+  return y, q, s
+
+
 def gelu_tanh(v: torch.Tensor) -> torch.Tensor:
   return torch.nn.functional.gelu(v, approximate="tanh")
 
