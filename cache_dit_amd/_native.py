@@ -22,6 +22,7 @@ QUANT_GEMM_FOLLOWS = 0x100  # cache hint, OR-ed into the scale mode of the per-r
 EPI_NONE = 0
 EPI_GELU_TANH = 1
 DT_F16, DT_BF16, DT_F32 = 0, 1, 2
+MAX_GROUP = 4  # members of cdit_fp8_gemm_rowwise_grouped
 STATIC_WS_CODE_BYTES, STATIC_WS_ROWS = 96 << 20, 65536  # cdit_fp8_linear_w8a8_static
 
 #: every symbol include/cdit_hip.h declares
@@ -33,6 +34,7 @@ EXPORTS = (
     "cdit_fp8_quant_tensorwise",
     "cdit_fp8_ln_modulate_quant",
     "cdit_fp8_gemm_rowwise",
+    "cdit_fp8_gemm_rowwise_grouped",
     "cdit_w8a16_gemm",
     "cdit_fp8_linear_w8a8",
     "cdit_fp8_linear_w8a8_static",
@@ -77,6 +79,11 @@ def _bind(L: ctypes.CDLL) -> None:
   L.cdit_fp8_gemm_rowwise.restype = ci
   L.cdit_fp8_gemm_rowwise.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci,
                                       vp]
+  L.cdit_fp8_gemm_rowwise_grouped.restype = ci
+  L.cdit_fp8_gemm_rowwise_grouped.argtypes = [vp, vp, i64, i64, i64, ci, ctypes.POINTER(vp),
+                                              ctypes.POINTER(vp), ctypes.POINTER(vp),
+                                              ctypes.POINTER(vp), ctypes.POINTER(i64), i64,
+                                              ctypes.POINTER(i64), ctypes.POINTER(ci), vp]
   L.cdit_fp8_linear_w8a8.restype = ci
   L.cdit_fp8_linear_w8a8.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci,
                                      ci, vp]

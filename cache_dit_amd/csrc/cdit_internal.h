@@ -41,8 +41,27 @@ struct GemmArgs {
   int out_dtype = CDIT_DT_BF16;  // CDIT_DT_*; the w8a16 kernels only build bf16
 };
 
+// GEMMs that share the A operand (same activation codes and scales: same M, K, lda, ldb)
+// and differ in the weight side. col_begin is filled by the launcher.
+constexpr int kMaxGroup = 4;
+struct GemmGroup {
+  int count;
+  int col_begin[kMaxGroup + 1];
+  const uint8_t* b[kMaxGroup];
+  const float* b_scale[kMaxGroup];
+  const uint16_t* bias[kMaxGroup];
+  uint16_t* out[kMaxGroup];
+  int N[kMaxGroup];
+  int64_t ldo[kMaxGroup];
+  int epilogue[kMaxGroup];
+};
+
 // variant < 0: choose by shape.
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream);
+// All members of `grp` in one launch (A side and ldb from `shared`). 0: launched; -1: not
+// taken (shape, alignment or variant without a grouped form); else a CDIT_E* code.
+int launch_gemm_fp8_grouped(const GemmArgs& shared, const GemmGroup& grp, int variant,
+                            hipStream_t stream);
 int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream);
 // One w8a8 Linear forward at M <= 16 in a single kernel (per-token quantizer + GEMM);
 // g.a is the bf16 activation, g.lda its leading dimension in elements. Returns 0 when

@@ -387,11 +387,24 @@ __device__ __forceinline__ void mfma_16x16x128_fp8(v4f& acc, const v8i& b, const
   }
 }
 
+// A group of GEMMs that share the A operand (the same activation codes and scales, so
+// the same M, K and lda) and differ in the weight: sibling Linears such as to_q / to_k /
+// to_v, and proj_mlp next to them in FLUX single blocks (reference dataflow:
+// src/cache_dit/caching/patch_functors/functor_flux.py:60-67). Their tiles are walked as
+// one tile stream by one persistent launch, as if the weights were stacked along N:
+// member p owns the tile columns [col_begin[p], col_begin[p + 1]). Every member has its
+// own weight, scale, bias, output and epilogue flag; ldb is common (GemmGroup, declared
+// with the launchers).
+struct NoGroup {};
+
 // OUT: dtype of the output and of the bias (CDIT_DT_*), a template parameter so that
-// the bf16 instances carry no trace of the others.
-template <class C, int OUT = CDIT_DT_BF16>
+// the bf16 instances carry no trace of the others. GROUPED: the launch walks the tiles
+// of a GemmGroup (the B-side fields of `g` are then unused); the instances without it
+// are unchanged by its existence.
+template <class C, int OUT = CDIT_DT_BF16, bool GROUPED = false>
 __global__ __launch_bounds__(C::THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void
-gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
+gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
+              std::conditional_t<GROUPED, GemmGroup, NoGroup> grp) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -412,12 +425,44 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
   // the end of the last step are the next tile's first. The epilogue of a tile
   // then runs with the next tile's panels landing in LDS, and its stores drain
   // while the next K loop is under way.
+  // B side of a tile: for a group, looked up from the tile column (the table sits in the
+  // kernel arguments: scalar loads with a uniform index)
+  auto member_of = [&](int tn, int* first_col) {
+    int p = 0;
+    if constexpr (GROUPED) {
+#pragma unroll
+      for (int i = 1; i < kMaxGroup; ++i)
+        if (i < grp.count && tn >= grp.col_begin[i]) p = i;
+      *first_col = grp.col_begin[p];
+    } else {
+      *first_col = 0;
+    }
+    return p;
+  };
+  auto b_of = [&](int p) -> const uint8_t* {
+    if constexpr (GROUPED) return grp.b[p];
+    return g.b;
+  };
+  auto n_of = [&](int p) -> int {
+    if constexpr (GROUPED) return grp.N[p];
+    return g.N;
+  };
+  auto grp_b_scale = [&](int p) -> const float* {
+    if constexpr (GROUPED) return grp.b_scale[p];
+    return g.b_scale;
+  };
+  auto grp_bias = [&](int p) -> const uint16_t* {
+    if constexpr (GROUPED) return grp.bias[p];
+    return g.bias;
+  };
   int m0, n0;  // tile being computed
+  int cur = 0;  // group member it belongs to
   {
-    int tm, tn;
+    int tm, tn, c0;
     tile_of_block<C::GROUP_M>(blockIdx.x, ntiles, tiles_m, tiles_n, &tm, &tn);
+    cur = member_of(tn, &c0);
     m0 = tm * C::BM;
-    n0 = tn * C::BN;
+    n0 = (tn - c0) * C::BN;
   }
 
   // DMA source: tile whose panels the DMA stream currently fetches. Instruction p
@@ -432,10 +477,10 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
   // and B: between two tiles without partial panels they are not recomputed (some 130
   // VALU instructions in the middle of the MFMA stream otherwise).
   bool off_clamped = true;  // the first call computes them
-  auto set_source = [&](int sm0, int sn0) {
+  auto set_source = [&](int sm0, int sn0, int member) {
     A = static_cast<const uint8_t*>(g.a) + (int64_t)sm0 * g.lda;
-    B = g.b + (int64_t)sn0 * g.ldb;
-    const int rows_a = g.M - sm0, rows_b = g.N - sn0;
+    B = b_of(member) + (int64_t)sn0 * g.ldb;
+    const int rows_a = g.M - sm0, rows_b = n_of(member) - sn0;
     const bool clamped = rows_a < C::BM || rows_b < C::BN;
     if (!clamped && !off_clamped) return;
     off_clamped = clamped;
@@ -452,7 +497,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
                     : (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
     }
   };
-  set_source(m0, n0);
+  set_source(m0, n0, cur);
   // buffer_load ... lds (MUBUF form: the compiler tracks it with vmcnt only, while
   // the global_load form makes it wait for all LDS reads at every use). With a
   // descriptor of zero records every lane is out of range: nothing is fetched and
@@ -517,7 +562,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
 
   for (int tile = blockIdx.x;; tile += gridDim.x) {
     const int next_tile = tile + gridDim.x;
-    int nm0 = 0, nn0 = 0;
+    int nm0 = 0, nn0 = 0, next_member = 0;
     // fragments of step 0 (in LDS since the prologue, or since the barrier of the
     // previous tile's last step). The last step of a tile reads them too, like
     // every step does for its successor, but keeping them across the epilogue
@@ -547,11 +592,12 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
       if (EVENTS && kt == KT - D) {
         // every DMA of this tile has been issued: the stream moves on
         if (next_tile < ntiles) {
-          int tm, tn;
+          int tm, tn, c0;
           tile_of_block<C::GROUP_M>(next_tile, ntiles, tiles_m, tiles_n, &tm, &tn);
+          next_member = member_of(tn, &c0);
           nm0 = tm * C::BM;
-          nn0 = tn * C::BN;
-          set_source(nm0, nn0);
+          nn0 = (tn - c0) * C::BN;
+          set_source(nm0, nn0, next_member);
         } else {
           nrec = 0;
         }
@@ -559,10 +605,13 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
       if (EVENTS && kt == KT - 2) {
         // buffer accesses: what lies beyond N (M) reads as zero, no bounds branches; a
         // null bias becomes an empty buffer
+        const float* const cur_b_scale = GROUPED ? grp_b_scale(cur) : g.b_scale;
+        const uint16_t* const cur_bias = GROUPED ? grp_bias(cur) : g.bias;
+        const int cur_n = n_of(cur);
         const __amdgpu_buffer_rsrc_t bs_buf = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<float*>(g.b_scale), 0, g.N * 4, 0x00020000);
+            const_cast<float*>(cur_b_scale), 0, cur_n * 4, 0x00020000);
         const __amdgpu_buffer_rsrc_t bi_buf = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<uint16_t*>(g.bias), 0, g.bias ? g.N * 2 : 0, 0x00020000);
+            const_cast<uint16_t*>(cur_bias), 0, cur_bias ? cur_n * 2 : 0, 0x00020000);
         const __amdgpu_buffer_rsrc_t as_buf = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<float*>(g.a_scale), 0, g.M * 4, 0x00020000);
         if constexpr (C::STAGE_EPI) {
@@ -703,8 +752,17 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     constexpr int OB = OUT == CDIT_DT_F32 ? 4 : 2;  // bytes per output element
     constexpr uint32_t kNoColumn = 0x80000000u;
     constexpr int kStoreOnce = 2;  // cache policy of the output stores: non-temporal (written once)
-    uint8_t* const out_wave = reinterpret_cast<uint8_t*>(g.out) +
-                              ((int64_t)(m0 + wm * C::WM) * g.ldo + (n0 + wn * C::WN)) * OB;
+    uint16_t* cur_out = g.out;
+    int64_t cur_ldo = g.ldo;
+    int cur_epilogue = g.epilogue;
+    if constexpr (GROUPED) {
+      cur_out = grp.out[cur];
+      cur_ldo = grp.ldo[cur];
+      cur_epilogue = grp.epilogue[cur];
+    }
+    const int cur_N = n_of(cur);
+    uint8_t* const out_wave = reinterpret_cast<uint8_t*>(cur_out) +
+                              ((int64_t)(m0 + wm * C::WM) * cur_ldo + (n0 + wn * C::WN)) * OB;
     const int rows_wave = g.M - (m0 + wm * C::WM);  // rows of the wave tile that exist
     // The memory pipeline merges the lanes of a store into one request only when
     // adjacent lanes write adjacent bytes: with lane = 16 kg + r16 holding row r16,
@@ -716,19 +774,19 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     constexpr bool PERMUTE = OUT != CDIT_DT_F32;
     const int st_row = PERMUTE ? lane >> 2 : r16, st_piece = PERMUTE ? lane & 3 : kg;
     const int bp_addr = 4 * (16 * (lane & 3) + (lane >> 2));
-    const uint32_t out_lane = ((uint32_t)st_row * (uint32_t)g.ldo + 8u * st_piece) * OB;
+    const uint32_t out_lane = ((uint32_t)st_row * (uint32_t)cur_ldo + 8u * st_piece) * OB;
     uint32_t out_off[TN / 2];
 #pragma unroll
     for (int u = 0; u < TN / 2; ++u)
-      out_off[u] = n0 + wn * C::WN + 8 * st_piece + 64 * (u >> 1) + 32 * (u & 1) < g.N
+      out_off[u] = n0 + wn * C::WN + 8 * st_piece + 64 * (u >> 1) + 32 * (u & 1) < cur_N
                        ? out_lane + (64 * (u >> 1) + 32 * (u & 1)) * OB
                        : kNoColumn;
     auto out_row_of = [&](int i) {
       // (made a scalar explicitly: a descriptor the compiler takes for divergent is
       // applied in a loop over its distinct values)
       const int rows = __builtin_amdgcn_readfirstlane(min(max(rows_wave - 16 * i, 0), 16));
-      return __builtin_amdgcn_make_buffer_rsrc(out_wave + (int64_t)(16 * i) * g.ldo * OB, 0,
-                                               rows * g.ldo * OB, 0x00020000);
+      return __builtin_amdgcn_make_buffer_rsrc(out_wave + (int64_t)(16 * i) * cur_ldo * OB, 0,
+                                               rows * cur_ldo * OB, 0x00020000);
     };
     // 16-bit outputs: the permuted words of a row of blocks are stored while the next
     // row is being computed, so the latency of the permutation is not waited for; the
@@ -797,7 +855,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
         __builtin_amdgcn_sched_barrier(0);
       }
     };
-    if (g.epilogue & CDIT_EPI_GELU_TANH) {
+    if (cur_epilogue & CDIT_EPI_GELU_TANH) {
       epilogue(std::true_type{});
     } else {
       epilogue(std::false_type{});
@@ -806,6 +864,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n) {
     if (next_tile >= ntiles) break;
     m0 = nm0;
     n0 = nn0;
+    cur = next_member;
   }
   // the zero-record DMA of the last D steps must not outlive the workgroup
   wait_vm<0>();
@@ -826,7 +885,33 @@ int launch_wide(const GemmArgs& g, hipStream_t stream) {
   const int ntiles = tiles_m * tiles_n;
   // one persistent workgroup per CU (its LDS and registers fill the CU)
   hipLaunchKernelGGL((gemm_fp8_wide<C, OUT>), dim3(ntiles < cus ? ntiles : cus), dim3(C::THREADS),
-                     C::LDS_BYTES, stream, g, tiles_m, tiles_n);
+                     C::LDS_BYTES, stream, g, tiles_m, tiles_n, NoGroup{});
+  return 0;
+}
+
+// The members' tiles as one launch: tile columns of member p are [col_begin[p], col_begin[p+1]).
+template <class C>
+int launch_wide_grouped(const GemmArgs& g, GemmGroup grp, hipStream_t stream) {
+  static bool lds_allowed[64];
+  if (int rc = allow_dynamic_lds(
+          reinterpret_cast<const void*>(&gemm_fp8_wide<C, CDIT_DT_BF16, true>), C::LDS_BYTES,
+          lds_allowed))
+    return rc;
+  const int cus = cu_count();
+  if (cus <= 0) {
+    set_error("cannot query the CU count of the current device");
+    return CDIT_EHIP;
+  }
+  const int tiles_m = (g.M + C::BM - 1) / C::BM;
+  int tiles_n = 0;
+  for (int p = 0; p < grp.count; ++p) {
+    grp.col_begin[p] = tiles_n;
+    tiles_n += (grp.N[p] + C::BN - 1) / C::BN;
+  }
+  for (int p = grp.count; p <= kMaxGroup; ++p) grp.col_begin[p] = tiles_n;
+  const int ntiles = tiles_m * tiles_n;
+  hipLaunchKernelGGL((gemm_fp8_wide<C, CDIT_DT_BF16, true>), dim3(ntiles < cus ? ntiles : cus),
+                     dim3(C::THREADS), C::LDS_BYTES, stream, g, tiles_m, tiles_n, grp);
   return 0;
 }
 
@@ -1116,6 +1201,11 @@ int launch_linear_fp8_skinny_fused(const GemmArgs& g, void* q_ws, float* scale_w
   return 0;
 }
 
+template <class Tiles, class WideOk>
+int choose_bf16_variant(Tiles tiles, WideOk wide_ok);
+template <class WideOk>
+int launch_bf16_variant(const GemmArgs& g, int variant, WideOk wide_ok, hipStream_t stream);
+
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {
     dim3 grid((g.N + 15) / 16, (g.M + 15) / 16);
@@ -1159,9 +1249,19 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     return 0;
   }
   if (variant < 0) {
-    auto tiles = [&](int bm, int bn) {
-      return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
-    };
+    variant = choose_bf16_variant(
+        [&](int bm, int bn) { return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn); },
+        wide_ok);
+  }
+  return launch_bf16_variant(g, variant, wide_ok, stream);
+}
+
+// Tile choice for a bf16-output problem whose tile count for a bm x bn tile is tiles(bm, bn)
+// (a single GEMM, or a group of GEMMs stacked along N).
+template <class Tiles, class WideOk>
+int choose_bf16_variant(Tiles tiles, WideOk wide_ok) {
+  int variant;
+  {
     // workgroups a round holds: one per CU (what launch_wide starts)
     const int64_t cus = cu_count() > 0 ? cu_count() : 256;
     if (tiles(256, 256) * 256 >= 160 * cus) {
@@ -1205,6 +1305,11 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
       }
     }
   }
+  return variant;
+}
+
+template <class WideOk>
+int launch_bf16_variant(const GemmArgs& g, int variant, WideOk wide_ok, hipStream_t stream) {
   switch (variant) {
     case 0: return launch_tiled<V0>(g, stream);
     case 1: return launch_tiled<V1>(g, stream);
@@ -1221,6 +1326,40 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     default:
       set_error("cdit_fp8_gemm_rowwise: unknown kernel variant %d", variant);
       return CDIT_EINVAL;
+  }
+}
+
+// The group as one launch. Returns 0 when launched, -1 when the group is not taken (the
+// caller then runs the members one by one), a CDIT_E* code on error.
+int launch_gemm_fp8_grouped(const GemmArgs& shared, const GemmGroup& grp, int variant,
+                            hipStream_t stream) {
+  if (grp.count < 2 || grp.count > kMaxGroup || shared.M <= 16 || shared.out_dtype != CDIT_DT_BF16)
+    return -1;
+  for (int p = 0; p < grp.count; ++p) {
+    GemmArgs g = shared;
+    g.b = grp.b[p];
+    g.b_scale = grp.b_scale[p];
+    g.bias = grp.bias[p];
+    g.out = grp.out[p];
+    g.N = grp.N[p];
+    g.ldo = grp.ldo[p];
+    if (!tiled_ok(g) || g.N <= 0) return -1;
+  }
+  auto wide_ok = [&](int depth) { return shared.K >= 128 * (depth > 3 ? depth : 3); };
+  auto tiles = [&](int bm, int bn) {
+    int64_t cols = 0;
+    for (int p = 0; p < grp.count; ++p) cols += (grp.N[p] + bn - 1) / bn;
+    return (int64_t)((shared.M + bm - 1) / bm) * cols;
+  };
+  if (variant < 0) variant = choose_bf16_variant(tiles, wide_ok);
+  switch (variant) {
+    case 12: return wide_ok(V12::DEPTH) ? launch_wide_grouped<V12>(shared, grp, stream) : -1;
+    case 14: return wide_ok(V14::DEPTH) ? launch_wide_grouped<V14>(shared, grp, stream) : -1;
+    case 15: return wide_ok(V15::DEPTH) ? launch_wide_grouped<V15>(shared, grp, stream) : -1;
+    case 16: return wide_ok(V16::DEPTH) ? launch_wide_grouped<V16>(shared, grp, stream) : -1;
+    case 17: return wide_ok(V17::DEPTH) ? launch_wide_grouped<V17>(shared, grp, stream) : -1;
+    case 18: return wide_ok(V18::DEPTH) ? launch_wide_grouped<V18>(shared, grp, stream) : -1;
+    default: return -1;  // the kernels without a tile stream have no grouped form
   }
 }
 

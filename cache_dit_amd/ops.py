@@ -127,6 +127,29 @@ def gemm_rowwise_into(a: torch.Tensor, a_scale: torch.Tensor, w: torch.Tensor,
         w.stride(0), out.stride(0), epilogue, encode_output_dtype(out.dtype), _stream_ptr(a)))
 
 
+def gemm_rowwise_grouped_into(a: torch.Tensor, a_scale: torch.Tensor, weights, w_scales, biases,
+                              outs, epilogues) -> None:
+  """Sibling GEMMs on one activation (a [M,K] e4m3 with scales [M]) as one launch: member
+  p is weights[p] [N_p,K] e4m3 with the same row stride, w_scales[p] fp32, biases[p] bf16
+  or None, outs[p] [M,N_p] bf16, epilogues[p]. Bit-identical to one gemm_rowwise_into per
+  member."""
+  import ctypes
+  n = len(weights)
+  M, K = a.shape
+  vp, i64 = ctypes.c_void_p, ctypes.c_int64
+  ldb = weights[0].stride(0)
+  if any(w.stride(0) != ldb or w.shape[1] != K for w in weights):
+    raise ValueError("gemm_rowwise_grouped_into: the weights must share K and the row stride")
+  with _DeviceOf(a):
+    _native.check(_native.load().cdit_fp8_gemm_rowwise_grouped(
+        a.data_ptr(), a_scale.data_ptr(), M, K, a.stride(0), n,
+        (vp * n)(*[w.data_ptr() for w in weights]), (vp * n)(*[s.data_ptr() for s in w_scales]),
+        (vp * n)(*[b.data_ptr() if b is not None else None for b in biases]),
+        (vp * n)(*[o.data_ptr() for o in outs]), (i64 * n)(*[w.shape[0] for w in weights]), ldb,
+        (i64 * n)(*[o.stride(0) for o in outs]), (ctypes.c_int * n)(*[int(e) for e in epilogues]),
+        _stream_ptr(a)))
+
+
 def w8a16_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
                bias: Optional[torch.Tensor], out: torch.Tensor, epilogue: int) -> None:
   M, K = x2.shape

@@ -167,6 +167,26 @@ int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale,
                           int epilogue, int out_dtype_id, void* stream);
 
 /*
+ * `count` (1 to 4) row-wise scaled FP8 GEMMs that share the A operand -- the same
+ * activation codes and scales, hence the same M, K and lda -- as ONE launch whose tile
+ * stream runs over all their output tiles: sibling Linears that read one activation, such
+ * as attn.to_q / to_k / to_v, and proj_mlp next to them in FLUX single blocks (reference
+ * dataflow src/cache_dit/caching/patch_functors/functor_flux.py:60-67; each is a separate
+ * torch._scaled_mm call there, _scaled_mm.py:62-91). Member p has its own weight b_q[p]
+ * [N[p],K] (common ldb), b_scale[p] [N[p]], bias[p] (bf16 [N[p]] or NULL; `bias` itself may
+ * be NULL), out[p] bf16 [M,N[p]] (ldo[p]) and epilogue[p] (`epilogue` may be NULL = none).
+ * The arrays live on the host and are read before the call returns. Results are those of
+ * `count` calls of cdit_fp8_gemm_rowwise with CDIT_DT_BF16, bit for bit; shapes the
+ * grouped kernel does not take are run that way.
+ */
+int cdit_fp8_gemm_rowwise_grouped(const void* a_q, const float* a_scale,
+                                  int64_t M, int64_t K, int64_t lda, int count,
+                                  const void* const* b_q, const float* const* b_scale,
+                                  const void* const* bias, void* const* out,
+                                  const int64_t* N, int64_t ldb, const int64_t* ldo,
+                                  const int* epilogue, void* stream);
+
+/*
  * Weight-only FP8 GEMM (w8a16): bf16 activations, e4m3 weights dequantized in
  * the mainloop, per-output-channel scale applied in the epilogue. Replaces
  * F.linear(x, W.dequantize(), bias) of torchao's Float8WeightOnlyConfig
