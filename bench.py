@@ -131,6 +131,9 @@ class HotPath:
     self.q = {mk: torch.empty(mk, dtype=torch.float8_e4m3fn, device=device) for mk in max_mk}
     self.s = {mk: torch.empty(mk[0], dtype=torch.float32, device=device) for mk in max_mk}
     self.out = torch.empty(max_mn, dtype=torch.bfloat16, device=device)
+    # a run of siblings writes its outputs side by side
+    run_mn = max(sum(self.layers[i][0] * self.layers[i][2] for i in run) for run in self.sibling_runs())
+    self.out2 = torch.empty(run_mn, dtype=torch.bfloat16, device=device)
 
   def step(self):
     """One pass: for every Linear the same library call its module forward makes
@@ -144,33 +147,71 @@ class HotPath:
       out = self.out[:M * N].view(M, N)
       ops.linear_w8a8_into(self.x[(M, K)], w, ws, b, out, self.q[(M, K)], self.s[(M, K)], 0, epi)
 
+  def sibling_runs(self):
+    """The Linears as runs of siblings: consecutive Linears that read the same activation in
+    the model (q/k/v of a stream; proj_mlp + q/k/v in FLUX single blocks; Wan's cross
+    attention k/v), each run a list of indices into self.layers."""
+    runs = []
+    for i, (name, *_) in enumerate(self.linears):
+      leaf = name.split(".", 2)[2]
+      same_input = leaf in ("attn.to_k", "attn.to_v", "attn.add_k_proj", "attn.add_v_proj",
+                            "attn1.to_k", "attn1.to_v", "attn2.to_v") or (
+                                name.startswith("single") and leaf == "attn.to_q")  # after proj_mlp
+      if same_input and runs:
+        runs[-1].append(i)
+      else:
+        runs.append([i])
+    return runs
+
   def step_shared_quant(self):
     """The same pass with one quantizer launch per distinct input: q/k/v (and
     proj_mlp in single blocks) read one activation, as share_activation_quant_
     arranges in a real model. Outputs are bit-identical to step()."""
     from cache_dit_amd import ops
-    names = [n for n, *_ in self.linears]
-    for name, (M, K, N, w, ws, b, epi) in zip(names, self.layers):
-      out = self.out[:M * N].view(M, N)
-      leaf = name.split(".", 2)[2]
-      reuse = leaf in ("attn.to_k", "attn.to_v", "attn.add_k_proj", "attn.add_v_proj") or (
-          name.startswith("single") and leaf == "attn.to_q")  # after proj_mlp
-      if not reuse:
-        ops.quant_rowwise_into(self.x[(M, K)], self.q[(M, K)], self.s[(M, K)], 0, gemm_follows=True)
-      ops.gemm_rowwise_into(self.q[(M, K)], self.s[(M, K)], w, ws, b, out, epi)
+    for run in self.sibling_runs():
+      M, K = self.layers[run[0]][:2]
+      ops.quant_rowwise_into(self.x[(M, K)], self.q[(M, K)], self.s[(M, K)], 0, gemm_follows=True)
+      for i in run:
+        _, _, N, w, ws, b, epi = self.layers[i]
+        ops.gemm_rowwise_into(self.q[(M, K)], self.s[(M, K)], w, ws, b, self.out[:M * N].view(M, N), epi)
+
+  def step_grouped(self):
+    """The pass as a model runs it with group_sibling_linears_: every run of siblings is one
+    quantizer launch and ONE grouped GEMM launch (cdit_fp8_gemm_rowwise_grouped); a Linear
+    without siblings is the fused quantizer + GEMM call of step(). Outputs are bit-identical
+    to step(); siblings write to disjoint parts of the output scratch."""
+    from cache_dit_amd import ops
+    for run in self.sibling_runs():
+      M, K = self.layers[run[0]][:2]
+      if len(run) == 1:
+        _, _, N, w, ws, b, epi = self.layers[run[0]]
+        ops.linear_w8a8_into(self.x[(M, K)], w, ws, b, self.out[:M * N].view(M, N), self.q[(M, K)],
+                             self.s[(M, K)], 0, epi)
+        continue
+      ops.quant_rowwise_into(self.x[(M, K)], self.q[(M, K)], self.s[(M, K)], 0, gemm_follows=True)
+      members = [self.layers[i] for i in run]
+      outs, at = [], 0
+      for _, _, N, *_ in members:
+        outs.append(self.out2[at:at + M * N].view(M, N))
+        at += M * N
+      ops.gemm_rowwise_grouped_into(self.q[(M, K)], self.s[(M, K)], [m[3] for m in members],
+                                    [m[4] for m in members], [m[5] for m in members], outs,
+                                    [m[6] for m in members])
 
 
 def step_leg(device, linears, mode, steps, warmup):
   """A step of another benchmark configuration (every quantized Linear of the model at
-  its real shape with its own weights), captured into a hipGraph and replayed like the
-  headline step. Returns ms per step, TFLOP/s and the Linear count."""
+  its real shape with its own weights; w8a8: siblings grouped as in the headline step),
+  captured into a hipGraph and replayed like the headline step. Returns ms per step,
+  TFLOP/s and the Linear count."""
   import torch
   hot = HotPath(device, linears, mode)
-  hot.step()
+  step = hot.step if mode == "w8a16" else hot.step_grouped
+  step()
   torch.cuda.synchronize()
   graph = torch.cuda.CUDAGraph()
   with torch.cuda.graph(graph):
-    hot.step()
+    step()
   for _ in range(warmup):
     graph.replay()
   torch.cuda.synchronize()
@@ -381,27 +422,54 @@ def cpu_baseline():
   }
 
 
-def dit_forward_ms(device):
-  """Full synthetic FLUX-shaped transformer forward (attention, norms, RoPE and
-  residual glue included), quantized with float8_per_row."""
+def dit_forward_ms(device, iters=5):
+  """Full synthetic FLUX-shaped transformer forward (attention, norms, RoPE and residual
+  glue included), quantized with float8_per_row and set up the way a serving loop would:
+  GELU-tanh folded into the producing Linear, sibling Linears grouped, the quantizer fused
+  into the modulated LayerNorms. Timed with eager launches and as one hipGraph replay.
+  Returns (eager ms, graph ms or None, note)."""
   try:
     import torch
     import cache_dit_amd
+    from cache_dit_amd.testing import dit_shapes
     from cache_dit_amd.testing.dit_shapes import FluxLikeTransformer, flux_like_inputs
   except Exception as e:
-    return None, f"synthetic transformer unavailable: {e}"[:160]
+    return None, None, f"synthetic transformer unavailable: {e}"[:160]
   torch.manual_seed(0)
   with torch.device(device):
     model = FluxLikeTransformer().to(torch.bfloat16)
   cache_dit_amd.quantize(model, cache_dit_amd.QuantizeConfig(quant_type="float8_per_row"))
-  from cache_dit_amd.testing import dit_shapes
   dit_shapes.fuse_gelu_epilogues(model)
   cache_dit_amd.share_activation_quant_(model)
   inputs = flux_like_inputs(device)
+  cache_dit_amd.group_sibling_linears_(model, lambda: model(**inputs))
+  dit_shapes.fuse_norm_quant(model, materialize=False)
+  graph_ms = None
   with torch.no_grad():
-    ms = _time_events(lambda: model(**inputs), 5, 2)
-  return ms, "float8_per_row, GELU-tanh fused into the producing Linear, shared activation " \
-             "quantization; bf16 SDPA attention, norms and RoPE in eager PyTorch"
+    ms = _time_events(lambda: model(**inputs), iters, 2)
+    try:
+      side = torch.cuda.Stream()
+      side.wait_stream(torch.cuda.current_stream())
+      with torch.cuda.stream(side):
+        model(**inputs)
+      torch.cuda.current_stream().wait_stream(side)
+      torch.cuda.synchronize()
+      graph = torch.cuda.CUDAGraph()
+      with torch.cuda.graph(graph):
+        model(**inputs)
+      graph_ms = _time_events(graph.replay, iters, 2)
+      del graph
+    except Exception as e:
+      graph_ms = None
+      note_err = f"; graph capture failed: {str(e)[:80]}"
+    else:
+      note_err = ""
+  del model
+  torch.cuda.empty_cache()
+  return ms, graph_ms, ("float8_per_row, GELU-tanh fused into the producing Linear, sibling Linears "
+                        "grouped on one shared quantization, quantizer fused into the modulated "
+                        "LayerNorms; bf16 SDPA attention, RMS norms, RoPE and residual glue in eager "
+                        "PyTorch ops" + note_err)
 
 
 def main():
@@ -418,6 +486,10 @@ def main():
                   help="run only the headline-shape kernels (the roofline legs) and print their "
                        "figures: the command to put under rocprofv3 when per-kernel averages "
                        "must not mix shapes")
+  ap.add_argument("--dit-only", action="store_true",
+                  help="run only the full synthetic transformer forward (eager and as a hipGraph "
+                       "replay): the command to put under rocprofv3 for the kernel mix of a whole "
+                       "DiT step")
   ap.add_argument("--pmc-sequence", action="store_true",
                   help="run only the launch sequence for rocprofv3 --pmc counter collection "
                        "(fill, plain copy, quantizer, fill, GEMM at the headline shape, 4 times)")
@@ -441,6 +513,11 @@ def main():
     pmc_sequence(device)
     print(json.dumps({"pmc_sequence": "done", "device": arch}))
     return
+  if args.dit_only:
+    ms, gms, note = dit_forward_ms(device, iters=args.steps)
+    print(json.dumps({"dit_step_ms": ms, "dit_step_ms_graph": gms, "dit_step_note": note,
+                      "device": arch}))
+    return
   if args.headline_only:
     print(json.dumps({"linear_headline": headline_kernels(device), "device": arch}))
     return
@@ -455,47 +532,41 @@ def main():
     hot.step()
   torch.cuda.synchronize()
   eager_ms = (time.perf_counter() - t0) / args.steps * 1e3
-  # the same step captured once into a hipGraph and replayed: what a serving loop
-  # does with a fixed-shape denoising step; removes the host launch cost
-  launch_mode = "hipGraph replay"
-  try:
-    graph = torch.cuda.CUDAGraph()
+  # The same step captured once into a hipGraph and replayed: what a serving loop does
+  # with a fixed-shape denoising step; removes the host launch cost. Three forms of the
+  # step, all with bit-identical outputs: every Linear on its own (quantizer + GEMM each);
+  # one quantizer launch per distinct activation (share_activation_quant_); and, the
+  # headline, sibling Linears also as one grouped GEMM launch (group_sibling_linears_).
+  def replay_ms(step_fn):
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
-      hot.step()
+      step_fn()
     torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-      hot.step()
+      step_fn()
     for _ in range(args.warmup):
       graph.replay()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(args.steps):  # exactly `steps` timed steps
       graph.replay()
     torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-  except Exception as e:  # capture unavailable: report the eager figure
-    launch_mode = f"eager (graph capture failed: {str(e)[:80]})"
-    dt = eager_ms * args.steps / 1e3
-  ms_per_step = dt / args.steps * 1e3
-  value = hot.flop / (dt / args.steps) / 1e12
-  # extra: the same step with shared activation quantization (304 quantizer launches)
+    return (time.perf_counter() - t0) / args.steps * 1e3
+
+  launch_mode = "hipGraph replay"
   try:
-    g2 = torch.cuda.CUDAGraph()
-    hot.step_shared_quant()
-    torch.cuda.synchronize()
-    with torch.cuda.graph(g2):
-      hot.step_shared_quant()
-    g2.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-      g2.replay()
-    torch.cuda.synchronize()
-    shared_ms = (time.perf_counter() - t0) / args.steps * 1e3
-  except Exception:
-    shared_ms = None
+    ungrouped_ms = replay_ms(hot.step)
+    shared_ms = replay_ms(hot.step_shared_quant)
+    ms_per_step = replay_ms(hot.step_grouped)
+  except Exception as e:  # capture unavailable: report the eager figure of the plain step
+    launch_mode = f"eager (graph capture failed: {str(e)[:80]})"
+    ungrouped_ms = shared_ms = None
+    ms_per_step = eager_ms
+  value = hot.flop / ms_per_step / 1e9
+  n_runs = len(hot.sibling_runs())
   n_layers = len(hot.layers)
   step_flop = hot.flop
   del hot
@@ -503,6 +574,7 @@ def main():
   if args.step_only:
     print(json.dumps({"value": value, "unit": "TFLOP/s", "ms_per_step": ms_per_step,
                       "launch": launch_mode, "eager_ms_per_step": eager_ms,
+                      "ungrouped_ms_per_step": ungrouped_ms,
                       "shared_quant_ms_per_step": shared_ms, "steps": args.steps,
                       "warmup": args.warmup, "device": arch}))
     return
@@ -539,7 +611,7 @@ def main():
     other["wan_step"] = step_leg(device, wan_step_linears(), "w8a8", few, 1)
     for k in ("qwen_step", "wan_step"):
       other[k]["frac_fp8_peak"] = other[k]["tflops"] / FP8_PEAK_TFLOPS
-  dit_ms, dit_note = (None, "skipped") if args.skip_dit else dit_forward_ms(device)
+  dit_ms, dit_graph_ms, dit_note = (None, None, "skipped") if args.skip_dit else dit_forward_ms(device)
   cpu = None if args.skip_cpu else cpu_baseline()
 
   line = {
@@ -557,16 +629,23 @@ def main():
       "data": "synthetic",
       "config": {
           "workload": "flux1_dev_shaped_step: all quantized Linears of one denoising step "
-                      "(19 double + 38 single blocks, 4096 img + 512 txt tokens), "
-                      "per-token quant + FP8 GEMM + epilogue each",
+                      "(19 double + 38 single blocks, 4096 img + 512 txt tokens): per-token "
+                      "quant + FP8 GEMM + epilogue; Linears that read one activation (q/k/v, "
+                      "proj_mlp + q/k/v) share its quantization and run as one grouped GEMM "
+                      "launch, bit-identical to running each on its own",
           "quant_type": "float8_per_row",
           "launch": launch_mode,
           "linears_per_step": n_layers,
+          "gemm_launches_per_step": n_runs,
           "linear_flop_per_step": step_flop,
           "batch": 1,
       },
       "frac_fp8_peak": value / FP8_PEAK_TFLOPS,
+      # the same step with every Linear on its own (eager launches, then replayed), and
+      # with shared quantization but one GEMM launch per Linear
       "eager_ms_per_step": eager_ms,
+      "ungrouped_ms_per_step": ungrouped_ms,
+      "ungrouped_tflops": None if not ungrouped_ms else step_flop / ungrouped_ms / 1e9,
       "shared_quant_ms_per_step": shared_ms,
       "linear_headline": head,
       # the other benchmark configurations as steps of their own (same construction as the
@@ -581,6 +660,7 @@ def main():
       "wan_step_tflops": other.get("wan_step", {}).get("tflops"),
       "other_configs": other,
       "dit_step_ms": dit_ms,
+      "dit_step_ms_graph": dit_graph_ms,
       "dit_step_note": dit_note,
       "roofline": roofline,
       "roofline_quant": roofline_quant,

@@ -21,6 +21,7 @@ from .nn import Fp8DynamicLinearPerTensor
 from .nn import Fp8WeightOnlyLinear
 from .nn import fuse_gelu_tanh_
 from .nn import share_activation_quant_
+from .nn import group_sibling_linears_
 from .ops import ln_modulate_quant
 from .utils import check_quantized
 
@@ -40,5 +41,6 @@ __all__ = [
     "Fp8WeightOnlyLinear",
     "fuse_gelu_tanh_",
     "share_activation_quant_",
+    "group_sibling_linears_",
     "ln_modulate_quant",
 ]

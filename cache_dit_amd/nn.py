@@ -66,6 +66,90 @@ class _Fp8LinearBase(nn.Linear):
       raise RuntimeError(f"{type(self).__name__}: input is on {x.device}; there is no CPU path")
 
 
+class _InputKey:
+  """Identity of an activation buffer: storage, offset, shape, strides and version
+  counter; keeps the tensor alive so that its address cannot be handed out again."""
+  __slots__ = ("x", "version")
+
+  def __init__(self, x2: torch.Tensor):
+    self.x, self.version = x2, x2._version
+
+  def matches(self, x2: torch.Tensor) -> bool:
+    x = self.x
+    return (self.version == x2._version and x.data_ptr() == x2.data_ptr() and x.shape == x2.shape
+            and x.stride() == x2.stride()
+            and x.untyped_storage().data_ptr() == x2.untyped_storage().data_ptr())
+
+
+class SiblingGroup:
+  """Two to four `float8_per_row` Linears that are handed the very same activation one
+  after the other (attn.to_q / to_k / to_v; proj_mlp + q/k/v in FLUX single blocks;
+  reference dataflow src/cache_dit/caching/patch_functors/functor_flux.py:60-67). The
+  first member called with an activation quantizes it once and computes every member's
+  output in ONE grouped GEMM launch; the others, called with the same unmodified buffer,
+  return theirs. Outputs are bit-identical to the ungrouped Linears. A member called with
+  anything else simply computes the group afresh, so a wrong guess costs time, not
+  correctness."""
+
+  def __init__(self, members):
+    members = list(members)
+    if not 2 <= len(members) <= _native.MAX_GROUP:
+      raise ValueError(f"a sibling group holds 2 to {_native.MAX_GROUP} Linears, got {len(members)}")
+    first = members[0]
+    for m in members:
+      if type(m) is not Fp8DynamicLinear:
+        raise TypeError("sibling groups are built from float8_per_row Linears")
+      if m.in_features != first.in_features or m._scale_mode_id != first._scale_mode_id:
+        raise ValueError("the members of a sibling group must share in_features and scale mode")
+    self.members = members
+    self.index = {id(m): i for i, m in enumerate(members)}
+    self.key = None  # _InputKey of the activation the pending outputs were computed from
+    self.outs = None
+    self.capture_id = 0
+
+  def forward_member(self, lin: "Fp8DynamicLinear", x: torch.Tensor) -> torch.Tensor:
+    x2 = ops._as_rows(x)
+    i = self.index[id(lin)]
+    capture_id = (_native.stream_capture_id(ops._stream_ptr(x2))
+                  if torch.cuda.is_current_stream_capturing() else 0)
+    if (self.key is not None and self.capture_id == capture_id and self.outs[i] is not None
+        and self.key.matches(x2)):
+      out, self.outs[i] = self.outs[i], None
+      if all(o is None for o in self.outs):
+        self.key = self.outs = None
+      return out.view(*x.shape[:-1], lin.out_features)
+    M = x2.shape[0]
+    members = self.members
+    outs = [torch.empty((M, m.out_features), dtype=torch.bfloat16, device=x2.device) for m in members]
+    if M > 0:
+      q, s = ops.shared_activation_quant(x2, lin._scale_mode_id)
+      ops.gemm_rowwise_grouped_into(q, s, [m.weight for m in members],
+                                    [m.weight_scale for m in members], [m.bias for m in members],
+                                    outs, [m.epilogue for m in members])
+    out, outs[i] = outs[i], None
+    self.key, self.outs, self.capture_id = _InputKey(x2), outs, capture_id
+    return out.view(*x.shape[:-1], lin.out_features)
+
+
+class _SiblingRecorder:
+  """Notes, during one forward, which Linears are called back to back with the same
+  activation buffer."""
+
+  def __init__(self):
+    self.runs, self.key = [], None
+
+  def note(self, lin, x):
+    x2 = ops._as_rows(x)
+    if self.key is not None and self.key.matches(x2) and all(lin is not m for m in self.runs[-1]):
+      self.runs[-1].append(lin)
+    else:
+      self.runs.append([lin])
+      self.key = _InputKey(x2)
+
+
+_recorder: Optional[_SiblingRecorder] = None
+
+
 class Fp8DynamicLinear(_Fp8LinearBase):
   """`float8_per_row` (w8a8 dynamic): per-token e4m3 activation quantization,
   e4m3 x e4m3 GEMM with fp32 accumulate, per-token x per-channel scales, bias,
@@ -75,11 +159,21 @@ class Fp8DynamicLinear(_Fp8LinearBase):
   opaque node with a fake implementation, the way the reference keeps this path
   traceable (src/cache_dit/quantization/torchao/_scaled_mm.py:94-137, :338-357)."""
 
+  sibling_group: Optional[SiblingGroup] = None
+
   def forward(self, x: torch.Tensor) -> torch.Tensor:
     self._check_input(x)
-    # sharing keeps the last activation's codes alive between calls; a compiled graph gets
-    # the stateless form (its front end owns the memory its graphs are captured into)
-    share = self.share_input_quant and not torch.compiler.is_compiling()
+    # sharing and grouping keep state between calls (the last activation's codes, the
+    # siblings' outputs); a compiled graph gets the stateless form (its front end owns the
+    # memory its graphs are captured into), and so do inference-mode tensors, which carry
+    # no version counter to tell a modified buffer by
+    stateless = torch.compiler.is_compiling()
+    if not stateless:
+      if _recorder is not None and not x.is_inference():
+        _recorder.note(self, x)
+      if self.sibling_group is not None and not x.is_inference():
+        return self.sibling_group.forward_member(self, x)
+    share = self.share_input_quant and not stateless
     return torch.ops.cdit.linear_w8a8(x, self.weight, self.weight_scale, self.bias,
                                       self._scale_mode_id, self.epilogue,
                                       ops.GRANULARITY_PER_ROW, share)
@@ -178,6 +272,43 @@ def share_activation_quant_(module: nn.Module, enable: bool = True) -> int:
   if not enable:
     ops.clear_shared_activation_quant()
   return n
+
+
+def group_sibling_linears_(module: nn.Module, run=None, enable: bool = True) -> int:
+  """Finds the `float8_per_row` Linears under `module` that are called back to back with
+  the very same activation and lets each such run (two to four Linears) compute its
+  outputs in one grouped GEMM launch on one shared quantization (SiblingGroup). `run` is a
+  callable that performs one forward of the model (e.g. `lambda: model(**inputs)`); it is
+  executed once under torch.no_grad() to observe the calls. Returns the number of groups
+  formed. enable=False removes every group under `module` (no `run` needed)."""
+  global _recorder
+  for m in module.modules():
+    if isinstance(m, Fp8DynamicLinear):
+      m.sibling_group = None
+  if not enable:
+    return 0
+  if run is None:
+    raise ValueError("group_sibling_linears_ needs `run`, a callable doing one forward")
+  mine = {id(m) for m in module.modules() if isinstance(m, Fp8DynamicLinear)}
+  _recorder = rec = _SiblingRecorder()
+  try:
+    with torch.no_grad():
+      run()
+  finally:
+    _recorder = None
+  groups = 0
+  for siblings in rec.runs:
+    siblings = [m for m in siblings if id(m) in mine and type(m) is Fp8DynamicLinear
+                and m.sibling_group is None]
+    siblings = [m for m in siblings if m.in_features == siblings[0].in_features
+                and m._scale_mode_id == siblings[0]._scale_mode_id]
+    while len(siblings) >= 2:
+      take, siblings = siblings[:_native.MAX_GROUP], siblings[_native.MAX_GROUP:]
+      g = SiblingGroup(take)
+      for m in take:
+        m.sibling_group = g
+      groups += 1
+  return groups
 
 
 def dequantize_weight(linear: _Fp8LinearBase) -> torch.Tensor:

@@ -131,3 +131,80 @@ def test_grouped_random_data_against_the_oracle_sampled_rows():
     ref = to.scaled_mm_rowwise(a[rows].cpu(), a_s[rows].cpu(), ws[p].cpu(), wss[p].cpu(), bs[p].cpu(),
                                gelu="fused" if p == 0 else None)
     assert max_rel_err(got[p][rows], ref) <= 1e-2, p
+
+
+def test_sibling_groups_in_a_model_are_found_and_bit_identical():
+  """group_sibling_linears_ on FLUX- and Wan-shaped toy models: the groups are the runs of
+  Linears fed the same buffer (q/k/v, add_q/k/v, proj_mlp + q/k/v; in Wan's cross
+  attention only to_k / to_v, which read the text), the output equals the ungrouped
+  model's bit for bit, also under graph capture and with the fused producer."""
+  import logging
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd import ops
+  from cache_dit_amd.testing import dit_shapes as ds
+  logging.getLogger("CACHE_DIT_AMD").setLevel(logging.WARNING)
+  torch.manual_seed(0)
+  kw = dict(dim=512, heads=4, mlp=2048, n_double=2, n_single=3, in_channels=64, text_dim=256,
+            pooled_dim=128)
+  model = ds.FluxLikeTransformer(**kw).to(torch.bfloat16).cuda()
+  cache_dit.quantize(model, cache_dit.QuantizeConfig())
+  ds.fuse_gelu_epilogues(model)
+  inputs = ds.flux_like_inputs("cuda", n_img=320, n_txt=64, in_channels=64, text_dim=256,
+                               pooled_dim=128)
+  with torch.no_grad():
+    y0 = model(**inputs)
+  n = cache_dit.group_sibling_linears_(model, lambda: model(**inputs))
+  assert n == 2 * 2 + 3 * 1
+  blk = model.single_transformer_blocks[0]
+  assert blk.proj_mlp.sibling_group is blk.attn.to_v.sibling_group
+  assert len(blk.proj_mlp.sibling_group.members) == 4 and blk.proj_out.sibling_group is None
+  with torch.no_grad():
+    ops.quant_launches = 0
+    y1 = model(**inputs)
+    # per double block 14 Linears, 6 of them in two groups; per single block 6, 4 in one group
+    assert ops.quant_launches == 2 * 2 + 3 * 1  # only the groups go through the shared lookup
+    assert torch.equal(y1, y0)
+    assert torch.equal(model(**inputs), y0)
+    # the fused producer hands its codes to the groups as well
+    ds.fuse_norm_quant(model)
+    ops.quant_launches = 0
+    y2 = model(**inputs)
+    assert ops.quant_launches == 0 and torch.isfinite(y2.float()).all()
+    ds.fuse_norm_quant(model, False)
+    # graph capture: the siblings' outputs live in the graph's pool
+    static = {k: v.clone() for k, v in inputs.items()}
+    model(**static)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+      model(**static)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+      ys = model(**static)
+    other = ds.flux_like_inputs("cuda", n_img=320, n_txt=64, in_channels=64, text_dim=256,
+                                pooled_dim=128, seed=5)
+    for src in (other, inputs):
+      want = model(**src)
+      torch.cuda.synchronize()
+      for k in static:
+        static[k].copy_(src[k])
+      graph.replay()
+      torch.cuda.synchronize()
+      assert torch.equal(ys, want)
+  with torch.inference_mode():  # no version counters: members compute on their own
+    assert torch.equal(model(**inputs), y0)
+  assert cache_dit.group_sibling_linears_(model, enable=False) == 0
+  assert blk.proj_mlp.sibling_group is None
+
+  wan = ds.WanLikeTransformer(dim=256, heads=2, ffn=512, n_layers=2, in_channels=64,
+                              text_dim=128).to(torch.bfloat16).cuda()
+  cache_dit.quantize(wan, cache_dit.QuantizeConfig())
+  winp = ds.wan_like_inputs("cuda", n_tokens=200, n_txt=48, in_channels=64, text_dim=128)
+  with torch.no_grad():
+    w0 = wan(**winp)
+    assert cache_dit.group_sibling_linears_(wan, lambda: wan(**winp)) == 2 * 2
+    b0 = wan.blocks[0]
+    assert len(b0.attn1.to_q.sibling_group.members) == 3
+    assert b0.attn2.to_q.sibling_group is None and len(b0.attn2.to_k.sibling_group.members) == 2
+    assert torch.equal(wan(**winp), w0)
