@@ -340,6 +340,43 @@ def headline_kernels(device):
       "quant_ms": quant_ms,
       "quant_gbps": (3.0 * M * K + 4.0 * M) / quant_ms / 1e6,
   }
+  # What bounds the quantizer at this size: the fixed cost of a launch of M one-wavefront
+  # workgroups. The same kernel with K = 0 (4608 workgroups that only write their scale)
+  # and on a single row, next to the 42 MB case; rocprofv3 --kernel-trace of this command
+  # gives the matching device-side durations (profiles/).
+  from cache_dit_amd import _native
+  L, stream = _native.load(), torch.cuda.current_stream().cuda_stream
+
+  def quant_raw(rows, cols):
+    def fn():
+      i = it["i"] = (it["i"] + 1) % nbuf
+      _native.check(L.cdit_fp8_quant_rowwise(xs[i].data_ptr(), rows, cols, K, qs[i].data_ptr(), K,
+                                             ss[i].data_ptr(), 0, stream))
+    return fn
+
+  res["quant_floor"] = {
+      "empty_4608_workgroups_us": _time_events(quant_raw(M, 0), 200, 20) * 1e3,
+      "one_row_us": _time_events(quant_raw(1, K), 200, 20) * 1e3,
+      "headline_us": quant_ms * 1e3,
+      "note": "HIP-event averages over back-to-back launches: K=0 (every workgroup only writes "
+              "its scale), one row of K=3072, and the 4608 x 3072 activation",
+  }
+  # the quantizer fused into its producer (LayerNorm + AdaLN modulation + quantization in one
+  # pass, bf16 output not written): same algorithmic bytes as the quantizer alone, 3MK + 4M
+  shift = torch.randn(K, device=device, generator=g).to(torch.bfloat16)
+  scale_mod = (torch.randn(K, device=device, generator=g) * 0.3).to(torch.bfloat16)
+
+  def ln_quant():
+    i = it["i"] = (it["i"] + 1) % nbuf
+    _native.check(L.cdit_fp8_ln_modulate_quant(xs[i].data_ptr(), M, K, K, shift.data_ptr(),
+                                               scale_mod.data_ptr(), K, M, 1e-6, None, K,
+                                               qs[i].data_ptr(), K, ss[i].data_ptr(), 0, stream))
+
+  lnq_ms = _time_events(ln_quant, 200, 20)
+  res["ln_modulate_quant_ms"] = lnq_ms
+  res["ln_modulate_quant_gbps"] = (3.0 * M * K + 4.0 * M) / lnq_ms / 1e6
+  for i in range(nbuf):  # the codes the later legs read are those of xs again
+    ops.quant_rowwise_into(xs[i], qs[i], ss[i], 0)
   res["gemm_frac_fp8_peak"] = res["gemm_tflops"] / FP8_PEAK_TFLOPS
   res["quant_frac_hbm_peak"] = res["quant_gbps"] / HBM_PEAK_GBPS
   res["linear_tflops"] = 2.0 * M * K * N / (gemm_ms + quant_ms) / 1e9

@@ -227,14 +227,44 @@ __global__ __launch_bounds__(64) void quant_tensorwise_cast(
 //   y = bf16(u + shift[k]);  then amax / scale / e4m3 cast of y as in quant_rowwise_regs.
 // shift and scale are bf16 [*, K]; row m uses their row m / rows_per_mod (one modulation
 // vector per batch element, broadcast over its tokens).
+// Sum over the wavefront, the same in every lane: four DPP steps inside each row of 16
+// lanes (the pattern of wave_max_u32: no LDS crossbar, no waits), then the four row sums
+// through scalars. The order of the additions is fixed, so the result does not depend on
+// where the wavefront runs.
 __device__ __forceinline__ float wave_sum_f32(float v) {
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
+  auto step = [](float a, int ctrl_id) {
+    int o;
+    const int ai = __float_as_int(a);
+    switch (ctrl_id) {
+      case 0: o = __builtin_amdgcn_update_dpp(0, ai, 0xB1, 0xf, 0xf, false); break;   // quad_perm [1,0,3,2]
+      case 1: o = __builtin_amdgcn_update_dpp(0, ai, 0x4E, 0xf, 0xf, false); break;   // quad_perm [2,3,0,1]
+      case 2: o = __builtin_amdgcn_update_dpp(0, ai, 0x141, 0xf, 0xf, false); break;  // row_half_mirror
+      default: o = __builtin_amdgcn_update_dpp(0, ai, 0x140, 0xf, 0xf, false); break;  // row_mirror
+    }
+    return a + __int_as_float(o);
+  };
+  v = step(v, 0);
+  v = step(v, 1);
+  v = step(v, 2);
+  v = step(v, 3);
+  const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return (a + b) + (c + d);
 }
 
 __device__ __forceinline__ uint32_t bf16_bits(float f) {
   return __float_as_uint(round_to_bf16(f)) >> 16;
+}
+
+// two fp32 -> packed bf16 pair, round to nearest even (v_cvt_pk_bf16_f32: one
+// instruction for what round_to_bf16 spells out in five integer operations per value)
+__device__ __forceinline__ uint32_t pk_bf16(float lo, float hi) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+  const v2f v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf));
 }
 
 // y bits of one element: x, scale, shift as fp32 (exact widenings of bf16 values)
@@ -245,10 +275,13 @@ __device__ __forceinline__ uint32_t modulate1(float x, float mean, float rstd, f
   return bf16_bits(u + sh);
 }
 
+// the same for a packed pair, every rounding step through the hardware converter
 __device__ __forceinline__ uint32_t modulate2(uint32_t xw, float mean, float rstd, uint32_t scw,
                                               uint32_t shw) {
-  return modulate1(bf16_lo(xw), mean, rstd, bf16_lo(scw), bf16_lo(shw)) |
-         (modulate1(bf16_hi(xw), mean, rstd, bf16_hi(scw), bf16_hi(shw)) << 16);
+  const uint32_t n = pk_bf16((bf16_lo(xw) - mean) * rstd, (bf16_hi(xw) - mean) * rstd);
+  const uint32_t t = pk_bf16(1.0f + bf16_lo(scw), 1.0f + bf16_hi(scw));
+  const uint32_t u = pk_bf16(bf16_lo(n) * bf16_lo(t), bf16_hi(n) * bf16_hi(t));
+  return pk_bf16(bf16_lo(u) + bf16_lo(shw), bf16_hi(u) + bf16_hi(shw));
 }
 
 template <int CH, bool WRITE_Y>
