@@ -22,7 +22,8 @@ QUANT_GEMM_FOLLOWS = 0x100  # cache hint, OR-ed into the scale mode of the per-r
 EPI_NONE = 0
 EPI_GELU_TANH = 1
 DT_F16, DT_BF16, DT_F32 = 0, 1, 2
-MAX_GROUP = 4  # members of cdit_fp8_gemm_rowwise_grouped
+MAX_GROUP = 8  # members of cdit_fp8_gemm_rowwise_grouped / _batched
+MAX_ACTS = 4  # activations of cdit_fp8_gemm_rowwise_batched
 STATIC_WS_CODE_BYTES, STATIC_WS_ROWS = 96 << 20, 65536  # cdit_fp8_linear_w8a8_static
 
 #: every symbol include/cdit_hip.h declares
@@ -35,6 +36,7 @@ EXPORTS = (
     "cdit_fp8_ln_modulate_quant",
     "cdit_fp8_gemm_rowwise",
     "cdit_fp8_gemm_rowwise_grouped",
+    "cdit_fp8_gemm_rowwise_batched",
     "cdit_w8a16_gemm",
     "cdit_fp8_linear_w8a8",
     "cdit_fp8_linear_w8a8_static",
@@ -84,6 +86,13 @@ def _bind(L: ctypes.CDLL) -> None:
                                               ctypes.POINTER(vp), ctypes.POINTER(vp),
                                               ctypes.POINTER(vp), ctypes.POINTER(i64), i64,
                                               ctypes.POINTER(i64), ctypes.POINTER(ci), vp]
+  L.cdit_fp8_gemm_rowwise_batched.restype = ci
+  L.cdit_fp8_gemm_rowwise_batched.argtypes = [ci, ctypes.POINTER(vp), ctypes.POINTER(vp),
+                                              ctypes.POINTER(i64), i64, i64, ctypes.POINTER(ci),
+                                              ctypes.POINTER(vp), ctypes.POINTER(vp),
+                                              ctypes.POINTER(vp), ctypes.POINTER(vp),
+                                              ctypes.POINTER(i64), i64, ctypes.POINTER(i64),
+                                              ctypes.POINTER(ci), vp]
   L.cdit_fp8_linear_w8a8.restype = ci
   L.cdit_fp8_linear_w8a8.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci,
                                      ci, vp]

@@ -310,74 +310,103 @@ int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale, const void* b_q
   return rc ? rc : after_launch(fn);
 }
 
-int cdit_fp8_gemm_rowwise_grouped(const void* a_q, const float* a_scale, int64_t M, int64_t K,
-                                  int64_t lda, int count, const void* const* b_q,
-                                  const float* const* b_scale, const void* const* bias,
-                                  void* const* out, const int64_t* N, int64_t ldb,
-                                  const int64_t* ldo, const int* epilogue, void* stream) {
-  const char* fn = "cdit_fp8_gemm_rowwise_grouped";
-  if (count < 1 || count > kMaxGroup) {
-    set_error("%s: count=%d, a group holds 1 to %d GEMMs", fn, count, kMaxGroup);
+// n_act activations, activation s with members_per_act[s] members (flattened in order).
+static int gemm_batched_impl(const char* fn, int n_act, const void* const* a_q,
+                             const float* const* a_scale, const int64_t* M, int64_t K, int64_t lda,
+                             const int* members_per_act, const void* const* b_q,
+                             const float* const* b_scale, const void* const* bias,
+                             void* const* out, const int64_t* N, int64_t ldb, const int64_t* ldo,
+                             const int* epilogue, void* stream) {
+  if (n_act < 1 || n_act > kMaxActs || !a_q || !a_scale || !M || !members_per_act) {
+    set_error("%s: 1 to %d activations with their arrays, got n_act=%d", fn, kMaxActs, n_act);
+    return CDIT_EINVAL;
+  }
+  int count = 0;
+  for (int s = 0; s < n_act; ++s) {
+    if (members_per_act[s] < 1) {
+      set_error("%s: activation %d has no member", fn, s);
+      return CDIT_EINVAL;
+    }
+    count += members_per_act[s];
+  }
+  if (count > kMaxGroup) {
+    set_error("%s: count=%d, a batch holds 1 to %d GEMMs", fn, count, kMaxGroup);
     return CDIT_EINVAL;
   }
   if (!b_q || !b_scale || !out || !N || !ldo) {
     set_error("%s: null array argument", fn);
     return CDIT_EINVAL;
   }
-  for (int p = 0; p < count; ++p) {
-    int rc = check_gemm(fn, a_q, b_q[p], b_scale[p], bias ? bias[p] : nullptr, out[p], M, N[p], K, lda,
-                        ldb, ldo[p], epilogue ? epilogue[p] : 0, CDIT_DT_BF16, false);
-    if (rc) return rc;
-  }
-  if (M == 0) return CDIT_OK;
-  if (!a_scale) {
-    set_error("%s: a_scale is null", fn);
-    return CDIT_EINVAL;
-  }
-  int rc = check_arch();
-  if (rc) return rc;
-  GemmArgs g;
-  g.a = a_q;
-  g.a_scale = a_scale;
-  g.b = static_cast<const uint8_t*>(b_q[0]);
-  g.b_scale = b_scale[0];
-  g.bias = static_cast<const uint16_t*>(bias ? bias[0] : nullptr);
-  g.out = static_cast<uint16_t*>(out[0]);
-  g.M = (int)M;
-  g.N = (int)N[0];
-  g.K = (int)K;
-  g.lda = lda;
-  g.ldb = ldb;
-  g.ldo = ldo[0];
-  g.epilogue = epilogue ? epilogue[0] : 0;
-  g.out_dtype = CDIT_DT_BF16;
   GemmGroup grp = {};
   grp.count = count;
+  grp.acts = n_act;
   bool any_empty = false;
-  for (int p = 0; p < count; ++p) {
-    grp.b[p] = static_cast<const uint8_t*>(b_q[p]);
-    grp.b_scale[p] = b_scale[p];
-    grp.bias[p] = static_cast<const uint16_t*>(bias ? bias[p] : nullptr);
-    grp.out[p] = static_cast<uint16_t*>(out[p]);
-    grp.N[p] = (int)N[p];
-    grp.ldo[p] = ldo[p];
-    grp.epilogue[p] = epilogue ? epilogue[p] : 0;
-    any_empty |= N[p] == 0;
+  for (int s = 0, p = 0; s < n_act; ++s) {
+    grp.first_member[s] = p;
+    for (int j = 0; j < members_per_act[s]; ++j, ++p) {
+      int rc = check_gemm(fn, a_q[s], b_q[p], b_scale[p], bias ? bias[p] : nullptr, out[p], M[s], N[p],
+                          K, lda, ldb, ldo[p], epilogue ? epilogue[p] : 0, CDIT_DT_BF16, false);
+      if (rc) return rc;
+      if (M[s] > 0 && N[p] > 0 && !a_scale[s]) {
+        set_error("%s: a_scale is null", fn);
+        return CDIT_EINVAL;
+      }
+      grp.b[p] = static_cast<const uint8_t*>(b_q[p]);
+      grp.b_scale[p] = b_scale[p];
+      grp.bias[p] = static_cast<const uint16_t*>(bias ? bias[p] : nullptr);
+      grp.out[p] = static_cast<uint16_t*>(out[p]);
+      grp.N[p] = (int)N[p];
+      grp.ldo[p] = ldo[p];
+      grp.epilogue[p] = epilogue ? epilogue[p] : 0;
+      any_empty |= N[p] == 0;
+    }
+    grp.a[s] = a_q[s];
+    grp.a_scale[s] = a_scale[s];
+    grp.M[s] = (int)M[s];
+    any_empty |= M[s] == 0;
   }
+  for (int s = n_act; s <= kMaxActs; ++s) grp.first_member[s] = count;
+  int rc = check_arch();
+  if (rc) return rc;
   if (!any_empty) {
-    rc = launch_gemm_fp8_grouped(g, grp, g_gemm_variant, static_cast<hipStream_t>(stream));
+    GemmArgs common = {};
+    common.K = (int)K;
+    common.lda = lda;
+    common.ldb = ldb;
+    common.out_dtype = CDIT_DT_BF16;
+    rc = launch_gemm_fp8_grouped(common, grp, g_gemm_variant, static_cast<hipStream_t>(stream));
     if (rc == 0) return after_launch(fn);
     if (rc > 0) return rc;
   }
-  // not taken as a group (a single member, an M <= 16 problem, an alignment only the
+  // not taken as a batch (a single member, an M <= 16 problem, an alignment only the
   // element-wise kernel takes): the members one after the other, same results
-  for (int p = 0; p < count; ++p) {
-    rc = cdit_fp8_gemm_rowwise(a_q, a_scale, b_q[p], b_scale[p], bias ? bias[p] : nullptr, out[p], M,
-                               N[p], K, lda, ldb, ldo[p], epilogue ? epilogue[p] : 0, CDIT_DT_BF16,
-                               stream);
-    if (rc) return rc;
-  }
+  for (int s = 0, p = 0; s < n_act; ++s)
+    for (int j = 0; j < members_per_act[s]; ++j, ++p) {
+      rc = cdit_fp8_gemm_rowwise(a_q[s], a_scale[s], b_q[p], b_scale[p], bias ? bias[p] : nullptr,
+                                 out[p], M[s], N[p], K, lda, ldb, ldo[p], epilogue ? epilogue[p] : 0,
+                                 CDIT_DT_BF16, stream);
+      if (rc) return rc;
+    }
   return CDIT_OK;
+}
+
+int cdit_fp8_gemm_rowwise_grouped(const void* a_q, const float* a_scale, int64_t M, int64_t K,
+                                  int64_t lda, int count, const void* const* b_q,
+                                  const float* const* b_scale, const void* const* bias,
+                                  void* const* out, const int64_t* N, int64_t ldb,
+                                  const int64_t* ldo, const int* epilogue, void* stream) {
+  return gemm_batched_impl("cdit_fp8_gemm_rowwise_grouped", 1, &a_q, &a_scale, &M, K, lda, &count,
+                           b_q, b_scale, bias, out, N, ldb, ldo, epilogue, stream);
+}
+
+int cdit_fp8_gemm_rowwise_batched(int n_act, const void* const* a_q, const float* const* a_scale,
+                                  const int64_t* M, int64_t K, int64_t lda,
+                                  const int* members_per_act, const void* const* b_q,
+                                  const float* const* b_scale, const void* const* bias,
+                                  void* const* out, const int64_t* N, int64_t ldb,
+                                  const int64_t* ldo, const int* epilogue, void* stream) {
+  return gemm_batched_impl("cdit_fp8_gemm_rowwise_batched", n_act, a_q, a_scale, M, K, lda,
+                           members_per_act, b_q, b_scale, bias, out, N, ldb, ldo, epilogue, stream);
 }
 
 int cdit_fp8_linear_w8a8(const void* x_bf16, const void* w_q, const float* w_scale,

@@ -41,12 +41,28 @@ struct GemmArgs {
   int out_dtype = CDIT_DT_BF16;  // CDIT_DT_*; the w8a16 kernels only build bf16
 };
 
-// GEMMs that share the A operand (same activation codes and scales: same M, K, lda, ldb)
-// and differ in the weight side. col_begin is filled by the launcher.
-constexpr int kMaxGroup = 4;
+// A batch of GEMMs run as one launch of the wide kernel. The batch holds up to kMaxActs
+// activations (A operands: codes, per-row scales, M); each activation has one or more
+// members (B side: weight, per-channel scale, bias, output, epilogue flag), up to kMaxGroup
+// members in all. K, lda and ldb are common. Members of one activation are walked as if their
+// weights were stacked along N (tile columns [col_begin[p], col_begin[p + 1]) of that
+// activation), activations one after the other. The fields marked (launcher) are filled by
+// launch_gemm_fp8_grouped for the tile shape it picks.
+constexpr int kMaxGroup = 8;
+constexpr int kMaxActs = 4;
 struct GemmGroup {
-  int count;
-  int col_begin[kMaxGroup + 1];
+  int count;  // members
+  int acts;   // activations
+  // per activation
+  const void* a[kMaxActs];
+  const float* a_scale[kMaxActs];
+  int M[kMaxActs];
+  int first_member[kMaxActs + 1];  // members of activation s: [first_member[s], first_member[s + 1])
+  int tile_begin[kMaxActs + 1];    // (launcher) first linear tile id of activation s
+  int tiles_m[kMaxActs];           // (launcher) tile rows of activation s
+  int tiles_n[kMaxActs];           // (launcher) tile columns of activation s, all its members
+  // per member
+  int col_begin[kMaxGroup + 1];    // (launcher) first tile column of member p inside its activation
   const uint8_t* b[kMaxGroup];
   const float* b_scale[kMaxGroup];
   const uint16_t* bias[kMaxGroup];
@@ -58,9 +74,10 @@ struct GemmGroup {
 
 // variant < 0: choose by shape.
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream);
-// All members of `grp` in one launch (A side and ldb from `shared`). 0: launched; -1: not
-// taken (shape, alignment or variant without a grouped form); else a CDIT_E* code.
-int launch_gemm_fp8_grouped(const GemmArgs& shared, const GemmGroup& grp, int variant,
+// All members of `grp` in one launch (K, lda, ldb and the output dtype from `common`; its other
+// fields are ignored). 0: launched; -1: not taken (shape, alignment or variant without a
+// grouped form); else a CDIT_E* code.
+int launch_gemm_fp8_grouped(const GemmArgs& common, const GemmGroup& grp, int variant,
                             hipStream_t stream);
 int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream);
 // One w8a8 Linear forward at M <= 16 in a single kernel (per-token quantizer + GEMM);

@@ -387,14 +387,13 @@ __device__ __forceinline__ void mfma_16x16x128_fp8(v4f& acc, const v8i& b, const
   }
 }
 
-// A group of GEMMs that share the A operand (the same activation codes and scales, so
-// the same M, K and lda) and differ in the weight: sibling Linears such as to_q / to_k /
-// to_v, and proj_mlp next to them in FLUX single blocks (reference dataflow:
-// src/cache_dit/caching/patch_functors/functor_flux.py:60-67). Their tiles are walked as
-// one tile stream by one persistent launch, as if the weights were stacked along N:
-// member p owns the tile columns [col_begin[p], col_begin[p + 1]). Every member has its
-// own weight, scale, bias, output and epilogue flag; ldb is common (GemmGroup, declared
-// with the launchers).
+// A batch of GEMMs as one launch (GemmGroup, declared with the launchers): sibling Linears
+// that read one activation -- to_q / to_k / to_v, and proj_mlp next to them in FLUX single
+// blocks (reference dataflow: src/cache_dit/caching/patch_functors/functor_flux.py:60-67) --
+// are members of that activation and are walked as if their weights were stacked along N;
+// independent Linears of the same stage on other activations (the text stream next to the
+// image stream of a double block) follow in the same tile stream. Every member has its own
+// weight, scale, bias, output and epilogue flag; K, lda and ldb are common.
 struct NoGroup {};
 
 // OUT: dtype of the output and of the bias (CDIT_DT_*), a template parameter so that
@@ -417,7 +416,8 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
   constexpr int NST = TM * (TN / 2) * (OUT == CDIT_DT_F32 ? 2 : 1);
   static_assert((D - 2) * C::ND + C::NDA + NST <= 63, "vmcnt is a 6-bit counter");
   const int KT = g.K / BKW;  // >= D (checked by the launcher)
-  const int ntiles = tiles_m * tiles_n;
+  int ntiles = tiles_m * tiles_n;
+  if constexpr (GROUPED) ntiles = grp.tile_begin[grp.acts];
 
   // The workgroup is persistent: it takes tiles blockIdx.x, blockIdx.x + gridDim.x,
   // ... and runs their K loops as one stream: the DMA of the last D steps of a
@@ -425,19 +425,53 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
   // the end of the last step are the next tile's first. The epilogue of a tile
   // then runs with the next tile's panels landing in LDS, and its stores drain
   // while the next K loop is under way.
-  // B side of a tile: for a group, looked up from the tile column (the table sits in the
-  // kernel arguments: scalar loads with a uniform index)
-  auto member_of = [&](int tn, int* first_col) {
-    int p = 0;
+  // Where a tile lives: for a batch, activation and member are looked up from the linear
+  // tile id (the table sits in the kernel arguments: scalar loads with uniform indices).
+  struct Where {
+    int act, member, m0, n0;
+  };
+  auto locate = [&](int t) -> Where {
+    Where w;
     if constexpr (GROUPED) {
+      constexpr int kXcd = 8;
+      int id = t;  // ids that run on one XCD are made consecutive, as tile_of_block does
+      if (ntiles % kXcd == 0) id = (t % kXcd) * (ntiles / kXcd) + t / kXcd;
+      int s = 0;
+#pragma unroll
+      for (int i = 1; i < kMaxActs; ++i)
+        if (i < grp.acts && id >= grp.tile_begin[i]) s = i;
+      int tm, tn;
+      tile_of_linear<C::GROUP_M>(id - grp.tile_begin[s], grp.tiles_m[s], grp.tiles_n[s], &tm, &tn);
+      int p = grp.first_member[s];
+      const int p_end = grp.first_member[s + 1];
 #pragma unroll
       for (int i = 1; i < kMaxGroup; ++i)
-        if (i < grp.count && tn >= grp.col_begin[i]) p = i;
-      *first_col = grp.col_begin[p];
+        if (i > p && i < p_end && tn >= grp.col_begin[i]) p = i;
+      w.act = s;
+      w.member = p;
+      w.m0 = tm * C::BM;
+      w.n0 = (tn - grp.col_begin[p]) * C::BN;
     } else {
-      *first_col = 0;
+      int tm, tn;
+      tile_of_block<C::GROUP_M>(t, ntiles, tiles_m, tiles_n, &tm, &tn);
+      w.act = 0;
+      w.member = 0;
+      w.m0 = tm * C::BM;
+      w.n0 = tn * C::BN;
     }
-    return p;
+    return w;
+  };
+  auto a_of = [&](int s) -> const uint8_t* {
+    if constexpr (GROUPED) return static_cast<const uint8_t*>(grp.a[s]);
+    return static_cast<const uint8_t*>(g.a);
+  };
+  auto a_scale_of = [&](int s) -> const float* {
+    if constexpr (GROUPED) return grp.a_scale[s];
+    return g.a_scale;
+  };
+  auto m_of = [&](int s) -> int {
+    if constexpr (GROUPED) return grp.M[s];
+    return g.M;
   };
   auto b_of = [&](int p) -> const uint8_t* {
     if constexpr (GROUPED) return grp.b[p];
@@ -455,14 +489,15 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
     if constexpr (GROUPED) return grp.bias[p];
     return g.bias;
   };
-  int m0, n0;  // tile being computed
-  int cur = 0;  // group member it belongs to
+  int m0, n0;          // tile being computed
+  int cur = 0;         // member it belongs to
+  int cur_act = 0;     // and its activation
   {
-    int tm, tn, c0;
-    tile_of_block<C::GROUP_M>(blockIdx.x, ntiles, tiles_m, tiles_n, &tm, &tn);
-    cur = member_of(tn, &c0);
-    m0 = tm * C::BM;
-    n0 = (tn - c0) * C::BN;
+    const Where w = locate(blockIdx.x);
+    cur = w.member;
+    cur_act = w.act;
+    m0 = w.m0;
+    n0 = w.n0;
   }
 
   // DMA source: tile whose panels the DMA stream currently fetches. Instruction p
@@ -477,10 +512,10 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
   // and B: between two tiles without partial panels they are not recomputed (some 130
   // VALU instructions in the middle of the MFMA stream otherwise).
   bool off_clamped = true;  // the first call computes them
-  auto set_source = [&](int sm0, int sn0, int member) {
-    A = static_cast<const uint8_t*>(g.a) + (int64_t)sm0 * g.lda;
+  auto set_source = [&](int sm0, int sn0, int member, int act) {
+    A = a_of(act) + (int64_t)sm0 * g.lda;
     B = b_of(member) + (int64_t)sn0 * g.ldb;
-    const int rows_a = g.M - sm0, rows_b = n_of(member) - sn0;
+    const int rows_a = m_of(act) - sm0, rows_b = n_of(member) - sn0;
     const bool clamped = rows_a < C::BM || rows_b < C::BN;
     if (!clamped && !off_clamped) return;
     off_clamped = clamped;
@@ -497,7 +532,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
                     : (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
     }
   };
-  set_source(m0, n0, cur);
+  set_source(m0, n0, cur, cur_act);
   // buffer_load ... lds (MUBUF form: the compiler tracks it with vmcnt only, while
   // the global_load form makes it wait for all LDS reads at every use). With a
   // descriptor of zero records every lane is out of range: nothing is fetched and
@@ -562,7 +597,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
 
   for (int tile = blockIdx.x;; tile += gridDim.x) {
     const int next_tile = tile + gridDim.x;
-    int nm0 = 0, nn0 = 0, next_member = 0;
+    int nm0 = 0, nn0 = 0, next_member = 0, next_act = 0;
     // fragments of step 0 (in LDS since the prologue, or since the barrier of the
     // previous tile's last step). The last step of a tile reads them too, like
     // every step does for its successor, but keeping them across the epilogue
@@ -592,12 +627,12 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
       if (EVENTS && kt == KT - D) {
         // every DMA of this tile has been issued: the stream moves on
         if (next_tile < ntiles) {
-          int tm, tn, c0;
-          tile_of_block<C::GROUP_M>(next_tile, ntiles, tiles_m, tiles_n, &tm, &tn);
-          next_member = member_of(tn, &c0);
-          nm0 = tm * C::BM;
-          nn0 = (tn - c0) * C::BN;
-          set_source(nm0, nn0, next_member);
+          const Where w = locate(next_tile);
+          next_member = w.member;
+          next_act = w.act;
+          nm0 = w.m0;
+          nn0 = w.n0;
+          set_source(nm0, nn0, next_member, next_act);
         } else {
           nrec = 0;
         }
@@ -613,7 +648,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
         const __amdgpu_buffer_rsrc_t bi_buf = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<uint16_t*>(cur_bias), 0, cur_bias ? cur_n * 2 : 0, 0x00020000);
         const __amdgpu_buffer_rsrc_t as_buf = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<float*>(g.a_scale), 0, g.M * 4, 0x00020000);
+            const_cast<float*>(a_scale_of(cur_act)), 0, m_of(cur_act) * 4, 0x00020000);
         if constexpr (C::STAGE_EPI) {
           // Four LDS-DMA instructions (every wave issues all four: the same bytes land
           // four times, and the waves' instruction counts stay equal) instead of TM +
@@ -763,7 +798,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
     const int cur_N = n_of(cur);
     uint8_t* const out_wave = reinterpret_cast<uint8_t*>(cur_out) +
                               ((int64_t)(m0 + wm * C::WM) * cur_ldo + (n0 + wn * C::WN)) * OB;
-    const int rows_wave = g.M - (m0 + wm * C::WM);  // rows of the wave tile that exist
+    const int rows_wave = m_of(cur_act) - (m0 + wm * C::WM);  // rows of the wave tile that exist
     // The memory pipeline merges the lanes of a store into one request only when
     // adjacent lanes write adjacent bytes: with lane = 16 kg + r16 holding row r16,
     // 16-byte piece kg, every lane is a request of its own (measured: 294 clocks per
@@ -865,6 +900,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
     m0 = nm0;
     n0 = nn0;
     cur = next_member;
+    cur_act = next_act;
   }
   // the zero-record DMA of the last D steps must not outlive the workgroup
   wait_vm<0>();
@@ -889,7 +925,7 @@ int launch_wide(const GemmArgs& g, hipStream_t stream) {
   return 0;
 }
 
-// The members' tiles as one launch: tile columns of member p are [col_begin[p], col_begin[p+1]).
+// The batch as one launch: fills the tile tables of `grp` for this tile shape.
 template <class C>
 int launch_wide_grouped(const GemmArgs& g, GemmGroup grp, hipStream_t stream) {
   static bool lds_allowed[64];
@@ -902,16 +938,22 @@ int launch_wide_grouped(const GemmArgs& g, GemmGroup grp, hipStream_t stream) {
     set_error("cannot query the CU count of the current device");
     return CDIT_EHIP;
   }
-  const int tiles_m = (g.M + C::BM - 1) / C::BM;
-  int tiles_n = 0;
-  for (int p = 0; p < grp.count; ++p) {
-    grp.col_begin[p] = tiles_n;
-    tiles_n += (grp.N[p] + C::BN - 1) / C::BN;
+  int ntiles = 0;
+  for (int s = 0; s < grp.acts; ++s) {
+    int cols = 0;
+    for (int p = grp.first_member[s]; p < grp.first_member[s + 1]; ++p) {
+      grp.col_begin[p] = cols;
+      cols += (grp.N[p] + C::BN - 1) / C::BN;
+    }
+    grp.tiles_m[s] = (grp.M[s] + C::BM - 1) / C::BM;
+    grp.tiles_n[s] = cols;
+    grp.tile_begin[s] = ntiles;
+    ntiles += grp.tiles_m[s] * cols;
   }
-  for (int p = grp.count; p <= kMaxGroup; ++p) grp.col_begin[p] = tiles_n;
-  const int ntiles = tiles_m * tiles_n;
+  for (int s = grp.acts; s <= kMaxActs; ++s) grp.tile_begin[s] = ntiles;
+  for (int p = grp.count; p <= kMaxGroup; ++p) grp.col_begin[p] = 0x7fffffff;
   hipLaunchKernelGGL((gemm_fp8_wide<C, CDIT_DT_BF16, true>), dim3(ntiles < cus ? ntiles : cus),
-                     dim3(C::THREADS), C::LDS_BYTES, stream, g, tiles_m, tiles_n, grp);
+                     dim3(C::THREADS), C::LDS_BYTES, stream, g, 0, 0, grp);
   return 0;
 }
 
@@ -1329,36 +1371,47 @@ int launch_bf16_variant(const GemmArgs& g, int variant, WideOk wide_ok, hipStrea
   }
 }
 
-// The group as one launch. Returns 0 when launched, -1 when the group is not taken (the
+// The batch as one launch. Returns 0 when launched, -1 when the batch is not taken (the
 // caller then runs the members one by one), a CDIT_E* code on error.
-int launch_gemm_fp8_grouped(const GemmArgs& shared, const GemmGroup& grp, int variant,
+int launch_gemm_fp8_grouped(const GemmArgs& common, const GemmGroup& grp, int variant,
                             hipStream_t stream) {
-  if (grp.count < 2 || grp.count > kMaxGroup || shared.M <= 16 || shared.out_dtype != CDIT_DT_BF16)
+  if (grp.count < 2 || grp.count > kMaxGroup || grp.acts < 1 || grp.acts > kMaxActs ||
+      common.out_dtype != CDIT_DT_BF16)
     return -1;
-  for (int p = 0; p < grp.count; ++p) {
-    GemmArgs g = shared;
-    g.b = grp.b[p];
-    g.b_scale = grp.b_scale[p];
-    g.bias = grp.bias[p];
-    g.out = grp.out[p];
-    g.N = grp.N[p];
-    g.ldo = grp.ldo[p];
-    if (!tiled_ok(g) || g.N <= 0) return -1;
+  for (int s = 0; s < grp.acts; ++s) {
+    if (grp.M[s] <= 16 || grp.first_member[s + 1] <= grp.first_member[s]) return -1;
+    for (int p = grp.first_member[s]; p < grp.first_member[s + 1]; ++p) {
+      GemmArgs g = common;
+      g.a = grp.a[s];
+      g.a_scale = grp.a_scale[s];
+      g.M = grp.M[s];
+      g.b = grp.b[p];
+      g.b_scale = grp.b_scale[p];
+      g.bias = grp.bias[p];
+      g.out = grp.out[p];
+      g.N = grp.N[p];
+      g.ldo = grp.ldo[p];
+      if (!tiled_ok(g) || g.N <= 0) return -1;
+    }
   }
-  auto wide_ok = [&](int depth) { return shared.K >= 128 * (depth > 3 ? depth : 3); };
+  auto wide_ok = [&](int depth) { return common.K >= 128 * (depth > 3 ? depth : 3); };
   auto tiles = [&](int bm, int bn) {
-    int64_t cols = 0;
-    for (int p = 0; p < grp.count; ++p) cols += (grp.N[p] + bn - 1) / bn;
-    return (int64_t)((shared.M + bm - 1) / bm) * cols;
+    int64_t t = 0;
+    for (int s = 0; s < grp.acts; ++s) {
+      int64_t cols = 0;
+      for (int p = grp.first_member[s]; p < grp.first_member[s + 1]; ++p) cols += (grp.N[p] + bn - 1) / bn;
+      t += (int64_t)((grp.M[s] + bm - 1) / bm) * cols;
+    }
+    return t;
   };
   if (variant < 0) variant = choose_bf16_variant(tiles, wide_ok);
   switch (variant) {
-    case 12: return wide_ok(V12::DEPTH) ? launch_wide_grouped<V12>(shared, grp, stream) : -1;
-    case 14: return wide_ok(V14::DEPTH) ? launch_wide_grouped<V14>(shared, grp, stream) : -1;
-    case 15: return wide_ok(V15::DEPTH) ? launch_wide_grouped<V15>(shared, grp, stream) : -1;
-    case 16: return wide_ok(V16::DEPTH) ? launch_wide_grouped<V16>(shared, grp, stream) : -1;
-    case 17: return wide_ok(V17::DEPTH) ? launch_wide_grouped<V17>(shared, grp, stream) : -1;
-    case 18: return wide_ok(V18::DEPTH) ? launch_wide_grouped<V18>(shared, grp, stream) : -1;
+    case 12: return wide_ok(V12::DEPTH) ? launch_wide_grouped<V12>(common, grp, stream) : -1;
+    case 14: return wide_ok(V14::DEPTH) ? launch_wide_grouped<V14>(common, grp, stream) : -1;
+    case 15: return wide_ok(V15::DEPTH) ? launch_wide_grouped<V15>(common, grp, stream) : -1;
+    case 16: return wide_ok(V16::DEPTH) ? launch_wide_grouped<V16>(common, grp, stream) : -1;
+    case 17: return wide_ok(V17::DEPTH) ? launch_wide_grouped<V17>(common, grp, stream) : -1;
+    case 18: return wide_ok(V18::DEPTH) ? launch_wide_grouped<V18>(common, grp, stream) : -1;
     default: return -1;  // the kernels without a tile stream have no grouped form
   }
 }

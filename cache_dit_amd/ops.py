@@ -150,6 +150,40 @@ def gemm_rowwise_grouped_into(a: torch.Tensor, a_scale: torch.Tensor, weights, w
         _stream_ptr(a)))
 
 
+def gemm_rowwise_batched_into(acts) -> None:
+  """Independent GEMMs of one stage as one launch. `acts` is a list of
+  (a [M,K] e4m3, a_scale [M], weights, w_scales, biases, outs, epilogues): one entry per
+  activation, its members listed as for gemm_rowwise_grouped_into; all activations and
+  weights share K and their row strides. Bit-identical to one gemm_rowwise_into per
+  member."""
+  import ctypes
+  vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+  a0 = acts[0][0]
+  K, lda, ldb = a0.shape[1], a0.stride(0), acts[0][2][0].stride(0)
+  ws, wss, bs, outs, epis, per_act = [], [], [], [], [], []
+  for a, a_s, weights, w_scales, biases, o, e in acts:
+    if a.shape[1] != K or a.stride(0) != lda or a.device != a0.device:
+      raise ValueError("gemm_rowwise_batched_into: the activations must share K, the row stride "
+                       "and the device")
+    if any(w.stride(0) != ldb or w.shape[1] != K for w in weights):
+      raise ValueError("gemm_rowwise_batched_into: the weights must share K and the row stride")
+    ws += weights
+    wss += w_scales
+    bs += biases
+    outs += o
+    epis += e
+    per_act.append(len(weights))
+  n, na = len(ws), len(acts)
+  with _DeviceOf(a0):
+    _native.check(_native.load().cdit_fp8_gemm_rowwise_batched(
+        na, (vp * na)(*[t[0].data_ptr() for t in acts]), (vp * na)(*[t[1].data_ptr() for t in acts]),
+        (i64 * na)(*[t[0].shape[0] for t in acts]), K, lda, (ci * na)(*per_act),
+        (vp * n)(*[w.data_ptr() for w in ws]), (vp * n)(*[s.data_ptr() for s in wss]),
+        (vp * n)(*[b.data_ptr() if b is not None else None for b in bs]),
+        (vp * n)(*[o.data_ptr() for o in outs]), (i64 * n)(*[w.shape[0] for w in ws]), ldb,
+        (i64 * n)(*[o.stride(0) for o in outs]), (ci * n)(*[int(e) for e in epis]), _stream_ptr(a0)))
+
+
 def w8a16_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
                bias: Optional[torch.Tensor], out: torch.Tensor, epilogue: int) -> None:
   M, K = x2.shape

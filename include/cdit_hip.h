@@ -167,7 +167,7 @@ int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale,
                           int epilogue, int out_dtype_id, void* stream);
 
 /*
- * `count` (1 to 4) row-wise scaled FP8 GEMMs that share the A operand -- the same
+ * `count` (1 to 8) row-wise scaled FP8 GEMMs that share the A operand -- the same
  * activation codes and scales, hence the same M, K and lda -- as ONE launch whose tile
  * stream runs over all their output tiles: sibling Linears that read one activation, such
  * as attn.to_q / to_k / to_v, and proj_mlp next to them in FLUX single blocks (reference
@@ -181,6 +181,26 @@ int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale,
  */
 int cdit_fp8_gemm_rowwise_grouped(const void* a_q, const float* a_scale,
                                   int64_t M, int64_t K, int64_t lda, int count,
+                                  const void* const* b_q, const float* const* b_scale,
+                                  const void* const* bias, void* const* out,
+                                  const int64_t* N, int64_t ldb, const int64_t* ldo,
+                                  const int* epilogue, void* stream);
+
+/*
+ * The general form of the call above: `n_act` (1 to 4) activations, activation s with
+ * members_per_act[s] GEMMs on it; the member arrays list the members of activation 0,
+ * then those of activation 1, ... (1 to 8 members in all). K, lda and ldb are common. For
+ * Linears of one stage that do not depend on each other, on the same or on different
+ * activations: in a FLUX double block attn.to_q/k/v on the image tokens and
+ * attn.add_q/k/v_proj on the text tokens, then to_out.0 and to_add_out, ff.net.0.proj and
+ * ff_context.net.0.proj, ... (dataflow src/cache_dit/caching/patch_functors/functor_flux.py:
+ * 48-80 and the double-stream block it patches around); small text-stream GEMMs then ride in
+ * the tile stream of the large image-stream ones instead of half filling the chip on their
+ * own. Same results as one cdit_fp8_gemm_rowwise call per member, bit for bit.
+ */
+int cdit_fp8_gemm_rowwise_batched(int n_act, const void* const* a_q, const float* const* a_scale,
+                                  const int64_t* M, int64_t K, int64_t lda,
+                                  const int* members_per_act,
                                   const void* const* b_q, const float* const* b_scale,
                                   const void* const* bias, void* const* out,
                                   const int64_t* N, int64_t ldb, const int64_t* ldo,

@@ -102,6 +102,77 @@ def test_every_tile_shape_exact_integers_against_the_oracle(variant):
     assert torch.equal(outs[p].cpu().view(torch.int16), ref.view(torch.int16)), f"member {p}"
 
 
+def _acts(spec, seed, integer=False):
+  """spec: list of (M, [N...]); one K for all. Returns the `acts` list for
+  gemm_rowwise_batched_into (outputs NaN-filled) and the per-member epilogue flags."""
+  out = []
+  for s, (M, K, Ns, epis) in enumerate(spec):
+    a, a_s, ws, wss, bs = _members(M, K, Ns, seed=seed + 17 * s, integer=integer, no_bias=(1,))
+    outs = [torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda") for N in Ns]
+    out.append((a, a_s, ws, wss, bs, outs, list(epis)))
+  return out
+
+
+@pytest.mark.parametrize("spec", [
+    # FLUX double block, stage by stage: image stream (4096 tokens) + text stream (512 tokens)
+    [(4096, 3072, [3072] * 3, [0] * 3), (512, 3072, [3072] * 3, [0] * 3)],
+    [(4096, 3072, [3072], [0]), (512, 3072, [3072], [0])],
+    [(4096, 3072, [12288], [1]), (512, 3072, [12288], [1])],
+    [(4096, 12288, [3072], [0]), (512, 12288, [3072], [0])],
+    # Qwen-Image: 6889 + 256 tokens
+    [(6889, 3072, [3072] * 3, [0] * 3), (256, 3072, [3072] * 3, [0] * 3)],
+    # ragged everything, three activations
+    [(300, 512, [520, 264], [0, 1]), (77, 512, [72], [0]), (1000, 512, [136, 8, 200], [1, 0, 0])],
+])
+def test_batched_equals_separate_launches(spec):
+  from cache_dit_amd import ops
+  acts = _acts(spec, seed=spec[0][0])
+  ops.gemm_rowwise_batched_into(acts)
+  torch.cuda.synchronize()
+  for s, (a, a_s, ws, wss, bs, outs, epis) in enumerate(acts):
+    want = _separate(a, a_s, ws, wss, bs, epis)
+    for p, (g, w) in enumerate(zip(outs, want)):
+      assert torch.equal(g.view(torch.int16), w.view(torch.int16)), f"activation {s} member {p}"
+
+
+def test_batched_launch_is_deterministic_over_repeats():
+  """The same batch twenty times over, alternating with other launches: every run gives
+  the same bits as the first and as the members on their own (a timing-dependent fault in
+  the tile stream would show as a run that differs)."""
+  from cache_dit_amd import ops
+  spec = [(6889, 3072, [3072] * 3, [0] * 3), (256, 3072, [3072] * 3, [0] * 3)]
+  acts = _acts(spec, seed=6889)
+  want = [_separate(a, a_s, ws, wss, bs, epis) for a, a_s, ws, wss, bs, outs, epis in acts]
+  other = _acts([(300, 512, [520, 264], [0, 1]), (77, 512, [72], [0])], seed=1)
+  for rep in range(20):
+    for _, _, _, _, _, outs, _ in acts:
+      for o in outs:
+        o.fill_(float("nan"))
+    ops.gemm_rowwise_batched_into(acts)
+    if rep % 3 == 0:
+      ops.gemm_rowwise_batched_into(other)
+    torch.cuda.synchronize()
+    for s, (_, _, _, _, _, outs, _) in enumerate(acts):
+      for p, (g, w) in enumerate(zip(outs, want[s])):
+        assert torch.equal(g.view(torch.int16), w.view(torch.int16)), (rep, s, p)
+
+
+@pytest.mark.parametrize("variant", [12, 14, 15, 16, 17, 18])
+def test_batched_every_tile_shape_exact_integers_against_the_oracle(variant):
+  from cache_dit_amd import _native, ops
+  spec = [(2100, 640, [1096, 520], [0, 0]), (333, 640, [3080], [0]), (40, 640, [264, 72], [0, 0])]
+  acts = _acts(spec, seed=variant, integer=True)
+  _native.set_gemm_variant(variant)
+  ops.gemm_rowwise_batched_into(acts)
+  torch.cuda.synchronize()
+  _native.set_gemm_variant(-1)
+  for s, (a, a_s, ws, wss, bs, outs, epis) in enumerate(acts):
+    for p in range(len(ws)):
+      ref = to.scaled_mm_rowwise(a.cpu(), a_s.cpu(), ws[p].cpu(), wss[p].cpu(),
+                                 None if bs[p] is None else bs[p].cpu())
+      assert torch.equal(outs[p].cpu().view(torch.int16), ref.view(torch.int16)), (s, p)
+
+
 def test_groups_the_grouped_kernel_does_not_take_still_run():
   """A single member, M <= 16 and a misaligned scale run member by member."""
   for M, Ns in ((7, [264, 520]), (300, [520])):
@@ -117,9 +188,17 @@ def test_groups_the_grouped_kernel_does_not_take_still_run():
     assert torch.equal(g.view(torch.int16), w.view(torch.int16))
   from cache_dit_amd import _native
   L = _native.load()
-  assert L.cdit_fp8_gemm_rowwise_grouped(None, None, 4, 64, 64, 5, None, None, None, None, None, 64,
+  assert L.cdit_fp8_gemm_rowwise_grouped(None, None, 4, 64, 64, 9, None, None, None, None, None, 64,
                                          None, None, None) == 1
-  assert b"a group holds" in L.cdit_last_error()
+  assert b"a batch holds" in L.cdit_last_error()
+  # a batch with an M <= 16 activation runs member by member
+  from cache_dit_amd import ops
+  acts = _acts([(300, 512, [520], [0]), (5, 512, [264], [0])], seed=8)
+  ops.gemm_rowwise_batched_into(acts)
+  torch.cuda.synchronize()
+  for a, a_s, ws, wss, bs, outs, epis in acts:
+    for g, w in zip(outs, _separate(a, a_s, ws, wss, bs, epis)):
+      assert torch.equal(g.view(torch.int16), w.view(torch.int16))
 
 
 def test_grouped_random_data_against_the_oracle_sampled_rows():
