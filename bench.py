@@ -132,7 +132,8 @@ class HotPath:
     self.s = {mk: torch.empty(mk[0], dtype=torch.float32, device=device) for mk in max_mk}
     self.out = torch.empty(max_mn, dtype=torch.bfloat16, device=device)
     # a run of siblings writes its outputs side by side
-    run_mn = max(sum(self.layers[i][0] * self.layers[i][2] for i in run) for run in self.sibling_runs())
+    run_mn = max(sum(self.layers[i][0] * self.layers[i][2] for run in stage for i in run)
+                 for stage in self.stages())
     self.out2 = torch.empty(run_mn, dtype=torch.bfloat16, device=device)
 
   def step(self):
@@ -162,6 +163,53 @@ class HotPath:
       else:
         runs.append([i])
     return runs
+
+  def stages(self):
+    """The sibling runs arranged in stages: runs of one stage are independent of each other
+    in the model (image-stream and text-stream Linears of a double-stream block at the same
+    point of the block; Wan's cross-attention query next to its key / value) and share K, so
+    that a block forward written against linear_batch launches each stage as one GEMM."""
+    partner = {"attn.add_q_proj": "attn.to_q", "attn.to_add_out": "attn.to_out.0",
+               "ff_context.net.0.proj": "ff.net.0.proj", "ff_context.net.2": "ff.net.2",
+               "txt_mlp.net.0.proj": "img_mlp.net.0.proj", "txt_mlp.net.2": "img_mlp.net.2",
+               "attn2.to_k": "attn2.to_q"}
+    stages, at = [], {}
+    for run in self.sibling_runs():
+      name = self.linears[run[0]][0]
+      block, leaf = name.rsplit(".", name.count(".") - 1)[0], name.split(".", 2)[2]
+      M, K = self.layers[run[0]][:2]
+      want = partner.get(leaf)
+      if want is not None and (block, want) in at and M > 16:
+        stages[at[(block, want)]].append(run)
+        continue
+      if M > 16 and not name.startswith("single"):
+        at[(block, leaf)] = len(stages)
+      stages.append([run])
+    return stages
+
+  def step_batched(self):
+    """The pass as block forwards written against linear_batch run it: one quantizer launch
+    per activation and ONE GEMM launch per stage (cdit_fp8_gemm_rowwise_batched). Outputs are
+    bit-identical to step()."""
+    from cache_dit_amd import ops
+    for stage in self.stages():
+      if len(stage) == 1 and len(stage[0]) == 1:
+        M, K, N, w, ws, b, epi = self.layers[stage[0][0]]
+        ops.linear_w8a8_into(self.x[(M, K)], w, ws, b, self.out[:M * N].view(M, N), self.q[(M, K)],
+                             self.s[(M, K)], 0, epi)
+        continue
+      acts, at = [], 0
+      for run in stage:
+        M, K = self.layers[run[0]][:2]
+        ops.quant_rowwise_into(self.x[(M, K)], self.q[(M, K)], self.s[(M, K)], 0, gemm_follows=True)
+        members = [self.layers[i] for i in run]
+        outs = []
+        for _, _, N, *_ in members:
+          outs.append(self.out2[at:at + M * N].view(M, N))
+          at += M * N
+        acts.append((self.q[(M, K)], self.s[(M, K)], [m[3] for m in members], [m[4] for m in members],
+                     [m[5] for m in members], outs, [m[6] for m in members]))
+      ops.gemm_rowwise_batched_into(acts)
 
   def step_shared_quant(self):
     """The same pass with one quantizer launch per distinct input: q/k/v (and
@@ -201,12 +249,12 @@ class HotPath:
 
 def step_leg(device, linears, mode, steps, warmup):
   """A step of another benchmark configuration (every quantized Linear of the model at
-  its real shape with its own weights; w8a8: siblings grouped as in the headline step),
+  its real shape with its own weights; w8a8: stages batched as in the headline step),
   captured into a hipGraph and replayed like the headline step. Returns ms per step,
   TFLOP/s and the Linear count."""
   import torch
   hot = HotPath(device, linears, mode)
-  step = hot.step if mode == "w8a16" else hot.step_grouped
+  step = hot.step if mode == "w8a16" else hot.step_batched
   step()
   torch.cuda.synchronize()
   graph = torch.cuda.CUDAGraph()
@@ -480,6 +528,7 @@ def dit_forward_ms(device, iters=5):
   cache_dit_amd.share_activation_quant_(model)
   inputs = flux_like_inputs(device)
   cache_dit_amd.group_sibling_linears_(model, lambda: model(**inputs))
+  dit_shapes.batch_streams(model)
   dit_shapes.fuse_norm_quant(model, materialize=False)
   graph_ms = None
   with torch.no_grad():
@@ -504,7 +553,8 @@ def dit_forward_ms(device, iters=5):
   del model
   torch.cuda.empty_cache()
   return ms, graph_ms, ("float8_per_row, GELU-tanh fused into the producing Linear, sibling Linears "
-                        "grouped on one shared quantization, quantizer fused into the modulated "
+                        "grouped on one shared quantization, image- and text-stream Linears of a "
+                        "stage batched into one launch, quantizer fused into the modulated "
                         "LayerNorms; bf16 SDPA attention, RMS norms, RoPE and residual glue in eager "
                         "PyTorch ops" + note_err)
 
@@ -570,10 +620,12 @@ def main():
   torch.cuda.synchronize()
   eager_ms = (time.perf_counter() - t0) / args.steps * 1e3
   # The same step captured once into a hipGraph and replayed: what a serving loop does
-  # with a fixed-shape denoising step; removes the host launch cost. Three forms of the
+  # with a fixed-shape denoising step; removes the host launch cost. Four forms of the
   # step, all with bit-identical outputs: every Linear on its own (quantizer + GEMM each);
-  # one quantizer launch per distinct activation (share_activation_quant_); and, the
-  # headline, sibling Linears also as one grouped GEMM launch (group_sibling_linears_).
+  # one quantizer launch per distinct activation (share_activation_quant_); sibling Linears
+  # also as one grouped GEMM launch (group_sibling_linears_); and, the headline, every stage
+  # of a block -- the siblings of the image stream together with those of the text stream --
+  # as one batched GEMM launch (block forwards written against linear_batch).
   def replay_ms(step_fn):
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -597,13 +649,14 @@ def main():
   try:
     ungrouped_ms = replay_ms(hot.step)
     shared_ms = replay_ms(hot.step_shared_quant)
-    ms_per_step = replay_ms(hot.step_grouped)
+    grouped_ms = replay_ms(hot.step_grouped)
+    ms_per_step = replay_ms(hot.step_batched)
   except Exception as e:  # capture unavailable: report the eager figure of the plain step
     launch_mode = f"eager (graph capture failed: {str(e)[:80]})"
-    ungrouped_ms = shared_ms = None
+    ungrouped_ms = shared_ms = grouped_ms = None
     ms_per_step = eager_ms
   value = hot.flop / ms_per_step / 1e9
-  n_runs = len(hot.sibling_runs())
+  n_runs = len(hot.stages())
   n_layers = len(hot.layers)
   step_flop = hot.flop
   del hot
@@ -612,7 +665,8 @@ def main():
     print(json.dumps({"value": value, "unit": "TFLOP/s", "ms_per_step": ms_per_step,
                       "launch": launch_mode, "eager_ms_per_step": eager_ms,
                       "ungrouped_ms_per_step": ungrouped_ms,
-                      "shared_quant_ms_per_step": shared_ms, "steps": args.steps,
+                      "shared_quant_ms_per_step": shared_ms,
+                      "grouped_ms_per_step": grouped_ms, "steps": args.steps,
                       "warmup": args.warmup, "device": arch}))
     return
 
@@ -668,8 +722,9 @@ def main():
           "workload": "flux1_dev_shaped_step: all quantized Linears of one denoising step "
                       "(19 double + 38 single blocks, 4096 img + 512 txt tokens): per-token "
                       "quant + FP8 GEMM + epilogue; Linears that read one activation (q/k/v, "
-                      "proj_mlp + q/k/v) share its quantization and run as one grouped GEMM "
-                      "launch, bit-identical to running each on its own",
+                      "proj_mlp + q/k/v) share its quantization, and the independent Linears of "
+                      "one stage of a block (image stream + text stream) run as one batched GEMM "
+                      "launch, bit-identical to running each Linear on its own",
           "quant_type": "float8_per_row",
           "launch": launch_mode,
           "linears_per_step": n_layers,
@@ -684,6 +739,10 @@ def main():
       "ungrouped_ms_per_step": ungrouped_ms,
       "ungrouped_tflops": None if not ungrouped_ms else step_flop / ungrouped_ms / 1e9,
       "shared_quant_ms_per_step": shared_ms,
+      # sibling Linears grouped per activation only (what group_sibling_linears_ gives a model
+      # whose block forwards are untouched)
+      "grouped_ms_per_step": grouped_ms,
+      "grouped_tflops": None if not grouped_ms else step_flop / grouped_ms / 1e9,
       "linear_headline": head,
       # the other benchmark configurations as steps of their own (same construction as the
       # headline step): config 3 = FLUX-shaped w8a16, config 4 = Qwen-Image-shaped w8a8,

@@ -22,6 +22,7 @@ from .nn import Fp8WeightOnlyLinear
 from .nn import fuse_gelu_tanh_
 from .nn import share_activation_quant_
 from .nn import group_sibling_linears_
+from .nn import linear_batch
 from .ops import ln_modulate_quant
 from .utils import check_quantized
 
@@ -42,5 +43,6 @@ __all__ = [
     "fuse_gelu_tanh_",
     "share_activation_quant_",
     "group_sibling_linears_",
+    "linear_batch",
     "ln_modulate_quant",
 ]

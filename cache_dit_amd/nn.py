@@ -311,6 +311,40 @@ def group_sibling_linears_(module: nn.Module, run=None, enable: bool = True) -> 
   return groups
 
 
+def linear_batch(pairs):
+  """Several quantized Linears of one stage in ONE GEMM launch. `pairs` is a list of
+  (x, [linear, ...]): every Linear of an entry is applied to that entry's activation; the
+  entries do not depend on each other (in a double-stream block: the image-stream and the
+  text-stream projections of the same stage, e.g. [(hidden, [to_q, to_k, to_v]),
+  (encoder, [add_q_proj, add_k_proj, add_v_proj])]). Returns the outputs in the same
+  nesting, bit-identical to calling the Linears one by one. For block forwards that are
+  written against this package; Linears that are not `float8_per_row` ones, a compiled
+  graph, or inference-mode tensors simply run one by one."""
+  flat = [lin for _, lins in pairs for lin in lins]
+  first = flat[0]
+  plain = (torch.compiler.is_compiling() or len(flat) > _native.MAX_GROUP
+           or len(pairs) > _native.MAX_ACTS
+           or any(type(lin) is not Fp8DynamicLinear or lin.in_features != first.in_features
+                  or lin._scale_mode_id != first._scale_mode_id for lin in flat)
+           or any(x.is_inference() or not x.is_cuda or x.dtype != torch.bfloat16 for x, _ in pairs))
+  if plain:
+    return [[lin(x) for lin in lins] for x, lins in pairs]
+  acts, result = [], []
+  for x, lins in pairs:
+    x2 = ops._as_rows(x)
+    M = x2.shape[0]
+    outs = [torch.empty((M, lin.out_features), dtype=torch.bfloat16, device=x2.device) for lin in lins]
+    result.append([o.view(*x.shape[:-1], lin.out_features) for o, lin in zip(outs, lins)])
+    if M == 0:
+      continue
+    q, s = ops.shared_activation_quant(x2, first._scale_mode_id)
+    acts.append((q, s, [lin.weight for lin in lins], [lin.weight_scale for lin in lins],
+                 [lin.bias for lin in lins], outs, [lin.epilogue for lin in lins]))
+  if acts:
+    ops.gemm_rowwise_batched_into(acts)
+  return result
+
+
 def dequantize_weight(linear: _Fp8LinearBase) -> torch.Tensor:
   """bf16 view of the quantized weight (for inspection and tests)."""
   return (linear.weight.to(torch.float32) * linear.weight_scale).to(torch.bfloat16)

@@ -149,7 +149,21 @@ class AdaLayerNormZero(_ModulatedNorm, nn.Module):
     return self._modulated(x, shift, scale), mods[2:]
 
 
+def _batch(pairs):
+  from ..nn import linear_batch
+  return linear_batch(pairs)
+
+
+def _ff_pair(ff_a: "FeedForward", xa, ff_b: "FeedForward", xb):
+  """Two FeedForwards on independent inputs, their Linears launched pairwise."""
+  (ha, ), (hb, ) = _batch([(xa, [ff_a.net[0].proj]), (xb, [ff_b.net[0].proj])])
+  ha, hb = ff_a.net[0].act(ha), ff_b.net[0].act(hb)  # identity once fused into the epilogue
+  (ya, ), (yb, ) = _batch([(ha, [ff_a.net[2]]), (hb, [ff_b.net[2]])])
+  return ya, yb
+
+
 class FluxAttention(nn.Module):
+  batch_streams = False  # see batch_streams(): image- and text-stream Linears in one launch
 
   def __init__(self, dim: int, heads: int, joint: bool):
     super().__init__()
@@ -166,13 +180,20 @@ class FluxAttention(nn.Module):
       self.to_add_out = nn.Linear(dim, dim)
 
   def forward(self, hidden, encoder=None, rope=None):
-    q = self.norm_q(_heads(self.to_q(hidden), self.heads))
-    k = self.norm_k(_heads(self.to_k(hidden), self.heads))
-    v = _heads(self.to_v(hidden), self.heads)
+    if self.joint and self.batch_streams:
+      (q, k, v), (eq, ek, ev) = _batch([(hidden, [self.to_q, self.to_k, self.to_v]),
+                                        (encoder, [self.add_q_proj, self.add_k_proj, self.add_v_proj])])
+    else:
+      q, k, v = self.to_q(hidden), self.to_k(hidden), self.to_v(hidden)
+      if self.joint:
+        eq, ek, ev = self.add_q_proj(encoder), self.add_k_proj(encoder), self.add_v_proj(encoder)
+    q = self.norm_q(_heads(q, self.heads))
+    k = self.norm_k(_heads(k, self.heads))
+    v = _heads(v, self.heads)
     if self.joint:
-      eq = self.norm_added_q(_heads(self.add_q_proj(encoder), self.heads))
-      ek = self.norm_added_k(_heads(self.add_k_proj(encoder), self.heads))
-      ev = _heads(self.add_v_proj(encoder), self.heads)
+      eq = self.norm_added_q(_heads(eq, self.heads))
+      ek = self.norm_added_k(_heads(ek, self.heads))
+      ev = _heads(ev, self.heads)
       q, k, v = torch.cat([eq, q], 2), torch.cat([ek, k], 2), torch.cat([ev, v], 2)
     if rope is not None:
       q, k = apply_rope(q, rope), apply_rope(k, rope)
@@ -180,6 +201,9 @@ class FluxAttention(nn.Module):
     if not self.joint:
       return o
     n_txt = encoder.shape[1]
+    if self.batch_streams:
+      (a, ), (ca, ) = _batch([(o[:, n_txt:], [self.to_out[0]]), (o[:, :n_txt], [self.to_add_out])])
+      return self.to_out[1](a), ca
     return self.to_out[1](self.to_out[0](o[:, n_txt:])), self.to_add_out(o[:, :n_txt])
 
 
@@ -197,9 +221,15 @@ class FluxTransformerBlock(_ModulatedNorm, nn.Module):
     ne, (c_gate_msa, c_shift_mlp, c_scale_mlp, c_gate_mlp) = self.norm1_context(encoder, temb)
     a, ca = self.attn(nh, ne, rope)
     hidden = hidden + gate_msa * a
-    hidden = hidden + gate_mlp * self.ff(self._modulated(hidden, shift_mlp, scale_mlp))
     encoder = encoder + c_gate_msa * ca
-    encoder = encoder + c_gate_mlp * self.ff_context(self._modulated(encoder, c_shift_mlp, c_scale_mlp))
+    if self.attn.batch_streams:
+      f, cf = _ff_pair(self.ff, self._modulated(hidden, shift_mlp, scale_mlp), self.ff_context,
+                       self._modulated(encoder, c_shift_mlp, c_scale_mlp))
+    else:
+      f = self.ff(self._modulated(hidden, shift_mlp, scale_mlp))
+      cf = self.ff_context(self._modulated(encoder, c_shift_mlp, c_scale_mlp))
+    hidden = hidden + gate_mlp * f
+    encoder = encoder + c_gate_mlp * cf
     return encoder, hidden
 
 
@@ -290,8 +320,14 @@ class QwenImageTransformerBlock(_ModulatedNorm, nn.Module):
     a, ca = self.attn(self._modulate(hidden, si1, sc1), self._modulate(encoder, ti1, tc1), rope)
     hidden = hidden + g1 * a
     encoder = encoder + tg1 * ca
-    hidden = hidden + g2 * self.img_mlp(self._modulate(hidden, si2, sc2))
-    encoder = encoder + tg2 * self.txt_mlp(self._modulate(encoder, ti2, tc2))
+    if self.attn.batch_streams:
+      f, cf = _ff_pair(self.img_mlp, self._modulate(hidden, si2, sc2), self.txt_mlp,
+                       self._modulate(encoder, ti2, tc2))
+    else:
+      f = self.img_mlp(self._modulate(hidden, si2, sc2))
+      cf = self.txt_mlp(self._modulate(encoder, ti2, tc2))
+    hidden = hidden + g2 * f
+    encoder = encoder + tg2 * cf
     return encoder, hidden
 
 
@@ -428,6 +464,20 @@ def fuse_gelu_epilogues(model: nn.Module) -> int:
       if isinstance(lin, _Fp8LinearBase) and not getattr(act, "_cdit_fused_into_linear", False):
         fuse_gelu_tanh_(lin, act)
         n += 1
+  return n
+
+
+def batch_streams(model: nn.Module, enable: bool = True) -> int:
+  """Switches the double-stream blocks of `model` (FLUX, Qwen-Image) to forwards that hand
+  the image-stream and the text-stream Linears of a stage to linear_batch: one GEMM launch
+  per stage instead of one per Linear, the small text-stream GEMMs riding along with the
+  large image-stream ones. Outputs are bit-identical. Returns the number of attention
+  modules switched."""
+  n = 0
+  for m in model.modules():
+    if isinstance(m, FluxAttention) and m.joint:
+      m.batch_streams = bool(enable)
+      n += 1
   return n
 
 

@@ -287,3 +287,69 @@ def test_sibling_groups_in_a_model_are_found_and_bit_identical():
     assert len(b0.attn1.to_q.sibling_group.members) == 3
     assert b0.attn2.to_q.sibling_group is None and len(b0.attn2.to_k.sibling_group.members) == 2
     assert torch.equal(wan(**winp), w0)
+
+
+def test_stream_batched_block_forwards_are_bit_identical():
+  """FLUX- and Qwen-Image-shaped toy models with the image- and text-stream Linears of a
+  stage handed to linear_batch (one launch per stage): same bits as the plain forwards,
+  also combined with the fused producer, under graph capture, and for models that are
+  not quantized at all (then the Linears just run one by one)."""
+  import logging
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd import ops
+  from cache_dit_amd.testing import dit_shapes as ds
+  logging.getLogger("CACHE_DIT_AMD").setLevel(logging.WARNING)
+  torch.manual_seed(0)
+  kw = dict(dim=512, heads=4, mlp=2048, n_double=2, n_single=2, in_channels=64, text_dim=256,
+            pooled_dim=128)
+  model = ds.FluxLikeTransformer(**kw).to(torch.bfloat16).cuda()
+  inputs = ds.flux_like_inputs("cuda", n_img=320, n_txt=64, in_channels=64, text_dim=256,
+                               pooled_dim=128)
+  with torch.no_grad():
+    y_bf16 = model(**inputs)
+    assert ds.batch_streams(model) == 2
+    assert torch.equal(model(**inputs), y_bf16)  # unquantized: plain Linears, one by one
+    ds.batch_streams(model, False)
+  cache_dit.quantize(model, cache_dit.QuantizeConfig())
+  ds.fuse_gelu_epilogues(model)
+  with torch.no_grad():
+    y0 = model(**inputs)
+    ds.batch_streams(model)
+    ops.quant_launches = 0
+    y1 = model(**inputs)
+    # per double block 4 stages x 2 streams go through the shared lookup; nothing else does
+    assert ops.quant_launches == 2 * 8
+    assert torch.equal(y1, y0)
+    ds.fuse_norm_quant(model)  # the modulated activations arrive with their codes
+    ops.quant_launches = 0
+    y2 = model(**inputs)
+    assert ops.quant_launches == 2 * 4 and torch.isfinite(y2.float()).all()
+    ds.fuse_norm_quant(model, False)
+    static = {k: v.clone() for k, v in inputs.items()}
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+      model(**static)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+      ys = model(**static)
+    other = ds.flux_like_inputs("cuda", n_img=320, n_txt=64, in_channels=64, text_dim=256,
+                                pooled_dim=128, seed=3)
+    want = model(**other)
+    for k in static:
+      static[k].copy_(other[k])
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(ys, want)
+  with torch.inference_mode():
+    assert torch.equal(model(**inputs), y0)
+
+  qwen = ds.QwenImageLikeTransformer(dim=256, heads=2, mlp=512, n_layers=2, in_channels=64,
+                                     text_dim=128).to(torch.bfloat16).cuda()
+  cache_dit.quantize(qwen, cache_dit.QuantizeConfig())
+  qin = ds.qwen_image_like_inputs("cuda", n_img=200, n_txt=24, in_channels=64, text_dim=128)
+  with torch.no_grad():
+    q0 = qwen(**qin)
+    assert ds.batch_streams(qwen) == 2
+    assert torch.equal(qwen(**qin), q0)
