@@ -12,7 +12,8 @@
 // Kernels in this file: gemm_fp8_wide (persistent, one wave per SIMD, the one every
 // large or medium problem runs; described in front of CfgWide), gemm_fp8_tiled (the
 // older kernel described next, kept for very short K), gemm_fp8_skinny and
-// linear_fp8_skinny_fused (M <= 16), gemm_fp8_generic (any shape and alignment).
+// linear_fp8_skinny_fused (M <= 16), linear_fp8_row1 (M = 1, K <= 4096),
+// gemm_fp8_generic (any shape and alignment).
 //
 // Tiled kernel: a workgroup of WGM x WGN wavefronts owns a BM x BN output
 // tile and walks K in steps of BK = 128 bytes. A and B panels are staged in
@@ -1163,6 +1164,125 @@ __global__ __launch_bounds__(256) void linear_fp8_skinny_fused(GemmArgs g, uint8
   }
 }
 
+// One activation row (M = 1: the modulation Linears of every block), K <= 4096. The
+// 16-row arrangement above makes every lane of a weight load a memory request of its own
+// (adjacent lanes read different rows); here a load instruction of the wavefront reads
+// 1 KiB of one weight row, lane l bytes 16 l .. 16 l + 15. A dot product does not care in
+// which order K is walked, so the MFMA's 16 "rows" are 16 interleaved K subsets of the
+// same weight row: with the activation codes fetched at the same positions, lane for lane,
+// D[i][i] is the partial dot product over subset i, the diagonal sums to the whole one and
+// the other 240 entries are never read (the matrix core has 17 times the rate this
+// stream needs). One MFMA takes two such 1 KiB pieces of a row. A wavefront owns R whole
+// rows, all of their loads in flight at once, and no partial sums cross wavefronts.
+// Measured at K = 3072 with a different weight matrix per launch, against the 16-row
+// kernel: 7.4 us instead of 10.1 at N = 9216 and 11.2 instead of 15.1 at N = 18432
+// (three rows per wavefront and four wavefronts were the best of 1-4 rows and 2-8
+// wavefronts; with this access pattern the non-temporal hint on the weight loads gains
+// 6-8 %, where it cost 10 % with the 16-row pattern).
+// FUSED: the row is quantized by every workgroup itself, as in linear_fp8_skinny_fused
+// (same codes, same scale, workgroup 0 writes them to the caller's workspaces); else
+// g.a holds the codes and g.a_scale the scale.
+constexpr int kRow1Rows = 3, kRow1Waves = 4;
+template <int CHK, bool FUSED>
+__global__ __launch_bounds__(64 * kRow1Waves) void linear_fp8_row1(GemmArgs g, uint8_t* q_ws,
+                                                                   float* scale_ws, int scale_mode) {
+  constexpr int R = kRow1Rows, WAVES = kRow1Waves, THREADS = 64 * WAVES;
+  constexpr int PP = (CHK * 128 + THREADS - 1) / THREADS;  // 8-element pieces of x per thread
+  __shared__ __attribute__((aligned(16))) uint8_t codes[FUSED ? CHK * 1024 : 16];
+  __shared__ uint32_t wave_amax[WAVES];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int row0 = (blockIdx.x * WAVES + wave) * R;
+  const v4i zero4 = {0, 0, 0, 0};
+  v4i w[R][CHK];
+#pragma unroll
+  for (int q = 0; q < R; ++q) {
+    const uint8_t* __restrict__ wp = g.b + (int64_t)min(row0 + q, g.N - 1) * g.ldb + lane * 16;
+#pragma unroll
+    for (int c = 0; c < CHK; ++c) {
+      const v4i* src = reinterpret_cast<const v4i*>(wp + c * 1024);
+      if (c * 1024 + lane * 16 < g.K) {
+        w[q][c] = __builtin_nontemporal_load(src);
+      } else {
+        w[q][c] = zero4;
+      }
+    }
+  }
+  v4i xa[CHK];
+  float as;
+  if constexpr (FUSED) {
+    // thread t quantizes the 8-element pieces t, t + THREADS, ...; pieces beyond K become
+    // zero codes (their weights are zeros too, but 0 x NaN is NaN)
+    const uint4* xr = static_cast<const uint4*>(g.a);
+    const int nchunks = g.K >> 3, t = threadIdx.x;
+    uint4 v[PP];
+    uint32_t am = 0u;
+#pragma unroll
+    for (int p = 0; p < PP; ++p) {
+      v[p] = t + p * THREADS < nchunks ? xr[t + p * THREADS] : uint4{0u, 0u, 0u, 0u};
+      am = absmax2(absmax2(absmax2(absmax2(am, v[p].x), v[p].y), v[p].z), v[p].w);
+    }
+    am = wave_max_u32(fold2(am));
+    if (lane == 0) wave_amax[wave] = am;
+    __syncthreads();
+    uint32_t amax = wave_amax[0];
+#pragma unroll
+    for (int i = 1; i < WAVES; ++i) amax = max(amax, wave_amax[i]);
+    as = row_scale(amax, scale_mode);
+    const bool fast = scale_in_fast_window(as);  // uniform
+    const float rcp = 1.0f / as;
+    uint2* dst = reinterpret_cast<uint2*>(codes);
+#pragma unroll
+    for (int p = 0; p < PP; ++p) {
+      const int c = t + p * THREADS;
+      uint2 code;
+      if (fast) {
+        code = uint2{quant4<true>(v[p].x, v[p].y, as, rcp), quant4<true>(v[p].z, v[p].w, as, rcp)};
+      } else {
+        code = uint2{quant4<false>(v[p].x, v[p].y, as, 0.0f), quant4<false>(v[p].z, v[p].w, as, 0.0f)};
+      }
+      if (c >= nchunks) code = uint2{0u, 0u};
+      if (c < CHK * 128) dst[c] = code;
+      if (blockIdx.x == 0 && c < nchunks) reinterpret_cast<uint2*>(q_ws)[c] = code;
+    }
+    if (blockIdx.x == 0 && t == 0) scale_ws[0] = as;
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < CHK; ++c) xa[c] = *reinterpret_cast<const v4i*>(codes + c * 1024 + lane * 16);
+  } else {
+    const uint8_t* __restrict__ ap = static_cast<const uint8_t*>(g.a) + lane * 16;
+#pragma unroll
+    for (int c = 0; c < CHK; ++c)
+      xa[c] = c * 1024 + lane * 16 < g.K ? *reinterpret_cast<const v4i*>(ap + c * 1024) : zero4;
+    as = g.a_scale[0];
+  }
+  // lane l holds D[4 (l >> 4) + e][l & 15]: the diagonal entry of lanes 0-3, 20-23, 40-43, 60-63
+  const int diag = (lane & 15) - 4 * (lane >> 4);
+  float mine = 0.0f;  // lane q keeps the dot product of row row0 + q
+#pragma unroll
+  for (int q = 0; q < R; ++q) {
+    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int c = 0; c < CHK; c += 2) {
+      const v4i w1 = c + 1 < CHK ? w[q][c + 1] : zero4, x1 = c + 1 < CHK ? xa[c + 1] : zero4;
+      const v8i wf = __builtin_shufflevector(w[q][c], w1, 0, 1, 2, 3, 4, 5, 6, 7);
+      const v8i af = __builtin_shufflevector(xa[c], x1, 0, 1, 2, 3, 4, 5, 6, 7);
+      acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, acc, 0, 0, 0, 0, 0, 0);
+    }
+    float d = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) d = diag == e ? acc[e] : d;
+    const float sum = wave_sum_f32(d);
+    mine = lane == q ? sum : mine;
+  }
+  const int n = row0 + lane;
+  if (lane < R && n < g.N) {
+    float t = mine * as * g.b_scale[n];
+    if (g.bias) t += bias_at(g, n);
+    if (g.epilogue & CDIT_EPI_GELU_TANH) t = gelu_tanh(t);
+    store_out(g, n, t);
+  }
+}
+
 // Any shape, any alignment: a 16x16 output tile per workgroup, one output
 // element per thread, scalar decode + FMA. Only for shapes the tiled kernel
 // cannot take (K not a multiple of 128, N not a multiple of 8, odd strides).
@@ -1227,8 +1347,42 @@ typedef CfgWide<128, 192, 4, 3> V16;                  // ... 64x96 wave tiles, D
 typedef CfgWide<64, 128, 8, 5> V17;                   // ... 32x64 wave tiles, DMA 5 steps ahead
 typedef CfgWide<128, 128, 4, 4> V18;                  // ... 64x64 wave tiles, DMA 4 steps ahead
 
+// The M = 1 kernel when the shape fits it (variant 51 forces it, 50 the 16-row kernel);
+// returns 1 when it is not taken.
+template <bool FUSED>
+int launch_row1(const GemmArgs& g, uint8_t* q_ws, float* scale_ws, int scale_mode, int variant,
+                hipStream_t stream) {
+  const bool ok = g.M == 1 && g.K >= 128 && g.K % 128 == 0 && g.K <= 4096 && g.ldb % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(g.a) % 16 == 0 && reinterpret_cast<uintptr_t>(g.b) % 16 == 0 &&
+                  (!FUSED || reinterpret_cast<uintptr_t>(q_ws) % 8 == 0) &&
+                  (variant < 0 || variant == 51);
+  if (!ok) return 1;
+  constexpr int rows_wg = kRow1Rows * kRow1Waves;
+  auto go = [&](auto chk_tag) {
+    hipLaunchKernelGGL((linear_fp8_row1<decltype(chk_tag)::value, FUSED>),
+                       dim3((g.N + rows_wg - 1) / rows_wg), dim3(64 * kRow1Waves), 0, stream, g, q_ws,
+                       scale_ws, scale_mode);
+  };
+  switch ((g.K + 1023) / 1024) {
+    case 1: go(std::integral_constant<int, 1>{}); break;
+    case 2: go(std::integral_constant<int, 2>{}); break;
+    case 3: go(std::integral_constant<int, 3>{}); break;
+    default: go(std::integral_constant<int, 4>{}); break;
+  }
+  return 0;
+}
+
 int launch_linear_fp8_skinny_fused(const GemmArgs& g, void* q_ws, float* scale_ws, int scale_mode,
                                    int variant, hipStream_t stream) {
+  // Bit-identical to the quantizer followed by cdit_fp8_gemm_rowwise only where that call
+  // would run the same M <= 16 kernels: arguments it would hand to the any-alignment kernel
+  // (N not a multiple of 8, misaligned scales, ...) take the two calls here as well.
+  GemmArgs two_step = g;
+  two_step.a = q_ws;
+  two_step.a_scale = scale_ws;
+  two_step.lda = g.K;
+  if (!tiled_ok(two_step)) return 1;
+  if (launch_row1<true>(g, static_cast<uint8_t*>(q_ws), scale_ws, scale_mode, variant, stream) == 0) return 0;
   const int64_t lds = (int64_t)g.M * (g.K + kFusedPad);
   const bool ok = g.M >= 1 && g.M <= 16 && (variant < 0 || variant == 50) && g.K >= 128 &&
                   g.K % 128 == 0 && g.N % 8 == 0 && lds <= 48 * 1024 && g.lda % 8 == 0 &&
@@ -1254,6 +1408,9 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
     hipLaunchKernelGGL(gemm_fp8_generic, grid, dim3(256), 0, stream, g);
     return 0;
   }
+  if ((variant < 0 || variant == 51) &&
+      launch_row1<false>(g, nullptr, nullptr, 0, variant, stream) == 0)
+    return 0;
   if ((variant < 0 && g.M <= 16) || variant == 50) {
     if (g.M > 16) {
       set_error("cdit_fp8_gemm_rowwise: the skinny kernel takes M <= 16, got %d", g.M);

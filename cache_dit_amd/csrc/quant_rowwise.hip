@@ -227,33 +227,6 @@ __global__ __launch_bounds__(64) void quant_tensorwise_cast(
 //   y = bf16(u + shift[k]);  then amax / scale / e4m3 cast of y as in quant_rowwise_regs.
 // shift and scale are bf16 [*, K]; row m uses their row m / rows_per_mod (one modulation
 // vector per batch element, broadcast over its tokens).
-// Sum over the wavefront, the same in every lane: four DPP steps inside each row of 16
-// lanes (the pattern of wave_max_u32: no LDS crossbar, no waits), then the four row sums
-// through scalars. The order of the additions is fixed, so the result does not depend on
-// where the wavefront runs.
-__device__ __forceinline__ float wave_sum_f32(float v) {
-  auto step = [](float a, int ctrl_id) {
-    int o;
-    const int ai = __float_as_int(a);
-    switch (ctrl_id) {
-      case 0: o = __builtin_amdgcn_update_dpp(0, ai, 0xB1, 0xf, 0xf, false); break;   // quad_perm [1,0,3,2]
-      case 1: o = __builtin_amdgcn_update_dpp(0, ai, 0x4E, 0xf, 0xf, false); break;   // quad_perm [2,3,0,1]
-      case 2: o = __builtin_amdgcn_update_dpp(0, ai, 0x141, 0xf, 0xf, false); break;  // row_half_mirror
-      default: o = __builtin_amdgcn_update_dpp(0, ai, 0x140, 0xf, 0xf, false); break;  // row_mirror
-    }
-    return a + __int_as_float(o);
-  };
-  v = step(v, 0);
-  v = step(v, 1);
-  v = step(v, 2);
-  v = step(v, 3);
-  const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
-  const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
-  const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
-  const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
-  return (a + b) + (c + d);
-}
-
 __device__ __forceinline__ uint32_t bf16_bits(float f) {
   return __float_as_uint(round_to_bf16(f)) >> 16;
 }

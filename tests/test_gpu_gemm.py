@@ -110,6 +110,127 @@ def test_skinny_exact_and_k_positions():
                      to.scaled_mm_rowwise(a.to(FP8), ones_m, w.to(FP8), ones_n))
 
 
+ONE_ROW_SHAPES = [(18432, 3072), (9216, 3072), (1000, 2048), (24, 128), (6152, 4096), (3080, 1024),
+                  (520, 1152), (264, 3968)]
+
+
+@pytest.mark.parametrize("N,K", ONE_ROW_SHAPES)
+@pytest.mark.parametrize("gelu", [0, 1])
+def test_one_row_kernel(N, K, gelu):
+  """M = 1 with K <= 4096 runs a kernel of its own (a wavefront reads whole weight rows, 1 KiB
+  per load, and walks K in an interleaved order): automatic choice, forced (51), against the
+  oracle and against the 16-row kernel (50); row counts that leave partial wavefronts and
+  workgroups, K with a partial last KiB."""
+  from cache_dit_amd import _native
+  p = _rand_problem(1, N, K, seed=N + K)
+  ref = to.scaled_mm_rowwise(*p, gelu="fused" if gelu else None)
+  auto = _run(*p, epilogue=gelu)
+  _assert_close(auto, ref)
+  _native.set_gemm_variant(51)
+  forced = _run(*p, epilogue=gelu)
+  assert torch.equal(forced, auto)
+  _native.set_gemm_variant(50)
+  _assert_close(_run(*p, epilogue=gelu), ref)
+
+
+@pytest.mark.parametrize("N,K", ONE_ROW_SHAPES)
+def test_one_row_kernel_exact_and_k_positions(N, K):
+  """Integer codes and power-of-two scales make every partial sum exact: bit-equal to the
+  oracle. Then a single 1 in the activation, at positions on both sides of every boundary
+  of the kernel's K walk (16-byte lane pieces, 1 KiB loads, the pair of loads of one MFMA),
+  against weights whose value encodes the K index: a mismatch between the positions the
+  weight and the activation operands are fetched from gives a wrong answer."""
+  from cache_dit_amd import _native
+  _native.set_gemm_variant(51)
+  g = torch.Generator().manual_seed(N + K)
+  a = torch.randint(-4, 5, (1, K), generator=g).float().to(FP8)
+  w = torch.randint(-4, 5, (N, K), generator=g).float().to(FP8)
+  a_s, w_s = torch.full((1, 1), 0.5), torch.full((N, 1), 0.25)
+  assert torch.equal(_run(a, a_s, w, w_s, None).cpu(), to.scaled_mm_rowwise(a, a_s, w, w_s))
+  w = (((torch.arange(K) * 7) % 15) + 1).float().repeat(N, 1) * (1 + (torch.arange(N) % 2)).reshape(-1, 1)
+  ones_n = torch.ones(N, 1)
+  for pos in (0, 15, 16, 31, 127, 128, 1007, 1023, 1024, 1040, 2047, 2048, 3071, 3072, K - 17, K - 1):
+    if pos >= K:
+      continue
+    a = torch.zeros(1, K)
+    a[0, pos] = 1.0
+    out = _run(a.to(FP8), torch.ones(1, 1), w.to(FP8), ones_n, None)
+    assert torch.equal(out.cpu(), to.scaled_mm_rowwise(a.to(FP8), torch.ones(1, 1), w.to(FP8), ones_n)), pos
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_one_row_kernel_writes_only_its_row(out_dtype):
+  """M = 1 into the first row of a larger buffer holding a sentinel, N that leaves a partial
+  wavefront: the other elements keep the sentinel, for every output type."""
+  from cache_dit_amd import _native
+  N, K = 1030, 3072
+  xq, xs, wq, ws, b = _rand_problem(1, N, K, seed=5)
+  if out_dtype == torch.float16:  # the bias has the output's type; an fp32 output takes none
+    b = b.to(torch.float16)
+  elif out_dtype == torch.float32:
+    b = None
+  ref = to.scaled_mm_rowwise(xq, xs, wq, ws, b, out_dtype=out_dtype)
+  buf = torch.full((2, N + 26), 7.0, dtype=out_dtype, device="cuda")
+  L = _native.load()
+  a, sa, w, sw = xq.cuda(), xs.cuda().reshape(-1), wq.cuda(), ws.cuda().reshape(-1).contiguous()
+  bias = None if b is None else b.cuda()
+  dt_id = {torch.bfloat16: _native.DT_BF16, torch.float16: _native.DT_F16, torch.float32: _native.DT_F32}[out_dtype]
+  rc = L.cdit_fp8_gemm_rowwise(a.data_ptr(), sa.data_ptr(), w.data_ptr(), sw.data_ptr(),
+                               None if bias is None else bias.data_ptr(), buf.data_ptr(), 1, N, K, K, K,
+                               buf.stride(0), 0, dt_id, None)
+  assert rc == 0, L.cdit_last_error()
+  torch.cuda.synchronize()
+  assert max_rel_err(buf[0, :N].cpu(), ref[0]) <= REL_TOL
+  assert (buf[0, N:] == 7.0).all() and (buf[1] == 7.0).all()
+
+
+@pytest.mark.parametrize("scale_mode", [0, 1])
+@pytest.mark.parametrize("kind", ["normal", "zero", "tiny", "huge", "nan", "inf"])
+def test_one_row_fused_linear_matches_the_two_calls(kind, scale_mode):
+  """cdit_fp8_linear_w8a8 at M = 1 (the row quantized inside the GEMM kernel) against the
+  quantizer and the GEMM called one after the other, bit for bit: also for a zero row, scales
+  outside the fast-division window and rows that hold a NaN or an infinity."""
+  from cache_dit_amd import _native, ops
+  N, K = 3080, 3072  # not a multiple of the 12 rows of a workgroup
+  g = torch.Generator(device="cuda").manual_seed(3 + scale_mode)
+  x = (torch.randn(1, K, generator=g, device="cuda") * 2).to(torch.bfloat16)
+  if kind == "zero":
+    x.zero_()
+  elif kind == "tiny":
+    x *= 1e-32
+  elif kind == "huge":
+    x *= 1e32
+  elif kind == "nan":
+    x[0, 1500] = float("nan")
+  elif kind == "inf":
+    x[0, 77] = float("inf")
+  w = (torch.randn(N, K, generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+  wq, w_s = ops.fp8_rowwise_quant(w)
+  w_s = w_s.reshape(-1).contiguous()
+  bias = (torch.randn(N, generator=g, device="cuda") * 0.1).to(torch.bfloat16)
+  L = _native.load()
+  q_ws = torch.full((1, K), 0x55, dtype=torch.uint8, device="cuda").view(FP8)
+  s_ws = torch.full((1,), -1.0, dtype=torch.float32, device="cuda")
+  out = torch.empty(1, N, dtype=torch.bfloat16, device="cuda")
+  rc = L.cdit_fp8_linear_w8a8(x.data_ptr(), wq.data_ptr(), w_s.data_ptr(), bias.data_ptr(),
+                              out.data_ptr(), q_ws.data_ptr(), s_ws.data_ptr(), 1, N, K, K, K, N,
+                              scale_mode, 0, 1, None)
+  assert rc == 0, L.cdit_last_error()
+  q2 = torch.empty(1, K, dtype=FP8, device="cuda")
+  s2 = torch.empty(1, dtype=torch.float32, device="cuda")
+  out2 = torch.empty(1, N, dtype=torch.bfloat16, device="cuda")
+  ops.quant_rowwise_into(x, q2, s2, scale_mode)
+  ops.gemm_rowwise_into(q2, s2, wq, w_s, bias, out2, 0)
+  torch.cuda.synchronize()
+  assert torch.equal(q_ws.view(torch.uint8), q2.view(torch.uint8))
+  assert torch.equal(s_ws.view(torch.int32), s2.view(torch.int32))
+  assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
+  if kind in ("nan", "inf"):
+    assert torch.isnan(out.float()).all()
+  else:
+    assert torch.isfinite(out.float()).all()
+
+
 def test_k_position_sensitivity():
   """One non-zero per row of A at a different K position per row against a weight
   whose value encodes its K index: a K-permutation mismatch between the A and B
