@@ -768,10 +768,16 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
     // columns do not exist get an offset beyond any descriptor. Per lane a 32-bit
     // byte offset (the launcher bounds 512 * ldo), per row of blocks a scalar base.
     if constexpr (C::STAGE_EPI) {
-      // staged two steps ago; landed before the barrier of the last step. (The
-      // compiler still puts a wait for all DMA in front of some of these reads: it
-      // cannot tell them from the panels in flight. Measured: no cost, the next tile's
-      // first steps are in the LDS by then.)
+      // Staged at the start of step KT-2. The wait of the last step lets (D-2) ND + NDA
+      // instructions fly, and ND + NDA were issued behind the staging by then: up to
+      // D = 3 that wait covers it, a deeper stream needs one of its own here (the two
+      // steps' 2 ND panel instructions are younger and may keep flying). Without it the
+      // first of these reads could run ahead of its DMA when that was slow (a cold TLB,
+      // the first launch of a process) and pick up what an earlier tile or kernel left.
+      // (The compiler puts a wait for all DMA in front of the later reads: it cannot tell
+      // them from the panels in flight. Measured: no cost, the next tile's first steps
+      // are in the LDS by then.)
+      if constexpr (D > 3) wait_vm<2 * C::ND>();
       auto read_staged = [&](const uint8_t* __restrict__ ep) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
@@ -1397,8 +1403,12 @@ int launch_linear_fp8_skinny_fused(const GemmArgs& g, void* q_ws, float* scale_w
   return 0;
 }
 
+struct TileChoice {
+  int variant;
+  int64_t cost;  // 1000 x CUs x tile area per full round over the CUs (K left out)
+};
 template <class Tiles, class WideOk>
-int choose_bf16_variant(Tiles tiles, WideOk wide_ok);
+TileChoice choose_bf16_variant(Tiles tiles, WideOk wide_ok);
 template <class WideOk>
 int launch_bf16_variant(const GemmArgs& g, int variant, WideOk wide_ok, hipStream_t stream);
 
@@ -1450,61 +1460,52 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   if (variant < 0) {
     variant = choose_bf16_variant(
         [&](int bm, int bn) { return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn); },
-        wide_ok);
+        wide_ok).variant;
   }
   return launch_bf16_variant(g, variant, wide_ok, stream);
 }
 
 // Tile choice for a bf16-output problem whose tile count for a bm x bn tile is tiles(bm, bn)
-// (a single GEMM, or a group of GEMMs stacked along N).
+// (a single GEMM, or a batch of GEMMs walked as one tile stream), with the modelled cost of
+// that choice; both branches count in the same unit.
 template <class Tiles, class WideOk>
-int choose_bf16_variant(Tiles tiles, WideOk wide_ok) {
-  int variant;
-  {
-    // workgroups a round holds: one per CU (what launch_wide starts)
-    const int64_t cus = cu_count() > 0 ? cu_count() : 256;
-    if (tiles(256, 256) * 256 >= 160 * cus) {
-      // Large problems take one of the large-tile wide kernels. Cost model, fitted to
-      // measured times: tile area times the number of rounds over the CUs, where a
-      // last, partial round of r tiles counts 0.4 + 0.6 r/CUs (the chip is power
-      // limited: with fewer CUs busy the clocks rise); ties go to the larger tile.
-      auto cost = [&](int bm, int bn, int pen) {
-        const int64_t t = tiles(bm, bn), full = t / cus, rem = t % cus;
-        return (full * 10 * cus + (rem ? 4 * cus + 6 * rem : 0)) * bm * bn * pen;
-      };
-      variant = 12;
-      int64_t best = cost(256, 256, 100);
-      const struct { int v, bm, bn, pen; } cand[] = {
-          {14, 288, 192, 101}, {15, 256, 192, 102}};
-      for (const auto& c : cand) {
-        const int64_t t = cost(c.bm, c.bn, c.pen);
-        if (t < best) {
-          best = t;
-          variant = c.v;
-        }
-      }
-    } else {
-      // Smaller problems (the text-stream Linears, M of a few hundred to a few
-      // thousand): whole rounds over the CUs times tile area, the small tiles
-      // penalised by their measured lower MFMA rate (per mille); ties go to the
-      // larger tile. Tiles whose prefetch depth K cannot feed are left out.
-      const struct { int v, bm, bn, pen, depth; } cand[] = {
-          {12, 256, 256, 1000, 2}, {14, 288, 192, 1000, 2}, {15, 256, 192, 1000, 2},
-          {16, 128, 192, 1124, 3}, {18, 128, 128, 1000, 4}, {17, 64, 128, 1493, 5}};
-      int64_t best = INT64_MAX;
-      // K < 256: the kernels without a K stream across tiles
-      variant = tiles(128, 128) >= cus ? 6 : 21;
-      for (const auto& c : cand) {
-        if (!wide_ok(c.depth)) continue;
-        const int64_t t = (tiles(c.bm, c.bn) + cus - 1) / cus * c.bm * c.bn * c.pen;
-        if (t < best) {
-          best = t;
-          variant = c.v;
-        }
-      }
+TileChoice choose_bf16_variant(Tiles tiles, WideOk wide_ok) {
+  // workgroups a round holds: one per CU (what launch_wide starts)
+  const int64_t cus = cu_count() > 0 ? cu_count() : 256;
+  TileChoice best;
+  if (tiles(256, 256) * 256 >= 160 * cus) {
+    // Large problems take one of the large-tile wide kernels. Cost model, fitted to
+    // measured times: tile area times the number of rounds over the CUs, where a
+    // last, partial round of r tiles counts 0.4 + 0.6 r/CUs (the chip is power
+    // limited: with fewer CUs busy the clocks rise); ties go to the larger tile.
+    auto cost = [&](int bm, int bn, int pen) {
+      const int64_t t = tiles(bm, bn), full = t / cus, rem = t % cus;
+      return (full * 10 * cus + (rem ? 4 * cus + 6 * rem : 0)) * bm * bn * pen;
+    };
+    best = {12, cost(256, 256, 100)};
+    const struct { int v, bm, bn, pen; } cand[] = {
+        {14, 288, 192, 101}, {15, 256, 192, 102}};
+    for (const auto& c : cand) {
+      const int64_t t = cost(c.bm, c.bn, c.pen);
+      if (t < best.cost) best = {c.v, t};
+    }
+  } else {
+    // Smaller problems (the text-stream Linears, M of a few hundred to a few
+    // thousand): whole rounds over the CUs times tile area, the small tiles
+    // penalised by their measured lower MFMA rate (per mille); ties go to the
+    // larger tile. Tiles whose prefetch depth K cannot feed are left out.
+    const struct { int v, bm, bn, pen, depth; } cand[] = {
+        {12, 256, 256, 1000, 2}, {14, 288, 192, 1000, 2}, {15, 256, 192, 1000, 2},
+        {16, 128, 192, 1124, 3}, {18, 128, 128, 1000, 4}, {17, 64, 128, 1493, 5}};
+    // K < 256: the kernels without a K stream across tiles (cost not modelled)
+    best = {tiles(128, 128) >= cus ? 6 : 21, INT64_MAX / 8};
+    for (const auto& c : cand) {
+      if (!wide_ok(c.depth)) continue;
+      const int64_t t = (tiles(c.bm, c.bn) + cus - 1) / cus * cus * c.bm * c.bn * c.pen;
+      if (t < best.cost) best = {c.v, t};
     }
   }
-  return variant;
+  return best;
 }
 
 template <class WideOk>
@@ -1561,7 +1562,70 @@ int launch_gemm_fp8_grouped(const GemmArgs& common, const GemmGroup& grp, int va
     }
     return t;
   };
-  if (variant < 0) variant = choose_bf16_variant(tiles, wide_ok);
+  if (variant < 0) {
+    const TileChoice whole = choose_bf16_variant(tiles, wide_ok);
+    variant = whole.variant;
+    if (grp.acts > 1) {
+      // One tile stream is not always the cheaper form: the tiles of a small activation
+      // can push a batch that filled whole rounds of large tiles into one more round
+      // (FLUX ff.net.0.proj: 4096 rows fill three rounds of 256 x 256 tiles exactly, the
+      // 512 text rows add a fourth, nearly empty one; on its own the text GEMM is one round
+      // of small tiles: measured 148 us as two launches, 173 as one). Compare with one
+      // launch per activation, each with the tile it would choose, plus what a further
+      // launch costs (about 3 us, in the unit of the model: a CU does about 4900 K-steps of
+      // one output element per us).
+      const int64_t cus = cu_count() > 0 ? cu_count() : 256;
+      int64_t apart = (grp.acts - 1) * (3 * 1000 * cus * 4900 / (common.K > 0 ? common.K : 1));
+      for (int s = 0; s < grp.acts; ++s) {
+        auto tiles_s = [&](int bm, int bn) {
+          int64_t cols = 0;
+          for (int p = grp.first_member[s]; p < grp.first_member[s + 1]; ++p) cols += (grp.N[p] + bn - 1) / bn;
+          return (int64_t)((grp.M[s] + bm - 1) / bm) * cols;
+        };
+        apart += choose_bf16_variant(tiles_s, wide_ok).cost;
+      }
+      if (apart < whole.cost) {
+        for (int s = 0; s < grp.acts; ++s) {
+          GemmGroup one = {};
+          one.acts = 1;
+          one.count = grp.first_member[s + 1] - grp.first_member[s];
+          one.a[0] = grp.a[s];
+          one.a_scale[0] = grp.a_scale[s];
+          one.M[0] = grp.M[s];
+          one.first_member[0] = 0;
+          one.first_member[1] = one.count;
+          for (int p = 0; p < one.count; ++p) {
+            const int src = grp.first_member[s] + p;
+            one.b[p] = grp.b[src];
+            one.b_scale[p] = grp.b_scale[src];
+            one.bias[p] = grp.bias[src];
+            one.out[p] = grp.out[src];
+            one.N[p] = grp.N[src];
+            one.ldo[p] = grp.ldo[src];
+            one.epilogue[p] = grp.epilogue[src];
+          }
+          int rc = one.count >= 2 ? launch_gemm_fp8_grouped(common, one, -1, stream) : -1;
+          if (rc > 0) return rc;
+          if (rc == 0) continue;
+          for (int p = 0; p < one.count; ++p) {  // a single member, or a group that is not taken
+            GemmArgs g = common;
+            g.a = one.a[0];
+            g.a_scale = one.a_scale[0];
+            g.M = one.M[0];
+            g.b = one.b[p];
+            g.b_scale = one.b_scale[p];
+            g.bias = one.bias[p];
+            g.out = one.out[p];
+            g.N = one.N[p];
+            g.ldo = one.ldo[p];
+            g.epilogue = one.epilogue[p];
+            if ((rc = launch_gemm_fp8(g, -1, stream))) return rc;
+          }
+        }
+        return 0;
+      }
+    }
+  }
   switch (variant) {
     case 12: return wide_ok(V12::DEPTH) ? launch_wide_grouped<V12>(common, grp, stream) : -1;
     case 14: return wide_ok(V14::DEPTH) ? launch_wide_grouped<V14>(common, grp, stream) : -1;

@@ -25,7 +25,10 @@ things the compiler may add that the kernels must not have:
   6. (w8a8 kernel) the waits of the first K steps of a tile count the output stores
      of the previous tile's epilogue, so every wave must issue all of them whatever
      part of the tile exists: the expected number of buffer stores, no global stores,
-     none under a lane mask or inside a loop over descriptor values.
+     none under a lane mask or inside a loop over descriptor values;
+  7. (w8a8 kernel) the epilogue operands staged in LDS by DMA are read after a vmcnt wait
+     that covers them: with a DMA stream more than 3 steps deep the waits of the K loop
+     do not, and the first LDS read after the last MFMA of a tile needs one of its own.
 """
 import os
 import re
@@ -179,3 +182,29 @@ def test_output_stores_are_unconditional(wide_kernels):
     counted += 1
   if any("gemm_fp8_wide" in n for n in wide_kernels):
     assert counted >= 3
+
+
+def test_staged_epilogue_operands_are_waited_for(wide_kernels):
+  """Rule 7. Between the end of a K loop (the pair of s_nop 15 in front of the epilogue)
+  and the first LDS read behind it, the instances whose DMA stream runs 4 or 5 steps ahead
+  wait with vmcnt(2 ND): the staging DMA is older than the 2 ND panel instructions of the
+  last two steps, nothing else may be in flight in front of the read."""
+  checked = 0
+  for name, code in wide_kernels.items():
+    m = re.search(r"gemm_fp8_wideINS0_7CfgWideILi(\d+)ELi(\d+)ELi\d+ELi(\d+)EEELi(\d)E", name)
+    if not m or int(m.group(3)) <= 3:
+      continue
+    bm, bn = int(m.group(1)), int(m.group(2))
+    nd = bm // 32 + bn // 32
+    ends = [i for i in range(len(code) - 1)
+            if code[i].startswith("s_nop 15") and code[i + 1].startswith("s_nop 15")]
+    assert ends, name
+    for e in ends:
+      first_read = next(i for i in range(e, len(code)) if code[i].startswith("ds_read"))
+      waits = [re.search(r"vmcnt\((\d+)\)", l) for l in code[e:first_read] if l.startswith("s_waitcnt")]
+      counts = [int(w.group(1)) for w in waits if w]
+      assert counts and min(counts) <= 2 * nd, \
+          f"{name}: LDS read {code[first_read]!r} after the K loop without a vmcnt wait <= {2 * nd}"
+    checked += 1
+  if any("gemm_fp8_wide" in n for n in wide_kernels):
+    assert checked >= 2
