@@ -188,9 +188,9 @@ class HotPath:
     return stages
 
   def step_batched(self):
-    """The pass as block forwards written against linear_batch run it: one quantizer launch
-    per activation and ONE GEMM launch per stage (cdit_fp8_gemm_rowwise_batched). Outputs are
-    bit-identical to step()."""
+    """The pass as block forwards written against linear_batch run it: ONE quantizer launch
+    (cdit_fp8_quant_rowwise_batched) and ONE GEMM launch (cdit_fp8_gemm_rowwise_batched) per
+    stage. Outputs are bit-identical to step()."""
     from cache_dit_amd import ops
     for stage in self.stages():
       if len(stage) == 1 and len(stage[0]) == 1:
@@ -199,9 +199,13 @@ class HotPath:
                              self.s[(M, K)], 0, epi)
         continue
       acts, at = [], 0
+      inputs = [self.layers[run[0]][:2] for run in stage]
+      if len(inputs) > 1:  # one quantizer launch for the activations of the stage
+        ops.quant_rowwise_batched_into([(self.x[mk], self.q[mk], self.s[mk]) for mk in inputs], 0)
+      else:
+        ops.quant_rowwise_into(self.x[inputs[0]], self.q[inputs[0]], self.s[inputs[0]], 0, gemm_follows=True)
       for run in stage:
         M, K = self.layers[run[0]][:2]
-        ops.quant_rowwise_into(self.x[(M, K)], self.q[(M, K)], self.s[(M, K)], 0, gemm_follows=True)
         members = [self.layers[i] for i in run]
         outs = []
         for _, _, N, *_ in members:

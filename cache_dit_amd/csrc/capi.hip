@@ -200,6 +200,66 @@ int cdit_fp8_quant_rowwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_
                            scale_mode, stream, false);
 }
 
+int cdit_fp8_quant_rowwise_batched(int n_act, const void* const* x_bf16, const int64_t* M,
+                                   int64_t K, const int64_t* ld_x, void* const* q_e4m3,
+                                   const int64_t* ld_q, float* const* scale, int scale_mode,
+                                   void* stream) {
+  const char* fn = "cdit_fp8_quant_rowwise_batched";
+  if (n_act < 1 || n_act > cdit::kMaxQuantActs || !x_bf16 || !M || !ld_x || !q_e4m3 || !ld_q || !scale) {
+    set_error("%s: 1 to %d activations and non-null argument arrays, got n_act=%d", fn,
+              cdit::kMaxQuantActs, n_act);
+    return CDIT_EINVAL;
+  }
+  const int mode = scale_mode >= 0 ? scale_mode & ~CDIT_QUANT_GEMM_FOLLOWS : scale_mode;
+  if (mode != CDIT_SCALE_BF16DIV && mode != CDIT_SCALE_FP32DIV) {
+    set_error("%s: unknown scale_mode %d", fn, scale_mode);
+    return CDIT_EINVAL;
+  }
+  cdit::QuantBatch batch = {};
+  int64_t rows = 0;
+  bool one_launch = K > 0 && K <= INT32_MAX;
+  for (int s = 0; s < n_act; ++s) {
+    if (M[s] < 0 || M[s] > INT32_MAX || K < 0 || K > INT32_MAX) {
+      set_error("%s: bad shape M[%d]=%lld K=%lld", fn, s, (long long)M[s], (long long)K);
+      return CDIT_EINVAL;
+    }
+    if (M[s] == 0) continue;
+    if (ld_x[s] < K || ld_q[s] < K) {
+      set_error("%s: leading dimension smaller than K (activation %d: ld_x=%lld ld_q=%lld K=%lld)",
+                fn, s, (long long)ld_x[s], (long long)ld_q[s], (long long)K);
+      return CDIT_EINVAL;
+    }
+    if (!scale[s] || (K > 0 && (!x_bf16[s] || !q_e4m3[s]))) {
+      set_error("%s: null pointer argument (activation %d)", fn, s);
+      return CDIT_EINVAL;
+    }
+    const int at = batch.acts++;
+    batch.row_begin[at] = (int)rows;
+    batch.x[at] = static_cast<const uint16_t*>(x_bf16[s]);
+    batch.ld_x[at] = ld_x[s];
+    batch.q[at] = static_cast<uint8_t*>(q_e4m3[s]);
+    batch.ld_q[at] = ld_q[s];
+    batch.scale[at] = scale[s];
+    rows += M[s];
+  }
+  if (batch.acts == 0) return CDIT_OK;
+  one_launch = one_launch && rows <= INT32_MAX && batch.acts > 1;
+  for (int s = batch.acts; s <= cdit::kMaxQuantActs; ++s) batch.row_begin[s] = (int)(one_launch ? rows : 0);
+  int rc = check_arch();
+  if (rc) return rc;
+  if (one_launch &&
+      cdit::launch_quant_rowwise_batched(batch, K, mode, static_cast<hipStream_t>(stream)) == 0)
+    return after_launch(fn);
+  // a single activation, or a batch the one-launch kernel does not take: one by one
+  for (int s = 0; s < n_act; ++s) {
+    if (M[s] == 0) continue;
+    rc = quant_rowwise_impl(fn, x_bf16[s], M[s], K, ld_x[s], q_e4m3[s], ld_q[s], scale[s], mode,
+                            stream, true);
+    if (rc) return rc;
+  }
+  return CDIT_OK;
+}
+
 int cdit_fp8_ln_modulate_quant(const void* x_bf16, int64_t M, int64_t K, int64_t ld_x,
                                const void* shift_bf16, const void* scale_bf16, int64_t ld_mod,
                                int64_t rows_per_mod, float eps, void* y_bf16, int64_t ld_y,

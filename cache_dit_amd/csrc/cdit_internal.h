@@ -15,6 +15,24 @@ int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void
                          int64_t ld_q, float* scale, int scale_mode, bool consumer_follows,
                          hipStream_t stream);
 
+// Up to kMaxQuantActs activations of one K quantized row-wise in one launch (the image- and
+// text-stream inputs of one stage of a double-stream block): global row r belongs to
+// activation s with row_begin[s] <= r < row_begin[s + 1].
+constexpr int kMaxQuantActs = 4;
+struct QuantBatch {
+  int acts;
+  int row_begin[kMaxQuantActs + 1];
+  const uint16_t* x[kMaxQuantActs];
+  int64_t ld_x[kMaxQuantActs];
+  uint8_t* q[kMaxQuantActs];
+  int64_t ld_q[kMaxQuantActs];
+  float* scale[kMaxQuantActs];
+};
+// 0: launched; 1: not taken (alignment, K beyond the register-resident kernel): the caller
+// launches the activations one by one.
+int launch_quant_rowwise_batched(const QuantBatch& batch, int64_t K, int scale_mode,
+                                 hipStream_t stream);
+
 int launch_quant_tensorwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void* q,
                             int64_t ld_q, float* scale, uint32_t* amax_ws, int scale_mode,
                             hipStream_t stream);

@@ -23,6 +23,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "cdit_internal.h"
 #include "quant_device.h"
 
@@ -30,17 +32,37 @@ namespace cdit {
 namespace {
 
 // Row resident in registers: CH 16-byte chunks per lane (K <= CH*512).
-template <int CH, bool NT_LOAD = false, bool NT_STORE = false>
+struct NoBatch {};
+
+// BATCHED: the rows of several activations in one launch (QuantBatch); x, q, scale and
+// their leading dimensions then come from the activation the row belongs to and M is the
+// total row count. The instances without it are unchanged by its existence.
+template <int CH, bool NT_LOAD = false, bool NT_STORE = false, bool BATCHED = false>
 __global__ __launch_bounds__(64) void quant_rowwise_regs(
     const uint16_t* __restrict__ x, int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q,
-    float* __restrict__ scale, int M, int K, int scale_mode) {
+    float* __restrict__ scale, int M, int K, int scale_mode,
+    std::conditional_t<BATCHED, QuantBatch, NoBatch> batch = {}) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int waves_per_block = blockDim.x >> 6;
   const int nchunks = K >> 3;
   for (int64_t row = (int64_t)blockIdx.x * waves_per_block + wave; row < M;
        row += (int64_t)gridDim.x * waves_per_block) {
-    const uint4* xr = reinterpret_cast<const uint4*>(x + row * ld_x);
+    const uint16_t* x_row = x + row * ld_x;
+    uint8_t* q_row = q + row * ld_q;
+    float* s_row = scale + row;
+    if constexpr (BATCHED) {
+      // wave-uniform: one row per wavefront (row_begin beyond the last activation holds M)
+      const int r = __builtin_amdgcn_readfirstlane((int)row);
+      int s = 0;
+#pragma unroll
+      for (int i = 1; i < kMaxQuantActs; ++i) s += r >= batch.row_begin[i];
+      const int64_t local = r - batch.row_begin[s];
+      x_row = batch.x[s] + local * batch.ld_x[s];
+      q_row = batch.q[s] + local * batch.ld_q[s];
+      s_row = batch.scale[s] + local;
+    }
+    const uint4* xr = reinterpret_cast<const uint4*>(x_row);
     uint4 v[CH];
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
@@ -67,8 +89,8 @@ __global__ __launch_bounds__(64) void quant_rowwise_regs(
     }
     m = wave_max_u32(fold2(m));
     const float s = row_scale(m, scale_mode);
-    if (lane == 0) scale[row] = s;
-    uint2* qr = reinterpret_cast<uint2*>(q + row * ld_q);
+    if (lane == 0) *s_row = s;
+    uint2* qr = reinterpret_cast<uint2*>(q_row);
     if (scale_in_fast_window(s)) {  // wave-uniform
       const float r = 1.0f / s;
 #pragma unroll
@@ -444,6 +466,51 @@ int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void
   hipLaunchKernelGGL(quant_rowwise_generic, grid, block, 0, stream, xp, ld_x, qp, ld_q, scale, Mi,
                      Ki, scale_mode);
   return 0;
+}
+
+int launch_quant_rowwise_batched(const QuantBatch& batch, int64_t K, int scale_mode,
+                                 hipStream_t stream) {
+  const int64_t M = batch.row_begin[batch.acts];
+  bool aligned = K % 8 == 0 && K > 0 && K <= 32 * 512;
+  for (int s = 0; s < batch.acts; ++s)
+    aligned = aligned && batch.ld_x[s] % 8 == 0 && batch.ld_q[s] % 8 == 0 &&
+              reinterpret_cast<uintptr_t>(batch.x[s]) % 16 == 0 &&
+              reinterpret_cast<uintptr_t>(batch.q[s]) % 8 == 0;
+  if (!aligned || M <= 0) return 1;
+  int64_t blocks = M < 256 * 256 ? M : 256 * 256;
+  dim3 grid((unsigned)blocks), block(64);
+  const int Mi = (int)M, Ki = (int)K;
+  const int need = (int)((K + 511) / 512);
+  // the codes are read by the GEMM that follows: cacheable stores; loads of a large batch
+  // carry the non-temporal hint (as launch_quant_rowwise chooses for one activation)
+  const bool nt_load = g_quant_variant >= 0 ? (g_quant_variant == 0 || g_quant_variant == 2)
+                                            : M * K * 2 > ((int64_t)64 << 20);
+#define CDIT_QUANT_CASE(CH)                                                                      \
+  if (need <= CH) {                                                                              \
+    if (nt_load) {                                                                               \
+      hipLaunchKernelGGL((quant_rowwise_regs<CH, true, false, true>), grid, block, 0, stream,    \
+                         nullptr, 0, nullptr, 0, nullptr, Mi, Ki, scale_mode, batch);            \
+    } else {                                                                                     \
+      hipLaunchKernelGGL((quant_rowwise_regs<CH, false, false, true>), grid, block, 0, stream,   \
+                         nullptr, 0, nullptr, 0, nullptr, Mi, Ki, scale_mode, batch);            \
+    }                                                                                            \
+    return 0;                                                                                    \
+  }
+  CDIT_QUANT_CASE(1)
+  CDIT_QUANT_CASE(2)
+  CDIT_QUANT_CASE(4)
+  CDIT_QUANT_CASE(6)
+  CDIT_QUANT_CASE(8)
+  CDIT_QUANT_CASE(10)
+  CDIT_QUANT_CASE(12)
+  CDIT_QUANT_CASE(16)
+  CDIT_QUANT_CASE(20)
+  CDIT_QUANT_CASE(24)
+  CDIT_QUANT_CASE(27)
+  CDIT_QUANT_CASE(30)
+  CDIT_QUANT_CASE(32)
+#undef CDIT_QUANT_CASE
+  return 1;
 }
 
 int launch_ln_modulate_quant(const void* x, int64_t M, int64_t K, int64_t ld_x, const void* shift,

@@ -329,7 +329,7 @@ def linear_batch(pairs):
            or any(x.is_inference() or not x.is_cuda or x.dtype != torch.bfloat16 for x, _ in pairs))
   if plain:
     return [[lin(x) for lin in lins] for x, lins in pairs]
-  acts, result = [], []
+  acts, result, rows = [], [], []
   for x, lins in pairs:
     x2 = ops._as_rows(x)
     M = x2.shape[0]
@@ -337,10 +337,13 @@ def linear_batch(pairs):
     result.append([o.view(*x.shape[:-1], lin.out_features) for o, lin in zip(outs, lins)])
     if M == 0:
       continue
-    q, s = ops.shared_activation_quant(x2, first._scale_mode_id)
-    acts.append((q, s, [lin.weight for lin in lins], [lin.weight_scale for lin in lins],
-                 [lin.bias for lin in lins], outs, [lin.epilogue for lin in lins]))
+    rows.append(x2)
+    acts.append([None, None, [lin.weight for lin in lins], [lin.weight_scale for lin in lins],
+                 [lin.bias for lin in lins], outs, [lin.epilogue for lin in lins]])
   if acts:
+    # one quantizer launch for the activations the cache does not hold, one GEMM launch
+    for act, (q, s) in zip(acts, ops.shared_activation_quant_many(rows, first._scale_mode_id)):
+      act[0], act[1] = q, s
     ops.gemm_rowwise_batched_into(acts)
   return result
 

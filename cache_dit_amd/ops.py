@@ -113,6 +113,26 @@ def quant_rowwise_into(x2: torch.Tensor, q: torch.Tensor, scale: torch.Tensor,
                                                         _stream_ptr(x2)))
 
 
+def quant_rowwise_batched_into(items, scale_mode_id: int) -> None:
+  """quant_rowwise_into for several activations of one K in a single launch. `items` is a
+  list of (x2 [M,K] bf16, q [M,K] e4m3, scale [M] fp32), at most _native.MAX_ACTS of them on
+  one device; the codes are taken to be read by a GEMM launched next. Bit-identical to one
+  quant_rowwise_into per item."""
+  import ctypes
+  n = len(items)
+  x0 = items[0][0]
+  K = x0.shape[1]
+  if any(x.shape[1] != K or x.device != x0.device for x, _, _ in items):
+    raise ValueError("quant_rowwise_batched_into: the activations must share K and the device")
+  vp, i64 = ctypes.c_void_p, ctypes.c_int64
+  with _DeviceOf(x0):
+    _native.check(_native.load().cdit_fp8_quant_rowwise_batched(
+        n, (vp * n)(*[x.data_ptr() for x, _, _ in items]), (i64 * n)(*[x.shape[0] for x, _, _ in items]),
+        K, (i64 * n)(*[x.stride(0) for x, _, _ in items]), (vp * n)(*[q.data_ptr() for _, q, _ in items]),
+        (i64 * n)(*[q.stride(0) for _, q, _ in items]), (vp * n)(*[s.data_ptr() for _, _, s in items]),
+        scale_mode_id, _stream_ptr(x0)))
+
+
 def gemm_rowwise_into(a: torch.Tensor, a_scale: torch.Tensor, w: torch.Tensor,
                       w_scale: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                       epilogue: int) -> None:
@@ -269,6 +289,46 @@ def shared_activation_quant(x2: torch.Tensor, scale_mode_id: int):
   quant_launches += 1
   _remember_quant(entries, capture_id, x2, scale_mode_id, q, s)
   return q, s
+
+
+def shared_activation_quant_many(x2s, scale_mode_id: int):
+  """shared_activation_quant for the activations of one stage: what the cache does not hold
+  is quantized in ONE launch (cdit_fp8_quant_rowwise_batched) when the activations share K
+  and the device. Returns [(codes, scales), ...] in the order of `x2s`."""
+  global quant_launches
+  x0 = x2s[0]
+  if (len(x2s) < 2 or len(x2s) > _native.MAX_ACTS
+      or any(x.is_inference() or x.shape[1] != x0.shape[1] or x.device != x0.device for x in x2s)):
+    return [shared_activation_quant(x, scale_mode_id) for x in x2s]
+  entries, capture_id = _shared_entries(x0)
+  result, missing = [None] * len(x2s), []
+  for i, x in enumerate(x2s):
+    for e in entries:
+      if e.matches(x, scale_mode_id):
+        result[i] = (e.q, e.s)
+        break
+    else:
+      if any(x is x2s[j] for j in missing):  # the same tensor twice in one stage
+        continue
+      missing.append(i)
+  if len(missing) == 1:
+    result[missing[0]] = shared_activation_quant(x2s[missing[0]], scale_mode_id)
+  elif missing:
+    items = []
+    for i in missing:
+      x = x2s[i]
+      q = torch.empty(x.shape, dtype=FP8, device=x.device)
+      s = torch.empty((x.shape[0], ), dtype=torch.float32, device=x.device)
+      items.append((x, q, s))
+    quant_rowwise_batched_into(items, scale_mode_id)
+    quant_launches += 1
+    for i, (x, q, s) in zip(missing, items):
+      _remember_quant(entries, capture_id, x, scale_mode_id, q, s)
+      result[i] = (q, s)
+  for i, x in enumerate(x2s):  # repeats of a tensor that was quantized just now
+    if result[i] is None:
+      result[i] = shared_activation_quant(x, scale_mode_id)
+  return result
 
 
 def clear_shared_activation_quant() -> None:

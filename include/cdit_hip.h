@@ -96,6 +96,23 @@ int cdit_fp8_quant_rowwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_
                            int scale_mode, void* stream);
 
 /*
+ * cdit_fp8_quant_rowwise on up to 4 activations of one K in a single launch: the inputs of
+ * the Linears of one stage that run as one batched GEMM (cdit_fp8_gemm_rowwise_batched), e.g.
+ * the image-stream and the text-stream activation of a double-stream block (reference
+ * dataflow: src/cache_dit/caching/patch_functors/functor_flux.py:48-80 patches the block
+ * forwards these Linears are called from). Activation s is x_bf16[s] [M[s], K] (ld_x[s]) ->
+ * q_e4m3[s] (ld_q[s]), scale[s] [M[s]]; codes and scales are those of one
+ * cdit_fp8_quant_rowwise call per activation, bit for bit (activations with M[s] == 0 are
+ * skipped; a batch the one-launch kernel does not take -- K not a multiple of 8, K > 16384,
+ * misaligned pointers -- runs as those calls). The codes are taken to be read by a GEMM
+ * launched next (CDIT_QUANT_GEMM_FOLLOWS is implied).
+ */
+int cdit_fp8_quant_rowwise_batched(int n_act, const void* const* x_bf16, const int64_t* M,
+                                   int64_t K, const int64_t* ld_x, void* const* q_e4m3,
+                                   const int64_t* ld_q, float* const* scale, int scale_mode,
+                                   void* stream);
+
+/*
  * Per-tensor dynamic FP8 quantization: one scale for the whole tensor. Replaces
  * torchao's Float8Tensor.from_hp(x, PerTensor()) as selected for the
  * "float8_per_tensor" quant type and the per-tensor fallback pass,

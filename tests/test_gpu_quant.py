@@ -211,3 +211,103 @@ def test_gemm_follows_hint_changes_nothing(mode):
   L = _native.load()  # an unknown mode stays an error with the flag set
   assert L.cdit_fp8_quant_rowwise(x.data_ptr(), 4, 64, 64, q0.data_ptr(), 64, s0.data_ptr(),
                                   0x100 | 5, None) == 1
+
+
+def _batched_case(shapes, K, mode_id, seed, specials=True):
+  """Activations [M_s, K] with outliers; a zero row, rows with scales outside the
+  fast-division window and a row that holds a NaN among them."""
+  g = torch.Generator(device="cuda").manual_seed(seed)
+  xs = []
+  for s, M in enumerate(shapes):
+    x = (torch.randn(M, K, generator=g, device="cuda") * (1 + s)).to(torch.bfloat16)
+    if specials and M >= 5 and K > 0:
+      x[0] = 0
+      x[1] *= 1e-32
+      x[2] *= 1e32
+      x[3, K // 2] = float("nan")
+      x[4, 0] = 100.0
+    xs.append(x)
+  return xs
+
+
+@pytest.mark.parametrize("mode_id", [0, 1])
+@pytest.mark.parametrize("shapes,K", [
+    ((4096, 512), 3072),          # FLUX double block: image + text stream
+    ((4096, 512), 12288),         # ... inputs of ff.net.2
+    ((6889, 256), 3072),          # Qwen-Image
+    ((5, 1, 77, 300), 1024),      # four activations, a single row among them
+    ((7, 0, 9), 640),             # an empty activation is skipped
+    ((33, 21), 16384),            # the longest row the register-resident kernel holds
+    ((33, 21), 16896),            # beyond it: runs as one launch per activation
+    ((12, 40), 200),              # K not a multiple of 8 in bytes of 16: likewise
+])
+def test_batched_quantizer_equals_one_launch_per_activation(shapes, K, mode_id):
+  """cdit_fp8_quant_rowwise_batched against cdit_fp8_quant_rowwise per activation: codes and
+  scales bit for bit, nothing written outside (outputs are windows of sentinel buffers)."""
+  from cache_dit_amd import ops
+  xs = _batched_case(shapes, K, mode_id, seed=sum(shapes) + K)
+  items, bufs = [], []
+  for x in xs:
+    M = x.shape[0]
+    qb = torch.full((M + 1, K + 16), 0x55, dtype=torch.uint8, device="cuda")
+    sb = torch.full((M + 1, ), -1.0, dtype=torch.float32, device="cuda")
+    bufs.append((qb, sb))
+    items.append((x, qb[:M, :K].view(torch.float8_e4m3fn), sb[:M]))
+  ops.quant_rowwise_batched_into(items, mode_id)
+  torch.cuda.synchronize()
+  for x, (qb, sb) in zip(xs, bufs):
+    M = x.shape[0]
+    q1 = torch.empty(M, K, dtype=torch.float8_e4m3fn, device="cuda")
+    s1 = torch.empty(M, dtype=torch.float32, device="cuda")
+    if M:
+      ops.quant_rowwise_into(x, q1, s1, mode_id)
+    torch.cuda.synchronize()
+    assert torch.equal(qb[:M, :K], q1.view(torch.uint8))
+    assert torch.equal(sb[:M].view(torch.int32), s1.view(torch.int32))
+    assert (qb[:, K:] == 0x55).all() and (qb[M] == 0x55).all() and sb[M] == -1.0
+
+
+def test_batched_quantizer_against_the_oracle_and_strided_inputs():
+  """Activations that are column windows of wider buffers (ld_x > K), against the CPU oracle."""
+  from cache_dit_amd import ops
+  K = 1536
+  g = torch.Generator().manual_seed(3)
+  wide = [torch.randn(M, K + 64, generator=g).to(torch.bfloat16) for M in (130, 70, 19)]
+  items = []
+  for w in wide:
+    x = w.cuda()[:, 8:8 + K]
+    items.append((x, torch.empty(x.shape, dtype=torch.float8_e4m3fn, device="cuda"),
+                  torch.empty(x.shape[0], dtype=torch.float32, device="cuda")))
+  ops.quant_rowwise_batched_into(items, 0)
+  torch.cuda.synchronize()
+  for w, (_, q, s) in zip(wide, items):
+    q_ref, s_ref = to.quantize_rowwise(w[:, 8:8 + K].contiguous(), "bf16div")
+    assert int((bits_u8(q) != bits_u8(q_ref)).sum()) == 0
+    assert int((bits_u32(s) != bits_u32(s_ref.reshape(-1))).sum()) == 0
+
+
+def test_batched_quantizer_argument_checks():
+  import ctypes
+  from cache_dit_amd import _native
+  L = _native.load()
+  x = torch.zeros(4, 64, dtype=torch.bfloat16, device="cuda")
+  q = torch.empty(4, 64, dtype=torch.uint8, device="cuda")
+  s = torch.empty(4, dtype=torch.float32, device="cuda")
+  vp, i64 = ctypes.c_void_p, ctypes.c_int64
+  EINVAL = 1  # CDIT_EINVAL
+
+  def call(n, M=4, K=64, ld=64, mode=0, xs=None):
+    k = max(n, 1)
+    return L.cdit_fp8_quant_rowwise_batched(
+        n, (vp * k)(*([x.data_ptr()] * k if xs is None else xs)), (i64 * k)(*[M] * k), K,
+        (i64 * k)(*[ld] * k), (vp * k)(*[q.data_ptr()] * k), (i64 * k)(*[64] * k),
+        (vp * k)(*[s.data_ptr()] * k), mode, None)
+
+  assert call(1) == 0 and call(2) == 0
+  assert call(0) == EINVAL and b"activations" in L.cdit_last_error()
+  assert call(5) == EINVAL
+  assert call(2, M=-1) == EINVAL and b"bad shape" in L.cdit_last_error()
+  assert call(2, ld=32) == EINVAL and b"leading dimension" in L.cdit_last_error()
+  assert call(2, mode=7) == EINVAL and b"scale_mode" in L.cdit_last_error()
+  assert call(2, xs=[x.data_ptr(), None]) == EINVAL and b"null pointer" in L.cdit_last_error()
+  torch.cuda.synchronize()
