@@ -588,6 +588,10 @@ def main():
                   help="run only the hot-path step legs (eager, hipGraph replay, shared "
                        "quantization) and print their figures: the command to put under "
                        "rocprofv3 for the kernel mix of one step")
+  ap.add_argument("--step-form", default="all",
+                  choices=["all", "batched", "grouped", "shared", "ungrouped"],
+                  help="with --step-only: time just this form of the step (default: all four "
+                       "and the eager launches), so that a kernel trace covers one form")
   args = ap.parse_args()
   if args.gpus != 1:
     sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
@@ -614,15 +618,18 @@ def main():
     return
 
   hot = HotPath(device)
-  for _ in range(args.warmup):
-    hot.step()
-  torch.cuda.synchronize()
-  # eager launches (988 kernel launches per step issued from Python)
-  t0 = time.perf_counter()
-  for _ in range(args.steps):
-    hot.step()
-  torch.cuda.synchronize()
-  eager_ms = (time.perf_counter() - t0) / args.steps * 1e3
+  one_form = args.step_form if args.step_only and args.step_form != "all" else None
+  eager_ms = None
+  if one_form is None:
+    for _ in range(args.warmup):
+      hot.step()
+    torch.cuda.synchronize()
+    # eager launches (988 kernel launches per step issued from Python)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+      hot.step()
+    torch.cuda.synchronize()
+    eager_ms = (time.perf_counter() - t0) / args.steps * 1e3
   # The same step captured once into a hipGraph and replayed: what a serving loop does
   # with a fixed-shape denoising step; removes the host launch cost. Four forms of the
   # step, all with bit-identical outputs: every Linear on its own (quantizer + GEMM each);
@@ -650,6 +657,14 @@ def main():
     return (time.perf_counter() - t0) / args.steps * 1e3
 
   launch_mode = "hipGraph replay"
+  if one_form is not None:
+    form = {"batched": hot.step_batched, "grouped": hot.step_grouped,
+            "shared": hot.step_shared_quant, "ungrouped": hot.step}[one_form]
+    ms = replay_ms(form)
+    print(json.dumps({"step_form": one_form, "ms_per_step": ms, "tflops": hot.flop / ms / 1e9,
+                      "launch": launch_mode, "steps": args.steps, "warmup": args.warmup,
+                      "device": arch}))
+    return
   try:
     ungrouped_ms = replay_ms(hot.step)
     shared_ms = replay_ms(hot.step_shared_quant)
