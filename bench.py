@@ -458,6 +458,50 @@ def headline_kernels(device):
     res["w8a16_frac_bf16_peak"] = res["w8a16_tflops"] / BF16_PEAK_TFLOPS
   except Exception as e:
     res["w8a16_note"] = str(e)[:120]
+  # the FP8 comm quantizers (scale packed behind each row) on an activation of the headline
+  # size and on its q/k/v as [B, S, 3, heads, head_dim]; GB/s over their algorithmic bytes
+  try:
+    heads, hd = 24, 128
+    yq = [torch.empty(M, K + 2, dtype=torch.uint8, device=device) for _ in range(nbuf)]
+    back = torch.empty(M, K, dtype=torch.bfloat16, device=device)
+    qkv = [torch.randn(1, M, 3, heads, hd, device=device, generator=g).to(torch.bfloat16)
+           for _ in range(3)]
+    pq = [torch.empty(3, M, 1, heads, hd + 4, dtype=torch.uint8, device=device) for _ in range(3)]
+    pback = torch.empty(1, M, heads, hd, dtype=torch.bfloat16, device=device)
+
+    def pt_quant():
+      i = it["i"] = (it["i"] + 1) % nbuf
+      _native.check(L.cdit_fp8_comm_per_token_quant(xs[i].data_ptr(), M, K, yq[i].data_ptr(), stream))
+
+    def pt_dequant():
+      i = it["i"] = (it["i"] + 1) % nbuf
+      _native.check(L.cdit_fp8_comm_per_token_dequant(yq[i].data_ptr(), M, K, back.data_ptr(), stream))
+
+    def qkv_quant():
+      i = it["i"] = (it["i"] + 1) % 3
+      x = qkv[i]
+      _native.check(L.cdit_fp8_comm_qkv_permute_quant(
+          x.data_ptr(), 1, M, 3, heads, hd, x.stride(0), x.stride(1), x.stride(2),
+          pq[i].data_ptr(), stream))
+
+    def qkv_dequant():
+      i = it["i"] = (it["i"] + 1) % 3
+      one = pq[i][0]  # [S, B, N, D + 4] bytes: strides are byte strides
+      _native.check(L.cdit_fp8_comm_qkv_permute_dequant(one.data_ptr(), M, 1, heads, hd, one.stride(0),
+                                                        one.stride(1), one.stride(2),
+                                                        pback.data_ptr(), stream))
+
+    rows = 3 * M * heads
+    res["comm_quant"] = {
+        "per_token_quant_gbps": (3.0 * K + 2) * M / _time_events(pt_quant, 200, 20) / 1e6,
+        "per_token_dequant_gbps": (3.0 * K + 2) * M / _time_events(pt_dequant, 200, 20) / 1e6,
+        "qkv_permute_quant_gbps": (3.0 * hd + 4) * rows / _time_events(qkv_quant, 100, 10) / 1e6,
+        "qkv_permute_dequant_gbps": (3.0 * hd + 4) * (rows / 3) / _time_events(qkv_dequant, 100, 10) / 1e6,
+        "note": "per token: 4608 x 3072 bf16 <-> codes + bf16 scale; qkv: [1, 4608, 3, 24, 128] "
+                "-> [3, 4608, 1, 24, 132], dequant of one of the three slices",
+    }
+  except Exception as e:
+    res["comm_quant_note"] = str(e)[:160]
   return res
 
 

@@ -78,16 +78,18 @@ __device__ __forceinline__ int align_of(const void* p) {
 //        1 = qkv form (fp32 scale, eps on the scale, true division).
 // Row r of `rows` rows: source x + src_off(r) (H bf16, 16-byte aligned when VEC), codes at
 // y + r * (H + tail) followed by the scale.
-template <int SCALE>
+// CH: 16-byte chunks per lane the row is held in (H <= 512 CH when vec): the register
+// budget, and with it the number of rows in flight per CU, follows the row length.
+template <int SCALE, int CH>
 __device__ __forceinline__ void quant_row(const uint16_t* __restrict__ xr, uint8_t* __restrict__ yr,
                                           int H, bool vec, int lane) {
   const int nchunks = H >> 3;
-  uint4 v[kMaxChunks];
+  uint4 v[CH];
   float amax = 0.0f;
   if (vec) {
     const uint4* xv = reinterpret_cast<const uint4*>(xr);
 #pragma unroll
-    for (int c = 0; c < kMaxChunks; ++c) {
+    for (int c = 0; c < CH; ++c) {
       const int idx = c * 64 + lane;
       if (c * 64 < nchunks) {  // wave-uniform: whole groups of 64 chunks
         v[c] = idx < nchunks ? xv[idx] : make_uint4(0, 0, 0, 0);
@@ -115,10 +117,61 @@ __device__ __forceinline__ void quant_row(const uint16_t* __restrict__ xr, uint8
     const float y = SCALE == 0 ? x * inv : x / scale;
     return y != y ? y : fminf(fmaxf(y, -kFp8Max), kFp8Max);
   };
-  if (vec) {
+  const int sh = (int)(reinterpret_cast<uintptr_t>(yr) & 7);  // wave-uniform
+  if (vec && (sh == 2 || sh == 4 || sh == 6)) {
+    // The row starts sh bytes behind an 8-byte boundary (the pitch H + 2 or D + 4 is not a
+    // multiple of 8): piece by piece 2- or 4-byte stores would quadruple the store count.
+    // The byte stream is shifted instead: the aligned 8-byte word k of the row holds the
+    // last sh bytes of piece k-1 and the first 8 - sh of piece k; a lane gets its left
+    // neighbour's piece with a wavefront shift (DPP), lane 0 the last piece of the previous
+    // group of 64 through a scalar. Only the first 8 - sh bytes of the row and its last sh
+    // bytes go out in 2-byte stores.
+    uint8_t* const base = yr - sh;
+    uint32_t carry_lo = 0, carry_hi = 0;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int idx = c * 64 + lane;
+      if (c * 64 < nchunks) {
+        uint32_t lo = 0, hi = 0;
+        if (idx < nchunks) {
+          lo = cvt4_fp8(q(bf16_lo(v[c].x)), q(bf16_hi(v[c].x)), q(bf16_lo(v[c].y)), q(bf16_hi(v[c].y)));
+          hi = cvt4_fp8(q(bf16_lo(v[c].z)), q(bf16_hi(v[c].z)), q(bf16_lo(v[c].w)), q(bf16_hi(v[c].w)));
+        }
+        // wave_shr:1 -- lane l takes lane l-1, lane 0 keeps the first operand
+        const uint32_t plo = (uint32_t)__builtin_amdgcn_update_dpp((int)carry_lo, (int)lo, 0x138, 0xf, 0xf, false);
+        const uint32_t phi = (uint32_t)__builtin_amdgcn_update_dpp((int)carry_hi, (int)hi, 0x138, 0xf, 0xf, false);
+        uint32_t wlo, whi;
+        if (sh == 2) {
+          wlo = __builtin_amdgcn_alignbyte(lo, phi, 2);
+          whi = __builtin_amdgcn_alignbyte(hi, lo, 2);
+        } else if (sh == 4) {
+          wlo = phi;
+          whi = lo;
+        } else {
+          wlo = __builtin_amdgcn_alignbyte(phi, plo, 2);
+          whi = __builtin_amdgcn_alignbyte(lo, phi, 2);
+        }
+        if (idx > 0 && idx < nchunks) *reinterpret_cast<uint2*>(base + 8 * (int64_t)idx) = uint2{wlo, whi};
+        const uint16_t hw[4] = {(uint16_t)lo, (uint16_t)(lo >> 16), (uint16_t)hi, (uint16_t)(hi >> 16)};
+        if (idx == 0) {  // head of the row: its first 8 - sh bytes
+#pragma unroll
+          for (int j = 0; j < 3; ++j)
+            if (2 * j < 8 - sh) reinterpret_cast<uint16_t*>(yr)[j] = hw[j];
+        }
+        if (idx == nchunks - 1) {  // tail: the last sh bytes of the last piece
+          uint16_t* t = reinterpret_cast<uint16_t*>(base + 8 * (int64_t)nchunks);
+#pragma unroll
+          for (int j = 1; j < 4; ++j)
+            if (2 * j >= 8 - sh) t[j - (8 - sh) / 2] = hw[j];
+        }
+        carry_lo = (uint32_t)__builtin_amdgcn_readlane((int)lo, 63);
+        carry_hi = (uint32_t)__builtin_amdgcn_readlane((int)hi, 63);
+      }
+    }
+  } else if (vec) {
     const int al = align_of(yr);
 #pragma unroll
-    for (int c = 0; c < kMaxChunks; ++c) {
+    for (int c = 0; c < CH; ++c) {
       const int idx = c * 64 + lane;
       if (c * 64 < nchunks && idx < nchunks) {
         const uint32_t lo = cvt4_fp8(q(bf16_lo(v[c].x)), q(bf16_hi(v[c].x)), q(bf16_lo(v[c].y)),
@@ -188,12 +241,13 @@ __device__ __forceinline__ void dequant_row(const uint8_t* __restrict__ xr, uint
   }
 }
 
+template <int CH>
 __global__ __launch_bounds__(64) void comm_per_token_quant(const uint16_t* __restrict__ x,
                                                            uint8_t* __restrict__ y, int64_t M, int H,
                                                            bool vec) {
   const int lane = threadIdx.x;
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x)
-    quant_row<0>(x + row * H, y + row * (H + 2), H, vec, lane);
+    quant_row<0, CH>(x + row * H, y + row * (H + 2), H, vec, lane);
 }
 
 __global__ __launch_bounds__(64) void comm_per_token_dequant(const uint8_t* __restrict__ x,
@@ -207,6 +261,7 @@ __global__ __launch_bounds__(64) void comm_per_token_dequant(const uint8_t* __re
 // One wavefront per head row. Output row index r = ((p * S + s) * B + b) * N + n of
 // [P,S,B,N,D+4]; the source row is x[b,s,p,n,:] (element strides for b, s, p; heads and
 // channels contiguous, as the reference kernel assumes).
+template <int CH>
 __global__ __launch_bounds__(64) void comm_qkv_permute_quant(
     const uint16_t* __restrict__ x, uint8_t* __restrict__ y, int B, int S, int P, int N, int D,
     int64_t sb, int64_t ss, int64_t sp, bool vec) {
@@ -218,7 +273,7 @@ __global__ __launch_bounds__(64) void comm_qkv_permute_quant(
     const int b = (int)(t % B);
     const int s = (int)((t / B) % S);
     const int p = (int)(t / ((int64_t)B * S));
-    quant_row<1>(x + b * sb + s * ss + p * sp + (int64_t)n * D, y + r * (D + 4), D, vec, lane);
+    quant_row<1, CH>(x + b * sb + s * ss + p * sp + (int64_t)n * D, y + r * (D + 4), D, vec, lane);
   }
 }
 
@@ -329,8 +384,16 @@ unsigned grid_for(int64_t rows) {
 int launch_comm_per_token_quant(const void* x, int64_t M, int64_t H, void* y, hipStream_t stream) {
   const bool vec = H % 8 == 0 && H <= kMaxChunks * 512 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(y) % 2 == 0;
-  hipLaunchKernelGGL(comm_per_token_quant, dim3(grid_for(M)), dim3(64), 0, stream,
-                     static_cast<const uint16_t*>(x), static_cast<uint8_t*>(y), M, (int)H, vec);
+  const int need = vec ? (int)((H + 511) / 512) : 1;
+#define CDIT_PT_Q(CH)                                                                          \
+  if (need <= CH) {                                                                            \
+    hipLaunchKernelGGL(comm_per_token_quant<CH>, dim3(grid_for(M)), dim3(64), 0, stream,        \
+                       static_cast<const uint16_t*>(x), static_cast<uint8_t*>(y), M, (int)H, vec); \
+    return 0;                                                                                  \
+  }
+  CDIT_PT_Q(1) CDIT_PT_Q(2) CDIT_PT_Q(4) CDIT_PT_Q(6) CDIT_PT_Q(8) CDIT_PT_Q(12) CDIT_PT_Q(16)
+  CDIT_PT_Q(24) CDIT_PT_Q(32)
+#undef CDIT_PT_Q
   return 0;
 }
 
@@ -359,9 +422,16 @@ int launch_comm_qkv_permute_quant(const void* x, int B, int S, int P, int N, int
 #undef CDIT_QKV_Q
     return 0;
   }
-  hipLaunchKernelGGL(comm_qkv_permute_quant, dim3(grid_for(rows)), dim3(64), 0,
-                     stream, static_cast<const uint16_t*>(x), static_cast<uint8_t*>(y), B, S, P, N, D, sb,
-                     ss, sp, vec);
+  const int need = vec ? (D + 511) / 512 : 1;
+#define CDIT_QKV_ROW(CH)                                                                          \
+  if (need <= CH) {                                                                               \
+    hipLaunchKernelGGL(comm_qkv_permute_quant<CH>, dim3(grid_for(rows)), dim3(64), 0, stream,      \
+                       static_cast<const uint16_t*>(x), static_cast<uint8_t*>(y), B, S, P, N, D, sb, \
+                       ss, sp, vec);                                                              \
+    return 0;                                                                                     \
+  }
+  CDIT_QKV_ROW(1) CDIT_QKV_ROW(4) CDIT_QKV_ROW(32)
+#undef CDIT_QKV_ROW
   return 0;
 }
 
