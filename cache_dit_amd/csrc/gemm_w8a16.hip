@@ -27,6 +27,7 @@
 #include <type_traits>
 
 #include "gemm_common.h"
+#include "quant_device.h"
 
 namespace cdit {
 namespace {
@@ -878,6 +879,79 @@ __global__ __launch_bounds__(256) void gemm_w8a16_skinny(GemmArgs g) {
   }
 }
 
+// One activation row (M = 1: the modulation Linears), K <= 4096, with the access pattern of
+// the w8a8 path's linear_fp8_row1: a load instruction of the wavefront reads 1 KiB of one
+// weight row (lane l bytes 16 l .. 16 l + 15) where the 16-row arrangement above makes every
+// lane a memory request of its own; the MFMA's 16 "rows" are 16 interleaved K subsets of that
+// row, the activation is fetched at the same positions lane for lane (32 bytes of bf16 per
+// 16 weight bytes), D[i][i] is the partial dot product over subset i and the diagonal sums
+// to the whole one. A wavefront owns three whole rows, all of their loads in flight at once.
+constexpr int kRow1Rows = 3, kRow1Waves = 4;
+template <int CHK>
+__global__ __launch_bounds__(64 * kRow1Waves) void gemm_w8a16_row1(GemmArgs g) {
+  constexpr int R = kRow1Rows;
+  typedef float v4f_ __attribute__((ext_vector_type(4)));
+  typedef unsigned int u4v __attribute__((ext_vector_type(4)));
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int row0 = (blockIdx.x * kRow1Waves + wave) * R;
+  const u4v zero4 = {0u, 0u, 0u, 0u};
+  u4v w[R][CHK];
+#pragma unroll
+  for (int q = 0; q < R; ++q) {
+    const uint8_t* __restrict__ wp = g.b + (int64_t)min(row0 + q, g.N - 1) * g.ldb + lane * 16;
+#pragma unroll
+    for (int c = 0; c < CHK; ++c) {
+      if (c * 1024 + lane * 16 < g.K) {
+        w[q][c] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wp + c * 1024));
+      } else {
+        w[q][c] = zero4;
+      }
+    }
+  }
+  const uint16_t* __restrict__ ap = static_cast<const uint16_t*>(g.a) + lane * 16;
+  const v8bf zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  v8bf xa[CHK][2];
+#pragma unroll
+  for (int c = 0; c < CHK; ++c) {
+    const bool in = c * 1024 + lane * 16 < g.K;
+    const v8bf* src = reinterpret_cast<const v8bf*>(ap + c * 1024);
+    xa[c][0] = in ? src[0] : zero8;
+    xa[c][1] = in ? src[1] : zero8;
+  }
+  // lane l holds D[4 (l >> 4) + e][l & 15]: the diagonal entry of lanes 0-3, 20-23, 40-43, 60-63
+  const int diag = (lane & 15) - 4 * (lane >> 4);
+  float mine = 0.0f;  // lane q keeps the dot product of row row0 + q
+#pragma unroll
+  for (int q = 0; q < R; ++q) {
+    v4f_ acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int c = 0; c < CHK; ++c) {
+      const uint32_t words[4] = {w[q][c][0], w[q][c][1], w[q][c][2], w[q][c][3]};
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const v2bf c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(words[2 * t], 1.0f, false);
+        const v2bf c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(words[2 * t], 1.0f, true);
+        const v2bf c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(words[2 * t + 1], 1.0f, false);
+        const v2bf c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(words[2 * t + 1], 1.0f, true);
+        const v8bf wf = {c0[0], c0[1], c1[0], c1[1], c2[0], c2[1], c3[0], c3[1]};
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xa[c][t], acc, 0, 0, 0);
+      }
+    }
+    float d = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) d = diag == e ? acc[e] : d;
+    const float sum = wave_sum_f32(d);
+    mine = lane == q ? sum : mine;
+  }
+  const int n = row0 + lane;
+  if (lane < R && n < g.N) {
+    float t = mine * g.b_scale[n];
+    if (g.bias) t += __uint_as_float((uint32_t)g.bias[n] << 16);
+    if (g.epilogue & CDIT_EPI_GELU_TANH) t = gelu_tanh(t);
+    g.out[n] = (uint16_t)(pack_bf16x2(t, 0.0f) & 0xffffu);
+  }
+}
+
 // Any shape: one output element per thread, scalar decode + FMA.
 __global__ __launch_bounds__(256) void gemm_w8a16_generic(GemmArgs g) {
   const int n = blockIdx.x * 16 + (threadIdx.x & 15);
@@ -936,6 +1010,18 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {
     dim3 grid((g.N + 15) / 16, (g.M + 15) / 16);
     hipLaunchKernelGGL(gemm_w8a16_generic, grid, dim3(256), 0, stream, g);
+    return 0;
+  }
+  if ((variant < 0 || variant == 51) && g.M == 1 && g.K % 128 == 0 && g.K <= 4096) {
+    // (tiled_ok has checked the alignment of the operands and of ldb)
+    constexpr int rows_wg = kRow1Rows * kRow1Waves;
+    const dim3 grid((g.N + rows_wg - 1) / rows_wg), block(64 * kRow1Waves);
+    switch ((g.K + 1023) / 1024) {
+      case 1: hipLaunchKernelGGL(gemm_w8a16_row1<1>, grid, block, 0, stream, g); break;
+      case 2: hipLaunchKernelGGL(gemm_w8a16_row1<2>, grid, block, 0, stream, g); break;
+      case 3: hipLaunchKernelGGL(gemm_w8a16_row1<3>, grid, block, 0, stream, g); break;
+      default: hipLaunchKernelGGL(gemm_w8a16_row1<4>, grid, block, 0, stream, g); break;
+    }
     return 0;
   }
   if ((variant < 0 && g.M <= 16 && g.K % 128 == 0) || variant == 50) {

@@ -80,6 +80,67 @@ def test_skinny_kernel(M, N, K, gelu):
   _assert_close(_run(x, wq, ws, b, epilogue=gelu), ref)
 
 
+ONE_ROW_SHAPES = [(18432, 3072), (9216, 3072), (1008, 2048), (24, 128), (6160, 4096), (3088, 1024),
+                  (528, 1152), (272, 3968)]
+
+
+@pytest.mark.parametrize("N,K", ONE_ROW_SHAPES)
+@pytest.mark.parametrize("gelu", [0, 1])
+def test_one_row_kernel(N, K, gelu):
+  """M = 1 with K <= 4096 runs a kernel of its own (whole weight rows per wavefront, K walked
+  in an interleaved order): automatic choice, forced (51), against the oracle and the 16-row
+  kernel (50); row counts that leave partial wavefronts, K with a partial last KiB."""
+  from cache_dit_amd import _native
+  x, wq, ws, b = _problem(1, N, K, seed=N + K)
+  ws = ws * (8 if gelu else 1)
+  ref = to.w8a16_linear(x, wq, ws, b, gelu="fused" if gelu else None, fused=True)
+  auto = _run(x, wq, ws, b, epilogue=gelu)
+  _assert_close(auto, ref)
+  _native.set_gemm_variant(51)
+  assert torch.equal(_run(x, wq, ws, b, epilogue=gelu), auto)
+  _native.set_gemm_variant(50)
+  _assert_close(_run(x, wq, ws, b, epilogue=gelu), ref)
+
+
+@pytest.mark.parametrize("N,K", ONE_ROW_SHAPES)
+def test_one_row_kernel_exact_and_k_positions(N, K):
+  """Integer operands: bit-equal to the oracle. Then a single 1 in the activation on both
+  sides of every boundary of the kernel's K walk (16-byte lane pieces, the two MFMAs of a
+  piece, 1 KiB loads) against weights whose value encodes the K index."""
+  from cache_dit_amd import _native
+  _native.set_gemm_variant(51)
+  g = torch.Generator().manual_seed(N + K)
+  x = torch.randint(-4, 5, (1, K), generator=g).to(torch.bfloat16)
+  w = torch.randint(-4, 5, (N, K), generator=g).float().to(FP8)
+  ws = torch.full((N, 1), 0.25)
+  assert torch.equal(_run(x, w, ws, None).cpu(), to.w8a16_linear(x, w, ws, fused=True))
+  w = ((((torch.arange(K) * 7) % 15) + 1).float().repeat(N, 1) * (1 + (torch.arange(N) % 2)).reshape(-1, 1)).to(FP8)
+  ones = torch.ones(N, 1)
+  for pos in (0, 7, 8, 15, 16, 31, 127, 128, 1007, 1023, 1024, 1040, 2047, 2048, 3071, 3072, K - 17, K - 1):
+    if pos >= K:
+      continue
+    x = torch.zeros(1, K)
+    x[0, pos] = 1.0
+    out = _run(x.to(torch.bfloat16), w, ones, None)
+    assert torch.equal(out.cpu(), to.w8a16_linear(x.to(torch.bfloat16), w, ones, fused=True)), pos
+
+
+def test_one_row_kernel_writes_only_its_row():
+  from cache_dit_amd import _native
+  N, K = 1040, 3072
+  x, wq, ws, b = _problem(1, N, K, seed=9)
+  ref = to.w8a16_linear(x, wq, ws, b, fused=True)
+  buf = torch.full((2, N + 24), 7.0, dtype=torch.bfloat16, device="cuda")
+  L = _native.load()
+  xg, w, sw, bias = x.cuda(), wq.cuda(), ws.cuda().reshape(-1).contiguous(), b.cuda()
+  rc = L.cdit_w8a16_gemm(xg.data_ptr(), w.data_ptr(), sw.data_ptr(), bias.data_ptr(), buf.data_ptr(),
+                         1, N, K, K, K, buf.stride(0), 0, _native.DT_BF16, None)
+  assert rc == 0, L.cdit_last_error()
+  torch.cuda.synchronize()
+  assert max_rel_err(buf[0, :N].cpu(), ref[0]) <= REL_TOL
+  assert (buf[0, N:] == 7.0).all() and (buf[1] == 7.0).all()
+
+
 def test_skinny_exact_and_every_code():
   from cache_dit_amd import _native
   g = torch.Generator().manual_seed(14)
