@@ -354,3 +354,51 @@ def test_stream_batched_block_forwards_are_bit_identical():
     q0 = qwen(**qin)
     assert ds.batch_streams(qwen) == 2
     assert torch.equal(qwen(**qin), q0)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_batched_random_shapes_exact_against_the_oracle(seed):
+  """Randomly drawn batches -- 1 to 4 activations of 17 to 700 rows, 1 to 3 members each with
+  N a multiple of 8 up to 600, K of 3 to 8 steps, random epilogue flags and missing biases,
+  a randomly forced tile shape or the automatic choice -- on integer-valued data, where every
+  partial sum is exact: the outputs must equal the CPU oracle bit for bit, and nothing but
+  the outputs may be written (each is a window of a sentinel-filled buffer)."""
+  import random
+  from cache_dit_amd import _native, ops
+  rnd = random.Random(seed)
+  K = 128 * rnd.randint(3, 8)
+  n_act = rnd.randint(1, 4)
+  budget = 8
+  acts, bufs = [], []
+  for s in range(n_act):
+    M = rnd.choice([17, 33, 64, 100, 255, 256, 257, 300, 511, 700])
+    n_mem = rnd.randint(1, min(3, budget - (n_act - s - 1)))
+    budget -= n_mem
+    Ns = [8 * rnd.randint(1, 75) for _ in range(n_mem)]
+    no_bias = tuple(i for i in range(n_mem) if rnd.random() < 0.3)
+    a, a_s, ws, wss, bs = _members(M, K, Ns, seed=1000 * seed + s, integer=True, no_bias=no_bias)
+    epis = [rnd.randint(0, 1) for _ in Ns]
+    outs = []
+    for N in Ns:
+      buf = torch.full((M + 1, N + 8), 7.0, dtype=torch.bfloat16, device="cuda")
+      bufs.append((buf, M, N))
+      outs.append(buf[:M, :N])
+    acts.append((a, a_s, ws, wss, bs, outs, epis))
+  variant = rnd.choice([-1, -1, 12, 14, 15, 16, 17, 18])
+  _native.set_gemm_variant(variant)
+  if n_act == 1 and len(acts[0][2]) == 1:
+    a, a_s, ws, wss, bs, outs, epis = acts[0]
+    ops.gemm_rowwise_into(a, a_s, ws[0], wss[0], bs[0], outs[0], epis[0])
+  else:
+    ops.gemm_rowwise_batched_into(acts)
+  torch.cuda.synchronize()
+  for s, (a, a_s, ws, wss, bs, outs, epis) in enumerate(acts):
+    for p, (w, sc, b, o, e) in enumerate(zip(ws, wss, bs, outs, epis)):
+      ref = to.scaled_mm_rowwise(a.cpu(), a_s.cpu(), w.cpu(), sc.cpu(), None if b is None else b.cpu(),
+                                 gelu="fused" if e else None)
+      if e:  # the GELU is not exact arithmetic: the oracle's tolerance
+        assert max_rel_err(o.cpu(), ref) <= 1e-2, (seed, variant, s, p)
+      else:
+        assert torch.equal(o.cpu().view(torch.int16), ref.view(torch.int16)), (seed, variant, s, p)
+  for buf, M, N in bufs:
+    assert (buf[M] == 7.0).all() and (buf[:, N:] == 7.0).all(), (seed, variant)
