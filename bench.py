@@ -193,6 +193,19 @@ class HotPath:
     stage. Outputs are bit-identical to step()."""
     from cache_dit_amd import ops
     for stage in self.stages():
+      if self.mode == "w8a16":  # weight-only: no quantizer, one GEMM launch per stage
+        acts, at = [], 0
+        for run in stage:
+          M, K = self.layers[run[0]][:2]
+          members = [self.layers[i] for i in run]
+          outs = []
+          for _, _, N, *_ in members:
+            outs.append(self.out2[at:at + M * N].view(M, N))
+            at += M * N
+          acts.append((self.x[(M, K)], [m[3] for m in members], [m[4] for m in members],
+                       [m[5] for m in members], outs, [m[6] for m in members]))
+        ops.w8a16_batched_into(acts)
+        continue
       if len(stage) == 1 and len(stage[0]) == 1:
         M, K, N, w, ws, b, epi = self.layers[stage[0][0]]
         ops.linear_w8a8_into(self.x[(M, K)], w, ws, b, self.out[:M * N].view(M, N), self.q[(M, K)],
@@ -253,28 +266,33 @@ class HotPath:
 
 def step_leg(device, linears, mode, steps, warmup):
   """A step of another benchmark configuration (every quantized Linear of the model at
-  its real shape with its own weights; w8a8: stages batched as in the headline step),
+  its real shape with its own weights; stages batched as in the headline step),
   captured into a hipGraph and replayed like the headline step. Returns ms per step,
   TFLOP/s and the Linear count."""
   import torch
   hot = HotPath(device, linears, mode)
-  step = hot.step if mode == "w8a16" else hot.step_batched
-  step()
-  torch.cuda.synchronize()
-  graph = torch.cuda.CUDAGraph()
-  with torch.cuda.graph(graph):
+
+  def replay_ms(step):
     step()
-  for _ in range(warmup):
-    graph.replay()
-  torch.cuda.synchronize()
-  t0 = time.perf_counter()
-  for _ in range(steps):
-    graph.replay()
-  torch.cuda.synchronize()
-  ms = (time.perf_counter() - t0) / steps * 1e3
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+      step()
+    for _ in range(warmup):
+      graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+      graph.replay()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3
+
+  ms = replay_ms(hot.step_batched)
   res = {"ms_per_step": ms, "tflops": hot.flop / ms / 1e9, "linears": len(hot.layers),
          "linear_flop_per_step": hot.flop}
-  del graph, hot
+  if mode == "w8a16":  # every Linear on its own, beside the batched stages
+    res["ungrouped_ms_per_step"] = replay_ms(hot.step)
+  del hot
   torch.cuda.empty_cache()
   return res
 

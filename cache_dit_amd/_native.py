@@ -39,6 +39,7 @@ EXPORTS = (
     "cdit_fp8_gemm_rowwise_grouped",
     "cdit_fp8_gemm_rowwise_batched",
     "cdit_w8a16_gemm",
+    "cdit_w8a16_gemm_batched",
     "cdit_fp8_linear_w8a8",
     "cdit_fp8_linear_w8a8_static",
     "cdit_fp8_comm_per_token_quant",
@@ -110,6 +111,8 @@ def _bind(L: ctypes.CDLL) -> None:
   L.cdit_fp8_comm_qkv_permute_quant.argtypes = [vp, i64, i64, i64, i64, i64, i64, i64, i64, vp, vp]
   L.cdit_fp8_comm_qkv_permute_dequant.restype = ci
   L.cdit_fp8_comm_qkv_permute_dequant.argtypes = [vp, i64, i64, i64, i64, i64, i64, i64, vp, vp]
+  L.cdit_w8a16_gemm_batched.restype = ci
+  L.cdit_w8a16_gemm_batched.argtypes = [ci, vp, vp, i64, i64, vp, vp, vp, vp, vp, vp, i64, vp, vp, vp]
   L.cdit_w8a16_gemm.restype = ci
   L.cdit_w8a16_gemm.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, vp]
 

@@ -371,13 +371,14 @@ int cdit_fp8_gemm_rowwise(const void* a_q, const float* a_scale, const void* b_q
 }
 
 // n_act activations, activation s with members_per_act[s] members (flattened in order).
-static int gemm_batched_impl(const char* fn, int n_act, const void* const* a_q,
+// weight_only: the w8a16 form (a_q holds bf16 activations, a_scale is null)
+static int gemm_batched_impl(const char* fn, bool weight_only, int n_act, const void* const* a_q,
                              const float* const* a_scale, const int64_t* M, int64_t K, int64_t lda,
                              const int* members_per_act, const void* const* b_q,
                              const float* const* b_scale, const void* const* bias,
                              void* const* out, const int64_t* N, int64_t ldb, const int64_t* ldo,
                              const int* epilogue, void* stream) {
-  if (n_act < 1 || n_act > kMaxActs || !a_q || !a_scale || !M || !members_per_act) {
+  if (n_act < 1 || n_act > kMaxActs || !a_q || (!a_scale && !weight_only) || !M || !members_per_act) {
     set_error("%s: 1 to %d activations with their arrays, got n_act=%d", fn, kMaxActs, n_act);
     return CDIT_EINVAL;
   }
@@ -405,9 +406,9 @@ static int gemm_batched_impl(const char* fn, int n_act, const void* const* a_q,
     grp.first_member[s] = p;
     for (int j = 0; j < members_per_act[s]; ++j, ++p) {
       int rc = check_gemm(fn, a_q[s], b_q[p], b_scale[p], bias ? bias[p] : nullptr, out[p], M[s], N[p],
-                          K, lda, ldb, ldo[p], epilogue ? epilogue[p] : 0, CDIT_DT_BF16, false);
+                          K, lda, ldb, ldo[p], epilogue ? epilogue[p] : 0, CDIT_DT_BF16, weight_only);
       if (rc) return rc;
-      if (M[s] > 0 && N[p] > 0 && !a_scale[s]) {
+      if (!weight_only && M[s] > 0 && N[p] > 0 && !a_scale[s]) {
         set_error("%s: a_scale is null", fn);
         return CDIT_EINVAL;
       }
@@ -421,7 +422,7 @@ static int gemm_batched_impl(const char* fn, int n_act, const void* const* a_q,
       any_empty |= N[p] == 0;
     }
     grp.a[s] = a_q[s];
-    grp.a_scale[s] = a_scale[s];
+    grp.a_scale[s] = weight_only ? nullptr : a_scale[s];
     grp.M[s] = (int)M[s];
     any_empty |= M[s] == 0;
   }
@@ -434,7 +435,9 @@ static int gemm_batched_impl(const char* fn, int n_act, const void* const* a_q,
     common.lda = lda;
     common.ldb = ldb;
     common.out_dtype = CDIT_DT_BF16;
-    rc = launch_gemm_fp8_grouped(common, grp, g_gemm_variant, static_cast<hipStream_t>(stream));
+    rc = weight_only
+             ? launch_gemm_w8a16_grouped(common, grp, g_gemm_variant, static_cast<hipStream_t>(stream))
+             : launch_gemm_fp8_grouped(common, grp, g_gemm_variant, static_cast<hipStream_t>(stream));
     if (rc == 0) return after_launch(fn);
     if (rc > 0) return rc;
   }
@@ -442,9 +445,13 @@ static int gemm_batched_impl(const char* fn, int n_act, const void* const* a_q,
   // element-wise kernel takes): the members one after the other, same results
   for (int s = 0, p = 0; s < n_act; ++s)
     for (int j = 0; j < members_per_act[s]; ++j, ++p) {
-      rc = cdit_fp8_gemm_rowwise(a_q[s], a_scale[s], b_q[p], b_scale[p], bias ? bias[p] : nullptr,
-                                 out[p], M[s], N[p], K, lda, ldb, ldo[p], epilogue ? epilogue[p] : 0,
-                                 CDIT_DT_BF16, stream);
+      rc = weight_only
+               ? cdit_w8a16_gemm(a_q[s], b_q[p], b_scale[p], bias ? bias[p] : nullptr, out[p], M[s],
+                                 N[p], K, lda, ldb, ldo[p], epilogue ? epilogue[p] : 0, CDIT_DT_BF16,
+                                 stream)
+               : cdit_fp8_gemm_rowwise(a_q[s], a_scale[s], b_q[p], b_scale[p],
+                                       bias ? bias[p] : nullptr, out[p], M[s], N[p], K, lda, ldb,
+                                       ldo[p], epilogue ? epilogue[p] : 0, CDIT_DT_BF16, stream);
       if (rc) return rc;
     }
   return CDIT_OK;
@@ -455,7 +462,7 @@ int cdit_fp8_gemm_rowwise_grouped(const void* a_q, const float* a_scale, int64_t
                                   const float* const* b_scale, const void* const* bias,
                                   void* const* out, const int64_t* N, int64_t ldb,
                                   const int64_t* ldo, const int* epilogue, void* stream) {
-  return gemm_batched_impl("cdit_fp8_gemm_rowwise_grouped", 1, &a_q, &a_scale, &M, K, lda, &count,
+  return gemm_batched_impl("cdit_fp8_gemm_rowwise_grouped", false, 1, &a_q, &a_scale, &M, K, lda, &count,
                            b_q, b_scale, bias, out, N, ldb, ldo, epilogue, stream);
 }
 
@@ -465,7 +472,16 @@ int cdit_fp8_gemm_rowwise_batched(int n_act, const void* const* a_q, const float
                                   const float* const* b_scale, const void* const* bias,
                                   void* const* out, const int64_t* N, int64_t ldb,
                                   const int64_t* ldo, const int* epilogue, void* stream) {
-  return gemm_batched_impl("cdit_fp8_gemm_rowwise_batched", n_act, a_q, a_scale, M, K, lda,
+  return gemm_batched_impl("cdit_fp8_gemm_rowwise_batched", false, n_act, a_q, a_scale, M, K, lda,
+                           members_per_act, b_q, b_scale, bias, out, N, ldb, ldo, epilogue, stream);
+}
+
+int cdit_w8a16_gemm_batched(int n_act, const void* const* x_bf16, const int64_t* M, int64_t K,
+                            int64_t lda, const int* members_per_act, const void* const* b_q,
+                            const float* const* b_scale, const void* const* bias,
+                            void* const* out, const int64_t* N, int64_t ldb, const int64_t* ldo,
+                            const int* epilogue, void* stream) {
+  return gemm_batched_impl("cdit_w8a16_gemm_batched", true, n_act, x_bf16, nullptr, M, K, lda,
                            members_per_act, b_q, b_scale, bias, out, N, ldb, ldo, epilogue, stream);
 }
 

@@ -98,6 +98,9 @@ int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream);
 int launch_gemm_fp8_grouped(const GemmArgs& common, const GemmGroup& grp, int variant,
                             hipStream_t stream);
 int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream);
+// The same for the weight-only GEMM (grp.a: bf16 activations; grp.a_scale unused).
+int launch_gemm_w8a16_grouped(const GemmArgs& common, const GemmGroup& grp, int variant,
+                              hipStream_t stream);
 // One w8a8 Linear forward at M <= 16 in a single kernel (per-token quantizer + GEMM);
 // g.a is the bf16 activation, g.lda its leading dimension in elements. Returns 0 when
 // launched, 1 when the shape or alignment is not taken (the caller then runs the

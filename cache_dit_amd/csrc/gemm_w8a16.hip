@@ -368,9 +368,18 @@ __device__ __forceinline__ void mfma_32x32x16_bf16(v16f& acc, const v8bf& w, con
   }
 }
 
-template <class C>
+struct NoGroup {};
+
+// GROUPED: the launch walks the tiles of a GemmGroup as one tile stream, as the w8a8
+// kernel's grouped form does (gemm_fp8.hip): sibling Linears on one activation are members
+// stacked along N, the Linears of the same stage on other activations follow; every member
+// has its own weight, scale, bias, output and epilogue flag, K and the row strides are
+// common (the B-side fields of `g` and grp.a_scale are unused). The instances without it are
+// unchanged by its existence.
+template <class C, bool GROUPED = false>
 __global__ __launch_bounds__(C::THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void
-gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
+gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n,
+                std::conditional_t<GROUPED, GemmGroup, NoGroup> grp) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -381,14 +390,70 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
   constexpr int TM = C::TM, TN = C::TN, H = C::H, A_ROW = C::A_ROW, B_ROW = C::B_ROW;
   constexpr int D = C::DEPTH;
   const int KT = g.K / BKE;  // >= D (checked by the launcher)
-  const int ntiles = tiles_m * tiles_n;
+  int ntiles = tiles_m * tiles_n;
+  if constexpr (GROUPED) ntiles = grp.tile_begin[grp.acts];
 
-  int m0, n0;  // tile being computed
+  // Where a tile lives: for a batch, activation and member are looked up from the linear
+  // tile id (the table sits in the kernel arguments: scalar loads with uniform indices).
+  struct Where {
+    int act, member, m0, n0;
+  };
+  auto locate = [&](int t) -> Where {
+    Where w;
+    if constexpr (GROUPED) {
+      constexpr int kXcd = 8;
+      int id = t;  // ids that run on one XCD are made consecutive, as tile_of_block does
+      if (ntiles % kXcd == 0) id = (t % kXcd) * (ntiles / kXcd) + t / kXcd;
+      int s = 0;
+#pragma unroll
+      for (int i = 1; i < kMaxActs; ++i)
+        if (i < grp.acts && id >= grp.tile_begin[i]) s = i;
+      int tm, tn;
+      tile_of_linear<C::GROUP_M>(id - grp.tile_begin[s], grp.tiles_m[s], grp.tiles_n[s], &tm, &tn);
+      int p = grp.first_member[s];
+      const int p_end = grp.first_member[s + 1];
+#pragma unroll
+      for (int i = 1; i < kMaxGroup; ++i)
+        if (i > p && i < p_end && tn >= grp.col_begin[i]) p = i;
+      w.act = s;
+      w.member = p;
+      w.m0 = tm * C::BM;
+      w.n0 = (tn - grp.col_begin[p]) * C::BN;
+    } else {
+      int tm, tn;
+      tile_of_block<C::GROUP_M>(t, ntiles, tiles_m, tiles_n, &tm, &tn);
+      w.act = 0;
+      w.member = 0;
+      w.m0 = tm * C::BM;
+      w.n0 = tn * C::BN;
+    }
+    return w;
+  };
+  auto a_of = [&](int s) -> const uint8_t* {
+    if constexpr (GROUPED) return static_cast<const uint8_t*>(grp.a[s]);
+    return static_cast<const uint8_t*>(g.a);
+  };
+  auto m_of = [&](int s) -> int {
+    if constexpr (GROUPED) return grp.M[s];
+    return g.M;
+  };
+  auto b_of = [&](int p) -> const uint8_t* {
+    if constexpr (GROUPED) return grp.b[p];
+    return g.b;
+  };
+  auto n_of = [&](int p) -> int {
+    if constexpr (GROUPED) return grp.N[p];
+    return g.N;
+  };
+  int m0, n0;       // tile being computed
+  int cur = 0;      // member it belongs to
+  int cur_act = 0;  // and its activation
   {
-    int tm, tn;
-    tile_of_block<C::GROUP_M>(blockIdx.x, ntiles, tiles_m, tiles_n, &tm, &tn);
-    m0 = tm * C::BM;
-    n0 = tn * C::BN;
+    const Where w = locate(blockIdx.x);
+    cur = w.member;
+    cur_act = w.act;
+    m0 = w.m0;
+    n0 = w.n0;
   }
 
   // DMA source: the tile whose panels the DMA stream currently fetches
@@ -399,10 +464,10 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
   // The lane offsets only depend on the tile through the clamps at the last rows of A
   // and B: between two tiles without partial panels they are not recomputed.
   bool off_clamped = true;  // the first call computes them
-  auto set_source = [&](int sm0, int sn0) {
-    A = static_cast<const uint8_t*>(g.a) + (int64_t)sm0 * g.lda * 2;
-    B = g.b + (int64_t)sn0 * g.ldb;
-    const int rows_a = g.M - sm0, rows_b = g.N - sn0;
+  auto set_source = [&](int sm0, int sn0, int member, int act) {
+    A = a_of(act) + (int64_t)sm0 * g.lda * 2;
+    B = b_of(member) + (int64_t)sn0 * g.ldb;
+    const int rows_a = m_of(act) - sm0, rows_b = n_of(member) - sn0;
     const bool clamped = rows_a < C::BM || rows_b < C::BN;
     if (!clamped && !off_clamped) return;
     off_clamped = clamped;
@@ -421,7 +486,7 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
       off[C::NDA + p] = (uint32_t)min(row, rows_b - 1) * (uint32_t)g.ldb + c * 16;
     }
   };
-  set_source(m0, n0);
+  set_source(m0, n0, cur, cur_act);
   auto dma_a = [&](int kt, int a_lds, int p) {
     const __amdgpu_buffer_rsrc_t rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(A), 0, nrec, 0x00020000);
@@ -496,7 +561,7 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
 
   for (int tile = blockIdx.x;; tile += gridDim.x) {
     const int next_tile = tile + gridDim.x;
-    int nm0 = 0, nn0 = 0;
+    int nm0 = 0, nn0 = 0, next_member = 0, next_act = 0;
     // fragments of step 0 (in LDS since the prologue, or since the barrier of the
     // previous tile's last step)
 #pragma unroll
@@ -515,11 +580,12 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
       if (EVENTS && kt == KT - D) {
         // every DMA of this tile has been issued: the stream moves on
         if (next_tile < ntiles) {
-          int tm, tn;
-          tile_of_block<C::GROUP_M>(next_tile, ntiles, tiles_m, tiles_n, &tm, &tn);
-          nm0 = tm * C::BM;
-          nn0 = tn * C::BN;
-          set_source(nm0, nn0);
+          const Where w = locate(next_tile);
+          next_member = w.member;
+          next_act = w.act;
+          nm0 = w.m0;
+          nn0 = w.n0;
+          set_source(nm0, nn0, next_member, next_act);
         } else {
           nrec = 0;
         }
@@ -529,10 +595,17 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
         // (every wave issues both: equal instruction counts; the same bytes land four
         // times) instead of 6 TN loads per lane at the start of the epilogue. What lies
         // beyond N reads as zero, a null bias is an empty buffer.
+        const float* cur_b_scale = g.b_scale;
+        const uint16_t* cur_bias = g.bias;
+        if constexpr (GROUPED) {
+          cur_b_scale = grp.b_scale[cur];
+          cur_bias = grp.bias[cur];
+        }
+        const int cur_n = n_of(cur);
         const __amdgpu_buffer_rsrc_t bs_buf = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<float*>(g.b_scale), 0, g.N * 4, 0x00020000);
+            const_cast<float*>(cur_b_scale), 0, cur_n * 4, 0x00020000);
         const __amdgpu_buffer_rsrc_t bi_buf = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<uint16_t*>(g.bias), 0, g.bias ? g.N * 2 : 0, 0x00020000);
+            const_cast<uint16_t*>(cur_bias), 0, cur_bias ? cur_n * 2 : 0, 0x00020000);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
             bs_buf, (__attribute__((address_space(3))) void*)(smem + C::EPI_BS), 16,
             n0 * 4 + 16 * lane, 0, 0, 0);
@@ -705,20 +778,29 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
     // hardware drops lanes beyond), lanes whose columns do not exist get an offset
     // beyond any descriptor -- no bounds branches, no 64-bit address arithmetic per store.
     constexpr uint32_t kNoColumn = 0x80000000u;
-    uint8_t* const out_wave = reinterpret_cast<uint8_t*>(g.out) +
-                              ((int64_t)(m0 + wm * C::WM) * g.ldo + (n0 + wn * C::WN)) * 2;
-    const int rows_wave = g.M - (m0 + wm * C::WM);
-    const uint32_t out_lane = ((uint32_t)(lane >> 2) * (uint32_t)g.ldo + 8u * (lane & 3)) * 2;
-    const uint32_t half_block = 16u * (uint32_t)g.ldo * 2;
+    uint16_t* cur_out = g.out;
+    int64_t cur_ldo = g.ldo;
+    int cur_epilogue = g.epilogue;
+    if constexpr (GROUPED) {
+      cur_out = grp.out[cur];
+      cur_ldo = grp.ldo[cur];
+      cur_epilogue = grp.epilogue[cur];
+    }
+    const int cur_N = n_of(cur);
+    uint8_t* const out_wave = reinterpret_cast<uint8_t*>(cur_out) +
+                              ((int64_t)(m0 + wm * C::WM) * cur_ldo + (n0 + wn * C::WN)) * 2;
+    const int rows_wave = m_of(cur_act) - (m0 + wm * C::WM);
+    const uint32_t out_lane = ((uint32_t)(lane >> 2) * (uint32_t)cur_ldo + 8u * (lane & 3)) * 2;
+    const uint32_t half_block = 16u * (uint32_t)cur_ldo * 2;
     uint32_t out_off[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-      out_off[j] = n0 + wn * C::WN + 32 * j + 8 * (lane & 3) < g.N ? out_lane + 64 * j : kNoColumn;
+      out_off[j] = n0 + wn * C::WN + 32 * j + 8 * (lane & 3) < cur_N ? out_lane + 64 * j : kNoColumn;
     uint32_t moved[8];
     auto store_moved = [&](int i, int j) {
       const int rows = __builtin_amdgcn_readfirstlane(min(max(rows_wave - 32 * i, 0), 32));
       const __amdgpu_buffer_rsrc_t block = __builtin_amdgcn_make_buffer_rsrc(
-          out_wave + (int64_t)(32 * i) * g.ldo * 2, 0, rows * g.ldo * 2, 0x00020000);
+          out_wave + (int64_t)(32 * i) * cur_ldo * 2, 0, rows * cur_ldo * 2, 0x00020000);
       __builtin_amdgcn_raw_buffer_store_b128(v4u{moved[0], moved[1], moved[2], moved[3]}, block,
                                              (int)out_off[j], 0, 2);
       __builtin_amdgcn_raw_buffer_store_b128(v4u{moved[4], moved[5], moved[6], moved[7]}, block,
@@ -765,7 +847,7 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
         }
       }
     };
-    if (g.epilogue & CDIT_EPI_GELU_TANH) {
+    if (cur_epilogue & CDIT_EPI_GELU_TANH) {
       epilogue(std::true_type{});
     } else {
       epilogue(std::false_type{});
@@ -774,6 +856,8 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n) {
     if (next_tile >= ntiles) break;
     m0 = nm0;
     n0 = nn0;
+    cur = next_member;
+    cur_act = next_act;
   }
   // the zero-record DMA of the last D steps must not outlive the workgroup
   wait_vm<0>();
@@ -794,7 +878,39 @@ int launch_wide(const GemmArgs& g, hipStream_t stream) {
   const int ntiles = tiles_m * tiles_n;
   // one persistent workgroup per CU (its LDS and registers fill the CU)
   hipLaunchKernelGGL(gemm_w8a16_wide<C>, dim3(ntiles < cus ? ntiles : cus), dim3(C::THREADS),
-                     C::LDS_BYTES, stream, g, tiles_m, tiles_n);
+                     C::LDS_BYTES, stream, g, tiles_m, tiles_n, NoGroup{});
+  return 0;
+}
+
+// A GemmGroup as one launch: the launcher fills the tile tables of the group for this tile
+// shape (grp is a copy).
+template <class C>
+int launch_wide_grouped(const GemmArgs& g, GemmGroup grp, hipStream_t stream) {
+  static bool lds_allowed[64];
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_w8a16_wide<C, true>),
+                                 C::LDS_BYTES, lds_allowed))
+    return rc;
+  const int cus = cu_count();
+  if (cus <= 0) {
+    set_error("cannot query the CU count of the current device");
+    return CDIT_EHIP;
+  }
+  int ntiles = 0;
+  for (int s = 0; s < grp.acts; ++s) {
+    int cols = 0;
+    for (int p = grp.first_member[s]; p < grp.first_member[s + 1]; ++p) {
+      grp.col_begin[p] = cols;
+      cols += (grp.N[p] + C::BN - 1) / C::BN;
+    }
+    grp.tiles_m[s] = (grp.M[s] + C::BM - 1) / C::BM;
+    grp.tiles_n[s] = cols;
+    grp.tile_begin[s] = ntiles;
+    ntiles += grp.tiles_m[s] * cols;
+  }
+  for (int s = grp.acts; s <= kMaxActs; ++s) grp.tile_begin[s] = ntiles;
+  for (int p = grp.count; p <= kMaxGroup; ++p) grp.col_begin[p] = 0x7fffffff;
+  hipLaunchKernelGGL((gemm_w8a16_wide<C, true>), dim3(ntiles < cus ? ntiles : cus), dim3(C::THREADS),
+                     C::LDS_BYTES, stream, g, 0, 0, grp);
   return 0;
 }
 
@@ -1006,6 +1122,44 @@ typedef CfgWW<128, 192, 4, 4> W10;          // wide: 64x96 wave tiles, DMA 4 ste
 typedef CfgWW<128, 128, 4, 5> W11;          // wide: 64x64 wave tiles, DMA 5 steps ahead
 typedef CfgWW<128, 64, 4, 6> W12;           // wide: 64x32 wave tiles, DMA 6 steps ahead
 
+namespace {
+struct TileChoice {
+  int variant;
+  int64_t cost;  // 1000 x CUs x tile area per full round over the CUs (K left out)
+};
+
+// Tile choice for a problem whose tile count for a bm x bn tile is tiles(bm, bn) (one GEMM,
+// or a batch walked as one tile stream). Same cost model as the w8a8 entry point: tile area
+// times rounds over the CUs (one persistent workgroup each), a last partial round of r tiles
+// counting 0.4 + 0.6 r/CUs; both branches count in the same unit.
+template <class Tiles, class WideOk>
+TileChoice choose_variant(Tiles tiles, WideOk wide_ok) {
+  const int64_t cus = cu_count() > 0 ? cu_count() : 256;
+  if (tiles(256, 256) * 256 >= 160 * cus && wide_ok(2)) {
+    auto cost = [&](int bm, int bn, int pen) {
+      const int64_t t = tiles(bm, bn), full = t / cus, rem = t % cus;
+      return (full * 10 * cus + (rem ? 4 * cus + 6 * rem : 0)) * bm * bn * pen;
+    };
+    const int64_t c8 = cost(256, 192, 103), c7 = cost(256, 256, 100);
+    return c8 < c7 ? TileChoice{8, c8} : TileChoice{7, c7};
+  }
+  // Smaller problems: whole rounds over the CUs times tile area, the small tiles
+  // penalised by their measured lower MFMA rate (per mille); ties go to the larger
+  // tile. Tiles whose prefetch depth K cannot feed are left out; without any wide
+  // tile (N not a multiple of 16, very short K) the 128x128 kernel runs.
+  const struct { int v, bm, bn, pen, depth; } cand[] = {
+      {7, 256, 256, 1000, 2}, {8, 256, 192, 1000, 2}, {10, 128, 192, 1300, 4},
+      {11, 128, 128, 1400, 5}, {12, 128, 64, 1700, 6}};
+  TileChoice best = {3, INT64_MAX / 8};  // the 128x128 kernel takes what no wide tile can
+  for (const auto& c : cand) {
+    if (!wide_ok(c.depth)) continue;
+    const int64_t t = (tiles(c.bm, c.bn) + cus - 1) / cus * cus * c.bm * c.bn * c.pen;
+    if (t < best.cost) best = {c.v, t};
+  }
+  return best;
+}
+}  // namespace
+
 int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {
     dim3 grid((g.N + 15) / 16, (g.M + 15) / 16);
@@ -1038,37 +1192,9 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
   // tile (before it, slower waves may still be reading the previous tile's)
   auto wide_ok = [&](int depth) { return g.K >= (depth > 3 ? depth : 3) * BKE && g.N % 16 == 0; };
   if (variant < 0) {
-    // Same cost model as the w8a8 entry point: tile area times rounds over the CUs (one
-    // persistent workgroup each), a last partial round of r tiles counting 0.4 + 0.6 r/CUs.
-    auto tiles = [&](int bm, int bn) {
-      return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
-    };
-    const int64_t cus = cu_count() > 0 ? cu_count() : 256;
-    auto cost = [&](int bm, int bn, int pen) {
-      const int64_t t = tiles(bm, bn), full = t / cus, rem = t % cus;
-      return (full * 10 * cus + (rem ? 4 * cus + 6 * rem : 0)) * bm * bn * pen;
-    };
-    if (tiles(256, 256) * 256 >= 160 * cus && wide_ok(2)) {
-      variant = cost(256, 192, 103) < cost(256, 256, 100) ? 8 : 7;
-    } else {
-      // Smaller problems: whole rounds over the CUs times tile area, the small tiles
-      // penalised by their measured lower MFMA rate (per mille); ties go to the larger
-      // tile. Tiles whose prefetch depth K cannot feed are left out; without any wide
-      // tile (N not a multiple of 16, very short K) the 128x128 kernel runs.
-      const struct { int v, bm, bn, pen, depth; } cand[] = {
-          {7, 256, 256, 1000, 2}, {8, 256, 192, 1000, 2}, {10, 128, 192, 1300, 4},
-          {11, 128, 128, 1400, 5}, {12, 128, 64, 1700, 6}};
-      int64_t best = INT64_MAX;
-      variant = 3;  // the 128x128 kernel takes what no wide tile can
-      for (const auto& c : cand) {
-        if (!wide_ok(c.depth)) continue;
-        const int64_t t = (tiles(c.bm, c.bn) + cus - 1) / cus * c.bm * c.bn * c.pen;
-        if (t < best) {
-          best = t;
-          variant = c.v;
-        }
-      }
-    }
+    variant = choose_variant(
+        [&](int bm, int bn) { return (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn); },
+        wide_ok).variant;
   }
   switch (variant) {
     case 0: return launch_tiled<W0>(g, stream);
@@ -1082,6 +1208,110 @@ int launch_gemm_w8a16(const GemmArgs& g, int variant, hipStream_t stream) {
     default:
       set_error("cdit_w8a16_gemm: unknown kernel variant %d", variant);
       return CDIT_EINVAL;
+  }
+}
+
+// The batch as one launch (or, where the cost model says so, one launch per activation).
+// Returns 0 when launched, -1 when the batch is not taken (the caller then runs the members
+// one by one), a CDIT_E* code on error.
+int launch_gemm_w8a16_grouped(const GemmArgs& common, const GemmGroup& grp, int variant,
+                              hipStream_t stream) {
+  if (grp.count < 2 || grp.count > kMaxGroup || grp.acts < 1 || grp.acts > kMaxActs ||
+      common.out_dtype != CDIT_DT_BF16)
+    return -1;
+  bool n16 = true;
+  for (int s = 0; s < grp.acts; ++s) {
+    if (grp.M[s] <= 16 || grp.first_member[s + 1] <= grp.first_member[s]) return -1;
+    for (int p = grp.first_member[s]; p < grp.first_member[s + 1]; ++p) {
+      GemmArgs g = common;
+      g.a = grp.a[s];
+      g.M = grp.M[s];
+      g.b = grp.b[p];
+      g.b_scale = grp.b_scale[p];
+      g.bias = grp.bias[p];
+      g.out = grp.out[p];
+      g.N = grp.N[p];
+      g.ldo = grp.ldo[p];
+      if (!tiled_ok(g) || g.N <= 0) return -1;
+      n16 = n16 && g.N % 16 == 0;
+    }
+  }
+  auto wide_ok = [&](int depth) { return common.K >= (depth > 3 ? depth : 3) * BKE && n16; };
+  auto tiles = [&](int bm, int bn) {
+    int64_t t = 0;
+    for (int s = 0; s < grp.acts; ++s) {
+      int64_t cols = 0;
+      for (int p = grp.first_member[s]; p < grp.first_member[s + 1]; ++p) cols += (grp.N[p] + bn - 1) / bn;
+      t += (int64_t)((grp.M[s] + bm - 1) / bm) * cols;
+    }
+    return t;
+  };
+  if (variant < 0) {
+    const TileChoice whole = choose_variant(tiles, wide_ok);
+    variant = whole.variant;
+    if (grp.acts > 1) {
+      // one tile stream against one launch per activation, as in the w8a8 launcher: a small
+      // activation can push a batch that filled whole rounds into one more, nearly empty one
+      // (a further launch costs about 3 us; a CU does about 2450 K elements of one output
+      // element per us at the bf16 rate)
+      const int64_t cus = cu_count() > 0 ? cu_count() : 256;
+      int64_t apart = (grp.acts - 1) * (3 * 1000 * cus * 2450 / (common.K > 0 ? common.K : 1));
+      for (int s = 0; s < grp.acts; ++s) {
+        auto tiles_s = [&](int bm, int bn) {
+          int64_t cols = 0;
+          for (int p = grp.first_member[s]; p < grp.first_member[s + 1]; ++p) cols += (grp.N[p] + bn - 1) / bn;
+          return (int64_t)((grp.M[s] + bm - 1) / bm) * cols;
+        };
+        apart += choose_variant(tiles_s, wide_ok).cost;
+      }
+      if (apart * 100 < whole.cost * 97) {
+        for (int s = 0; s < grp.acts; ++s) {
+          GemmGroup one = {};
+          one.acts = 1;
+          one.count = grp.first_member[s + 1] - grp.first_member[s];
+          one.a[0] = grp.a[s];
+          one.M[0] = grp.M[s];
+          one.first_member[0] = 0;
+          one.first_member[1] = one.count;
+          for (int p = 0; p < one.count; ++p) {
+            const int src = grp.first_member[s] + p;
+            one.b[p] = grp.b[src];
+            one.b_scale[p] = grp.b_scale[src];
+            one.bias[p] = grp.bias[src];
+            one.out[p] = grp.out[src];
+            one.N[p] = grp.N[src];
+            one.ldo[p] = grp.ldo[src];
+            one.epilogue[p] = grp.epilogue[src];
+          }
+          int rc = one.count >= 2 ? launch_gemm_w8a16_grouped(common, one, -1, stream) : -1;
+          if (rc > 0) return rc;
+          if (rc == 0) continue;
+          for (int p = 0; p < one.count; ++p) {  // a single member, or a group that is not taken
+            GemmArgs g = common;
+            g.a = one.a[0];
+            g.M = one.M[0];
+            g.b = one.b[p];
+            g.b_scale = one.b_scale[p];
+            g.bias = one.bias[p];
+            g.out = one.out[p];
+            g.N = one.N[p];
+            g.ldo = one.ldo[p];
+            g.epilogue = one.epilogue[p];
+            if ((rc = launch_gemm_w8a16(g, -1, stream))) return rc;
+          }
+        }
+        return 0;
+      }
+    }
+  }
+  switch (variant) {
+    case 7: return wide_ok(W7::DEPTH) ? launch_wide_grouped<W7>(common, grp, stream) : -1;
+    case 8: return wide_ok(W8::DEPTH) ? launch_wide_grouped<W8>(common, grp, stream) : -1;
+    case 9: return wide_ok(W9::DEPTH) ? launch_wide_grouped<W9>(common, grp, stream) : -1;
+    case 10: return wide_ok(W10::DEPTH) ? launch_wide_grouped<W10>(common, grp, stream) : -1;
+    case 11: return wide_ok(W11::DEPTH) ? launch_wide_grouped<W11>(common, grp, stream) : -1;
+    case 12: return wide_ok(W12::DEPTH) ? launch_wide_grouped<W12>(common, grp, stream) : -1;
+    default: return -1;  // the kernels without a tile stream have no grouped form
   }
 }
 

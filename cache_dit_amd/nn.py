@@ -82,7 +82,8 @@ class _InputKey:
 
 
 class SiblingGroup:
-  """Two to four `float8_per_row` Linears that are handed the very same activation one
+  """Two to eight `float8_per_row` Linears (or `float8_weight_only` ones, which skip the
+  quantization) that are handed the very same activation one
   after the other (attn.to_q / to_k / to_v; proj_mlp + q/k/v in FLUX single blocks;
   reference dataflow src/cache_dit/caching/patch_functors/functor_flux.py:60-67). The
   first member called with an activation quantizes it once and computes every member's
@@ -96,11 +97,14 @@ class SiblingGroup:
     if not 2 <= len(members) <= _native.MAX_GROUP:
       raise ValueError(f"a sibling group holds 2 to {_native.MAX_GROUP} Linears, got {len(members)}")
     first = members[0]
+    if type(first) not in (Fp8DynamicLinear, Fp8WeightOnlyLinear):
+      raise TypeError("sibling groups are built from float8_per_row or float8_weight_only Linears")
     for m in members:
-      if type(m) is not Fp8DynamicLinear:
-        raise TypeError("sibling groups are built from float8_per_row Linears")
+      if type(m) is not type(first):
+        raise TypeError("the members of a sibling group must be of one quant type")
       if m.in_features != first.in_features or m._scale_mode_id != first._scale_mode_id:
         raise ValueError("the members of a sibling group must share in_features and scale mode")
+    self.weight_only = type(first) is Fp8WeightOnlyLinear
     self.members = members
     self.index = {id(m): i for i, m in enumerate(members)}
     self.key = None  # _InputKey of the activation the pending outputs were computed from
@@ -121,7 +125,10 @@ class SiblingGroup:
     M = x2.shape[0]
     members = self.members
     outs = [torch.empty((M, m.out_features), dtype=torch.bfloat16, device=x2.device) for m in members]
-    if M > 0:
+    if M > 0 and self.weight_only:
+      ops.w8a16_batched_into([(x2, [m.weight for m in members], [m.weight_scale for m in members],
+                               [m.bias for m in members], outs, [m.epilogue for m in members])])
+    elif M > 0:
       q, s = ops.shared_activation_quant(x2, lin._scale_mode_id)
       ops.gemm_rowwise_grouped_into(q, s, [m.weight for m in members],
                                     [m.weight_scale for m in members], [m.bias for m in members],
@@ -196,8 +203,15 @@ class Fp8WeightOnlyLinear(_Fp8LinearBase):
   """`float8_weight_only` (w8a16): bf16 activations, e4m3 weights dequantized in
   the GEMM mainloop, per-channel scale in the epilogue."""
 
+  sibling_group: Optional[SiblingGroup] = None
+
   def forward(self, x: torch.Tensor) -> torch.Tensor:
     self._check_input(x)
+    if not torch.compiler.is_compiling() and not x.is_inference():  # as in Fp8DynamicLinear
+      if _recorder is not None:
+        _recorder.note(self, x)
+      if self.sibling_group is not None:
+        return self.sibling_group.forward_member(self, x)
     return torch.ops.cdit.w8a16_mm(x, self.weight.t(), self.weight_scale, self.bias,
                                    _native.DT_BF16, self.epilogue)
 
@@ -275,21 +289,23 @@ def share_activation_quant_(module: nn.Module, enable: bool = True) -> int:
 
 
 def group_sibling_linears_(module: nn.Module, run=None, enable: bool = True) -> int:
-  """Finds the `float8_per_row` Linears under `module` that are called back to back with
-  the very same activation and lets each such run (two to four Linears) compute its
-  outputs in one grouped GEMM launch on one shared quantization (SiblingGroup). `run` is a
+  """Finds the `float8_per_row` (or `float8_weight_only`) Linears under `module` that are
+  called back to back with the very same activation and lets each such run (two to eight
+  Linears of one quant type) compute its outputs in one grouped GEMM launch, for
+  `float8_per_row` on one shared quantization (SiblingGroup). `run` is a
   callable that performs one forward of the model (e.g. `lambda: model(**inputs)`); it is
   executed once under torch.no_grad() to observe the calls. Returns the number of groups
   formed. enable=False removes every group under `module` (no `run` needed)."""
   global _recorder
+  groupable = (Fp8DynamicLinear, Fp8WeightOnlyLinear)
   for m in module.modules():
-    if isinstance(m, Fp8DynamicLinear):
+    if type(m) in groupable:
       m.sibling_group = None
   if not enable:
     return 0
   if run is None:
     raise ValueError("group_sibling_linears_ needs `run`, a callable doing one forward")
-  mine = {id(m) for m in module.modules() if isinstance(m, Fp8DynamicLinear)}
+  mine = {id(m) for m in module.modules() if type(m) in groupable}
   _recorder = rec = _SiblingRecorder()
   try:
     with torch.no_grad():
@@ -298,9 +314,10 @@ def group_sibling_linears_(module: nn.Module, run=None, enable: bool = True) -> 
     _recorder = None
   groups = 0
   for siblings in rec.runs:
-    siblings = [m for m in siblings if id(m) in mine and type(m) is Fp8DynamicLinear
+    siblings = [m for m in siblings if id(m) in mine and type(m) in groupable
                 and m.sibling_group is None]
-    siblings = [m for m in siblings if m.in_features == siblings[0].in_features
+    siblings = [m for m in siblings if type(m) is type(siblings[0])
+                and m.in_features == siblings[0].in_features
                 and m._scale_mode_id == siblings[0]._scale_mode_id]
     while len(siblings) >= 2:
       take, siblings = siblings[:_native.MAX_GROUP], siblings[_native.MAX_GROUP:]
@@ -318,13 +335,15 @@ def linear_batch(pairs):
   text-stream projections of the same stage, e.g. [(hidden, [to_q, to_k, to_v]),
   (encoder, [add_q_proj, add_k_proj, add_v_proj])]). Returns the outputs in the same
   nesting, bit-identical to calling the Linears one by one. For block forwards that are
-  written against this package; Linears that are not `float8_per_row` ones, a compiled
-  graph, or inference-mode tensors simply run one by one."""
+  written against this package; `float8_per_row` Linears (one quantizer launch for the
+  stage as well) or `float8_weight_only` ones; other Linears, mixed types, a compiled graph
+  or inference-mode tensors simply run one by one."""
   flat = [lin for _, lins in pairs for lin in lins]
   first = flat[0]
   plain = (torch.compiler.is_compiling() or len(flat) > _native.MAX_GROUP
            or len(pairs) > _native.MAX_ACTS
-           or any(type(lin) is not Fp8DynamicLinear or lin.in_features != first.in_features
+           or type(first) not in (Fp8DynamicLinear, Fp8WeightOnlyLinear)
+           or any(type(lin) is not type(first) or lin.in_features != first.in_features
                   or lin._scale_mode_id != first._scale_mode_id for lin in flat)
            or any(x.is_inference() or not x.is_cuda or x.dtype != torch.bfloat16 for x, _ in pairs))
   if plain:
@@ -340,7 +359,9 @@ def linear_batch(pairs):
     rows.append(x2)
     acts.append([None, None, [lin.weight for lin in lins], [lin.weight_scale for lin in lins],
                  [lin.bias for lin in lins], outs, [lin.epilogue for lin in lins]])
-  if acts:
+  if acts and type(first) is Fp8WeightOnlyLinear:
+    ops.w8a16_batched_into([(x2, *act[2:]) for x2, act in zip(rows, acts)])
+  elif acts:
     # one quantizer launch for the activations the cache does not hold, one GEMM launch
     for act, (q, s) in zip(acts, ops.shared_activation_quant_many(rows, first._scale_mode_id)):
       act[0], act[1] = q, s

@@ -204,6 +204,43 @@ def gemm_rowwise_batched_into(acts) -> None:
         (i64 * n)(*[o.stride(0) for o in outs]), (ci * n)(*[int(e) for e in epis]), _stream_ptr(a0)))
 
 
+def w8a16_batched_into(acts) -> None:
+  """Independent weight-only GEMMs of one stage as one launch. `acts` is a list of
+  (x2 [M,K] bf16, weights, w_scales, biases, outs, epilogues): one entry per activation, its
+  members e4m3 [N_p,K] weights with a common row stride, fp32 scales, bf16 biases or None,
+  bf16 outputs [M,N_p] and epilogue flags. Activations whose row strides differ are
+  launched apart. Bit-identical to one w8a16_into per member."""
+  import ctypes
+  vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+  x0 = acts[0][0]
+  if any(t[0].stride(0) != x0.stride(0) for t in acts[1:]):
+    for t in acts:
+      w8a16_batched_into([t])
+    return
+  K, lda, ldb = x0.shape[1], x0.stride(0), acts[0][1][0].stride(0)
+  ws, wss, bs, outs, epis, per_act = [], [], [], [], [], []
+  for x, weights, w_scales, biases, o, e in acts:
+    if x.shape[1] != K or x.device != x0.device or x.dtype != torch.bfloat16 or x.stride(1) != 1:
+      raise ValueError("w8a16_batched_into: the activations must be bf16 rows of one K on one device")
+    if any(w.stride(0) != ldb or w.shape[1] != K for w in weights):
+      raise ValueError("w8a16_batched_into: the weights must share K and the row stride")
+    ws += weights
+    wss += w_scales
+    bs += biases
+    outs += o
+    epis += e
+    per_act.append(len(weights))
+  n, na = len(ws), len(acts)
+  with _DeviceOf(x0):
+    _native.check(_native.load().cdit_w8a16_gemm_batched(
+        na, (vp * na)(*[t[0].data_ptr() for t in acts]), (i64 * na)(*[t[0].shape[0] for t in acts]),
+        K, lda, (ci * na)(*per_act), (vp * n)(*[w.data_ptr() for w in ws]),
+        (vp * n)(*[s.data_ptr() for s in wss]),
+        (vp * n)(*[b.data_ptr() if b is not None else None for b in bs]),
+        (vp * n)(*[o.data_ptr() for o in outs]), (i64 * n)(*[w.shape[0] for w in ws]), ldb,
+        (i64 * n)(*[o.stride(0) for o in outs]), (ci * n)(*[int(e) for e in epis]), _stream_ptr(x0)))
+
+
 def w8a16_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
                bias: Optional[torch.Tensor], out: torch.Tensor, epilogue: int) -> None:
   M, K = x2.shape

@@ -241,6 +241,25 @@ int cdit_w8a16_gemm(const void* x_bf16, const void* b_q, const float* b_scale,
                     int epilogue, int out_dtype_id, void* stream);
 
 /*
+ * cdit_w8a16_gemm for the Linears of one stage as one launch: up to 4 activations
+ * (x_bf16[s] bf16 [M[s], K], common lda) with members_per_act[s] weight-only Linears each, up to
+ * 8 members in all, listed activation by activation (member p: b_q[p] e4m3 [N[p], K] with the
+ * common ldb, b_scale[p], bias[p] bf16 or NULL, out[p] bf16 [M, N[p]] with ldo[p], epilogue[p]).
+ * The weight-only counterpart of cdit_fp8_gemm_rowwise_batched: sibling Linears that read one
+ * activation (attn.to_q / to_k / to_v, proj_mlp next to them; reference dataflow
+ * src/cache_dit/caching/patch_functors/functor_flux.py:60-67) and the same stage of the other
+ * stream of a double-stream block, which the reference runs as one `F.linear` on a dequantized
+ * weight each (Float8WeightOnlyConfig, src/cache_dit/quantization/torchao/quantize_ao.py:604-610).
+ * Bit-identical to one cdit_w8a16_gemm call per member; what the tile stream does not take
+ * (M <= 16, N not a multiple of 16, a single member) runs as those calls.
+ */
+int cdit_w8a16_gemm_batched(int n_act, const void* const* x_bf16, const int64_t* M, int64_t K,
+                            int64_t lda, const int* members_per_act, const void* const* b_q,
+                            const float* const* b_scale, const void* const* bias,
+                            void* const* out, const int64_t* N, int64_t ldb, const int64_t* ldo,
+                            const int* epilogue, void* stream);
+
+/*
  * One quantized nn.Linear forward in the w8a8 dynamic mode: the two calls above
  * back to back on `stream` (per-token quantization of x into the caller's
  * workspace, then the scaled GEMM), saving one trip through the caller's FFI;

@@ -296,3 +296,162 @@ def test_very_large_output_stride_takes_a_kernel_with_64_bit_offsets():
     ref = to.w8a16_linear(x.cpu(), w.cpu(), sw.cpu().reshape(-1, 1), None, fused=True)
     assert torch.equal(buf[:, :N].cpu(), ref)
     assert bool((buf[:, N:] == -7.0).all())
+
+
+def _stage(spec, seed, integer=False):
+  """spec: list of (M, K, [N...], [epilogue...]). Returns the `acts` list of
+  ops.w8a16_batched_into with NaN-filled outputs."""
+  acts = []
+  for s, (M, K, Ns, epis) in enumerate(spec):
+    g = torch.Generator(device="cuda").manual_seed(seed + 17 * s)
+    if integer:
+      x = torch.randint(-3, 4, (M, K), generator=g, device="cuda").to(torch.bfloat16)
+    else:
+      x = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
+    ws, wss, bs = [], [], []
+    for i, N in enumerate(Ns):
+      if integer:
+        ws.append(torch.randint(-3, 4, (N, K), generator=g, device="cuda").float().to(FP8))
+        wss.append(torch.full((N,), 0.25, device="cuda"))
+        b = torch.randint(-8, 9, (N,), generator=g, device="cuda").float().to(torch.bfloat16)
+      else:
+        ws.append(torch.randn(N, K, generator=g, device="cuda").to(FP8))
+        wss.append(torch.rand(N, generator=g, device="cuda") * 0.01 + 0.001)
+        b = (torch.randn(N, generator=g, device="cuda") * 0.1).to(torch.bfloat16)
+      bs.append(None if i == 1 else b)
+    outs = [torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda") for N in Ns]
+    acts.append((x, ws, wss, bs, outs, list(epis)))
+  return acts
+
+
+def _one_by_one(x, ws, wss, bs, epis):
+  from cache_dit_amd import ops
+  outs = []
+  for w, s, b, e in zip(ws, wss, bs, epis):
+    o = torch.empty((x.shape[0], w.shape[0]), dtype=torch.bfloat16, device="cuda")
+    ops.w8a16_into(x, w, s, b, o, e)
+    outs.append(o)
+  return outs
+
+
+@pytest.mark.parametrize("spec", [
+    # FLUX single block: proj_mlp (GELU) + q/k/v on one activation
+    [(4608, 3072, [12288, 3072, 3072, 3072], [1, 0, 0, 0])],
+    # FLUX double block, stage by stage: image stream (4096 tokens) + text stream (512 tokens)
+    [(4096, 3072, [3072] * 3, [0] * 3), (512, 3072, [3072] * 3, [0] * 3)],
+    [(4096, 3072, [3072], [0]), (512, 3072, [3072], [0])],
+    [(4096, 3072, [12288], [1]), (512, 3072, [12288], [1])],
+    [(4096, 12288, [3072], [0]), (512, 12288, [3072], [0])],
+    # ragged everything, three activations
+    [(300, 512, [528, 272], [0, 1]), (77, 512, [80], [0]), (1000, 512, [144, 16, 208], [1, 0, 0])],
+    # what the tile stream does not take runs as single calls: N not a multiple of 16, M <= 16
+    [(300, 512, [520, 264], [0, 0])],
+    [(300, 512, [528], [0]), (9, 512, [272], [0])],
+])
+def test_batched_equals_one_launch_per_member(spec):
+  from cache_dit_amd import ops
+  acts = _stage(spec, seed=spec[0][0])
+  ops.w8a16_batched_into(acts)
+  torch.cuda.synchronize()
+  for s, (x, ws, wss, bs, outs, epis) in enumerate(acts):
+    want = _one_by_one(x, ws, wss, bs, epis)
+    for p, (g, w) in enumerate(zip(outs, want)):
+      assert torch.equal(g.view(torch.int16), w.view(torch.int16)), f"activation {s} member {p}"
+
+
+@pytest.mark.parametrize("variant", [7, 8, 9, 10, 11, 12])
+def test_batched_every_tile_shape_exact_integers_against_the_oracle(variant):
+  from cache_dit_amd import _native, ops
+  spec = [(2100, 640, [1104, 528], [0, 0]), (333, 640, [3088], [0]), (40, 640, [272, 80], [0, 0])]
+  acts = _stage(spec, seed=variant, integer=True)
+  _native.set_gemm_variant(variant)
+  ops.w8a16_batched_into(acts)
+  torch.cuda.synchronize()
+  for s, (x, ws, wss, bs, outs, epis) in enumerate(acts):
+    for p, (w, sc, b, o) in enumerate(zip(ws, wss, bs, outs)):
+      ref = to.w8a16_linear(x.cpu(), w.cpu(), sc.cpu(), None if b is None else b.cpu(), fused=True)
+      assert torch.equal(o.cpu().view(torch.int16), ref.view(torch.int16)), (variant, s, p)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_batched_random_shapes_exact_against_the_oracle(seed):
+  """Randomly drawn batches (1 to 4 activations of 17 to 700 rows, 1 to 3 members each with N
+  a multiple of 16 up to 608, K of 3 to 8 steps of 64, a randomly forced tile shape or the
+  automatic choice) on integer-valued data: bit-equal to the CPU oracle, nothing written
+  outside the outputs (windows of sentinel-filled buffers)."""
+  import random
+  from cache_dit_amd import _native, ops
+  rnd = random.Random(seed)
+  K = 64 * rnd.randint(6, 16)
+  n_act = rnd.randint(1, 4)
+  budget = 8
+  acts, bufs = [], []
+  for s in range(n_act):
+    M = rnd.choice([17, 33, 64, 100, 255, 256, 257, 300, 511, 700])
+    n_mem = rnd.randint(1, min(3, budget - (n_act - s - 1)))
+    budget -= n_mem
+    Ns = [16 * rnd.randint(1, 38) for _ in range(n_mem)]
+    (x, ws, wss, bs, _, _), = _stage([(M, K, Ns, [0] * n_mem)], seed=1000 * seed + s, integer=True)
+    outs = []
+    for N in Ns:
+      buf = torch.full((M + 1, N + 8), 7.0, dtype=torch.bfloat16, device="cuda")
+      bufs.append((buf, M, N))
+      outs.append(buf[:M, :N])
+    acts.append((x, ws, wss, bs, outs, [0] * n_mem))
+  variant = rnd.choice([-1, -1, 7, 8, 9, 10, 11, 12])
+  _native.set_gemm_variant(variant)
+  ops.w8a16_batched_into(acts)
+  torch.cuda.synchronize()
+  for s, (x, ws, wss, bs, outs, epis) in enumerate(acts):
+    for p, (w, sc, b, o) in enumerate(zip(ws, wss, bs, outs)):
+      ref = to.w8a16_linear(x.cpu(), w.cpu(), sc.cpu(), None if b is None else b.cpu(), fused=True)
+      assert torch.equal(o.cpu().view(torch.int16), ref.view(torch.int16)), (seed, variant, s, p)
+  for buf, M, N in bufs:
+    assert (buf[M] == 7.0).all() and (buf[:, N:] == 7.0).all(), (seed, variant)
+
+
+def test_weight_only_sibling_groups_and_stream_batches_in_a_model():
+  """float8_weight_only model: group_sibling_linears_ and the stream-batched block forwards
+  give the bits of the plain forwards, eager and under graph capture."""
+  import logging
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd.testing import dit_shapes as ds
+  logging.getLogger("CACHE_DIT_AMD").setLevel(logging.WARNING)
+  torch.manual_seed(0)
+  kw = dict(dim=512, heads=4, mlp=2048, n_double=2, n_single=3, in_channels=64, text_dim=256,
+            pooled_dim=128)
+  model = ds.FluxLikeTransformer(**kw).to(torch.bfloat16).cuda()
+  cache_dit.quantize(model, cache_dit.QuantizeConfig(quant_type="float8_weight_only"))
+  ds.fuse_gelu_epilogues(model)
+  inputs = ds.flux_like_inputs("cuda", n_img=320, n_txt=64, in_channels=64, text_dim=256,
+                               pooled_dim=128)
+  with torch.no_grad():
+    y0 = model(**inputs)
+    assert cache_dit.group_sibling_linears_(model, lambda: model(**inputs)) == 2 * 2 + 3 * 1
+    blk = model.single_transformer_blocks[0]
+    assert len(blk.proj_mlp.sibling_group.members) == 4 and blk.proj_mlp.sibling_group.weight_only
+    assert torch.equal(model(**inputs), y0)
+    assert ds.batch_streams(model) == 2
+    assert torch.equal(model(**inputs), y0)
+    static = {k: v.clone() for k, v in inputs.items()}
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+      model(**static)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+      ys = model(**static)
+    other = ds.flux_like_inputs("cuda", n_img=320, n_txt=64, in_channels=64, text_dim=256,
+                                pooled_dim=128, seed=5)
+    for src in (other, inputs):
+      want = model(**src)
+      torch.cuda.synchronize()
+      for k in static:
+        static[k].copy_(src[k])
+      graph.replay()
+      torch.cuda.synchronize()
+      assert torch.equal(ys, want)
+    ds.batch_streams(model, False)
+    assert cache_dit.group_sibling_linears_(model, enable=False) == 0
+    assert torch.equal(model(**inputs), y0)
