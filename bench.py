@@ -595,6 +595,7 @@ def dit_forward_ms(device, iters=5):
   inputs = flux_like_inputs(device)
   cache_dit_amd.group_sibling_linears_(model, lambda: model(**inputs))
   dit_shapes.batch_streams(model)
+  dit_shapes.fuse_cat_quant(model)
   dit_shapes.fuse_norm_quant(model, materialize=False)
   graph_ms = None
   with torch.no_grad():
@@ -621,7 +622,7 @@ def dit_forward_ms(device, iters=5):
   return ms, graph_ms, ("float8_per_row, GELU-tanh fused into the producing Linear, sibling Linears "
                         "grouped on one shared quantization, image- and text-stream Linears of a "
                         "stage batched into one launch, quantizer fused into the modulated "
-                        "LayerNorms; bf16 SDPA attention, RMS norms, RoPE and residual glue in eager "
+                        "LayerNorms and reading proj_out's two sources in place; bf16 SDPA attention, RMS norms, RoPE and residual glue in eager "
                         "PyTorch ops" + note_err)
 
 

@@ -23,6 +23,7 @@ from .nn import fuse_gelu_tanh_
 from .nn import share_activation_quant_
 from .nn import group_sibling_linears_
 from .nn import linear_batch
+from .nn import linear_on_cat
 from .ops import ln_modulate_quant
 from .utils import check_quantized
 
@@ -44,5 +45,6 @@ __all__ = [
     "share_activation_quant_",
     "group_sibling_linears_",
     "linear_batch",
+    "linear_on_cat",
     "ln_modulate_quant",
 ]

@@ -33,6 +33,7 @@ EXPORTS = (
     "cdit_device_arch",
     "cdit_fp8_quant_rowwise",
     "cdit_fp8_quant_rowwise_batched",
+    "cdit_fp8_quant_rowwise_cat2",
     "cdit_fp8_quant_tensorwise",
     "cdit_fp8_ln_modulate_quant",
     "cdit_fp8_gemm_rowwise",
@@ -75,6 +76,8 @@ def _bind(L: ctypes.CDLL) -> None:
   L.cdit_debug_set_quant_hints.argtypes = [ci]
   L.cdit_fp8_quant_rowwise.restype = ci
   L.cdit_fp8_quant_rowwise.argtypes = [vp, i64, i64, i64, vp, i64, vp, ci, vp]
+  L.cdit_fp8_quant_rowwise_cat2.restype = ci
+  L.cdit_fp8_quant_rowwise_cat2.argtypes = [vp, i64, i64, vp, i64, i64, i64, vp, i64, vp, ci, vp]
   L.cdit_fp8_quant_rowwise_batched.restype = ci
   L.cdit_fp8_quant_rowwise_batched.argtypes = [ci, vp, vp, i64, vp, vp, vp, vp, ci, vp]
   L.cdit_fp8_ln_modulate_quant.restype = ci

@@ -200,6 +200,43 @@ int cdit_fp8_quant_rowwise(const void* x_bf16, int64_t M, int64_t K, int64_t ld_
                            scale_mode, stream, false);
 }
 
+int cdit_fp8_quant_rowwise_cat2(const void* x1_bf16, int64_t K1, int64_t ld_x1,
+                                const void* x2_bf16, int64_t K2, int64_t ld_x2, int64_t M,
+                                void* q_e4m3, int64_t ld_q, float* scale, int scale_mode,
+                                void* stream) {
+  const char* fn = "cdit_fp8_quant_rowwise_cat2";
+  const int mode = scale_mode >= 0 ? scale_mode & ~CDIT_QUANT_GEMM_FOLLOWS : scale_mode;
+  if (M < 0 || K1 <= 0 || K2 <= 0 || M > INT32_MAX || K1 + K2 > INT32_MAX) {
+    set_error("%s: bad shape M=%lld K1=%lld K2=%lld", fn, (long long)M, (long long)K1, (long long)K2);
+    return CDIT_EINVAL;
+  }
+  if (mode != CDIT_SCALE_BF16DIV && mode != CDIT_SCALE_FP32DIV) {
+    set_error("%s: unknown scale_mode %d", fn, scale_mode);
+    return CDIT_EINVAL;
+  }
+  if (M == 0) return CDIT_OK;
+  if (ld_x1 < K1 || ld_x2 < K2 || ld_q < K1 + K2) {
+    set_error("%s: leading dimension smaller than the row (ld_x1=%lld ld_x2=%lld ld_q=%lld)", fn,
+              (long long)ld_x1, (long long)ld_x2, (long long)ld_q);
+    return CDIT_EINVAL;
+  }
+  if (!x1_bf16 || !x2_bf16 || !q_e4m3 || !scale) {
+    set_error("%s: null pointer argument", fn);
+    return CDIT_EINVAL;
+  }
+  int rc = check_arch();
+  if (rc) return rc;
+  if (cdit::launch_quant_rowwise_cat2(x1_bf16, K1, ld_x1, x2_bf16, K2, ld_x2, M, q_e4m3, ld_q, scale,
+                                      mode, static_cast<hipStream_t>(stream)) != 0) {
+    set_error("%s: K1 and K2 must be multiples of 8 with K1 + K2 <= 16384, rows 16-byte aligned "
+              "(K1=%lld K2=%lld ld_x1=%lld ld_x2=%lld ld_q=%lld): concatenate and call "
+              "cdit_fp8_quant_rowwise instead", fn, (long long)K1, (long long)K2, (long long)ld_x1,
+              (long long)ld_x2, (long long)ld_q);
+    return CDIT_EINVAL;
+  }
+  return after_launch(fn);
+}
+
 int cdit_fp8_quant_rowwise_batched(int n_act, const void* const* x_bf16, const int64_t* M,
                                    int64_t K, const int64_t* ld_x, void* const* q_e4m3,
                                    const int64_t* ld_q, float* const* scale, int scale_mode,

@@ -32,6 +32,11 @@ struct QuantBatch {
 // launches the activations one by one.
 int launch_quant_rowwise_batched(const QuantBatch& batch, int64_t K, int scale_mode,
                                  hipStream_t stream);
+// Rows that are the concatenation [x1 | x2] of two sources quantized as one row. 0: launched;
+// 1: not taken (alignment, K1 + K2 beyond the register-resident kernel).
+int launch_quant_rowwise_cat2(const void* x1, int64_t K1, int64_t ld_x1, const void* x2, int64_t K2,
+                              int64_t ld_x2, int64_t M, void* q, int64_t ld_q, float* scale,
+                              int scale_mode, hipStream_t stream);
 
 int launch_quant_tensorwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void* q,
                             int64_t ld_q, float* scale, uint32_t* amax_ws, int scale_mode,

@@ -123,6 +123,62 @@ __global__ __launch_bounds__(64) void quant_rowwise_regs(
   }
 }
 
+// The regs kernel on a row that is the concatenation of two source rows, [x1 | x2]: the
+// input of FLUX single blocks' proj_out is torch.cat([attn_output, mlp_hidden_states], dim=2)
+// (reference dataflow src/cache_dit/caching/patch_functors/functor_flux.py:68-80), read by
+// that quantized Linear only -- quantizing the two sources in place of their copy saves the
+// copy's write and the quantizer's read of it. n1 = chunks (8 elements) of x1 per row; the
+// codes go to one [M, K1 + K2] buffer and are those of the quantizer on the concatenation.
+template <int CH, bool NT_LOAD>
+__global__ __launch_bounds__(64) void quant_rowwise_cat_regs(
+    const uint16_t* __restrict__ x1, int64_t ld_x1, int n1, const uint16_t* __restrict__ x2,
+    int64_t ld_x2, uint8_t* __restrict__ q, int64_t ld_q, float* __restrict__ scale, int M, int K,
+    int scale_mode) {
+  const int lane = threadIdx.x & 63;
+  const int nchunks = K >> 3;
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+    const uint4* r1 = reinterpret_cast<const uint4*>(x1 + row * ld_x1);
+    const uint4* r2 = reinterpret_cast<const uint4*>(x2 + row * ld_x2) - n1;
+    auto load = [&](int idx) -> uint4 {
+      const uint4* src = (idx < n1 ? r1 : r2) + idx;
+      if constexpr (NT_LOAD) {
+        typedef unsigned int u4v __attribute__((ext_vector_type(4)));
+        const u4v t = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(src));
+        return make_uint4(t[0], t[1], t[2], t[3]);
+      } else {
+        return *src;
+      }
+    };
+    uint4 v[CH];
+    uint32_t m = 0;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int idx = c * 64 + lane;
+      v[c] = idx < nchunks ? load(idx) : make_uint4(0, 0, 0, 0);
+      m = absmax2(absmax2(absmax2(absmax2(m, v[c].x), v[c].y), v[c].z), v[c].w);
+    }
+    m = wave_max_u32(fold2(m));
+    const float s = row_scale(m, scale_mode);
+    if (lane == 0) scale[row] = s;
+    uint2* qr = reinterpret_cast<uint2*>(q + row * ld_q);
+    if (scale_in_fast_window(s)) {  // wave-uniform
+      const float r = 1.0f / s;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int idx = c * 64 + lane;
+        if (idx < nchunks)
+          qr[idx] = uint2{quant4<true>(v[c].x, v[c].y, s, r), quant4<true>(v[c].z, v[c].w, s, r)};
+      }
+    } else {  // cold path: re-reads the row
+#pragma unroll 1
+      for (int idx = lane; idx < nchunks; idx += 64) {
+        const uint4 w = load(idx);
+        qr[idx] = uint2{quant4<false>(w.x, w.y, s, 0.0f), quant4<false>(w.z, w.w, s, 0.0f)};
+      }
+    }
+  }
+}
+
 // Any K, any alignment: one wavefront per row, two passes over the row with
 // element-wise loads (the second pass hits L2). Slow path for odd shapes.
 __global__ __launch_bounds__(64) void quant_rowwise_generic(
@@ -466,6 +522,50 @@ int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void
   hipLaunchKernelGGL(quant_rowwise_generic, grid, block, 0, stream, xp, ld_x, qp, ld_q, scale, Mi,
                      Ki, scale_mode);
   return 0;
+}
+
+// 0: launched; 1: not taken (K1 or K2 not a multiple of 8, rows not 16-byte aligned,
+// K1 + K2 beyond the register-resident kernel).
+int launch_quant_rowwise_cat2(const void* x1, int64_t K1, int64_t ld_x1, const void* x2, int64_t K2,
+                              int64_t ld_x2, int64_t M, void* q, int64_t ld_q, float* scale,
+                              int scale_mode, hipStream_t stream) {
+  const int64_t K = K1 + K2;
+  const bool aligned = K1 % 8 == 0 && K2 % 8 == 0 && K <= 32 * 512 && ld_x1 % 8 == 0 && ld_x2 % 8 == 0 &&
+                       ld_q % 8 == 0 && reinterpret_cast<uintptr_t>(x1) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(x2) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(q) % 8 == 0;
+  if (!aligned || M <= 0) return 1;
+  dim3 grid((unsigned)(M < 256 * 256 ? M : 256 * 256)), block(64);
+  const int need = (int)((K + 511) / 512);
+  // the codes are read by the GEMM that follows: plain stores; loads of a large activation
+  // carry the non-temporal hint (as launch_quant_rowwise chooses)
+  const bool nt_load = M * K * 2 > ((int64_t)64 << 20);
+  const uint16_t* p1 = static_cast<const uint16_t*>(x1);
+  const uint16_t* p2 = static_cast<const uint16_t*>(x2);
+#define CDIT_QUANT_CASE(CH)                                                                         \
+  if (need <= CH) {                                                                                 \
+    if (nt_load) {                                                                                  \
+      hipLaunchKernelGGL((quant_rowwise_cat_regs<CH, true>), grid, block, 0, stream, p1, ld_x1,     \
+                         (int)(K1 / 8), p2, ld_x2, static_cast<uint8_t*>(q), ld_q, scale, (int)M,   \
+                         (int)K, scale_mode);                                                       \
+    } else {                                                                                        \
+      hipLaunchKernelGGL((quant_rowwise_cat_regs<CH, false>), grid, block, 0, stream, p1, ld_x1,    \
+                         (int)(K1 / 8), p2, ld_x2, static_cast<uint8_t*>(q), ld_q, scale, (int)M,   \
+                         (int)K, scale_mode);                                                       \
+    }                                                                                               \
+    return 0;                                                                                       \
+  }
+  CDIT_QUANT_CASE(2)
+  CDIT_QUANT_CASE(4)
+  CDIT_QUANT_CASE(8)
+  CDIT_QUANT_CASE(12)
+  CDIT_QUANT_CASE(16)
+  CDIT_QUANT_CASE(20)
+  CDIT_QUANT_CASE(24)
+  CDIT_QUANT_CASE(30)
+  CDIT_QUANT_CASE(32)
+#undef CDIT_QUANT_CASE
+  return 1;
 }
 
 int launch_quant_rowwise_batched(const QuantBatch& batch, int64_t K, int scale_mode,

@@ -369,6 +369,21 @@ def linear_batch(pairs):
   return result
 
 
+def linear_on_cat(linear: nn.Module, xs) -> torch.Tensor:
+  """`linear(torch.cat(xs, dim=-1))` for two sources without the concatenated tensor when
+  `linear` is a `float8_per_row` Linear: the per-token quantizer reads the sources in place
+  (FLUX single blocks: `proj_out(torch.cat([attn_output, mlp_hidden_states], dim=2))`,
+  reference dataflow src/cache_dit/caching/patch_functors/functor_flux.py:68-80).
+  Bit-identical to the plain expression, which is what runs for any other module, number of
+  sources or dtype."""
+  xs = list(xs)
+  if (type(linear) is Fp8DynamicLinear and len(xs) == 2 and linear.sibling_group is None
+      and all(x.is_cuda and x.dtype == torch.bfloat16 for x in xs)):
+    return torch.ops.cdit.linear_w8a8_cat2(xs[0], xs[1], linear.weight, linear.weight_scale,
+                                           linear.bias, linear._scale_mode_id, linear.epilogue)
+  return linear(torch.cat(xs, dim=-1))
+
+
 def dequantize_weight(linear: _Fp8LinearBase) -> torch.Tensor:
   """bf16 view of the quantized weight (for inspection and tests)."""
   return (linear.weight.to(torch.float32) * linear.weight_scale).to(torch.bfloat16)

@@ -133,6 +133,23 @@ def quant_rowwise_batched_into(items, scale_mode_id: int) -> None:
         scale_mode_id, _stream_ptr(x0)))
 
 
+def quant_rowwise_cat2_into(x1: torch.Tensor, x2: torch.Tensor, q: torch.Tensor, scale: torch.Tensor,
+                            scale_mode_id: int) -> None:
+  """Quantizes the rows [x1 | x2] (bf16 [M,K1] and [M,K2]) into q [M,K1+K2] / scale [M] without
+  the concatenated tensor; the results are those of quant_rowwise_into on torch.cat."""
+  with _DeviceOf(x1):
+    _native.check(_native.load().cdit_fp8_quant_rowwise_cat2(
+        x1.data_ptr(), x1.shape[1], x1.stride(0), x2.data_ptr(), x2.shape[1], x2.stride(0),
+        x1.shape[0], q.data_ptr(), q.stride(0), scale.data_ptr(), scale_mode_id, _stream_ptr(x1)))
+
+
+def cat2_quant_ok(x1: torch.Tensor, x2: torch.Tensor) -> bool:
+  """Whether quant_rowwise_cat2_into takes these two row blocks (else: concatenate)."""
+  return (x1.shape[0] == x2.shape[0] and x1.shape[1] % 8 == 0 and x2.shape[1] % 8 == 0
+          and x1.shape[1] + x2.shape[1] <= 16384 and x1.stride(0) % 8 == 0 and x2.stride(0) % 8 == 0
+          and x1.data_ptr() % 16 == 0 and x2.data_ptr() % 16 == 0)
+
+
 def gemm_rowwise_into(a: torch.Tensor, a_scale: torch.Tensor, w: torch.Tensor,
                       w_scale: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                       epilogue: int) -> None:
@@ -405,6 +422,11 @@ torch.library.define(
     "int epilogue=0, int granularity=0, bool share_input_quant=False) -> Tensor",
 )
 torch.library.define(
+    "cdit::linear_w8a8_cat2",
+    "(Tensor x1, Tensor x2, Tensor weight, Tensor weight_scale, Tensor? bias, int scale_mode=0, "
+    "int epilogue=0) -> Tensor",
+)
+torch.library.define(
     "cdit::w8a16_mm",
     "(Tensor x, Tensor b_data, Tensor b_scale, Tensor? bias, int out_dtype_id, "
     "int epilogue=0) -> Tensor",
@@ -630,6 +652,47 @@ def _linear_w8a8(x, weight, weight_scale, bias, scale_mode=0, epilogue=0, granul
       q, s = activation_workspace(M, K, x2.device)
       linear_w8a8_into(x2, w, w_s, bias, out, q, s, int(scale_mode), int(epilogue))
   return out.view(*x.shape[:-1], N)
+
+
+@torch.library.impl("cdit::linear_w8a8_cat2", "CUDA")
+def _linear_w8a8_cat2(x1, x2, weight, weight_scale, bias, scale_mode=0, epilogue=0):
+  """cdit::linear_w8a8 (per-token scales) on torch.cat([x1, x2], dim=-1) without that tensor:
+  the two sources are quantized as one row (cdit_fp8_quant_rowwise_cat2). FLUX single blocks
+  feed proj_out this way (reference dataflow
+  src/cache_dit/caching/patch_functors/functor_flux.py:68-80). Bit-identical to the op on the
+  concatenation; sources the kernel does not take are concatenated."""
+  name = "cdit::linear_w8a8_cat2"
+  if x1.dtype != torch.bfloat16 or x2.dtype != torch.bfloat16:
+    raise ValueError(f"{name}: x1 and x2 must be bfloat16, got {x1.dtype} and {x2.dtype}")
+  if x1.shape[:-1] != x2.shape[:-1]:
+    raise ValueError(f"{name}: leading shapes differ: {tuple(x1.shape)} and {tuple(x2.shape)}")
+  N, K = weight.shape
+  if x1.shape[-1] + x2.shape[-1] != K:
+    raise ValueError(f"{name}: shape mismatch [{x1.shape[-1]} | {x2.shape[-1]}] x weight "
+                     f"{tuple(weight.shape)}")
+  a, b = _as_rows(x1), _as_rows(x2)
+  if not cat2_quant_ok(a, b) or a.shape[0] <= 16 or scale_mode not in (0, 1):
+    return torch.ops.cdit.linear_w8a8(torch.cat([x1, x2], dim=-1), weight, weight_scale, bias,
+                                      scale_mode, epilogue, GRANULARITY_PER_ROW, False)
+  if weight.dtype != FP8 or weight_scale.numel() != N or weight_scale.dtype != torch.float32:
+    raise ValueError(f"{name}: weight must be float8_e4m3fn [N,K] with {N} float32 scales")
+  if bias is not None and (bias.numel() != N or bias.dtype != torch.bfloat16):
+    raise ValueError(f"{name}: bias must hold {N} bfloat16 values")
+  w = weight if weight.stride(-1) == 1 else weight.contiguous()
+  w_s = weight_scale if weight_scale.is_contiguous() else weight_scale.contiguous()
+  if bias is not None and not bias.is_contiguous():
+    bias = bias.contiguous()
+  M = a.shape[0]
+  out = torch.empty((M, N), dtype=torch.bfloat16, device=x1.device)
+  q, s = activation_workspace(M, K, a.device)
+  quant_rowwise_cat2_into(a, b, q, s, int(scale_mode))
+  gemm_rowwise_into(q, s, w, w_s, bias, out, int(epilogue))
+  return out.view(*x1.shape[:-1], N)
+
+
+@torch.library.register_fake("cdit::linear_w8a8_cat2")
+def _fake_linear_w8a8_cat2(x1, x2, weight, weight_scale, bias, scale_mode=0, epilogue=0):
+  return x1.new_empty((*x1.shape[:-1], weight.shape[0]), dtype=torch.bfloat16)
 
 
 @torch.library.register_fake("cdit::linear_w8a8")

@@ -243,11 +243,15 @@ class FluxSingleTransformerBlock(nn.Module):
     self.act_mlp = nn.GELU(approximate="tanh")
     self.attn = FluxAttention(dim, heads, joint=False)
     self.proj_out = nn.Linear(dim + mlp, dim)
+    self.fuse_cat = False  # fuse_cat_quant: proj_out quantizes [attn | mlp] without the copy
 
   def forward(self, hidden, temb, rope):
     normed, (gate, ) = self.norm(hidden, temb)
     mlp = self.act_mlp(self.proj_mlp(normed))
     attn = self.attn(normed, rope=rope)
+    if self.fuse_cat:
+      from ..nn import linear_on_cat
+      return hidden + gate * linear_on_cat(self.proj_out, [attn, mlp])
     return hidden + gate * self.proj_out(torch.cat([attn, mlp], dim=2))
 
 
@@ -477,6 +481,18 @@ def batch_streams(model: nn.Module, enable: bool = True) -> int:
   for m in model.modules():
     if isinstance(m, FluxAttention) and m.joint:
       m.batch_streams = bool(enable)
+      n += 1
+  return n
+
+
+def fuse_cat_quant(model: nn.Module, enable: bool = True) -> int:
+  """Switches the single-stream blocks of `model` to `linear_on_cat`: proj_out's quantizer
+  reads the attention output and the MLP activation in place instead of their torch.cat
+  copy. Outputs are bit-identical. Returns the number of blocks switched."""
+  n = 0
+  for m in model.modules():
+    if isinstance(m, FluxSingleTransformerBlock):
+      m.fuse_cat = bool(enable)
       n += 1
   return n
 

@@ -113,6 +113,22 @@ int cdit_fp8_quant_rowwise_batched(int n_act, const void* const* x_bf16, const i
                                    void* stream);
 
 /*
+ * cdit_fp8_quant_rowwise on rows that are the concatenation [x1 | x2] of two sources, without
+ * the concatenated tensor: FLUX single blocks feed proj_out with
+ * torch.cat([attn_output, mlp_hidden_states], dim=2) (reference dataflow
+ * src/cache_dit/caching/patch_functors/functor_flux.py:68-80), which only that quantized Linear
+ * reads. x1 bf16 [M,K1] (ld_x1), x2 bf16 [M,K2] (ld_x2) -> q e4m3 [M,K1+K2] (ld_q), scale [M]:
+ * the codes and scales of cdit_fp8_quant_rowwise on the concatenation, bit for bit. K1 and K2
+ * must be multiples of 8, K1 + K2 <= 16384, rows 16-byte aligned (CDIT_EINVAL otherwise:
+ * concatenate and use cdit_fp8_quant_rowwise). The codes are taken to be read by a GEMM
+ * launched next.
+ */
+int cdit_fp8_quant_rowwise_cat2(const void* x1_bf16, int64_t K1, int64_t ld_x1,
+                                const void* x2_bf16, int64_t K2, int64_t ld_x2, int64_t M,
+                                void* q_e4m3, int64_t ld_q, float* scale, int scale_mode,
+                                void* stream);
+
+/*
  * Per-tensor dynamic FP8 quantization: one scale for the whole tensor. Replaces
  * torchao's Float8Tensor.from_hp(x, PerTensor()) as selected for the
  * "float8_per_tensor" quant type and the per-tensor fallback pass,

@@ -87,6 +87,10 @@ def test_fake_impls_shapes_and_dtypes():
     w = torch.empty(12288, 3072, dtype=FP8, device="cuda")
     y = torch.ops.cdit.linear_w8a8(x, w, torch.empty(12288, 1, device="cuda"), None)
     assert y.shape == (2, 77, 12288) and y.dtype == torch.bfloat16 and y.device.type == "cuda"
+    w2 = torch.empty(3072, 3072 + 12288, dtype=FP8, device="cuda")
+    y = torch.ops.cdit.linear_w8a8_cat2(x, torch.empty(2, 77, 12288, dtype=torch.bfloat16, device="cuda"),
+                                        w2, torch.empty(3072, 1, device="cuda"), None)
+    assert y.shape == (2, 77, 3072) and y.dtype == torch.bfloat16 and y.device.type == "cuda"
 
 
 def _meta_quantized_linear(cls_name, in_f, out_f):

@@ -508,3 +508,43 @@ def test_mixed_precision_plan_and_fallback_on_device(with_plan):
       y = lin(x.cuda())
       y_ref = _oracle_linear(kind, x, w, None if rlin.bias is None else rlin.bias.detach())
       assert max_rel_err(y, y_ref) <= 1e-2, (name, kind, max_rel_err(y, y_ref))
+
+
+def test_linear_on_cat_equals_the_linear_on_the_concatenation():
+  """linear_on_cat(proj_out, [attn, mlp]) against proj_out(torch.cat(...)): same bits, eager,
+  compiled (fullgraph) and for the cases that fall back to concatenating (another quant type,
+  three sources, few rows); and a FLUX-shaped model with fuse_cat_quant equals itself without."""
+  import logging
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd.testing import dit_shapes as ds
+  logging.getLogger("CACHE_DIT_AMD").setLevel(logging.WARNING)
+  torch.manual_seed(0)
+  lin = torch.nn.Linear(512 + 2048, 512).to(torch.bfloat16).cuda()
+  holder = torch.nn.Sequential(lin)
+  cache_dit.quantize(holder, cache_dit.QuantizeConfig())
+  a = torch.randn(2, 300, 512, device="cuda").to(torch.bfloat16)
+  b = torch.randn(2, 300, 2048, device="cuda").to(torch.bfloat16)
+  with torch.no_grad():
+    want = lin(torch.cat([a, b], dim=-1))
+    assert torch.equal(cache_dit.linear_on_cat(lin, [a, b]), want)
+    compiled = torch.compile(lambda u, v: cache_dit.linear_on_cat(lin, [u, v]), fullgraph=True)
+    assert torch.equal(compiled(a, b), want)
+    # few rows, three sources: the plain expression
+    assert torch.equal(cache_dit.linear_on_cat(lin, [a[:1, :4], b[:1, :4]]),
+                       lin(torch.cat([a[:1, :4], b[:1, :4]], dim=-1)))
+    assert torch.equal(cache_dit.linear_on_cat(lin, [a, b[..., :1024], b[..., 1024:]]), want)
+  wo = torch.nn.Sequential(torch.nn.Linear(512 + 2048, 512).to(torch.bfloat16).cuda())
+  cache_dit.quantize(wo, cache_dit.QuantizeConfig(quant_type="float8_weight_only"))
+  with torch.no_grad():
+    assert torch.equal(cache_dit.linear_on_cat(wo[0], [a, b]), wo[0](torch.cat([a, b], dim=-1)))
+
+  kw = dict(dim=512, heads=4, mlp=2048, n_double=1, n_single=3, in_channels=64, text_dim=256,
+            pooled_dim=128)
+  model = ds.FluxLikeTransformer(**kw).to(torch.bfloat16).cuda()
+  cache_dit.quantize(model, cache_dit.QuantizeConfig())
+  inputs = ds.flux_like_inputs("cuda", n_img=320, n_txt=64, in_channels=64, text_dim=256,
+                               pooled_dim=128)
+  with torch.no_grad():
+    y0 = model(**inputs)
+    assert ds.fuse_cat_quant(model) == 3
+    assert torch.equal(model(**inputs), y0)

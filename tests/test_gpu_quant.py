@@ -311,3 +311,57 @@ def test_batched_quantizer_argument_checks():
   assert call(2, mode=7) == EINVAL and b"scale_mode" in L.cdit_last_error()
   assert call(2, xs=[x.data_ptr(), None]) == EINVAL and b"null pointer" in L.cdit_last_error()
   torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("mode_id", [0, 1])
+@pytest.mark.parametrize("M,K1,K2", [(4608, 3072, 12288), (300, 512, 2048), (77, 8, 8), (33, 4096, 12288),
+                                     (5, 1000, 24)])
+def test_concatenating_quantizer_equals_the_quantizer_on_the_concatenation(M, K1, K2, mode_id):
+  """cdit_fp8_quant_rowwise_cat2 on [x1 | x2] (column windows of wider buffers) against
+  cdit_fp8_quant_rowwise on torch.cat: codes and scales bit for bit, nothing written outside;
+  rows with a zero block, scales outside the fast-division window and a NaN among them."""
+  from cache_dit_amd import ops
+  g = torch.Generator(device="cuda").manual_seed(M + K1 + K2)
+  w1 = (torch.randn(M, K1 + 16, generator=g, device="cuda") * 3).to(torch.bfloat16)
+  w2 = torch.randn(M, K2 + 8, generator=g, device="cuda").to(torch.bfloat16)
+  x1, x2 = w1[:, 8:8 + K1], w2[:, :K2]
+  if M >= 5:
+    x1[0] = 0
+    x1[1] *= 1e-32
+    x2[1] *= 1e-32
+    x2[2] *= 1e32
+    x2[3, K2 // 2] = float("nan")
+    x1[4] = 0
+    x2[4] = 0
+  K = K1 + K2
+  qb = torch.full((M + 1, K + 16), 0x55, dtype=torch.uint8, device="cuda")
+  sb = torch.full((M + 1, ), -1.0, dtype=torch.float32, device="cuda")
+  ops.quant_rowwise_cat2_into(x1, x2, qb[:M, :K].view(torch.float8_e4m3fn), sb[:M], mode_id)
+  cat = torch.cat([x1, x2], dim=1)
+  q1 = torch.empty(M, K, dtype=torch.float8_e4m3fn, device="cuda")
+  s1 = torch.empty(M, dtype=torch.float32, device="cuda")
+  ops.quant_rowwise_into(cat, q1, s1, mode_id)
+  torch.cuda.synchronize()
+  assert torch.equal(qb[:M, :K], q1.view(torch.uint8))
+  assert torch.equal(sb[:M].view(torch.int32), s1.view(torch.int32))
+  assert (qb[:, K:] == 0x55).all() and (qb[M] == 0x55).all() and sb[M] == -1.0
+
+
+def test_concatenating_quantizer_argument_checks():
+  from cache_dit_amd import _native
+  L = _native.load()
+  x = torch.zeros(4, 64, dtype=torch.bfloat16, device="cuda")
+  q = torch.empty(4, 128, dtype=torch.uint8, device="cuda")
+  s = torch.empty(4, dtype=torch.float32, device="cuda")
+
+  def call(K1=64, K2=64, ld1=64, ld2=64, ldq=128, mode=0, x2=x):
+    return L.cdit_fp8_quant_rowwise_cat2(x.data_ptr(), K1, ld1, x2.data_ptr() if x2 is not None else None,
+                                         K2, ld2, 4, q.data_ptr(), ldq, s.data_ptr(), mode, None)
+
+  assert call() == 0
+  assert call(K1=0) == 1 and b"bad shape" in L.cdit_last_error()
+  assert call(ldq=100) == 1 and b"leading dimension" in L.cdit_last_error()
+  assert call(mode=5) == 1 and b"scale_mode" in L.cdit_last_error()
+  assert call(x2=None) == 1 and b"null pointer" in L.cdit_last_error()
+  assert call(K1=60, ld1=64) == 1 and b"multiples of 8" in L.cdit_last_error()
+  torch.cuda.synchronize()
