@@ -626,6 +626,41 @@ def dit_forward_ms(device, iters=5):
                         "PyTorch ops" + note_err)
 
 
+def dit_forward_compiled_ms(device, iters=5):
+  """The same transformer with its blocks compiled by torch.compile (regional compilation,
+  fullgraph): every converted Linear is one registered op, the Linears of a stage one
+  batched op (cdit::linear_w8a8_batch), so Inductor fuses the element-wise glue around
+  them. Returns (ms, seconds spent compiling, cosine against the eager forward) or
+  (None, None, note)."""
+  try:
+    import torch
+    import cache_dit_amd
+    from cache_dit_amd.testing import dit_shapes
+    torch.manual_seed(0)
+    with torch.device(device):
+      model = dit_shapes.FluxLikeTransformer().to(torch.bfloat16)
+    cache_dit_amd.quantize(model, cache_dit_amd.QuantizeConfig(quant_type="float8_per_row"))
+    dit_shapes.fuse_gelu_epilogues(model)
+    dit_shapes.batch_streams(model, single_blocks=True)
+    inputs = dit_shapes.flux_like_inputs(device)
+    with torch.no_grad():
+      want = model(**inputs)
+      t0 = time.perf_counter()
+      for blk in list(model.transformer_blocks) + list(model.single_transformer_blocks):
+        blk.compile(fullgraph=True)
+      got = model(**inputs)
+      torch.cuda.synchronize()
+      compile_s = time.perf_counter() - t0
+      ms = _time_events(lambda: model(**inputs), iters, 2)
+    cos = torch.nn.functional.cosine_similarity(want.float().flatten(), got.float().flatten(),
+                                                dim=0).item()
+    del model
+    torch.cuda.empty_cache()
+    return ms, compile_s, cos
+  except Exception as e:  # no Inductor back end on this box, or a compile failure
+    return None, None, f"torch.compile leg failed: {str(e)[:160]}"
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -633,6 +668,8 @@ def main():
   ap.add_argument("--warmup", type=int, default=3)
   ap.add_argument("--skip-cpu", action="store_true", help="skip the cpu_baseline leg")
   ap.add_argument("--skip-dit", action="store_true", help="skip the full-transformer forward")
+  ap.add_argument("--skip-compiled", action="store_true",
+                  help="skip the torch.compile leg of the full-transformer forward")
   ap.add_argument("--skip-other-configs", action="store_true",
                   help="skip the step legs of the other benchmark configurations (FLUX-shaped "
                        "w8a16, Qwen-Image-shaped and Wan-shaped w8a8)")
@@ -673,8 +710,11 @@ def main():
     return
   if args.dit_only:
     ms, gms, note = dit_forward_ms(device, iters=args.steps)
-    print(json.dumps({"dit_step_ms": ms, "dit_step_ms_graph": gms, "dit_step_note": note,
-                      "device": arch}))
+    out = {"dit_step_ms": ms, "dit_step_ms_graph": gms, "dit_step_note": note, "device": arch}
+    if not args.skip_compiled:
+      cms, cs, cos = dit_forward_compiled_ms(device, iters=args.steps)
+      out.update({"dit_step_ms_compiled": cms, "dit_compile_seconds": cs, "dit_compiled_cosine": cos})
+    print(json.dumps(out))
     return
   if args.headline_only:
     print(json.dumps({"linear_headline": headline_kernels(device), "device": arch}))
@@ -785,6 +825,9 @@ def main():
     for k in ("qwen_step", "wan_step"):
       other[k]["frac_fp8_peak"] = other[k]["tflops"] / FP8_PEAK_TFLOPS
   dit_ms, dit_graph_ms, dit_note = (None, None, "skipped") if args.skip_dit else dit_forward_ms(device)
+  dit_compiled = (None, None, "skipped")
+  if not args.skip_dit and not args.skip_compiled:
+    dit_compiled = dit_forward_compiled_ms(device)
   cpu = None if args.skip_cpu else cpu_baseline()
 
   line = {
@@ -840,6 +883,11 @@ def main():
       "dit_step_ms": dit_ms,
       "dit_step_ms_graph": dit_graph_ms,
       "dit_step_note": dit_note,
+      # the same forward with its blocks under torch.compile (Inductor fuses the glue around
+      # the registered ops), seconds spent compiling, cosine against the eager forward
+      "dit_step_ms_compiled": dit_compiled[0],
+      "dit_compile_seconds": dit_compiled[1],
+      "dit_compiled_cosine": dit_compiled[2],
       "roofline": roofline,
       "roofline_quant": roofline_quant,
       "cpu_baseline": cpu,

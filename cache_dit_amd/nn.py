@@ -336,18 +336,35 @@ def linear_batch(pairs):
   (encoder, [add_q_proj, add_k_proj, add_v_proj])]). Returns the outputs in the same
   nesting, bit-identical to calling the Linears one by one. For block forwards that are
   written against this package; `float8_per_row` Linears (one quantizer launch for the
-  stage as well) or `float8_weight_only` ones; other Linears, mixed types, a compiled graph
-  or inference-mode tensors simply run one by one."""
+  stage as well) or `float8_weight_only` ones; other Linears, mixed types or inference-mode
+  tensors simply run one by one. Inside a compiled graph the stage is one traceable op
+  (`cdit::linear_w8a8_batch` / `cdit::w8a16_batch`) without the shared-quantization state."""
   flat = [lin for _, lins in pairs for lin in lins]
   first = flat[0]
-  plain = (torch.compiler.is_compiling() or len(flat) > _native.MAX_GROUP
+  plain = (len(flat) > _native.MAX_GROUP
            or len(pairs) > _native.MAX_ACTS
            or type(first) not in (Fp8DynamicLinear, Fp8WeightOnlyLinear)
            or any(type(lin) is not type(first) or lin.in_features != first.in_features
                   or lin._scale_mode_id != first._scale_mode_id for lin in flat)
-           or any(x.is_inference() or not x.is_cuda or x.dtype != torch.bfloat16 for x, _ in pairs))
+           or any(not x.is_cuda or x.dtype != torch.bfloat16 for x, _ in pairs))
+  compiling = torch.compiler.is_compiling()
+  if not plain and not compiling:  # (no version counters on inference tensors: nothing is shared)
+    plain = any(x.is_inference() for x, _ in pairs)
   if plain:
     return [[lin(x) for lin in lins] for x, lins in pairs]
+  if compiling:
+    # a compiled graph gets the stateless form: one traceable op for the whole stage
+    op = (torch.ops.cdit.w8a16_batch if type(first) is Fp8WeightOnlyLinear
+          else torch.ops.cdit.linear_w8a8_batch)
+    args = ([x for x, _ in pairs], [lin.weight for lin in flat],
+            [lin.weight_scale.reshape(-1) for lin in flat], [lin.bias for lin in flat],
+            [len(lins) for _, lins in pairs], [lin.epilogue for lin in flat])
+    outs = op(*args) if type(first) is Fp8WeightOnlyLinear else op(*args, first._scale_mode_id)
+    result, p = [], 0
+    for _, lins in pairs:
+      result.append(list(outs[p:p + len(lins)]))
+      p += len(lins)
+    return result
   acts, result, rows = [], [], []
   for x, lins in pairs:
     x2 = ops._as_rows(x)

@@ -427,6 +427,16 @@ torch.library.define(
     "int epilogue=0) -> Tensor",
 )
 torch.library.define(
+    "cdit::linear_w8a8_batch",
+    "(Tensor[] xs, Tensor[] weights, Tensor[] weight_scales, Tensor?[] biases, "
+    "int[] members_per_act, int[] epilogues, int scale_mode=0) -> Tensor[]",
+)
+torch.library.define(
+    "cdit::w8a16_batch",
+    "(Tensor[] xs, Tensor[] weights, Tensor[] weight_scales, Tensor?[] biases, "
+    "int[] members_per_act, int[] epilogues) -> Tensor[]",
+)
+torch.library.define(
     "cdit::w8a16_mm",
     "(Tensor x, Tensor b_data, Tensor b_scale, Tensor? bias, int out_dtype_id, "
     "int epilogue=0) -> Tensor",
@@ -693,6 +703,113 @@ def _linear_w8a8_cat2(x1, x2, weight, weight_scale, bias, scale_mode=0, epilogue
 @torch.library.register_fake("cdit::linear_w8a8_cat2")
 def _fake_linear_w8a8_cat2(x1, x2, weight, weight_scale, bias, scale_mode=0, epilogue=0):
   return x1.new_empty((*x1.shape[:-1], weight.shape[0]), dtype=torch.bfloat16)
+
+
+def _batch_check(name, xs, weights, weight_scales, biases, members_per_act, epilogues):
+  n = len(weights)
+  if (len(xs) != len(members_per_act) or sum(members_per_act) != n or len(weight_scales) != n
+      or len(biases) != n or len(epilogues) != n or not 1 <= len(xs) <= _native.MAX_ACTS
+      or n > _native.MAX_GROUP or any(c < 1 for c in members_per_act)):
+    raise ValueError(f"{name}: 1 to {_native.MAX_ACTS} activations with 1 to {_native.MAX_GROUP} "
+                     "members in all, listed activation by activation")
+  K = xs[0].shape[-1]
+  for x in xs:
+    if x.dtype != torch.bfloat16 or x.shape[-1] != K:
+      raise ValueError(f"{name}: activations must be bfloat16 [..., {K}]")
+  for w, s, b in zip(weights, weight_scales, biases):
+    if w.dtype != FP8 or w.dim() != 2 or w.shape[1] != K or w.stride(-1) != 1:
+      raise ValueError(f"{name}: weights must be float8_e4m3fn [N, {K}] rows")
+    if s.numel() != w.shape[0] or s.dtype != torch.float32 or not s.is_contiguous():
+      raise ValueError(f"{name}: weight_scales must hold N contiguous float32 values")
+    if b is not None and (b.numel() != w.shape[0] or b.dtype != torch.bfloat16 or not b.is_contiguous()):
+      raise ValueError(f"{name}: biases must hold N contiguous bfloat16 values")
+
+
+def _batch_outputs(xs, weights, members_per_act):
+  rows, outs, shaped, p = [], [], [], 0
+  for x, c in zip(xs, members_per_act):
+    x2 = _as_rows(x)
+    rows.append(x2)
+    mine = [torch.empty((x2.shape[0], w.shape[0]), dtype=torch.bfloat16, device=x.device)
+            for w in weights[p:p + c]]
+    outs.append(mine)
+    shaped += [o.view(*x.shape[:-1], o.shape[1]) for o in mine]
+    p += c
+  return rows, outs, shaped
+
+
+@torch.library.impl("cdit::linear_w8a8_batch", "CUDA")
+def _linear_w8a8_batch(xs, weights, weight_scales, biases, members_per_act, epilogues, scale_mode=0):
+  """The float8_per_row Linears of one stage on up to four activations as one quantizer
+  launch and one GEMM launch (cdit_fp8_quant_rowwise_batched + cdit_fp8_gemm_rowwise_batched)
+  behind a single traceable op: xs[s] bf16 [..., K]; the members of activation s are the
+  next members_per_act[s] entries of weights (e4m3 [N_p, K]), weight_scales, biases and
+  epilogues. Returns one bf16 [..., N_p] per member, bit-identical to cdit::linear_w8a8 per
+  member."""
+  _batch_check("cdit::linear_w8a8_batch", xs, weights, weight_scales, biases, members_per_act,
+               epilogues)
+  rows, outs, shaped = _batch_outputs(xs, weights, members_per_act)
+  live = [i for i, r in enumerate(rows) if r.shape[0] > 0]
+  if not live:
+    return shaped
+  items = []
+  for i in live:
+    r = rows[i]
+    items.append((r, torch.empty(r.shape, dtype=FP8, device=r.device),
+                  torch.empty((r.shape[0], ), dtype=torch.float32, device=r.device)))
+  if len(items) > 1:
+    quant_rowwise_batched_into(items, int(scale_mode))
+  else:
+    quant_rowwise_into(items[0][0], items[0][1], items[0][2], int(scale_mode), gemm_follows=True)
+  starts = [sum(members_per_act[:i]) for i in range(len(xs))]
+  acts = []
+  for (r, q, sc), i in zip(items, live):
+    a, b = starts[i], starts[i] + members_per_act[i]
+    acts.append((q, sc, list(weights[a:b]), list(weight_scales[a:b]), list(biases[a:b]), outs[i],
+                 [int(e) for e in epilogues[a:b]]))
+  if len(acts) == 1 and len(acts[0][2]) == 1:
+    q, sc, w, ws, b, o, e = acts[0]
+    gemm_rowwise_into(q, sc, w[0], ws[0], b[0], o[0], e[0])
+  else:
+    gemm_rowwise_batched_into(acts)
+  return shaped
+
+
+@torch.library.impl("cdit::w8a16_batch", "CUDA")
+def _w8a16_batch(xs, weights, weight_scales, biases, members_per_act, epilogues):
+  """The float8_weight_only counterpart of cdit::linear_w8a8_batch (cdit_w8a16_gemm_batched)."""
+  _batch_check("cdit::w8a16_batch", xs, weights, weight_scales, biases, members_per_act, epilogues)
+  rows, outs, shaped = _batch_outputs(xs, weights, members_per_act)
+  starts = [sum(members_per_act[:i]) for i in range(len(xs))]
+  acts = []
+  for i, r in enumerate(rows):
+    if r.shape[0] == 0:
+      continue
+    a, b = starts[i], starts[i] + members_per_act[i]
+    acts.append((r, list(weights[a:b]), list(weight_scales[a:b]), list(biases[a:b]), outs[i],
+                 [int(e) for e in epilogues[a:b]]))
+  if acts:
+    w8a16_batched_into(acts)
+  return shaped
+
+
+def _fake_batch(xs, weights, members_per_act):
+  out, p = [], 0
+  for x, c in zip(xs, members_per_act):
+    out += [x.new_empty((*x.shape[:-1], w.shape[0]), dtype=torch.bfloat16) for w in weights[p:p + c]]
+    p += c
+  return out
+
+
+@torch.library.register_fake("cdit::linear_w8a8_batch")
+def _fake_linear_w8a8_batch(xs, weights, weight_scales, biases, members_per_act, epilogues,
+                            scale_mode=0):
+  return _fake_batch(xs, weights, members_per_act)
+
+
+@torch.library.register_fake("cdit::w8a16_batch")
+def _fake_w8a16_batch(xs, weights, weight_scales, biases, members_per_act, epilogues):
+  return _fake_batch(xs, weights, members_per_act)
 
 
 @torch.library.register_fake("cdit::linear_w8a8")

@@ -179,8 +179,10 @@ class FluxAttention(nn.Module):
       self.norm_added_q, self.norm_added_k = RMSNorm(hd), RMSNorm(hd)
       self.to_add_out = nn.Linear(dim, dim)
 
-  def forward(self, hidden, encoder=None, rope=None):
-    if self.joint and self.batch_streams:
+  def forward(self, hidden, encoder=None, rope=None, qkv=None):
+    if qkv is not None:  # computed by the caller together with other Linears on `hidden`
+      q, k, v = qkv
+    elif self.joint and self.batch_streams:
       (q, k, v), (eq, ek, ev) = _batch([(hidden, [self.to_q, self.to_k, self.to_v]),
                                         (encoder, [self.add_q_proj, self.add_k_proj, self.add_v_proj])])
     else:
@@ -244,11 +246,18 @@ class FluxSingleTransformerBlock(nn.Module):
     self.attn = FluxAttention(dim, heads, joint=False)
     self.proj_out = nn.Linear(dim + mlp, dim)
     self.fuse_cat = False  # fuse_cat_quant: proj_out quantizes [attn | mlp] without the copy
+    self.batch_siblings = False  # batch_streams(single_blocks=True): proj_mlp + q/k/v in one launch
 
   def forward(self, hidden, temb, rope):
     normed, (gate, ) = self.norm(hidden, temb)
-    mlp = self.act_mlp(self.proj_mlp(normed))
-    attn = self.attn(normed, rope=rope)
+    if self.batch_siblings:
+      (mlp, q, k, v), = _batch([(normed, [self.proj_mlp, self.attn.to_q, self.attn.to_k,
+                                          self.attn.to_v])])
+      mlp = self.act_mlp(mlp)
+      attn = self.attn(normed, rope=rope, qkv=(q, k, v))
+    else:
+      mlp = self.act_mlp(self.proj_mlp(normed))
+      attn = self.attn(normed, rope=rope)
     if self.fuse_cat:
       from ..nn import linear_on_cat
       return hidden + gate * linear_on_cat(self.proj_out, [attn, mlp])
@@ -471,17 +480,21 @@ def fuse_gelu_epilogues(model: nn.Module) -> int:
   return n
 
 
-def batch_streams(model: nn.Module, enable: bool = True) -> int:
+def batch_streams(model: nn.Module, enable: bool = True, single_blocks: bool = False) -> int:
   """Switches the double-stream blocks of `model` (FLUX, Qwen-Image) to forwards that hand
   the image-stream and the text-stream Linears of a stage to linear_batch: one GEMM launch
   per stage instead of one per Linear, the small text-stream GEMMs riding along with the
-  large image-stream ones. Outputs are bit-identical. Returns the number of attention
-  modules switched."""
+  large image-stream ones. single_blocks=True does the same for proj_mlp + q/k/v of FLUX
+  single blocks (in eager code group_sibling_linears_ finds those by itself; a compiled
+  graph needs the explicit call). Outputs are bit-identical. Returns the number of
+  double-stream attention modules switched."""
   n = 0
   for m in model.modules():
     if isinstance(m, FluxAttention) and m.joint:
       m.batch_streams = bool(enable)
       n += 1
+    if isinstance(m, FluxSingleTransformerBlock):
+      m.batch_siblings = bool(enable) and single_blocks
   return n
 
 

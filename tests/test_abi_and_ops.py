@@ -87,6 +87,13 @@ def test_fake_impls_shapes_and_dtypes():
     w = torch.empty(12288, 3072, dtype=FP8, device="cuda")
     y = torch.ops.cdit.linear_w8a8(x, w, torch.empty(12288, 1, device="cuda"), None)
     assert y.shape == (2, 77, 12288) and y.dtype == torch.bfloat16 and y.device.type == "cuda"
+    ys = torch.ops.cdit.linear_w8a8_batch(
+        [x, torch.empty(5, 3072, dtype=torch.bfloat16, device="cuda")], [w, w, w],
+        [torch.empty(12288, device="cuda")] * 3, [None, None, None], [2, 1], [0, 1, 0])
+    assert [tuple(y.shape) for y in ys] == [(2, 77, 12288), (2, 77, 12288), (5, 12288)]
+    ys = torch.ops.cdit.w8a16_batch([x], [w, w], [torch.empty(12288, device="cuda")] * 2, [None, None],
+                                    [2], [0, 0])
+    assert [tuple(y.shape) for y in ys] == [(2, 77, 12288)] * 2 and ys[0].dtype == torch.bfloat16
     w2 = torch.empty(3072, 3072 + 12288, dtype=FP8, device="cuda")
     y = torch.ops.cdit.linear_w8a8_cat2(x, torch.empty(2, 77, 12288, dtype=torch.bfloat16, device="cuda"),
                                         w2, torch.empty(3072, 1, device="cuda"), None)

@@ -548,3 +548,51 @@ def test_linear_on_cat_equals_the_linear_on_the_concatenation():
     y0 = model(**inputs)
     assert ds.fuse_cat_quant(model) == 3
     assert torch.equal(model(**inputs), y0)
+
+
+def test_compiled_blocks_run_the_batched_ops():
+  """Blocks of a FLUX-shaped toy model under torch.compile(fullgraph=True) with the Linears of
+  a stage handed to linear_batch: inside a compiled graph a stage is one cdit::linear_w8a8_batch
+  (or cdit::w8a16_batch) op; the op equals the per-Linear ops bit for bit, the compiled model
+  agrees with the eager one to the accuracy of the re-fused glue."""
+  import logging
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd.testing import dit_shapes as ds
+  logging.getLogger("CACHE_DIT_AMD").setLevel(logging.WARNING)
+  for quant_type in ("float8_per_row", "float8_weight_only"):
+    torch.manual_seed(0)
+    lins = [torch.nn.Linear(512, n).to(torch.bfloat16).cuda() for n in (512, 1024, 256, 512)]
+    holder = torch.nn.ModuleList(lins)
+    cache_dit.quantize(holder, cache_dit.QuantizeConfig(quant_type=quant_type))
+    x = torch.randn(2, 150, 512, device="cuda").to(torch.bfloat16)
+    e = torch.randn(2, 40, 512, device="cuda").to(torch.bfloat16)
+    op = (torch.ops.cdit.linear_w8a8_batch if quant_type == "float8_per_row"
+          else torch.ops.cdit.w8a16_batch)
+    with torch.no_grad():
+      outs = op([x, e], [l.weight for l in lins], [l.weight_scale.reshape(-1) for l in lins],
+                [l.bias for l in lins], [3, 1], [0, 1, 0, 0])
+      lins[1].epilogue = 1
+      want = [lins[0](x), lins[1](x), lins[2](x), lins[3](e)]
+      for o, w in zip(outs, want):
+        assert torch.equal(o, w)
+      fn = torch.compile(lambda a, b: cache_dit.linear_batch([(a, lins[:3]), (b, lins[3:])]),
+                         fullgraph=True)
+      (o0, o1, o2), (o3, ) = fn(x, e)
+      for o, w in zip((o0, o1, o2, o3), want):
+        assert torch.equal(o, w)
+
+    kw = dict(dim=512, heads=4, mlp=2048, n_double=2, n_single=2, in_channels=64, text_dim=256,
+              pooled_dim=128)
+    model = ds.FluxLikeTransformer(**kw).to(torch.bfloat16).cuda()
+    cache_dit.quantize(model, cache_dit.QuantizeConfig(quant_type=quant_type))
+    ds.fuse_gelu_epilogues(model)
+    inputs = ds.flux_like_inputs("cuda", n_img=320, n_txt=64, in_channels=64, text_dim=256,
+                                 pooled_dim=128)
+    with torch.no_grad():
+      y0 = model(**inputs)
+      ds.batch_streams(model, single_blocks=True)
+      assert torch.equal(model(**inputs), y0)  # eager: the stateful batched path
+      for blk in list(model.transformer_blocks) + list(model.single_transformer_blocks):
+        blk.compile(fullgraph=True)
+      y1 = model(**inputs)
+    assert cosine(y1, y0) >= 0.999
