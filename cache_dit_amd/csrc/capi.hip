@@ -156,7 +156,7 @@ int cdit_set_gemm_variant(int variant) {
 
 int cdit_debug_set_quant_hints(int hints) {
   int prev = cdit::g_quant_variant;
-  cdit::g_quant_variant = hints >= 0 && hints <= 3 ? hints : -1;
+  cdit::g_quant_variant = hints >= 0 && hints <= 7 ? hints : -1;
   return prev;
 }
 

@@ -123,6 +123,87 @@ __global__ __launch_bounds__(64) void quant_rowwise_regs(
   }
 }
 
+// Two wavefronts share a row, each keeps half of it in registers: half the registers per
+// wavefront, twice the wavefronts in flight, and a row's loads, arithmetic and stores
+// overlap between its two halves; the two partial maxima meet in LDS. Measured against one
+// wavefront per row (codes read by a GEMM next; us): 4608 x 15360 40.0 -> 36.2, 4096 x 12288
+// 27.5 -> 25.9, 4608 x 3072 9.0 -> 8.5, 32760 x 5120 87.1 -> 85.4. BATCHED as in
+// quant_rowwise_regs.
+template <int CH, bool NT_LOAD, bool NT_STORE, bool BATCHED = false>
+__global__ __launch_bounds__(128) void quant_rowwise_split2(
+    const uint16_t* __restrict__ x, int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q,
+    float* __restrict__ scale, int M, int K, int scale_mode,
+    std::conditional_t<BATCHED, QuantBatch, NoBatch> batch = {}) {
+  __shared__ uint32_t part[2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nchunks = K >> 3;
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+    const uint16_t* x_row = x + row * ld_x;
+    uint8_t* q_row = q + row * ld_q;
+    float* s_row = scale + row;
+    if constexpr (BATCHED) {
+      const int r = __builtin_amdgcn_readfirstlane((int)row);
+      int s = 0;
+#pragma unroll
+      for (int i = 1; i < kMaxQuantActs; ++i) s += r >= batch.row_begin[i];
+      const int64_t local = r - batch.row_begin[s];
+      x_row = batch.x[s] + local * batch.ld_x[s];
+      q_row = batch.q[s] + local * batch.ld_q[s];
+      s_row = batch.scale[s] + local;
+    }
+    const uint4* xr = reinterpret_cast<const uint4*>(x_row);
+    uint4 v[CH];
+    uint32_t m = 0;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int idx = (2 * c + wave) * 64 + lane;
+      if (idx < nchunks) {
+        if constexpr (NT_LOAD) {
+          typedef unsigned int u4v __attribute__((ext_vector_type(4)));
+          const u4v t = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(xr + idx));
+          v[c] = make_uint4(t[0], t[1], t[2], t[3]);
+        } else {
+          v[c] = xr[idx];
+        }
+      } else {
+        v[c] = make_uint4(0, 0, 0, 0);
+      }
+      m = absmax2(absmax2(absmax2(absmax2(m, v[c].x), v[c].y), v[c].z), v[c].w);
+    }
+    m = wave_max_u32(fold2(m));
+    if (lane == 0) part[wave] = m;
+    __syncthreads();
+    m = max(part[0], part[1]);
+    __syncthreads();  // part is free for the next row
+    const float s = row_scale(m, scale_mode);
+    if (threadIdx.x == 0) *s_row = s;
+    uint2* qr = reinterpret_cast<uint2*>(q_row);
+    if (scale_in_fast_window(s)) {  // uniform
+      const float r = 1.0f / s;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int idx = (2 * c + wave) * 64 + lane;
+        if (idx < nchunks) {
+          const uint2 o = {quant4<true>(v[c].x, v[c].y, s, r), quant4<true>(v[c].z, v[c].w, s, r)};
+          if constexpr (NT_STORE) {
+            typedef unsigned int u2v __attribute__((ext_vector_type(2)));
+            const u2v t = {o.x, o.y};
+            __builtin_nontemporal_store(t, reinterpret_cast<u2v*>(qr + idx));
+          } else {
+            qr[idx] = o;
+          }
+        }
+      }
+    } else {  // cold path: re-reads the row
+#pragma unroll 1
+      for (int idx = threadIdx.x; idx < nchunks; idx += 128) {
+        const uint4 w = xr[idx];
+        qr[idx] = uint2{quant4<false>(w.x, w.y, s, 0.0f), quant4<false>(w.z, w.w, s, 0.0f)};
+      }
+    }
+  }
+}
+
 // The regs kernel on a row that is the concatenation of two source rows, [x1 | x2]: the
 // input of FLUX single blocks' proj_out is torch.cat([attn_output, mlp_hidden_states], dim=2)
 // (reference dataflow src/cache_dit/caching/patch_functors/functor_flux.py:68-80), read by
@@ -488,15 +569,46 @@ int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void
   dim3 grid((unsigned)blocks), block(kThreads);
   const int Mi = (int)M, Ki = (int)K;
   const int need = (int)((K + 511) / 512);  // 16-byte chunks per lane
+  // Cache hints (0: loads and stores non-temporal, 1: neither, 2: loads, 3: stores) and,
+  // from 4 on, the same hints with two wavefronts per row. Codes that a GEMM reads next
+  // keep their stores cacheable; activations beyond 64 MB are loaded non-temporally; two
+  // wavefronts per row wherever a GEMM follows, and for a stand-alone call on long rows or
+  // large activations (one wavefront per row is the faster at 4608 x 3072 on its own:
+  // 8.0 against 8.2 us).
+  const bool large = M * K * 2 > ((int64_t)64 << 20);
   const int hints = g_quant_variant >= 0 ? g_quant_variant
-                    : consumer_follows   ? (M * K * 2 > ((int64_t)64 << 20) ? 2 : 1)
-                    : M * K * 2 > ((int64_t)64 << 20) ? 0 : 3;
+                    : consumer_follows   ? (large ? 6 : 5)
+                    : large              ? 4
+                    : K >= 8192          ? 7
+                                         : 3;
+  if (aligned && hints >= 4 && need >= 2 && need <= 32) {
+    dim3 b2(128);
+    const int h = hints - 4;
+#define CDIT_SPLIT_LAUNCH(CH, NL, NS)                                                          \
+  hipLaunchKernelGGL((quant_rowwise_split2<CH, NL, NS>), grid, b2, 0, stream, xp, ld_x, qp, ld_q, \
+                     scale, Mi, Ki, scale_mode)
+#define CDIT_SPLIT_CASE(CH)                                                                    \
+  if (need <= 2 * CH) {                                                                        \
+    switch (h) {                                                                               \
+      case 0: CDIT_SPLIT_LAUNCH(CH, true, true); break;                                        \
+      case 2: CDIT_SPLIT_LAUNCH(CH, true, false); break;                                       \
+      case 3: CDIT_SPLIT_LAUNCH(CH, false, true); break;                                       \
+      default: CDIT_SPLIT_LAUNCH(CH, false, false); break;                                     \
+    }                                                                                          \
+    return 0;                                                                                  \
+  }
+    CDIT_SPLIT_CASE(1) CDIT_SPLIT_CASE(2) CDIT_SPLIT_CASE(3) CDIT_SPLIT_CASE(4) CDIT_SPLIT_CASE(5)
+    CDIT_SPLIT_CASE(6) CDIT_SPLIT_CASE(8) CDIT_SPLIT_CASE(10) CDIT_SPLIT_CASE(12) CDIT_SPLIT_CASE(14)
+    CDIT_SPLIT_CASE(15) CDIT_SPLIT_CASE(16)
+#undef CDIT_SPLIT_CASE
+#undef CDIT_SPLIT_LAUNCH
+  }
 #define CDIT_QUANT_LAUNCH(CH, NL, NS)                                                        \
   hipLaunchKernelGGL((quant_rowwise_regs<CH, NL, NS>), grid, block, 0, stream, xp, ld_x, qp,   \
                      ld_q, scale, Mi, Ki, scale_mode)
 #define CDIT_QUANT_CASE(CH)                                                                  \
   if (aligned && need <= CH) {                                                               \
-    switch (hints) {                                                                         \
+    switch (hints & 3) {                                                                         \
       case 0: CDIT_QUANT_LAUNCH(CH, true, true); break;                                      \
       case 2: CDIT_QUANT_LAUNCH(CH, true, false); break;                                     \
       case 3: CDIT_QUANT_LAUNCH(CH, false, true); break;                                     \
@@ -583,33 +695,43 @@ int launch_quant_rowwise_batched(const QuantBatch& batch, int64_t K, int scale_m
   const int need = (int)((K + 511) / 512);
   // the codes are read by the GEMM that follows: cacheable stores; loads of a large batch
   // carry the non-temporal hint (as launch_quant_rowwise chooses for one activation)
-  const bool nt_load = g_quant_variant >= 0 ? (g_quant_variant == 0 || g_quant_variant == 2)
+  const bool nt_load = g_quant_variant >= 0 ? ((g_quant_variant & 3) == 0 || (g_quant_variant & 3) == 2)
                                             : M * K * 2 > ((int64_t)64 << 20);
+  dim3 b2(128);
 #define CDIT_QUANT_CASE(CH)                                                                      \
-  if (need <= CH) {                                                                              \
+  if (need >= 2 && need <= 2 * CH) {                                                             \
     if (nt_load) {                                                                               \
-      hipLaunchKernelGGL((quant_rowwise_regs<CH, true, false, true>), grid, block, 0, stream,    \
+      hipLaunchKernelGGL((quant_rowwise_split2<CH, true, false, true>), grid, b2, 0, stream,     \
                          nullptr, 0, nullptr, 0, nullptr, Mi, Ki, scale_mode, batch);            \
     } else {                                                                                     \
-      hipLaunchKernelGGL((quant_rowwise_regs<CH, false, false, true>), grid, block, 0, stream,   \
+      hipLaunchKernelGGL((quant_rowwise_split2<CH, false, false, true>), grid, b2, 0, stream,    \
                          nullptr, 0, nullptr, 0, nullptr, Mi, Ki, scale_mode, batch);            \
     }                                                                                            \
     return 0;                                                                                    \
   }
   CDIT_QUANT_CASE(1)
   CDIT_QUANT_CASE(2)
+  CDIT_QUANT_CASE(3)
   CDIT_QUANT_CASE(4)
+  CDIT_QUANT_CASE(5)
   CDIT_QUANT_CASE(6)
   CDIT_QUANT_CASE(8)
   CDIT_QUANT_CASE(10)
   CDIT_QUANT_CASE(12)
+  CDIT_QUANT_CASE(14)
+  CDIT_QUANT_CASE(15)
   CDIT_QUANT_CASE(16)
-  CDIT_QUANT_CASE(20)
-  CDIT_QUANT_CASE(24)
-  CDIT_QUANT_CASE(27)
-  CDIT_QUANT_CASE(30)
-  CDIT_QUANT_CASE(32)
 #undef CDIT_QUANT_CASE
+  if (need == 1) {  // rows of up to 512 elements: one wavefront each
+    if (nt_load) {
+      hipLaunchKernelGGL((quant_rowwise_regs<1, true, false, true>), grid, block, 0, stream, nullptr, 0,
+                         nullptr, 0, nullptr, Mi, Ki, scale_mode, batch);
+    } else {
+      hipLaunchKernelGGL((quant_rowwise_regs<1, false, false, true>), grid, block, 0, stream, nullptr,
+                         0, nullptr, 0, nullptr, Mi, Ki, scale_mode, batch);
+    }
+    return 0;
+  }
   return 1;
 }
 
