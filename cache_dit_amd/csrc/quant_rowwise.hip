@@ -123,18 +123,18 @@ __global__ __launch_bounds__(64) void quant_rowwise_regs(
   }
 }
 
-// Two wavefronts share a row, each keeps half of it in registers: half the registers per
-// wavefront, twice the wavefronts in flight, and a row's loads, arithmetic and stores
-// overlap between its two halves; the two partial maxima meet in LDS. Measured against one
+// WAVES (two or four) wavefronts share a row, each keeps its part of it in registers: fewer
+// registers per wavefront, more wavefronts in flight, and a row's loads, arithmetic and
+// stores overlap between its parts; the partial maxima meet in LDS. Measured against one
 // wavefront per row (codes read by a GEMM next; us): 4608 x 15360 40.0 -> 36.2, 4096 x 12288
 // 27.5 -> 25.9, 4608 x 3072 9.0 -> 8.5, 32760 x 5120 87.1 -> 85.4. BATCHED as in
 // quant_rowwise_regs.
-template <int CH, bool NT_LOAD, bool NT_STORE, bool BATCHED = false>
-__global__ __launch_bounds__(128) void quant_rowwise_split2(
+template <int CH, bool NT_LOAD, bool NT_STORE, bool BATCHED = false, int WAVES = 2>
+__global__ __launch_bounds__(64 * WAVES) void quant_rowwise_split2(
     const uint16_t* __restrict__ x, int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q,
     float* __restrict__ scale, int M, int K, int scale_mode,
     std::conditional_t<BATCHED, QuantBatch, NoBatch> batch = {}) {
-  __shared__ uint32_t part[2];
+  __shared__ uint32_t part[WAVES];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nchunks = K >> 3;
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(128) void quant_rowwise_split2(
     uint32_t m = 0;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-      const int idx = (2 * c + wave) * 64 + lane;
+      const int idx = (WAVES * c + wave) * 64 + lane;
       if (idx < nchunks) {
         if constexpr (NT_LOAD) {
           typedef unsigned int u4v __attribute__((ext_vector_type(4)));
@@ -173,7 +173,9 @@ __global__ __launch_bounds__(128) void quant_rowwise_split2(
     m = wave_max_u32(fold2(m));
     if (lane == 0) part[wave] = m;
     __syncthreads();
-    m = max(part[0], part[1]);
+    m = part[0];
+#pragma unroll
+    for (int i = 1; i < WAVES; ++i) m = max(m, part[i]);
     __syncthreads();  // part is free for the next row
     const float s = row_scale(m, scale_mode);
     if (threadIdx.x == 0) *s_row = s;
@@ -182,7 +184,7 @@ __global__ __launch_bounds__(128) void quant_rowwise_split2(
       const float r = 1.0f / s;
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
-        const int idx = (2 * c + wave) * 64 + lane;
+        const int idx = (WAVES * c + wave) * 64 + lane;
         if (idx < nchunks) {
           const uint2 o = {quant4<true>(v[c].x, v[c].y, s, r), quant4<true>(v[c].z, v[c].w, s, r)};
           if constexpr (NT_STORE) {
@@ -196,7 +198,7 @@ __global__ __launch_bounds__(128) void quant_rowwise_split2(
       }
     } else {  // cold path: re-reads the row
 #pragma unroll 1
-      for (int idx = threadIdx.x; idx < nchunks; idx += 128) {
+      for (int idx = threadIdx.x; idx < nchunks; idx += 64 * WAVES) {
         const uint4 w = xr[idx];
         qr[idx] = uint2{quant4<false>(w.x, w.y, s, 0.0f), quant4<false>(w.z, w.w, s, 0.0f)};
       }
@@ -582,24 +584,28 @@ int launch_quant_rowwise(const void* x, int64_t M, int64_t K, int64_t ld_x, void
                     : K >= 8192          ? 7
                                          : 3;
   if (aligned && hints >= 4 && need >= 2 && need <= 32) {
-    dim3 b2(128);
-    const int h = hints - 4;
-#define CDIT_SPLIT_LAUNCH(CH, NL, NS)                                                          \
-  hipLaunchKernelGGL((quant_rowwise_split2<CH, NL, NS>), grid, b2, 0, stream, xp, ld_x, qp, ld_q, \
-                     scale, Mi, Ki, scale_mode)
-#define CDIT_SPLIT_CASE(CH)                                                                    \
-  if (need <= 2 * CH) {                                                                        \
-    switch (h) {                                                                               \
-      case 0: CDIT_SPLIT_LAUNCH(CH, true, true); break;                                        \
-      case 2: CDIT_SPLIT_LAUNCH(CH, true, false); break;                                       \
-      case 3: CDIT_SPLIT_LAUNCH(CH, false, true); break;                                       \
-      default: CDIT_SPLIT_LAUNCH(CH, false, false); break;                                     \
-    }                                                                                          \
-    return 0;                                                                                  \
+    // several wavefronts per row: two up to 3584 elements, four beyond (measured: four gain
+    // another 2-4 % from K = 5120 on and lose 3-8 % at K = 3072)
+    const int h = hints & 3;
+#define CDIT_SPLIT_LAUNCH(W, CH, NL, NS)                                                        \
+  hipLaunchKernelGGL((quant_rowwise_split2<CH, NL, NS, false, W>), grid, dim3(64 * W), 0, stream, \
+                     xp, ld_x, qp, ld_q, scale, Mi, Ki, scale_mode)
+#define CDIT_SPLIT_CASE(W, CH)                                                                  \
+  if (need <= W * CH) {                                                                         \
+    switch (h) {                                                                                \
+      case 0: CDIT_SPLIT_LAUNCH(W, CH, true, true); break;                                      \
+      case 2: CDIT_SPLIT_LAUNCH(W, CH, true, false); break;                                     \
+      case 3: CDIT_SPLIT_LAUNCH(W, CH, false, true); break;                                     \
+      default: CDIT_SPLIT_LAUNCH(W, CH, false, false); break;                                   \
+    }                                                                                           \
+    return 0;                                                                                   \
   }
-    CDIT_SPLIT_CASE(1) CDIT_SPLIT_CASE(2) CDIT_SPLIT_CASE(3) CDIT_SPLIT_CASE(4) CDIT_SPLIT_CASE(5)
-    CDIT_SPLIT_CASE(6) CDIT_SPLIT_CASE(8) CDIT_SPLIT_CASE(10) CDIT_SPLIT_CASE(12) CDIT_SPLIT_CASE(14)
-    CDIT_SPLIT_CASE(15) CDIT_SPLIT_CASE(16)
+    if (need < 8) {
+      CDIT_SPLIT_CASE(2, 1) CDIT_SPLIT_CASE(2, 2) CDIT_SPLIT_CASE(2, 3) CDIT_SPLIT_CASE(2, 4)
+    } else {
+      CDIT_SPLIT_CASE(4, 2) CDIT_SPLIT_CASE(4, 3) CDIT_SPLIT_CASE(4, 4) CDIT_SPLIT_CASE(4, 5)
+      CDIT_SPLIT_CASE(4, 6) CDIT_SPLIT_CASE(4, 7) CDIT_SPLIT_CASE(4, 8)
+    }
 #undef CDIT_SPLIT_CASE
 #undef CDIT_SPLIT_LAUNCH
   }
@@ -697,30 +703,23 @@ int launch_quant_rowwise_batched(const QuantBatch& batch, int64_t K, int scale_m
   // carry the non-temporal hint (as launch_quant_rowwise chooses for one activation)
   const bool nt_load = g_quant_variant >= 0 ? ((g_quant_variant & 3) == 0 || (g_quant_variant & 3) == 2)
                                             : M * K * 2 > ((int64_t)64 << 20);
-  dim3 b2(128);
-#define CDIT_QUANT_CASE(CH)                                                                      \
-  if (need >= 2 && need <= 2 * CH) {                                                             \
+#define CDIT_QUANT_CASE(W, CH)                                                                   \
+  if (need <= W * CH) {                                                                          \
     if (nt_load) {                                                                               \
-      hipLaunchKernelGGL((quant_rowwise_split2<CH, true, false, true>), grid, b2, 0, stream,     \
-                         nullptr, 0, nullptr, 0, nullptr, Mi, Ki, scale_mode, batch);            \
+      hipLaunchKernelGGL((quant_rowwise_split2<CH, true, false, true, W>), grid, dim3(64 * W), 0, \
+                         stream, nullptr, 0, nullptr, 0, nullptr, Mi, Ki, scale_mode, batch);    \
     } else {                                                                                     \
-      hipLaunchKernelGGL((quant_rowwise_split2<CH, false, false, true>), grid, b2, 0, stream,    \
-                         nullptr, 0, nullptr, 0, nullptr, Mi, Ki, scale_mode, batch);            \
+      hipLaunchKernelGGL((quant_rowwise_split2<CH, false, false, true, W>), grid, dim3(64 * W), 0, \
+                         stream, nullptr, 0, nullptr, 0, nullptr, Mi, Ki, scale_mode, batch);    \
     }                                                                                            \
     return 0;                                                                                    \
   }
-  CDIT_QUANT_CASE(1)
-  CDIT_QUANT_CASE(2)
-  CDIT_QUANT_CASE(3)
-  CDIT_QUANT_CASE(4)
-  CDIT_QUANT_CASE(5)
-  CDIT_QUANT_CASE(6)
-  CDIT_QUANT_CASE(8)
-  CDIT_QUANT_CASE(10)
-  CDIT_QUANT_CASE(12)
-  CDIT_QUANT_CASE(14)
-  CDIT_QUANT_CASE(15)
-  CDIT_QUANT_CASE(16)
+  if (need >= 2 && need < 8) {  // wavefronts per row as in launch_quant_rowwise
+    CDIT_QUANT_CASE(2, 1) CDIT_QUANT_CASE(2, 2) CDIT_QUANT_CASE(2, 3) CDIT_QUANT_CASE(2, 4)
+  } else if (need >= 8) {
+    CDIT_QUANT_CASE(4, 2) CDIT_QUANT_CASE(4, 3) CDIT_QUANT_CASE(4, 4) CDIT_QUANT_CASE(4, 5)
+    CDIT_QUANT_CASE(4, 6) CDIT_QUANT_CASE(4, 7) CDIT_QUANT_CASE(4, 8)
+  }
 #undef CDIT_QUANT_CASE
   if (need == 1) {  // rows of up to 512 elements: one wavefront each
     if (nt_load) {
