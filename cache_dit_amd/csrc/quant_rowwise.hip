@@ -212,12 +212,13 @@ __global__ __launch_bounds__(64 * WAVES) void quant_rowwise_split2(
 // that quantized Linear only -- quantizing the two sources in place of their copy saves the
 // copy's write and the quantizer's read of it. n1 = chunks (8 elements) of x1 per row; the
 // codes go to one [M, K1 + K2] buffer and are those of the quantizer on the concatenation.
-template <int CH, bool NT_LOAD>
-__global__ __launch_bounds__(64) void quant_rowwise_cat_regs(
+template <int CH, bool NT_LOAD, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void quant_rowwise_cat_regs(
     const uint16_t* __restrict__ x1, int64_t ld_x1, int n1, const uint16_t* __restrict__ x2,
     int64_t ld_x2, uint8_t* __restrict__ q, int64_t ld_q, float* __restrict__ scale, int M, int K,
     int scale_mode) {
-  const int lane = threadIdx.x & 63;
+  __shared__ uint32_t part[WAVES];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nchunks = K >> 3;
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
     const uint4* r1 = reinterpret_cast<const uint4*>(x1 + row * ld_x1);
@@ -236,25 +237,33 @@ __global__ __launch_bounds__(64) void quant_rowwise_cat_regs(
     uint32_t m = 0;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-      const int idx = c * 64 + lane;
+      const int idx = (WAVES * c + wave) * 64 + lane;
       v[c] = idx < nchunks ? load(idx) : make_uint4(0, 0, 0, 0);
       m = absmax2(absmax2(absmax2(absmax2(m, v[c].x), v[c].y), v[c].z), v[c].w);
     }
     m = wave_max_u32(fold2(m));
+    if constexpr (WAVES > 1) {  // the wavefronts of a row meet in LDS, as in quant_rowwise_split2
+      if (lane == 0) part[wave] = m;
+      __syncthreads();
+      m = part[0];
+#pragma unroll
+      for (int i = 1; i < WAVES; ++i) m = max(m, part[i]);
+      __syncthreads();
+    }
     const float s = row_scale(m, scale_mode);
-    if (lane == 0) scale[row] = s;
+    if (threadIdx.x == 0) scale[row] = s;
     uint2* qr = reinterpret_cast<uint2*>(q + row * ld_q);
-    if (scale_in_fast_window(s)) {  // wave-uniform
+    if (scale_in_fast_window(s)) {  // uniform
       const float r = 1.0f / s;
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
-        const int idx = c * 64 + lane;
+        const int idx = (WAVES * c + wave) * 64 + lane;
         if (idx < nchunks)
           qr[idx] = uint2{quant4<true>(v[c].x, v[c].y, s, r), quant4<true>(v[c].z, v[c].w, s, r)};
       }
     } else {  // cold path: re-reads the row
 #pragma unroll 1
-      for (int idx = lane; idx < nchunks; idx += 64) {
+      for (int idx = threadIdx.x; idx < nchunks; idx += 64 * WAVES) {
         const uint4 w = load(idx);
         qr[idx] = uint2{quant4<false>(w.x, w.y, s, 0.0f), quant4<false>(w.z, w.w, s, 0.0f)};
       }
@@ -653,35 +662,34 @@ int launch_quant_rowwise_cat2(const void* x1, int64_t K1, int64_t ld_x1, const v
                        reinterpret_cast<uintptr_t>(x2) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(q) % 8 == 0;
   if (!aligned || M <= 0) return 1;
-  dim3 grid((unsigned)(M < 256 * 256 ? M : 256 * 256)), block(64);
+  dim3 grid((unsigned)(M < 256 * 256 ? M : 256 * 256));
   const int need = (int)((K + 511) / 512);
   // the codes are read by the GEMM that follows: plain stores; loads of a large activation
   // carry the non-temporal hint (as launch_quant_rowwise chooses)
   const bool nt_load = M * K * 2 > ((int64_t)64 << 20);
   const uint16_t* p1 = static_cast<const uint16_t*>(x1);
   const uint16_t* p2 = static_cast<const uint16_t*>(x2);
-#define CDIT_QUANT_CASE(CH)                                                                         \
-  if (need <= CH) {                                                                                 \
+#define CDIT_QUANT_CASE(W, CH)                                                                      \
+  if (need <= W * CH) {                                                                             \
     if (nt_load) {                                                                                  \
-      hipLaunchKernelGGL((quant_rowwise_cat_regs<CH, true>), grid, block, 0, stream, p1, ld_x1,     \
-                         (int)(K1 / 8), p2, ld_x2, static_cast<uint8_t*>(q), ld_q, scale, (int)M,   \
-                         (int)K, scale_mode);                                                       \
+      hipLaunchKernelGGL((quant_rowwise_cat_regs<CH, true, W>), grid, dim3(64 * W), 0, stream, p1,  \
+                         ld_x1, (int)(K1 / 8), p2, ld_x2, static_cast<uint8_t*>(q), ld_q, scale,   \
+                         (int)M, (int)K, scale_mode);                                               \
     } else {                                                                                        \
-      hipLaunchKernelGGL((quant_rowwise_cat_regs<CH, false>), grid, block, 0, stream, p1, ld_x1,    \
-                         (int)(K1 / 8), p2, ld_x2, static_cast<uint8_t*>(q), ld_q, scale, (int)M,   \
-                         (int)K, scale_mode);                                                       \
+      hipLaunchKernelGGL((quant_rowwise_cat_regs<CH, false, W>), grid, dim3(64 * W), 0, stream, p1, \
+                         ld_x1, (int)(K1 / 8), p2, ld_x2, static_cast<uint8_t*>(q), ld_q, scale,   \
+                         (int)M, (int)K, scale_mode);                                               \
     }                                                                                               \
     return 0;                                                                                       \
   }
-  CDIT_QUANT_CASE(2)
-  CDIT_QUANT_CASE(4)
-  CDIT_QUANT_CASE(8)
-  CDIT_QUANT_CASE(12)
-  CDIT_QUANT_CASE(16)
-  CDIT_QUANT_CASE(20)
-  CDIT_QUANT_CASE(24)
-  CDIT_QUANT_CASE(30)
-  CDIT_QUANT_CASE(32)
+  if (need < 2) {  // wavefronts per row as in launch_quant_rowwise
+    CDIT_QUANT_CASE(1, 1)
+  } else if (need < 8) {
+    CDIT_QUANT_CASE(2, 1) CDIT_QUANT_CASE(2, 2) CDIT_QUANT_CASE(2, 3) CDIT_QUANT_CASE(2, 4)
+  } else {
+    CDIT_QUANT_CASE(4, 2) CDIT_QUANT_CASE(4, 3) CDIT_QUANT_CASE(4, 4) CDIT_QUANT_CASE(4, 5)
+    CDIT_QUANT_CASE(4, 6) CDIT_QUANT_CASE(4, 7) CDIT_QUANT_CASE(4, 8)
+  }
 #undef CDIT_QUANT_CASE
   return 1;
 }
