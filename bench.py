@@ -848,12 +848,13 @@ def main():
                       "(19 double + 38 single blocks, 4096 img + 512 txt tokens): per-token "
                       "quant + FP8 GEMM + epilogue; Linears that read one activation (q/k/v, "
                       "proj_mlp + q/k/v) share its quantization, and the independent Linears of "
-                      "one stage of a block (image stream + text stream) run as one batched GEMM "
-                      "launch, bit-identical to running each Linear on its own",
+                      "one stage of a block (image stream + text stream) run as one quantizer "
+                      "launch and one batched GEMM launch (two where the tile cost model splits "
+                      "the stage), bit-identical to running each Linear on its own",
           "quant_type": "float8_per_row",
           "launch": launch_mode,
           "linears_per_step": n_layers,
-          "gemm_launches_per_step": n_runs,
+          "stages_per_step": n_runs,
           "linear_flop_per_step": step_flop,
           "batch": 1,
       },
