@@ -455,3 +455,21 @@ def test_weight_only_sibling_groups_and_stream_batches_in_a_model():
     ds.batch_streams(model, False)
     assert cache_dit.group_sibling_linears_(model, enable=False) == 0
     assert torch.equal(model(**inputs), y0)
+
+  # Qwen-Image- and Wan-shaped toy models: stream batches and sibling groups of weight-only Linears
+  qwen = ds.QwenImageLikeTransformer(dim=256, heads=2, mlp=512, n_layers=2, in_channels=64,
+                                     text_dim=128).to(torch.bfloat16).cuda()
+  cache_dit.quantize(qwen, cache_dit.QuantizeConfig(quant_type="float8_weight_only"))
+  qin = ds.qwen_image_like_inputs("cuda", n_img=200, n_txt=24, in_channels=64, text_dim=128)
+  wan = ds.WanLikeTransformer(dim=256, heads=2, ffn=512, n_layers=2, in_channels=64,
+                              text_dim=128).to(torch.bfloat16).cuda()
+  cache_dit.quantize(wan, cache_dit.QuantizeConfig(quant_type="float8_weight_only"))
+  winp = ds.wan_like_inputs("cuda", n_tokens=200, n_txt=48, in_channels=64, text_dim=128)
+  with torch.no_grad():
+    q0 = qwen(**qin)
+    assert ds.batch_streams(qwen) == 2
+    assert torch.equal(qwen(**qin), q0)
+    w0 = wan(**winp)
+    assert cache_dit.group_sibling_linears_(wan, lambda: wan(**winp)) == 2 * 2
+    assert wan.blocks[0].attn1.to_q.sibling_group.weight_only
+    assert torch.equal(wan(**winp), w0)
