@@ -47,8 +47,9 @@ EXPORTS = (
     "cdit_fp8_comm_per_token_dequant",
     "cdit_fp8_comm_qkv_permute_quant",
     "cdit_fp8_comm_qkv_permute_dequant",
-    "cdit_set_gemm_variant",
+    "cdit_debug_set_gemm_variant",
     "cdit_debug_set_quant_hints",
+    "cdit_debug_mfma_only",
     "cdit_stream_capture_id",
 )
 
@@ -70,10 +71,12 @@ def _bind(L: ctypes.CDLL) -> None:
   L.cdit_device_arch.argtypes = [ctypes.c_char_p, ci]
   L.cdit_stream_capture_id.restype = ci
   L.cdit_stream_capture_id.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64)]
-  L.cdit_set_gemm_variant.restype = ci
-  L.cdit_set_gemm_variant.argtypes = [ci]
+  L.cdit_debug_set_gemm_variant.restype = ci
+  L.cdit_debug_set_gemm_variant.argtypes = [ci]
   L.cdit_debug_set_quant_hints.restype = ci
   L.cdit_debug_set_quant_hints.argtypes = [ci]
+  L.cdit_debug_mfma_only.restype = ci
+  L.cdit_debug_mfma_only.argtypes = [vp, ci, ci, ci, ctypes.POINTER(ctypes.c_double), vp]
   L.cdit_fp8_quant_rowwise.restype = ci
   L.cdit_fp8_quant_rowwise.argtypes = [vp, i64, i64, i64, vp, i64, vp, ci, vp]
   L.cdit_fp8_quant_rowwise_cat2.restype = ci
@@ -164,7 +167,7 @@ def device_arch() -> str:
 
 
 def set_gemm_variant(variant: int) -> int:
-  return load().cdit_set_gemm_variant(int(variant))
+  return load().cdit_debug_set_gemm_variant(int(variant))
 
 
 def stream_capture_id(stream: int) -> int:

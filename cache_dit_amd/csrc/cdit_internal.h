@@ -121,6 +121,12 @@ int launch_comm_qkv_permute_quant(const void* x, int B, int S, int P, int N, int
 int launch_comm_qkv_permute_dequant(const void* qx, int S, int B, int N, int D, int64_t qs, int64_t qb,
                                     int64_t qn, void* x, hipStream_t stream);
 
+// Measurement aid: `blocks` workgroups of four wavefronts run `iters` rounds of 16 MFMAs
+// (v_mfma_f32_16x16x128_f8f6f4) on register operands; out: blocks * 256 floats. *flop gets the
+// floating-point operations of the launch.
+int launch_mfma_only(float* out, int blocks, int iters, bool random_operands, double* flop,
+                     hipStream_t stream);
+
 void set_error(const char* fmt, ...);
 
 }  // namespace cdit

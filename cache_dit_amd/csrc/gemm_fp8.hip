@@ -295,7 +295,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_tiled(GemmArgs g, int til
 // rows lane bit 3 is row bit 4, hence swz_b. Before they are stored the packed words
 // change lanes once more (ds_bpermute_b32) so that adjacent lanes hold adjacent
 // bytes: the memory pipeline only merges those into one request (see the epilogue).
-template <int BM_, int BN_, int GROUP_M_, int DEPTH_ = 2>
+template <int BM_, int BN_, int GROUP_M_, int DEPTH_ = 2, bool FULL_LINE_ = true>
 struct CfgWide {
   static constexpr int BM = BM_, BN = BN_, GROUP_M = GROUP_M_;
   // K steps the DMA stream runs ahead of the MFMAs. 2 for the large tiles (their
@@ -327,6 +327,27 @@ struct CfgWide {
   static_assert(TM * TN <= 64, "accumulators: at most 256 registers");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
   static_assert(DEPTH >= 2 && (DEPTH - 2) * ND + NDA < 63, "DMA instructions in flight: vmcnt has 6 bits");
+
+  // Which columns of the tile a wave owns. A pair of B fragments gives a lane 8 consecutive
+  // output columns and the four lanes of a row 32 columns = 64 bytes of a 16-bit output: half
+  // a 128-byte memory line. FULL_LINE: two neighbouring pairs are stored together, 8 lanes on
+  // the 128 contiguous bytes of a row, so that every store instruction writes whole lines
+  // (with 16 rows x 64 bytes per instruction a line leaves the L2 in two halves under the
+  // write-once hint). A wave tile is then LP line-wide column blocks of 64 plus, where WN is
+  // an odd multiple of 32, one half-line block; the line-wide blocks of wave column wn start
+  // at 64 LP wn, the half-line blocks follow behind all of them at 128 LP + 32 wn, so that
+  // every line-wide block starts on a line boundary of the tile (WN = 96: wave column 0 owns
+  // columns 0..63 and 128..159, wave column 1 owns 64..127 and 160..191).
+  static constexpr bool FULL_LINE = FULL_LINE_;
+  static constexpr int NPAIR = TN / 2;               // fragment pairs per row of blocks
+  static constexpr int LP = FULL_LINE ? WN / 64 : 0;  // pairs of pairs stored as whole lines
+  static constexpr int NHALF = NPAIR - 2 * LP;        // pairs stored as half lines
+  static constexpr bool SPLIT_COLS = FULL_LINE && WN % 64 != 0;
+  // first column (inside the tile) of fragment pair u in wave column wn
+  __host__ __device__ static constexpr int colbase(int u, int wn) {
+    if (!SPLIT_COLS) return wn * WN + 32 * u;
+    return u < 2 * LP ? wn * 64 * LP + 32 * u : 128 * LP + 32 * wn + 32 * (u - 2 * LP);
+  }
 
   // Issue schedule of a K step: which LDS reads and DMA instructions go in front of
   // which MFMA. An LDS read pair or a DMA instruction holds the wave's instruction
@@ -556,11 +577,17 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
   // operand read map
   const int r16 = lane & 15, kg = lane >> 4;
   const int brow = 8 * (r16 >> 2) + (r16 & 3);
-  uint32_t rd_a[2], rd_b[2];
+  // B fragments: pair u of this wave reads panel rows colbase(u, wn) + brow (+ 4 for the
+  // second fragment of the pair). The pairs stored as whole lines are contiguous from
+  // colbase(0, wn) on; the half-line pair (SPLIT_COLS) has a base of its own, rd_bh. All
+  // bases are multiples of 32, which leaves swz_b (row bits 1 and 4) to brow alone.
+  uint32_t rd_a[2], rd_b[2], rd_bh[2];
 #pragma unroll
   for (int e = 0; e < 2; ++e) {
     rd_a[e] = (wm * C::WM + r16) * BKW + (((2 * kg + e) ^ swz_a(wm * C::WM + r16)) << 4);
-    rd_b[e] = (wn * C::WN + brow) * BKW + (((2 * kg + e) ^ swz_b(wn * C::WN + brow)) << 4);
+    const uint32_t chunk = ((2 * kg + e) ^ swz_b(brow)) << 4;
+    rd_b[e] = (C::colbase(0, wn) + brow) * BKW + chunk;
+    rd_bh[e] = (C::colbase(C::NPAIR - 1, wn) + brow) * BKW + chunk;
   }
   // __restrict__: loads through a restrict-qualified pointer carry alias scope
   // information. Without it the compiler assumes that an LDS read may alias any
@@ -573,9 +600,10 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
   auto read_b = [&](const uint8_t* __restrict__ st, int j) -> v8i {
-    const int ro = 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
-    const v4i lo = *reinterpret_cast<const v4i*>(st + rd_b[0] + ro * BKW);
-    const v4i hi = *reinterpret_cast<const v4i*>(st + rd_b[1] + ro * BKW);
+    const bool half = C::SPLIT_COLS && (j >> 1) >= 2 * C::LP;
+    const int ro = (half ? 0 : 32 * (j >> 1)) + 4 * (j & 1);
+    const v4i lo = *reinterpret_cast<const v4i*>(st + (half ? rd_bh[0] : rd_b[0]) + ro * BKW);
+    const v4i hi = *reinterpret_cast<const v4i*>(st + (half ? rd_bh[1] : rd_b[1]) + ro * BKW);
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
 
@@ -609,8 +637,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
     // epilogue operands of this tile, fetched two steps before they are needed:
     // acc[i][4t+q][e] is out[m][n] with
     //   m = m0 + wm*WM + 16i + (lane&15),
-    //   n = n0 + wn*WN + 64t + 32(q>>1) + 8(lane>>4) + 4(q&1) + e
-    const int nw = n0 + wn * C::WN + 8 * kg;
+    //   n = n0 + colbase(2t + (q>>1), wn) + 8(lane>>4) + 4(q&1) + e
     const int mw = m0 + wm * C::WM + r16;
     v4f bs[TN];
     uint2 bi[TN];  // bias stays packed (bf16 pairs) until used: registers are scarce
@@ -668,7 +695,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
         } else {
 #pragma unroll
           for (int j = 0; j < TN; ++j) {
-            const int n = nw + 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
+            const int n = n0 + C::colbase(j >> 1, wn) + 8 * kg + 4 * (j & 1);
             bs[j] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(bs_buf, n * 4, 0, 0));
             bi[j] = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(bi_buf, n * 2, 0, 0));
           }
@@ -781,7 +808,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
       auto read_staged = [&](const uint8_t* __restrict__ ep) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          const int c = wn * C::WN + 8 * kg + 64 * (j >> 2) + 32 * ((j >> 1) & 1) + 4 * (j & 1);
+          const int c = C::colbase(j >> 1, wn) + 8 * kg + 4 * (j & 1);
           bs[j] = *reinterpret_cast<const v4f*>(ep + C::EPI_BS + c * 4);
           bi[j] = *reinterpret_cast<const uint2*>(ep + C::EPI_BI + c * 2);
         }
@@ -803,26 +830,42 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
       cur_epilogue = grp.epilogue[cur];
     }
     const int cur_N = n_of(cur);
-    uint8_t* const out_wave = reinterpret_cast<uint8_t*>(cur_out) +
-                              ((int64_t)(m0 + wm * C::WM) * cur_ldo + (n0 + wn * C::WN)) * OB;
+    uint8_t* const out_wave =
+        reinterpret_cast<uint8_t*>(cur_out) + ((int64_t)(m0 + wm * C::WM) * cur_ldo + n0) * OB;
     const int rows_wave = m_of(cur_act) - (m0 + wm * C::WM);  // rows of the wave tile that exist
     // The memory pipeline merges the lanes of a store into one request only when
     // adjacent lanes write adjacent bytes: with lane = 16 kg + r16 holding row r16,
     // 16-byte piece kg, every lane is a request of its own (measured: 294 clocks per
     // store instruction with four waves storing, against 77 when lanes 4r .. 4r+3 hold
-    // the 64 contiguous bytes of row r). 16-bit outputs are therefore moved to that
-    // arrangement with ds_bpermute_b32 (the LDS crossbar, no LDS memory) before they
-    // are stored: lane L takes the packed words of lane 16 (L & 3) + (L >> 2).
+    // the 64 contiguous bytes of row r). 16-bit outputs are therefore moved with
+    // ds_bpermute_b32 (the LDS crossbar, no LDS memory) before they are stored.
+    // Half-line pairs: lane L takes the packed words of lane 16 (L & 3) + (L >> 2) and
+    // holds piece L & 3 of row L >> 2 (16 rows x 64 bytes per store instruction).
+    // Whole lines (pairs 2v and 2v+1 together, 64 columns): first the two halves of a row
+    // of 16 lanes trade words (DPP row_ror:8 under a bank mask), P = {rows 0-7: pair 2v |
+    // rows 8-15: pair 2v+1 of the row 8 above}, Q = {rows 0-7: pair 2v of the row 8 below |
+    // rows 8-15: pair 2v+1}; then lane L = 8 row + piece takes P (store A, block rows 0-7)
+    // and Q (store B, block rows 8-15) from lane 16 (piece & 3) + 8 (piece >> 2) + row: 8
+    // lanes on the 128 contiguous bytes of a row, 8 rows per store instruction.
     constexpr bool PERMUTE = OUT != CDIT_DT_F32;
+    constexpr int LP = PERMUTE ? C::LP : 0, NP = TN / 2, NH = NP - 2 * LP;
     const int st_row = PERMUTE ? lane >> 2 : r16, st_piece = PERMUTE ? lane & 3 : kg;
     const int bp_addr = 4 * (16 * (lane & 3) + (lane >> 2));
+    const int bp_line = 4 * (16 * (lane & 3) + 8 * ((lane >> 2) & 1) + (lane >> 3));
     const uint32_t out_lane = ((uint32_t)st_row * (uint32_t)cur_ldo + 8u * st_piece) * OB;
-    uint32_t out_off[TN / 2];
+    const uint32_t out_lane_line = ((uint32_t)(lane >> 3) * (uint32_t)cur_ldo + 8u * (lane & 7)) * OB;
+    const uint32_t rows8 = 8u * (uint32_t)cur_ldo * OB;  // block rows 8-15 of a whole-line store
+    uint32_t out_off[NH > 0 ? NH : 1], out_off_line[LP > 0 ? LP : 1];
 #pragma unroll
-    for (int u = 0; u < TN / 2; ++u)
-      out_off[u] = n0 + wn * C::WN + 8 * st_piece + 64 * (u >> 1) + 32 * (u & 1) < cur_N
-                       ? out_lane + (64 * (u >> 1) + 32 * (u & 1)) * OB
-                       : kNoColumn;
+    for (int h = 0; h < NH; ++h) {
+      const int col = C::colbase(2 * LP + h, wn);
+      out_off[h] = n0 + col + 8 * st_piece < cur_N ? out_lane + col * OB : kNoColumn;
+    }
+#pragma unroll
+    for (int v = 0; v < LP; ++v) {
+      const int col = C::colbase(2 * v, wn);
+      out_off_line[v] = n0 + col + 8 * (lane & 7) < cur_N ? out_lane_line + col * OB : kNoColumn;
+    }
     auto out_row_of = [&](int i) {
       // (made a scalar explicitly: a descriptor the compiler takes for divergent is
       // applied in a loop over its distinct values)
@@ -833,13 +876,22 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
     // 16-bit outputs: the permuted words of a row of blocks are stored while the next
     // row is being computed, so the latency of the permutation is not waited for; the
     // last row's after the two copies of the epilogue have joined
-    uint32_t moved[TN / 2][4];
+    uint32_t moved[NH > 0 ? NH : 1][4], moved_a[LP > 0 ? LP : 1][4], moved_b[LP > 0 ? LP : 1][4];
     auto store_moved = [&](int i) {
       const __amdgpu_buffer_rsrc_t row = out_row_of(i);
 #pragma unroll
-      for (int u = 0; u < TN / 2; ++u)
+      for (int v = 0; v < LP; ++v) {
         __builtin_amdgcn_raw_buffer_store_b128(
-            v4u{moved[u][0], moved[u][1], moved[u][2], moved[u][3]}, row, (int)out_off[u], 0, kStoreOnce);
+            v4u{moved_a[v][0], moved_a[v][1], moved_a[v][2], moved_a[v][3]}, row,
+            (int)out_off_line[v], 0, kStoreOnce);
+        __builtin_amdgcn_raw_buffer_store_b128(
+            v4u{moved_b[v][0], moved_b[v][1], moved_b[v][2], moved_b[v][3]}, row,
+            (int)(out_off_line[v] + rows8), 0, kStoreOnce);
+      }
+#pragma unroll
+      for (int h = 0; h < NH; ++h)
+        __builtin_amdgcn_raw_buffer_store_b128(
+            v4u{moved[h][0], moved[h][1], moved[h][2], moved[h][3]}, row, (int)out_off[h], 0, kStoreOnce);
     };
     auto epilogue = [&](auto gelu_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
@@ -872,7 +924,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
             __builtin_amdgcn_raw_buffer_store_b128(
                 v4u{__float_as_uint(v[4]), __float_as_uint(v[5]), __float_as_uint(v[6]),
                     __float_as_uint(v[7])},
-                out_row, (int)(out_off[u] + 16u), 0, kStoreOnce);
+                out_row, (int)(out_off[u] + 16u), 0, kStoreOnce);  // (fp32: every pair is a half-line pair)
           } else {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -889,10 +941,22 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
           __builtin_amdgcn_sched_barrier(0);
           if (i > 0) store_moved(i - 1);
 #pragma unroll
-          for (int u = 0; u < TN / 2; ++u)
+          for (int v = 0; v < LP; ++v)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const int w0 = (int)pk[2 * v][k], w1 = (int)pk[2 * v + 1][k];
+              // row_ror:8 = 0x128; bank mask 0xc: lanes 8-15 of a row take the other half's
+              // word, lanes 0-7 keep `old`; 0x3 the other way round
+              const int p = __builtin_amdgcn_update_dpp(w0, w1, 0x128, 0xf, 0xc, false);
+              const int q = __builtin_amdgcn_update_dpp(w1, w0, 0x128, 0xf, 0x3, false);
+              moved_a[v][k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_line, p);
+              moved_b[v][k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_line, q);
+            }
+#pragma unroll
+          for (int h = 0; h < NH; ++h)
 #pragma unroll
             for (int k = 0; k < 4; ++k)
-              moved[u][k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_addr, (int)pk[u][k]);
+              moved[h][k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_addr, (int)pk[2 * LP + h][k]);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -1338,7 +1402,7 @@ bool tiled_ok(const GemmArgs& g) {
 }  // namespace
 
 // Kernel variants. The entry point picks one by shape; tests and the tuning hook
-// (cdit_set_gemm_variant) can force any of them.
+// (cdit_debug_set_gemm_variant) can force any of them.
 //          BM   BN  WGM WGN direct epiLDS groupM stages
 typedef Cfg<256, 256, 2, 2, false, false, 8> V0;      // register staging, direct stores
 typedef Cfg<256, 256, 2, 2, true, true, 8> V1;        // LDS-DMA, 2 stages, 4 waves
@@ -1352,6 +1416,10 @@ typedef CfgWide<256, 192, 4> V15;                     // ... 128x96 wave tiles
 typedef CfgWide<128, 192, 4, 3> V16;                  // ... 64x96 wave tiles, DMA 3 steps ahead
 typedef CfgWide<64, 128, 8, 5> V17;                   // ... 32x64 wave tiles, DMA 5 steps ahead
 typedef CfgWide<128, 128, 4, 4> V18;                  // ... 64x64 wave tiles, DMA 4 steps ahead
+// the two large tiles with contiguous wave columns and half-line output stores (16 rows x 64
+// bytes per store instruction), kept to measure the whole-line stores against: variants 112, 114
+typedef CfgWide<256, 256, 4, 2, false> V12H;
+typedef CfgWide<288, 192, 4, 2, false> V14H;
 
 // The M = 1 kernel when the shape fits it (variant 51 forces it, 50 the 16-row kernel);
 // returns 1 when it is not taken.
@@ -1523,6 +1591,8 @@ int launch_bf16_variant(const GemmArgs& g, int variant, WideOk wide_ok, hipStrea
     case 16: return wide_ok(V16::DEPTH) ? launch_wide<V16>(g, stream) : launch_tiled<V6>(g, stream);
     case 17: return wide_ok(V17::DEPTH) ? launch_wide<V17>(g, stream) : launch_tiled<V6>(g, stream);
     case 18: return wide_ok(V18::DEPTH) ? launch_wide<V18>(g, stream) : launch_tiled<V6>(g, stream);
+    case 112: return wide_ok(V12H::DEPTH) ? launch_wide<V12H>(g, stream) : launch_tiled<V6>(g, stream);
+    case 114: return wide_ok(V14H::DEPTH) ? launch_wide<V14H>(g, stream) : launch_tiled<V6>(g, stream);
     default:
       set_error("cdit_fp8_gemm_rowwise: unknown kernel variant %d", variant);
       return CDIT_EINVAL;
@@ -1637,6 +1707,55 @@ int launch_gemm_fp8_grouped(const GemmArgs& common, const GemmGroup& grp, int va
     case 18: return wide_ok(V18::DEPTH) ? launch_wide_grouped<V18>(common, grp, stream) : -1;
     default: return -1;  // the kernels without a tile stream have no grouped form
   }
+}
+
+// ---------------------------------------------------------------------------
+// Measurement aid: a loop of nothing but the wide kernel's MFMA instruction on register
+// operands (one wave per SIMD, four per workgroup, 16 independent accumulators), so that the
+// rate the matrix cores sustain before a byte is moved can be timed on the part at hand.
+// RANDOM: operands are pseudo-random e4m3 codes with |value| <= 1.75 (what the benchmark's
+// weights are drawn from); otherwise every code is 1.0. The clock a power-limited part
+// settles at depends on the operand bits, and with it the ceiling of any FP8 kernel.
+namespace {
+template <bool RANDOM>
+__global__ __launch_bounds__(256) void mfma_only_loop(float* out, int iters) {
+  constexpr int NACC = 16, NOP = 4;
+  v8i a[NOP], b[NOP];
+  uint32_t h = (blockIdx.x * 256u + threadIdx.x) * 2654435761u + 12345u;
+#pragma unroll
+  for (int o = 0; o < NOP; ++o)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      h = h * 1664525u + 1013904223u;
+      a[o][i] = RANDOM ? (int)((h ^ (h >> 13)) & 0xBFBFBFBFu) : 0x38383838;
+      h = h * 1664525u + 1013904223u;
+      b[o][i] = RANDOM ? (int)((h ^ (h >> 11)) & 0xBFBFBFBFu) : 0x38383838;
+    }
+  v4f acc[NACC];
+#pragma unroll
+  for (int j = 0; j < NACC; ++j) acc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < NACC; ++j)
+      acc[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[j % NOP], b[(j / NOP) % NOP], acc[j],
+                                                                0, 0, 0, 0, 0, 0);
+  }
+  float sum = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NACC; ++j) sum += (acc[j][0] + acc[j][1]) + (acc[j][2] + acc[j][3]);
+  out[blockIdx.x * 256 + threadIdx.x] = sum;
+}
+}  // namespace
+
+int launch_mfma_only(float* out, int blocks, int iters, bool random_operands, double* flop,
+                     hipStream_t stream) {
+  if (random_operands) {
+    hipLaunchKernelGGL(mfma_only_loop<true>, dim3(blocks), dim3(256), 0, stream, out, iters);
+  } else {
+    hipLaunchKernelGGL(mfma_only_loop<false>, dim3(blocks), dim3(256), 0, stream, out, iters);
+  }
+  if (flop) *flop = (double)blocks * 4.0 * iters * 16.0 * (2.0 * 16 * 16 * 128);
+  return 0;
 }
 
 }  // namespace cdit

@@ -367,14 +367,27 @@ int cdit_stream_capture_id(void* stream, uint64_t* id);
  * safe and must not be called while another thread is inside the library. A production
  * caller never needs them (the default, -1, is the automatic choice).
  *
- * cdit_set_gemm_variant: forces the kernel variant the GEMM entry points pick (-1 = by
+ * cdit_debug_set_gemm_variant: forces the kernel variant the GEMM entry points pick (-1 = by
  * shape). Returns the previous value. The tests use it to run every variant on one shape.
  * cdit_debug_set_quant_hints: forces the cache hints of the per-row quantizer (0: loads
  * and stores non-temporal, 1: neither, 2: loads, 3: stores; anything else = -1 = by
  * size). Returns the previous value. Results never depend on it.
  */
-int cdit_set_gemm_variant(int variant);
+int cdit_debug_set_gemm_variant(int variant);
 int cdit_debug_set_quant_hints(int hints);
+
+/*
+ * Measurement aid, not part of the operator interface (no counterpart in the reference):
+ * launches `blocks` workgroups of four wavefronts that run `iters` rounds of 16 independent
+ * v_mfma_f32_16x16x128_f8f6f4 instructions (the FP8 GEMM's instruction) on register
+ * operands and nothing else, with pseudo-random e4m3 operands (random_operands != 0) or
+ * all-ones operands. out_f32: blocks * 256 floats of device memory (written so that the loop
+ * is not dead code). *flop (host memory, may be null) receives the floating-point operations
+ * of the launch. Timing it gives the rate the matrix cores of the part at hand sustain before
+ * a byte is moved: the ceiling bench.py reports next to the GEMM's rate.
+ */
+int cdit_debug_mfma_only(void* out_f32, int blocks, int iters, int random_operands, double* flop,
+                         void* stream);
 
 #ifdef __cplusplus
 }

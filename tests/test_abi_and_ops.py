@@ -55,7 +55,7 @@ def test_argument_validation_without_gpu():
   assert L.cdit_w8a16_gemm(one, one, None, None, one, 4, 4, 32, 32, 32, 4, 0, 1, None) == 1
   assert b"null pointer" in L.cdit_last_error()
   assert L.cdit_w8a16_gemm(one, one, one, None, one, 0, 4, 32, 32, 32, 4, 0, 1, None) == 0
-  assert L.cdit_set_gemm_variant(3) == -1 and L.cdit_set_gemm_variant(-1) == 3
+  assert L.cdit_debug_set_gemm_variant(3) == -1 and L.cdit_debug_set_gemm_variant(-1) == 3
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -158,7 +158,7 @@ def test_output_stores_are_unconditional(wide_kernels):
   branch); for 16-bit outputs the stores of the last row of blocks follow the join."""
   counted = 0
   for name, code in wide_kernels.items():
-    m = re.search(r"gemm_fp8_wideINS0_7CfgWideILi(\d+)ELi(\d+)ELi\d+ELi\d+EEELi(\d)E", name)
+    m = re.search(r"gemm_fp8_wideINS0_7CfgWideILi(\d+)ELi(\d+)ELi\d+ELi\d+ELb[01]EEELi(\d)E", name)
     if not m:
       continue
     bm, bn, out = int(m.group(1)), int(m.group(2)), int(m.group(3))
@@ -191,7 +191,7 @@ def test_staged_epilogue_operands_are_waited_for(wide_kernels):
   last two steps, nothing else may be in flight in front of the read."""
   checked = 0
   for name, code in wide_kernels.items():
-    m = re.search(r"gemm_fp8_wideINS0_7CfgWideILi(\d+)ELi(\d+)ELi\d+ELi(\d+)EEELi(\d)E", name)
+    m = re.search(r"gemm_fp8_wideINS0_7CfgWideILi(\d+)ELi(\d+)ELi\d+ELi(\d+)ELb[01]EEELi(\d)E", name)
     if not m or int(m.group(3)) <= 3:
       continue
     bm, bn = int(m.group(1)), int(m.group(2))
