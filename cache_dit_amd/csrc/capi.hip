@@ -148,7 +148,7 @@ int cdit_stream_capture_id(void* stream, uint64_t* id) {
   return CDIT_OK;
 }
 
-int cdit_set_gemm_variant(int variant) {
+int cdit_debug_set_gemm_variant(int variant) {
   int prev = g_gemm_variant;
   g_gemm_variant = variant;
   return prev;
@@ -158,6 +158,20 @@ int cdit_debug_set_quant_hints(int hints) {
   int prev = cdit::g_quant_variant;
   cdit::g_quant_variant = hints >= 0 && hints <= 7 ? hints : -1;
   return prev;
+}
+
+int cdit_debug_mfma_only(void* out_f32, int blocks, int iters, int random_operands, double* flop,
+                         void* stream) {
+  const char* fn = "cdit_debug_mfma_only";
+  if (!out_f32 || blocks < 1 || blocks > 65536 || iters < 1) {
+    set_error("%s: out is null, or blocks=%d / iters=%d out of range", fn, blocks, iters);
+    return CDIT_EINVAL;
+  }
+  int rc = check_arch();
+  if (rc) return rc;
+  rc = launch_mfma_only(static_cast<float*>(out_f32), blocks, iters, random_operands != 0, flop,
+                        static_cast<hipStream_t>(stream));
+  return rc ? rc : after_launch(fn);
 }
 
 // consumer_follows: the codes are read by a GEMM launched right behind (the fused
@@ -331,6 +345,8 @@ int cdit_fp8_ln_modulate_quant(const void* x_bf16, int64_t M, int64_t K, int64_t
     set_error("%s: null pointer argument", fn);
     return CDIT_EINVAL;
   }
+  // one modulation vector for all rows may be spelled with any large count
+  if (rows_per_mod > M) rows_per_mod = M;
   int rc = check_arch();
   if (rc) return rc;
   rc = launch_ln_modulate_quant(x_bf16, M, K, ld_x, shift_bf16, scale_bf16, ld_mod, rows_per_mod,

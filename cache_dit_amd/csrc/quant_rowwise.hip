@@ -418,92 +418,285 @@ __device__ __forceinline__ uint32_t modulate1(float x, float mean, float rstd, f
   return bf16_bits(u + sh);
 }
 
-// the same for a packed pair, every rounding step through the hardware converter
-__device__ __forceinline__ uint32_t modulate2(uint32_t xw, float mean, float rstd, uint32_t scw,
-                                              uint32_t shw) {
-  const uint32_t n = pk_bf16((bf16_lo(xw) - mean) * rstd, (bf16_hi(xw) - mean) * rstd);
-  const uint32_t t = pk_bf16(1.0f + bf16_lo(scw), 1.0f + bf16_hi(scw));
-  const uint32_t u = pk_bf16(bf16_lo(n) * bf16_lo(t), bf16_hi(n) * bf16_hi(t));
-  return pk_bf16(bf16_lo(u) + bf16_lo(shw), bf16_hi(u) + bf16_hi(shw));
+// Wave-wide reductions that leave the result in lane 63: four butterfly steps inside each
+// row of 16 lanes (DPP quad_perm / row_half_mirror / row_mirror), then the row results travel
+// up with row_bcast:15 into rows 1 and 3 and row_bcast:31 into rows 2 and 3. Six DPP
+// instructions, a fixed order of operations.
+template <class Op>
+__device__ __forceinline__ uint32_t wave_reduce_to_lane63(uint32_t v, Op op) {
+  v = op(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  v = op(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  v = op(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, false));  // row_half_mirror
+  v = op(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xf, 0xf, false));  // row_mirror
+  // rows 1 and 3 take in lane 15 of the row below them; the other rows keep their value
+  v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)Op::identity(), (int)v, 0x142, 0xa, 0xf, false));
+  // rows 2 and 3 take in lane 31
+  v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)Op::identity(), (int)v, 0x143, 0xc, 0xf, false));
+  return v;
+}
+struct AddF32 {
+  static __device__ __forceinline__ uint32_t identity() { return 0u; }  // +0.0f
+  __device__ __forceinline__ uint32_t operator()(uint32_t a, uint32_t b) const {
+    return __float_as_uint(__uint_as_float(a) + __uint_as_float(b));
+  }
+};
+struct MaxU32 {
+  static __device__ __forceinline__ uint32_t identity() { return 0u; }
+  __device__ __forceinline__ uint32_t operator()(uint32_t a, uint32_t b) const { return a > b ? a : b; }
+};
+
+// x.lo * y.lo + x.hi * y.hi + acc of two packed bf16 pairs in one instruction
+// (v_dot2c_f32_bf16). The products are exact in fp32; how the three-term sum is rounded
+// inside is the instruction's own business, which row statistics tolerate.
+__device__ __forceinline__ float dot_pair(uint32_t a, uint32_t b, float acc) {
+  typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf, a), __builtin_bit_cast(v2bf, b), acc,
+                                         false);
 }
 
-template <int CH, bool WRITE_Y>
-__global__ __launch_bounds__(64) void ln_modulate_quant_regs(
+// fp32 -> nearest-even bf16, widened back to fp32, in one instruction: v_cvt_pk_bf16_f32 with
+// a zero in the low half leaves the rounded value's bits where an fp32 has them.
+__device__ __forceinline__ float round_bf16_wide(float f) { return __uint_as_float(pk_bf16(0.0f, f)); }
+
+// two widened bf16 values -> packed pair (their high halves), one byte permute
+__device__ __forceinline__ uint32_t pack_wide(float lo, float hi) {
+  return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+}
+
+// A workgroup of WAVES wavefronts owns `rows_per_wg` consecutive rows; chunk (WAVES c + wave)
+// * 64 + lane of a row belongs to this thread, CH chunks of 8 elements per thread.
+//  * What is the same for every row of a modulation vector stays in registers from row to row,
+//    widened to fp32: t = bf16(1 + scale[k]) (0 beyond K) and shift[k].
+//  * The next row is fetched while the current one is worked on (two register sets, taken in
+//    turn). Every load and store of the row loop is a buffer access without a branch around
+//    it (beyond the row: zeros read, nothing written; the scale leaves through a lane offset
+//    beyond its descriptor for every thread but one), so that the compiler can count the
+//    accesses in flight: with a store under a lane mask it waits for everything (vmcnt(0))
+//    where it needs the prefetched row, which puts the latency of the previous row's stores
+//    into every row.
+//  * Statistics in one pass over the packed row: sum and sum of squares with one
+//    v_dot2c_f32_bf16 each per pair, var = E[x^2] - mean^2; when that difference has lost more
+//    than two bits to cancellation (mean^2 > 4 var, a zero or negative result, non-finite
+//    input) the deviations are summed in a second pass as the unfused LayerNorm does. One
+//    workgroup reduction for both sums, one for the amax: lane 63 of every wavefront
+//    leaves its partial result in an LDS slot (slots alternate with the row parity, so one
+//    barrier each).
+//  * Per element: widen, one FMA for (x - mean) rstd (as x rstd - mean rstd), then every step
+//    that the unfused bf16 op sequence rounds is one v_cvt_pk_bf16_f32 that rounds and
+//    widens at once; amax as integer maxima of the raw bits, positive and negative values
+//    apart (a NaN pattern is the largest of either kind, as in torch.amax); the e4m3 cast
+//    as in the stand-alone quantizer. About 14 VALU instructions per element.
+template <int CH, bool WRITE_Y, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void ln_modulate_quant_rows(
     const uint16_t* __restrict__ x, int64_t ld_x, const uint16_t* __restrict__ shift,
     const uint16_t* __restrict__ scale_mod, int64_t ld_mod, int rows_per_mod, float eps,
     uint16_t* __restrict__ y, int64_t ld_y, uint8_t* __restrict__ q, int64_t ld_q,
-    float* __restrict__ scale, int M, int K, int scale_mode) {
-  const int lane = threadIdx.x & 63;
+    float* __restrict__ scale, int M, int K, int scale_mode, int rows_per_wg) {
+  constexpr int kCached = 0;
+  typedef unsigned int u4v __attribute__((ext_vector_type(4)));
+  typedef unsigned int u2v __attribute__((ext_vector_type(2)));
+  __shared__ float red_f[2][8][2];
+  __shared__ uint32_t red_m[2][8];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int nchunks = K >> 3;
   const float inv_k = 1.0f / (float)K;
-  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
-    const uint4* xr = reinterpret_cast<const uint4*>(x + row * ld_x);
-    const int64_t mod_row = (row / rows_per_mod) * ld_mod;
-    const uint4* shr = reinterpret_cast<const uint4*>(shift + mod_row);
-    const uint4* scr = reinterpret_cast<const uint4*>(scale_mod + mod_row);
-    uint4 v[CH];
-    float sum = 0.0f;
+  const int row0 = blockIdx.x * rows_per_wg;
+  const int row_end = min(M, row0 + rows_per_wg);
+  if (row0 >= row_end) return;
+  int idx[CH];
+#pragma unroll
+  for (int c = 0; c < CH; ++c) idx[c] = (WAVES * c + wave) * 64 + lane;
+  auto row_buf = [&](const void* base, int64_t byte0, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(static_cast<const uint8_t*>(base)) + byte0, 0, bytes, 0x00020000);
+  };
+
+  float t_f[CH][8], sh_f[CH][8];  // modulation vectors of the current modulation row
+  int cur_mod = -1;
+  auto load_mod = [&](int mod) {
+    const __amdgpu_buffer_rsrc_t shb = row_buf(shift, (int64_t)mod * ld_mod * 2, K * 2);
+    const __amdgpu_buffer_rsrc_t scb = row_buf(scale_mod, (int64_t)mod * ld_mod * 2, K * 2);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-      const int idx = c * 64 + lane;
-      v[c] = idx < nchunks ? xr[idx] : make_uint4(0, 0, 0, 0);
-      sum += (bf16_lo(v[c].x) + bf16_hi(v[c].x)) + (bf16_lo(v[c].y) + bf16_hi(v[c].y)) +
-             (bf16_lo(v[c].z) + bf16_hi(v[c].z)) + (bf16_lo(v[c].w) + bf16_hi(v[c].w));
+      const u4v sh = __builtin_amdgcn_raw_buffer_load_b128(shb, idx[c] * 16, 0, kCached);
+      const u4v sc = __builtin_amdgcn_raw_buffer_load_b128(scb, idx[c] * 16, 0, kCached);
+      const bool valid = idx[c] < nchunks;  // beyond K: t = 0, so that y = 0 there
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        t_f[c][2 * e] = valid ? round_bf16_wide(1.0f + bf16_lo(sc[e])) : 0.0f;
+        t_f[c][2 * e + 1] = valid ? round_bf16_wide(1.0f + bf16_hi(sc[e])) : 0.0f;
+        sh_f[c][2 * e] = bf16_lo(sh[e]);
+        sh_f[c][2 * e + 1] = bf16_hi(sh[e]);
+      }
     }
-    const float mean = wave_sum_f32(sum) * inv_k;
-    float ss = 0.0f;
+    cur_mod = mod;
+  };
+  auto load_row = [&](int row, u4v (&dst)[CH]) {
+    const __amdgpu_buffer_rsrc_t xb = row_buf(x, (int64_t)row * ld_x * 2, K * 2);
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      if (c * 64 + lane < nchunks) {
-        const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+    for (int c = 0; c < CH; ++c) dst[c] = __builtin_amdgcn_raw_buffer_load_b128(xb, idx[c] * 16, 0, kCached);
+  };
+  // sum of (a, b) over the workgroup, the same in every thread
+  auto block_sum2 = [&](float& a, float& b, float (*slot)[2]) {
+    a = __uint_as_float(wave_reduce_to_lane63(__float_as_uint(a), AddF32{}));
+    b = __uint_as_float(wave_reduce_to_lane63(__float_as_uint(b), AddF32{}));
+    if constexpr (WAVES == 1) {
+      a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(a), 63));
+      b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(b), 63));
+    } else {
+      if (lane == 63) {
+        slot[wave][0] = a;
+        slot[wave][1] = b;
+      }
+      __syncthreads();
+      a = slot[0][0] + slot[1][0];
+      b = slot[0][1] + slot[1][1];
+#pragma unroll
+      for (int w = 2; w < WAVES; w += 2) {  // a fixed order of additions
+        a += slot[w][0] + slot[w + 1][0];
+        b += slot[w][1] + slot[w + 1][1];
+      }
+    }
+  };
+  auto block_max = [&](uint32_t m, uint32_t* slot) -> uint32_t {
+    m = wave_reduce_to_lane63(m, MaxU32{});
+    if constexpr (WAVES == 1) return (uint32_t)__builtin_amdgcn_readlane((int)m, 63);
+    if (lane == 63) slot[wave] = m;
+    __syncthreads();
+    uint32_t r = max(slot[0], slot[1]);
+#pragma unroll
+    for (int w = 2; w < WAVES; w += 2) r = max(r, max(slot[w], slot[w + 1]));
+    return r;
+  };
+
+  // One row: `cur` holds it, `nxt` receives the row after it (the last row once more where
+  // there is none: a load that is never used, so that the count of accesses stays fixed).
+  auto one_row = [&](int row, u4v (&cur)[CH], u4v (&nxt)[CH]) {
+    const int par = row & 1;
+    const int mod = row / rows_per_mod;
+    if (mod != cur_mod) load_mod(mod);  // uniform, rare
+    load_row(min(row + 1, row_end - 1), nxt);
+
+    float sum = 0.0f, sq = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        sum = dot_pair(cur[c][e], 0x3f803f80u, sum);
+        sq = dot_pair(cur[c][e], cur[c][e], sq);
+      }
+    block_sum2(sum, sq, red_f[par]);
+    const float mean = sum * inv_k;
+    float var = sq * inv_k - mean * mean;
+    if (!(mean * mean <= 4.0f * var)) {  // uniform; also taken by var <= 0 and by NaN
+      float ss = 0.0f, unused = 0.0f;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const bool valid = idx[c] < nchunks;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float a = bf16_lo(w[e]) - mean, b = bf16_hi(w[e]) - mean;
+          uint32_t w = cur[c][e];
+          asm volatile("" : "+v"(w));  // keeps this path's widening inside the (cold) branch
+          const float a = valid ? bf16_lo(w) - mean : 0.0f;
+          const float b = valid ? bf16_hi(w) - mean : 0.0f;
           ss = __fmaf_rn(a, a, ss);
           ss = __fmaf_rn(b, b, ss);
         }
       }
+      __syncthreads();  // the slots of this parity are read by everyone before they are reused
+      block_sum2(ss, unused, red_f[par]);
+      var = ss * inv_k;
     }
-    const float var = wave_sum_f32(ss) * inv_k;
-    const float rstd = 1.0f / sqrtf(var + eps);
-    uint32_t m = 0;
+    // (v_rsq_f32, about an ulp: the statistics are fp32 sums in an order of their own anyway)
+    const float rstd = __builtin_amdgcn_rsqf(var + eps);
+    const float off = -mean * rstd;
+
+    uint32_t mpos = 0, mneg = 0;  // signed and unsigned maxima of the raw bits
+    float yv[CH][8];
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-      const int idx = c * 64 + lane;
-      if (idx < nchunks) {
-        const uint4 sh = shr[idx], sc = scr[idx];
-        v[c].x = modulate2(v[c].x, mean, rstd, sc.x, sh.x);
-        v[c].y = modulate2(v[c].y, mean, rstd, sc.y, sh.y);
-        v[c].z = modulate2(v[c].z, mean, rstd, sc.z, sh.z);
-        v[c].w = modulate2(v[c].w, mean, rstd, sc.w, sh.w);
-        if constexpr (WRITE_Y) reinterpret_cast<uint4*>(y + row * ld_y)[idx] = v[c];
-        m = absmax2(m, v[c].x);
-        m = absmax2(m, v[c].y);
-        m = absmax2(m, v[c].z);
-        m = absmax2(m, v[c].w);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float n0 = round_bf16_wide(__fmaf_rn(bf16_lo(cur[c][e]), rstd, off));
+        const float n1 = round_bf16_wide(__fmaf_rn(bf16_hi(cur[c][e]), rstd, off));
+        const float u0 = round_bf16_wide(n0 * t_f[c][2 * e]);
+        const float u1 = round_bf16_wide(n1 * t_f[c][2 * e + 1]);
+        const float y0 = round_bf16_wide(u0 + sh_f[c][2 * e]);
+        const float y1 = round_bf16_wide(u1 + sh_f[c][2 * e + 1]);
+        yv[c][2 * e] = y0;
+        yv[c][2 * e + 1] = y1;
+        const int b0 = __float_as_int(y0), b1 = __float_as_int(y1);
+        mpos = (uint32_t)max(max((int)mpos, b0), b1);          // v_max3_i32: the largest positive pattern
+        mneg = max(max(mneg, (uint32_t)b0), (uint32_t)b1);     // v_max3_u32: the largest negative one
+      }
+      if constexpr (WRITE_Y) {
+        const __amdgpu_buffer_rsrc_t yb = row_buf(y, (int64_t)row * ld_y * 2, K * 2);
+        const u4v packed = {pack_wide(yv[c][0], yv[c][1]), pack_wide(yv[c][2], yv[c][3]),
+                            pack_wide(yv[c][4], yv[c][5]), pack_wide(yv[c][6], yv[c][7])};
+        __builtin_amdgcn_raw_buffer_store_b128(packed, yb, idx[c] * 16, 0, kCached);
       }
     }
-    m = wave_max_u32(fold2(m));
+    // magnitude bits of the larger of the two (mneg only counts when it is a negative pattern)
+    const uint32_t mag_neg = (mneg & 0x80000000u) ? (mneg & 0x7fffffffu) : 0u;
+    uint32_t m = max(mpos, mag_neg) >> 16;  // bf16 bit pattern of max |y|
+    m = block_max(m, red_m[par]);
     const float s = row_scale(m, scale_mode);
-    if (lane == 0) scale[row] = s;
-    uint2* qr = reinterpret_cast<uint2*>(q + row * ld_q);
-    const bool fast = scale_in_fast_window(s);  // wave-uniform
-    const float r = fast ? 1.0f / s : 0.0f;
+    // thread 0 writes the scale; everyone else's offset lies beyond the 4-byte descriptor
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(s), row_buf(scale, (int64_t)row * 4, 4),
+                                          threadIdx.x == 0 ? 0 : 4, 0, kCached);
+    u2v o[CH];
+    if (scale_in_fast_window(s)) {  // uniform
+      const float r = 1.0f / s;
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      const int idx = c * 64 + lane;
-      if (idx < nchunks) {
-        uint2 o;
-        if (fast) {
-          o.x = quant4<true>(v[c].x, v[c].y, s, r);
-          o.y = quant4<true>(v[c].z, v[c].w, s, r);
-        } else {
-          o.x = quant4<false>(v[c].x, v[c].y, s, 0.0f);
-          o.y = quant4<false>(v[c].z, v[c].w, s, 0.0f);
+      for (int c = 0; c < CH; ++c) {
+        uint32_t p[2] = {0u, 0u};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float a = div_scale<true>(yv[c][2 * e], s, r), b = div_scale<true>(yv[c][2 * e + 1], s, r);
+          p[e >> 1] = (e & 1) ? __builtin_amdgcn_cvt_pk_fp8_f32(a, b, p[e >> 1], true)
+                              : __builtin_amdgcn_cvt_pk_fp8_f32(a, b, p[e >> 1], false);
         }
-        qr[idx] = o;
+        o[c] = u2v{p[0], p[1]};
+      }
+    } else {
+#pragma unroll 1
+      for (int c = 0; c < CH; ++c) {
+        uint32_t p[2] = {0u, 0u};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float a = clamp448(yv[c][2 * e] / s), b = clamp448(yv[c][2 * e + 1] / s);
+          p[e >> 1] = (e & 1) ? __builtin_amdgcn_cvt_pk_fp8_f32(a, b, p[e >> 1], true)
+                              : __builtin_amdgcn_cvt_pk_fp8_f32(a, b, p[e >> 1], false);
+        }
+        o[c] = u2v{p[0], p[1]};
       }
     }
+    const __amdgpu_buffer_rsrc_t qb = row_buf(q, (int64_t)row * ld_q, K);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) __builtin_amdgcn_raw_buffer_store_b64(o[c], qb, idx[c] * 8, 0, kCached);
+  };
+
+  u4v va[CH], vb[CH];
+  load_row(row0, va);
+  {
+    // As many stores as a row issues, every lane beyond its descriptor (nothing is written):
+    // the first row then meets the same sequence of accesses in flight as every later one,
+    // and the wait for its data is the same count (the compiler takes the smaller of the two
+    // otherwise, which makes every other row wait for stores of the row before it).
+    const __amdgpu_buffer_rsrc_t none = row_buf(scale, 0, 0);
+    if constexpr (WRITE_Y) {
+#pragma unroll
+      for (int c = 0; c < CH; ++c) __builtin_amdgcn_raw_buffer_store_b128(va[0], none, 0, 0, kCached);
+    }
+    __builtin_amdgcn_raw_buffer_store_b32(0u, none, 0, 0, kCached);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) __builtin_amdgcn_raw_buffer_store_b64(u2v{0u, 0u}, none, 0, 0, kCached);
+  }
+  for (int row = row0;;) {
+    one_row(row, va, vb);
+    if (++row >= row_end) break;
+    one_row(row, vb, va);
+    if (++row >= row_end) break;
   }
 }
 
@@ -742,6 +935,18 @@ int launch_quant_rowwise_batched(const QuantBatch& batch, int64_t K, int scale_m
   return 1;
 }
 
+// CUs of the current device, `fallback` when the query fails
+static int64_t cu_count_or(int64_t fallback) {
+  static int cached[64];  // per device ordinal; the answer cannot change
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fallback;
+  if (dev >= 0 && dev < 64 && cached[dev] > 0) return cached[dev];
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+    return fallback;
+  if (dev >= 0 && dev < 64) cached[dev] = n;
+  return n;
+}
+
 int launch_ln_modulate_quant(const void* x, int64_t M, int64_t K, int64_t ld_x, const void* shift,
                              const void* scale_mod, int64_t ld_mod, int64_t rows_per_mod, float eps,
                              void* y, int64_t ld_y, void* q, int64_t ld_q, float* scale,
@@ -760,27 +965,45 @@ int launch_ln_modulate_quant(const void* x, int64_t M, int64_t K, int64_t ld_x, 
   if (blocks > kMaxBlocks) blocks = kMaxBlocks;
   dim3 grid((unsigned)blocks), block(64);
   const int need = (int)((K + 511) / 512);
-#define CDIT_LNQ_CASE(CH)                                                                       \
-  if (aligned && need <= CH) {                                                                  \
-    if (y)                                                                                      \
-      hipLaunchKernelGGL((ln_modulate_quant_regs<CH, true>), grid, block, 0, stream, xp, ld_x,   \
-                         shp, scp, ld_mod, (int)rows_per_mod, eps, yp, ld_y, qp, ld_q, scale,    \
-                         (int)M, (int)K, scale_mode);                                           \
-    else                                                                                        \
-      hipLaunchKernelGGL((ln_modulate_quant_regs<CH, false>), grid, block, 0, stream, xp, ld_x,  \
-                         shp, scp, ld_mod, (int)rows_per_mod, eps, yp, ld_y, qp, ld_q, scale,    \
-                         (int)M, (int)K, scale_mode);                                           \
-    return 0;                                                                                   \
+  // Wavefronts per row: the fewest of 1, 2, 4, 8 that leave a thread at most three chunks of 8
+  // elements (the row, the prefetched next row and the two modulation vectors live in
+  // registers: 153 at three chunks, three wavefronts per SIMD); rows beyond 12288 elements
+  // take four chunks at eight wavefronts (K <= 16384). Workgroups: about six wavefronts'
+  // worth per SIMD (twice what is resident at once), each with the same number of
+  // consecutive rows.
+  if (aligned && need <= 32) {
+    int waves = 8;
+    for (int w = 1; w <= 8; w *= 2)
+      if ((need + w - 1) / w <= 3) {
+        waves = w;
+        break;
+      }
+    const int ch = (need + waves - 1) / waves;
+    const int64_t cus = cu_count_or(256);
+    // (measured at 4608 x 3072: 16.1 us with 16 wavefronts' worth of workgroups per CU, 15.2
+    // with 20 or 24; four wavefronts of two chunks per row instead of two of three: 17.4-17.7)
+    const int64_t target = cus * 24 / waves;
+    const int rows_per_wg = (int)((M + target - 1) / target);
+    const dim3 rgrid((unsigned)((M + rows_per_wg - 1) / rows_per_wg));
+#define CDIT_LNQ_LAUNCH(W, CH, WY)                                                              \
+  hipLaunchKernelGGL((ln_modulate_quant_rows<CH, WY, W>), rgrid, dim3(64 * W), 0, stream, xp,   \
+                     ld_x, shp, scp, ld_mod, (int)rows_per_mod, eps, yp, ld_y, qp, ld_q, scale, \
+                     (int)M, (int)K, scale_mode, rows_per_wg)
+#define CDIT_LNQ_CASE(W, CH)                  \
+  if (waves == W && ch <= CH) {               \
+    if (y)                                    \
+      CDIT_LNQ_LAUNCH(W, CH, true);           \
+    else                                      \
+      CDIT_LNQ_LAUNCH(W, CH, false);          \
+    return 0;                                 \
   }
-  CDIT_LNQ_CASE(1)
-  CDIT_LNQ_CASE(2)
-  CDIT_LNQ_CASE(4)
-  CDIT_LNQ_CASE(6)
-  CDIT_LNQ_CASE(8)
-  CDIT_LNQ_CASE(10)
-  CDIT_LNQ_CASE(12)
-  CDIT_LNQ_CASE(16)
+    CDIT_LNQ_CASE(1, 1) CDIT_LNQ_CASE(1, 2) CDIT_LNQ_CASE(1, 3)
+    CDIT_LNQ_CASE(2, 2) CDIT_LNQ_CASE(2, 3)
+    CDIT_LNQ_CASE(4, 2) CDIT_LNQ_CASE(4, 3)
+    CDIT_LNQ_CASE(8, 2) CDIT_LNQ_CASE(8, 3) CDIT_LNQ_CASE(8, 4)
 #undef CDIT_LNQ_CASE
+#undef CDIT_LNQ_LAUNCH
+  }
   hipLaunchKernelGGL(ln_modulate_quant_generic, grid, block, 0, stream, xp, ld_x, shp, scp, ld_mod,
                      (int)rows_per_mod, eps, yp, ld_y, qp, ld_q, scale, (int)M, (int)K, scale_mode);
   return 0;

@@ -88,10 +88,51 @@ def _require_cuda(name: str, *tensors: Optional[torch.Tensor]) -> None:
 # These take already-validated 2-D tensors and write into caller-provided outputs.
 
 
+#: Buffers whose bf16 values were never written: ln_modulate_quant(materialize=False) returns
+#: such a tensor, and only its FP8 codes (handed over through the shared-quantization lookup)
+#: mean anything. storage address -> (weak reference to the storage, version counter at
+#: hand-over). The storage object lives as long as any view of the buffer does, so the entry
+#: covers every reshape and slice of it and disappears with the last of them.
+_codes_only: dict = {}
+
+
+def _mark_codes_only(y: torch.Tensor) -> None:
+  import weakref
+  st = y.untyped_storage()
+  key = st.data_ptr()
+  _codes_only[key] = (weakref.ref(st, lambda _r, k=key: _codes_only.pop(k, None)), y._version)
+
+
+def is_codes_only(x: torch.Tensor) -> bool:
+  """Whether x aliases a buffer that ln_modulate_quant(materialize=False) left unwritten
+  (and nobody has written through PyTorch since)."""
+  if not _codes_only or x.is_inference():
+    return False
+  st = x.untyped_storage()
+  entry = _codes_only.get(st.data_ptr())
+  return entry is not None and entry[0]() is st and entry[1] == x._version
+
+
+def _reject_codes_only(what: str, *xs: torch.Tensor) -> None:
+  """Every path that reads an activation's bf16 values calls this first: reading a
+  codes-only buffer would quantize (or multiply) uninitialised memory without any error."""
+  if not _codes_only:
+    return
+  for x in xs:
+    if is_codes_only(x):
+      raise RuntimeError(
+          f"{what}: this activation comes from ln_modulate_quant(materialize=False), which "
+          "writes FP8 codes only, and its codes were not found by the consumer (they are handed "
+          "over per device and stream to float8_per_row Linears with share_activation_quant_ "
+          "switched on, a few activations deep). Call ln_modulate_quant with materialize=True "
+          "for this consumer.")
+
+
 def quant_tensorwise_into(x2: torch.Tensor, q: torch.Tensor, scale: torch.Tensor,
                           amax_ws: torch.Tensor, scale_mode_id: int) -> None:
   """Per-tensor quantizer: one scale for all of x2, written to every scale[m].
   amax_ws: 4 bytes of device scratch (an int32 tensor of one element)."""
+  _reject_codes_only("quant_tensorwise_into", x2)
   M, K = x2.shape
   with _DeviceOf(x2):
     _native.check(_native.load().cdit_fp8_quant_tensorwise(x2.data_ptr(), M, K, x2.stride(0),
@@ -104,6 +145,7 @@ def quant_rowwise_into(x2: torch.Tensor, q: torch.Tensor, scale: torch.Tensor,
                        scale_mode_id: int, gemm_follows: bool = False) -> None:
   """gemm_follows: the codes are read by a GEMM launched next on this stream (a cache
   hint for the quantizer; the results are the same)."""
+  _reject_codes_only("quant_rowwise_into", x2)
   M, K = x2.shape
   mode = scale_mode_id | (_native.QUANT_GEMM_FOLLOWS if gemm_follows else 0)
   with _DeviceOf(x2):
@@ -118,6 +160,7 @@ def quant_rowwise_batched_into(items, scale_mode_id: int) -> None:
   list of (x2 [M,K] bf16, q [M,K] e4m3, scale [M] fp32), at most _native.MAX_ACTS of them on
   one device; the codes are taken to be read by a GEMM launched next. Bit-identical to one
   quant_rowwise_into per item."""
+  _reject_codes_only("quant_rowwise_batched_into", *[x for x, _, _ in items])
   import ctypes
   n = len(items)
   x0 = items[0][0]
@@ -137,6 +180,7 @@ def quant_rowwise_cat2_into(x1: torch.Tensor, x2: torch.Tensor, q: torch.Tensor,
                             scale_mode_id: int) -> None:
   """Quantizes the rows [x1 | x2] (bf16 [M,K1] and [M,K2]) into q [M,K1+K2] / scale [M] without
   the concatenated tensor; the results are those of quant_rowwise_into on torch.cat."""
+  _reject_codes_only("quant_rowwise_cat2_into", x1, x2)
   with _DeviceOf(x1):
     _native.check(_native.load().cdit_fp8_quant_rowwise_cat2(
         x1.data_ptr(), x1.shape[1], x1.stride(0), x2.data_ptr(), x2.shape[1], x2.stride(0),
@@ -227,6 +271,7 @@ def w8a16_batched_into(acts) -> None:
   members e4m3 [N_p,K] weights with a common row stride, fp32 scales, bf16 biases or None,
   bf16 outputs [M,N_p] and epilogue flags. Activations whose row strides differ are
   launched apart. Bit-identical to one w8a16_into per member."""
+  _reject_codes_only("w8a16_batched_into", *[t[0] for t in acts])
   import ctypes
   vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
   x0 = acts[0][0]
@@ -260,6 +305,7 @@ def w8a16_batched_into(acts) -> None:
 
 def w8a16_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
                bias: Optional[torch.Tensor], out: torch.Tensor, epilogue: int) -> None:
+  _reject_codes_only("w8a16_into", x2)
   M, K = x2.shape
   N = w.shape[0]
   with _DeviceOf(x2):
@@ -393,6 +439,7 @@ def linear_w8a8_into(x2: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor,
                      bias: Optional[torch.Tensor], out: torch.Tensor, q_ws: torch.Tensor,
                      s_ws: torch.Tensor, scale_mode_id: int, epilogue: int) -> None:
   """Quantizer + GEMM of one Linear forward in a single library call."""
+  _reject_codes_only("linear_w8a8_into", x2)
   M, K = x2.shape
   N = w.shape[0]
   with _DeviceOf(x2):
@@ -605,13 +652,19 @@ def ln_modulate_quant(x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor,
   lookup on; the bf16 tensor is then always written and nothing is handed over."""
   _require_cuda("ln_modulate_quant", x, shift, scale)
   mode_id = _native.SCALE_MODE_IDS[scale_mode]
-  no_handover = x.is_inference() or torch.is_inference_mode_enabled()
-  y, q, s = torch.ops.cdit.ln_modulate_quant(x, shift, scale, float(eps), mode_id,
-                                             bool(materialize or no_handover))
+  # no hand-over (the bf16 tensor is then always written): inference-mode tensors carry no
+  # version counter, and a graph being traced by torch.compile never shares codes (its
+  # Linears run with sharing off)
+  no_handover = (x.is_inference() or torch.is_inference_mode_enabled()
+                 or torch.compiler.is_compiling())
+  write_y = bool(materialize or no_handover)
+  y, q, s = torch.ops.cdit.ln_modulate_quant(x, shift, scale, float(eps), mode_id, write_y)
   if not no_handover and y.numel() > 0:
     y2 = y.view(-1, y.shape[-1])
     entries, capture_id = _shared_entries(y2)
     _remember_quant(entries, capture_id, y2, mode_id, q.view(y2.shape), s.view(-1))
+    if not write_y:
+      _mark_codes_only(y)  # a consumer that does not find the codes raises
   return y
 
 

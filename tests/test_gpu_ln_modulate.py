@@ -114,3 +114,126 @@ def test_codes_are_handed_to_the_consuming_linears():
   assert cosine(y3, y0) >= 0.9999
   ds.fuse_norm_quant(model, False)
   cache_dit.share_activation_quant_(model, False)
+
+
+def _codes_only_activation(M=64, K=512, seed=3):
+  """y = ln_modulate_quant(..., materialize=False): its bf16 values are never written."""
+  from cache_dit_amd import ops
+  x, shift, scale = _inputs((1, M, K), 1, seed=seed)
+  xg, sh, sc = x.cuda(), shift.cuda(), scale.cuda()
+  y = ops.ln_modulate_quant(xg, sh, sc, materialize=False)
+  want = ops.ln_modulate_quant(xg.clone(), sh, sc, materialize=True)
+  return y, want
+
+
+def _linear(quant_type, K=512, N=256, share=False):
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd import nn as cnn
+  torch.manual_seed(0)
+  lin = torch.nn.Linear(K, N, dtype=torch.bfloat16).cuda()
+  cnn.convert_linear_(lin, quant_type)
+  if share:
+    lin.share_input_quant = True
+  return lin
+
+
+def test_codes_only_activation_reaches_its_consumer_or_raises():
+  """The tensor ln_modulate_quant(materialize=False) returns holds no values. A consumer
+  that finds the delivered codes uses them; every consumer that would read the bf16
+  values instead must raise, never quantize uninitialised memory."""
+  from cache_dit_amd import ops
+  assert torch.cuda.is_available()
+  # the happy path: a sharing float8_per_row Linear, also through a reshaped view
+  y, want = _codes_only_activation()
+  assert ops.is_codes_only(y) and ops.is_codes_only(y.view(-1, y.shape[-1])[8:])
+  lin = _linear("float8_per_row", share=True)
+  assert torch.equal(lin(y), lin(want))
+  assert torch.equal(lin(y.view(-1, y.shape[-1])), lin(want.view(-1, want.shape[-1])))
+  # a Linear that does not share its input quantization
+  y, _ = _codes_only_activation(seed=4)
+  with pytest.raises(RuntimeError, match="materialize=True"):
+    _linear("float8_per_row", share=False)(y)
+  # weight-only and per-tensor Linears read the bf16 values
+  with pytest.raises(RuntimeError, match="materialize=True"):
+    _linear("float8_weight_only")(y)
+  with pytest.raises(RuntimeError, match="materialize=True"):
+    _linear("float8_per_tensor")(y)
+  # a slice is another activation (other shape): not in the lookup, and it aliases the buffer
+  with pytest.raises(RuntimeError, match="materialize=True"):
+    _linear("float8_per_row", share=True)(y[:, :32])
+  # the entry evicted by other quantizations on the stream
+  y, _ = _codes_only_activation(seed=5)
+  lin = _linear("float8_per_row", share=True)
+  for i in range(ops._SHARED_QUANT_ENTRIES + 1):
+    lin(torch.randn(8, 512, device="cuda").to(torch.bfloat16))
+  with pytest.raises(RuntimeError, match="materialize=True"):
+    lin(y)
+  # a consumer on another stream
+  y, _ = _codes_only_activation(seed=6)
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side), pytest.raises(RuntimeError, match="materialize=True"):
+    lin(y)
+  torch.cuda.current_stream().wait_stream(side)
+  # written through PyTorch afterwards: an ordinary activation again
+  y, _ = _codes_only_activation(seed=7)
+  y.copy_(torch.ones_like(y))
+  assert not ops.is_codes_only(y)
+  out = _linear("float8_weight_only")(y)
+  assert torch.isfinite(out.float()).all()
+  # sibling groups: per-row members find the codes, weight-only members raise
+  from cache_dit_amd import nn as cnn
+  y, want = _codes_only_activation(seed=8)
+  a, b = _linear("float8_per_row"), _linear("float8_per_row")
+  g = cnn.SiblingGroup([a, b])
+  a.sibling_group = b.sibling_group = g
+  ya, yb = a(y), b(y)
+  a.sibling_group = b.sibling_group = None
+  a.share_input_quant = b.share_input_quant = True
+  assert torch.equal(ya, a(want)) and torch.equal(yb, b(want))
+  y, _ = _codes_only_activation(seed=9)
+  a, b = _linear("float8_weight_only"), _linear("float8_weight_only")
+  a.sibling_group = b.sibling_group = cnn.SiblingGroup([a, b])
+  with pytest.raises(RuntimeError, match="materialize=True"):
+    a(y)
+
+
+def test_codes_only_is_never_produced_under_compile_or_inference_mode():
+  """Where nothing can be handed over the bf16 values are written whatever the caller asked."""
+  from cache_dit_amd import ops
+  x, shift, scale = _inputs((1, 32, 512), 1, seed=11)
+  xg, sh, sc = x.cuda(), shift.cuda(), scale.cuda()
+  want = ops.ln_modulate_quant(xg, sh, sc, materialize=True)
+  with torch.inference_mode():
+    y = ops.ln_modulate_quant(xg, sh, sc, materialize=False)
+  assert torch.equal(y, want) and not ops.is_codes_only(y)
+  lin = _linear("float8_weight_only")
+
+  def f(x):
+    return lin(ops.ln_modulate_quant(x, sh, sc, materialize=False))
+
+  try:
+    got = torch.compile(f, fullgraph=False)(xg)
+  except Exception as e:  # no Inductor back end on the box
+    pytest.skip(f"torch.compile unavailable: {str(e)[:80]}")
+  assert torch.equal(got, lin(want))
+
+
+def test_rows_per_mod_beyond_the_row_count_means_one_vector():
+  """The C entry point takes any count >= M for 'one modulation vector for every row'."""
+  import ctypes
+  from cache_dit_amd import _native
+  x, shift, scale = _inputs((1, 40, 512), 1, seed=12)
+  xg, sh, sc = x.cuda().view(40, 512), shift.cuda(), scale.cuda()
+  L, stream = _native.load(), torch.cuda.current_stream().cuda_stream
+  outs = []
+  for rows_per_mod in (40, 1 << 32, (1 << 63) - 1):
+    q = torch.empty(40, 512, dtype=torch.uint8, device="cuda")
+    s = torch.empty(40, dtype=torch.float32, device="cuda")
+    _native.check(L.cdit_fp8_ln_modulate_quant(xg.data_ptr(), 40, 512, 512, sh.data_ptr(), sc.data_ptr(),
+                                               512, rows_per_mod, 1e-6, None, 512, q.data_ptr(), 512,
+                                               s.data_ptr(), 0, stream))
+    torch.cuda.synchronize()
+    outs.append((q.cpu(), s.cpu()))
+  for q, s in outs[1:]:
+    assert torch.equal(q, outs[0][0]) and torch.equal(s, outs[0][1])
