@@ -17,8 +17,27 @@ import torch
 from torch import nn
 
 from . import _native, ops
+from .logger import init_logger
+
+logger = init_logger(__name__)
 
 FP8 = torch.float8_e4m3fn
+
+_warned_inference_bypass = False
+
+
+def _note_inference_bypass(what: str) -> None:
+  """Sharing, grouping and stage batching key their state on the activation's version
+  counter, which inference-mode tensors do not have: under torch.inference_mode() every
+  Linear runs on its own. Said once per process, since the slower path is otherwise silent."""
+  global _warned_inference_bypass
+  if not _warned_inference_bypass:
+    _warned_inference_bypass = True
+    logger.warning(
+        f"{what}: the input is an inference-mode tensor (no version counter), so shared "
+        "activation quantization, sibling groups and stage batching are bypassed and every "
+        "Linear launches its own quantizer and GEMM. Run under torch.no_grad() instead of "
+        "torch.inference_mode() to keep them.")
 
 #: scale rounding used for activations and weights (see ops.fp8_rowwise_quant)
 DEFAULT_SCALE_MODE = "bf16div"
@@ -110,18 +129,36 @@ class SiblingGroup:
     self.key = None  # _InputKey of the activation the pending outputs were computed from
     self.outs = None
     self.capture_id = 0
+    self.stream = None  # (device index, raw stream) the pending outputs were launched on
+
+  def drop_pending(self) -> None:
+    """Forgets the outputs no sibling has collected (and the activation they came from)."""
+    self.key = self.outs = None
 
   def forward_member(self, lin: "Fp8DynamicLinear", x: torch.Tensor) -> torch.Tensor:
+    """Not thread-safe: a group's state belongs to the thread that runs the model."""
+    global _pending_group
     x2 = ops._as_rows(x)
     i = self.index[id(lin)]
     capture_id = (_native.stream_capture_id(ops._stream_ptr(x2))
                   if torch.cuda.is_current_stream_capturing() else 0)
-    if (self.key is not None and self.capture_id == capture_id and self.outs[i] is not None
-        and self.key.matches(x2)):
+    stream = (x2.device.index, ops._stream_ptr(x2))
+    # pending outputs are only handed out on the stream they were launched on (another
+    # stream would read them without any ordering) and inside the capture they belong to
+    if (self.key is not None and self.capture_id == capture_id and self.stream == stream
+        and self.outs[i] is not None and self.key.matches(x2)):
       out, self.outs[i] = self.outs[i], None
       if all(o is None for o in self.outs):
-        self.key = self.outs = None
+        self.drop_pending()
+        if _pending_group is self:
+          _pending_group = None
       return out.view(*x.shape[:-1], lin.out_features)
+    # A group that computes afresh while another still holds uncollected outputs: that
+    # forward left its siblings early (an exception, a skipped branch); its leftovers (up to
+    # M x sum(N) bf16) are released here rather than kept until its next call.
+    if _pending_group is not None and _pending_group is not self:
+      _pending_group.drop_pending()
+    _pending_group = self
     M = x2.shape[0]
     members = self.members
     outs = [torch.empty((M, m.out_features), dtype=torch.bfloat16, device=x2.device) for m in members]
@@ -134,8 +171,23 @@ class SiblingGroup:
                                     [m.weight_scale for m in members], [m.bias for m in members],
                                     outs, [m.epilogue for m in members])
     out, outs[i] = outs[i], None
-    self.key, self.outs, self.capture_id = _InputKey(x2), outs, capture_id
+    self.key, self.outs, self.capture_id, self.stream = _InputKey(x2), outs, capture_id, stream
     return out.view(*x.shape[:-1], lin.out_features)
+
+
+#: the sibling group whose outputs are waiting to be collected, if any (one at a time: the
+#: siblings of a group are called back to back)
+_pending_group: Optional[SiblingGroup] = None
+
+
+def release_pending_outputs() -> None:
+  """Drops the outputs a sibling group computed ahead for members that were never called
+  (a forward that raised or returned between two siblings). Happens by itself at the next
+  grouped call; for a caller that wants the memory back right away."""
+  global _pending_group
+  if _pending_group is not None:
+    _pending_group.drop_pending()
+    _pending_group = None
 
 
 class _SiblingRecorder:
@@ -176,10 +228,14 @@ class Fp8DynamicLinear(_Fp8LinearBase):
     # no version counter to tell a modified buffer by
     stateless = torch.compiler.is_compiling()
     if not stateless:
-      if _recorder is not None and not x.is_inference():
-        _recorder.note(self, x)
-      if self.sibling_group is not None and not x.is_inference():
-        return self.sibling_group.forward_member(self, x)
+      if x.is_inference():
+        if self.sibling_group is not None or self.share_input_quant:
+          _note_inference_bypass(type(self).__name__)
+      else:
+        if _recorder is not None:
+          _recorder.note(self, x)
+        if self.sibling_group is not None:
+          return self.sibling_group.forward_member(self, x)
     share = self.share_input_quant and not stateless
     return torch.ops.cdit.linear_w8a8(x, self.weight, self.weight_scale, self.bias,
                                       self._scale_mode_id, self.epilogue,
@@ -207,11 +263,15 @@ class Fp8WeightOnlyLinear(_Fp8LinearBase):
 
   def forward(self, x: torch.Tensor) -> torch.Tensor:
     self._check_input(x)
-    if not torch.compiler.is_compiling() and not x.is_inference():  # as in Fp8DynamicLinear
-      if _recorder is not None:
-        _recorder.note(self, x)
-      if self.sibling_group is not None:
-        return self.sibling_group.forward_member(self, x)
+    if not torch.compiler.is_compiling():  # as in Fp8DynamicLinear
+      if x.is_inference():
+        if self.sibling_group is not None:
+          _note_inference_bypass(type(self).__name__)
+      else:
+        if _recorder is not None:
+          _recorder.note(self, x)
+        if self.sibling_group is not None:
+          return self.sibling_group.forward_member(self, x)
     return torch.ops.cdit.w8a16_mm(x, self.weight.t(), self.weight_scale, self.bias,
                                    _native.DT_BF16, self.epilogue)
 
@@ -350,6 +410,8 @@ def linear_batch(pairs):
   compiling = torch.compiler.is_compiling()
   if not plain and not compiling:  # (no version counters on inference tensors: nothing is shared)
     plain = any(x.is_inference() for x, _ in pairs)
+    if plain:
+      _note_inference_bypass("linear_batch")
   if plain:
     return [[lin(x) for lin in lins] for x, lins in pairs]
   if compiling:
