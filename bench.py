@@ -299,10 +299,11 @@ def step_leg(device, linears, mode, steps, warmup):
 
 def pmc_sequence(device):
   """Launch sequence for counter collection: run under `rocprofv3 --pmc FETCH_SIZE`, then
-  under `--pmc WRITE_SIZE`, each in a run of its own. Four times over: a 512 MiB fill (to
-  push earlier data out of the caches), a plain device copy of the bf16 activation (known
-  size: the scale of the counters), the quantizer on that activation, another fill, the
-  FP8 GEMM on the codes; all at the headline shape."""
+  under `--pmc WRITE_SIZE`, each in a run of its own. Four times over, each kernel behind a
+  512 MiB fill (to push earlier data out of the caches): a plain device copy of the bf16
+  activation (known size: the scale of the counters), the quantizer on that activation, the
+  FP8 GEMM on the codes, the fused LayerNorm + modulate + quantizer, the weight-only GEMM
+  and the grouped GEMM of a FLUX single block; all at the headline shape."""
   import torch
   from cache_dit_amd import ops
   M, K, N = HEADLINE
@@ -316,6 +317,18 @@ def pmc_sequence(device):
   out = torch.empty(M, N, dtype=torch.bfloat16, device=device)
   y = torch.empty(M, K, dtype=torch.bfloat16, device=device)
   flush = torch.empty(1 << 29, dtype=torch.uint8, device=device)
+  # further kernels of the path, for their own counter summaries: the fused LayerNorm +
+  # modulate + quantizer, the weight-only GEMM, and the grouped GEMM of a FLUX single block
+  # (proj_mlp + q/k/v on one activation: 12288 + 3 x 3072 columns on 256 x 256 tiles)
+  from cache_dit_amd import _native
+  L, stream = _native.load(), torch.cuda.current_stream().cuda_stream
+  shift = torch.randn(K, device=device, generator=g).to(torch.bfloat16)
+  scale_mod = (torch.randn(K, device=device, generator=g) * 0.3).to(torch.bfloat16)
+  sib_n = (N, K, K, K)
+  sib_w = [_rand_fp8((n, K), g, device) for n in sib_n]
+  sib_s = [torch.rand(n, device=device, generator=g) * 1e-3 for n in sib_n]
+  sib_b = [torch.randn(n, device=device, generator=g).to(torch.bfloat16) for n in sib_n]
+  sib_out = [torch.empty(M, n, dtype=torch.bfloat16, device=device) for n in sib_n]
   for i in range(4):
     flush.zero_()
     y.copy_(x[i])  # plain copy: reads 2MK, writes 2MK bytes
@@ -323,6 +336,15 @@ def pmc_sequence(device):
     ops.quant_rowwise_into(x[i], q[i], s, 0)
     flush.zero_()
     ops.gemm_rowwise_into(q[i], s, w[i], ws, b, out, 0)
+    flush.zero_()
+    _native.check(L.cdit_fp8_ln_modulate_quant(x[i].data_ptr(), M, K, K, shift.data_ptr(),
+                                               scale_mod.data_ptr(), K, M, 1e-6, None, K,
+                                               q[i].data_ptr(), K, s.data_ptr(), 0, stream))
+    flush.zero_()
+    ops.w8a16_into(x[i], w[i], ws, b, out, 0)
+    flush.zero_()
+    ops.quant_rowwise_into(x[i], q[i], s, 0)
+    ops.gemm_rowwise_grouped_into(q[i], s, sib_w, sib_s, sib_b, sib_out, [1, 0, 0, 0])
   torch.cuda.synchronize()
 
 
@@ -391,6 +413,14 @@ def headline_kernels(device):
   # of this part keeps rising over the first second or two of a run of GEMMs (10 % between
   # the first hundred launches and the settled value). Blocks of 100 launches until two
   # consecutive blocks agree within 0.5 %, for at least 1.5 and at most 4 seconds.
+  # The quantizer is timed twice, as the median of five blocks of 100 launches each: before
+  # the GEMM legs (cooler part, higher clocks) and after them (the state it runs in inside a
+  # step). Both are reported; roofline_quant quotes the later one.
+  def quant_median_ms():
+    blocks = sorted(_time_events(quant, 100, 20 if k == 0 else 0) for k in range(5))
+    return blocks[2], blocks[0], blocks[-1]
+
+  quant_before = quant_median_ms()
   t_start, prev = time.perf_counter(), _time_events(gemm, 100, 100)
   while time.perf_counter() - t_start < 4.0:
     cur = _time_events(gemm, 100, 0)
@@ -400,7 +430,8 @@ def headline_kernels(device):
       break
   gemm_ms = _time_events(gemm, 100, 10)
   gemm_gelu_ms = _time_events(gemm_gelu, 100, 10)
-  quant_ms = _time_events(quant, 200, 20)
+  quant_after = quant_median_ms()
+  quant_ms = quant_after[0]
   res = {
       "shape": {"M": M, "K": K, "N": N},
       "gemm_ms": gemm_ms,
@@ -409,6 +440,9 @@ def headline_kernels(device):
       "gemm_gelu_tflops": 2.0 * M * K * N / gemm_gelu_ms / 1e9,
       "quant_ms": quant_ms,
       "quant_gbps": (3.0 * M * K + 4.0 * M) / quant_ms / 1e6,
+      # median, fastest and slowest of five blocks of 100 back-to-back launches (ms)
+      "quant_ms_before_gemm_legs": list(quant_before),
+      "quant_ms_after_gemm_legs": list(quant_after),
   }
   # What bounds the quantizer at this size: the fixed cost of a launch of M one-wavefront
   # workgroups. The same kernel with K = 0 (4608 workgroups that only write their scale)
@@ -442,7 +476,7 @@ def headline_kernels(device):
                                                scale_mod.data_ptr(), K, M, 1e-6, None, K,
                                                qs[i].data_ptr(), K, ss[i].data_ptr(), 0, stream))
 
-  lnq_ms = _time_events(ln_quant, 200, 20)
+  lnq_ms = sorted(_time_events(ln_quant, 100, 20 if k == 0 else 0) for k in range(5))[2]
   res["ln_modulate_quant_ms"] = lnq_ms
   res["ln_modulate_quant_gbps"] = (3.0 * M * K + 4.0 * M) / lnq_ms / 1e6
   for i in range(nbuf):  # the codes the later legs read are those of xs again
@@ -523,6 +557,68 @@ def headline_kernels(device):
   return res
 
 
+def mfma_only_ceiling(device):
+  """What the matrix cores of this part sustain on the GEMM's own instruction
+  (v_mfma_f32_16x16x128_f8f6f4) with nothing else going on: 256 workgroups of four
+  wavefronts, register operands, no memory traffic (cdit_debug_mfma_only). With all-ones
+  operands the part holds its rated clock; with random e4m3 operands (the benchmark's data)
+  the power limit lowers it. The random-operand figure is the ceiling of any FP8 kernel on
+  this data before a byte is moved. Each case: two warm-up launches, then the median of
+  three launches of about 15 ms."""
+  import ctypes
+  import torch
+  from cache_dit_amd import _native
+  L, stream = _native.load(), torch.cuda.current_stream().cuda_stream
+  blocks, iters = 256, 60000
+  out = torch.empty(blocks * 256, dtype=torch.float32, device=device)
+  res = {}
+  for key, rnd in (("constant_operands_tflops", 0), ("random_operands_tflops", 1)):
+    flop = ctypes.c_double(0.0)
+
+    def fn():
+      _native.check(L.cdit_debug_mfma_only(out.data_ptr(), blocks, iters, rnd, ctypes.byref(flop), stream))
+
+    times = sorted(_time_events(fn, 1, 2 if k == 0 else 0) for k in range(3))
+    res[key] = flop.value / times[1] / 1e9
+  res["note"] = ("loop of v_mfma_f32_16x16x128_f8f6f4 on register operands, 256 workgroups x 4 "
+                 "wavefronts, 16 independent accumulators, no memory traffic; HIP events")
+  return res
+
+
+def quant_large_shapes(device):
+  """The per-row quantizer on the largest activation of each benchmark configuration
+  (FLUX proj_out input 4608 x 15360, Qwen-Image MLP hidden 6889 x 12288, Wan hidden
+  32760 x 5120 and FFN hidden 32760 x 13824): algorithmic bytes 3MK + 4M over the median of
+  five blocks of launches, rotating over two buffer sets (each beyond the 256 MiB last-level
+  cache together with its codes)."""
+  import torch
+  from cache_dit_amd import ops
+  out = []
+  g = torch.Generator(device=device).manual_seed(2)
+  for name, M, K in (("flux proj_out input", 4608, 15360), ("qwen img_mlp.net.2 input", 6889, 12288),
+                     ("wan hidden", 32760, 5120), ("wan ffn.net.2 input", 32760, 13824)):
+    xs = [torch.randn(M, K, device=device, generator=g).to(torch.bfloat16) for _ in range(2)]
+    qs = [torch.empty(M, K, dtype=torch.float8_e4m3fn, device=device) for _ in range(2)]
+    sc = [torch.empty(M, dtype=torch.float32, device=device) for _ in range(2)]
+    it = {"i": 0}
+
+    def quant():
+      i = it["i"] = it["i"] ^ 1
+      ops.quant_rowwise_into(xs[i], qs[i], sc[i], 0)
+
+    n = max(10, min(100, int(2.0e10 / (3.0 * M * K))))  # about 3 ms per block at 6 TB/s
+    blocks = sorted(_time_events(quant, n, 4 if k == 0 else 0) for k in range(5))
+    nbytes = 3.0 * M * K + 4.0 * M
+    gbps = nbytes / blocks[2] / 1e6
+    out.append({"kernel": f"per-row quantizer, {name} (M={M} K={K})", "bound": "hbm",
+                "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+                "traffic": None, "algorithmic_bytes": nbytes, "us": blocks[2] * 1e3,
+                "us_fastest_block": blocks[0] * 1e3, "us_slowest_block": blocks[-1] * 1e3})
+    del xs, qs, sc
+    torch.cuda.empty_cache()
+  return out
+
+
 def cpu_baseline():
   """The CPU restatement of the reference path (oracle.torch_oracle: eager PyTorch
   CPU ops) on benchmark config 1 (M=4608, K=3072, N=3072): activation quantization +
@@ -536,9 +632,14 @@ def cpu_baseline():
   except ValueError:
     pass
   torch.set_num_threads(cores)
+  # benchmark config 1, drawn exactly as the parity tests draw it (seed 0, CPU generator,
+  # fp32 then bf16): x ~N(0,1) with max(1, floor(0.001 K)) = 3 channels picked by
+  # randperm scaled by 20, W ~N(0,0.02), bias ~N(0,0.01)
   g = torch.Generator().manual_seed(0)
   M, K, N = 4608, 3072, 3072
-  x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+  x = torch.randn(1, M, K, generator=g)
+  x[..., torch.randperm(K, generator=g)[:max(1, int(0.001 * K))]] *= 20.0
+  x = x.to(torch.bfloat16).reshape(M, K)
   w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
   b = (torch.randn(N, generator=g) * 0.01).to(torch.bfloat16)
   wq, ws = to.quantize_rowwise(w)
@@ -565,7 +666,7 @@ def cpu_baseline():
       "unit": "TFLOP/s",
       "cores": torch.get_num_threads(),
       "kind": "port",
-      "sample": f"benchmark config 1 linear (M={M} K={K} N={N}): per-token quant + scaled matmul "
+      "sample": f"benchmark config 1 linear (M={M} K={K} N={N}, 3 outlier channels x20): per-token quant + scaled matmul "
                 f"+ bias in eager PyTorch CPU ops, median of {len(times)} runs ({total_s:.0f} s of "
                 f"CPU work), {t*1e3:.0f} ms/linear",
       "quant_gbps": (3.0 * M * K + 4.0 * M) / tq / 1e9,
@@ -717,7 +818,9 @@ def main():
     print(json.dumps(out))
     return
   if args.headline_only:
-    print(json.dumps({"linear_headline": headline_kernels(device), "device": arch}))
+    print(json.dumps({"linear_headline": headline_kernels(device),
+                      "mfma_only": mfma_only_ceiling(device),
+                      "roofline_quant_large": quant_large_shapes(device), "device": arch}))
     return
 
   hot = HotPath(device)
@@ -793,6 +896,8 @@ def main():
     return
 
   head = headline_kernels(device)
+  ceiling = mfma_only_ceiling(device)
+  quant_large = quant_large_shapes(device)
   M, K, N = HEADLINE
   roofline = {
       "kernel": "gemm_fp8_wide<288x192> (w8a8 GEMM + scale/bias epilogue) at M=4608 K=3072 "
@@ -805,6 +910,10 @@ def main():
       # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain
       # copy of known size (read from profiles/traffic.json); algorithmic 165.2 MB
       "traffic": measured_traffic("gemm_fp8_wide_headline"),
+      # the same instruction with nothing else going on, timed in this run (mfma_only): the
+      # rate the power-limited part sustains on random e4m3 operands, and the GEMM against it
+      "mfma_only_tflops": ceiling["random_operands_tflops"],
+      "frac_of_mfma_only": head["gemm_tflops"] / ceiling["random_operands_tflops"],
   }
   roofline_quant = {
       "kernel": "quant_rowwise_regs at M=4608 K=3072",
@@ -891,6 +1000,16 @@ def main():
       "dit_compiled_cosine": dit_compiled[2],
       "roofline": roofline,
       "roofline_quant": roofline_quant,
+      # the same kernel on the largest activation of each benchmark configuration
+      "roofline_quant_large": quant_large,
+      "roofline_ln_modulate_quant": {
+          "kernel": "ln_modulate_quant (LayerNorm + AdaLN modulation + per-row quantizer in one "
+                    "pass) at M=4608 K=3072",
+          "bound": "hbm", "achieved": head["ln_modulate_quant_gbps"], "peak": HBM_PEAK_GBPS,
+          "unit": "GB/s", "frac": head["ln_modulate_quant_gbps"] / HBM_PEAK_GBPS,
+          "traffic": measured_traffic("ln_modulate_quant_headline"),
+      },
+      "mfma_only": ceiling,
       "cpu_baseline": cpu,
       "device": arch,
   }
