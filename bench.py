@@ -692,12 +692,11 @@ def dit_forward_ms(device, iters=5):
     model = FluxLikeTransformer().to(torch.bfloat16)
   cache_dit_amd.quantize(model, cache_dit_amd.QuantizeConfig(quant_type="float8_per_row"))
   dit_shapes.fuse_gelu_epilogues(model)
-  cache_dit_amd.share_activation_quant_(model)
   inputs = flux_like_inputs(device)
-  cache_dit_amd.group_sibling_linears_(model, lambda: model(**inputs))
-  dit_shapes.batch_streams(model)
-  dit_shapes.fuse_cat_quant(model)
-  dit_shapes.fuse_norm_quant(model, materialize=False)
+  # the model's block and attention code stays as it is: the stage patch functor hooks the
+  # attention modules and rebinds the block forwards (cache_dit_amd.patch_functors)
+  cache_dit_amd.apply_stage_patch(model, batch_stages=True, single_blocks=True, fuse_cat=True,
+                                  fuse_norm_quant=True, materialize=False)
   graph_ms = None
   with torch.no_grad():
     ms = _time_events(lambda: model(**inputs), iters, 2)

@@ -24,6 +24,10 @@ from .nn import share_activation_quant_
 from .nn import group_sibling_linears_
 from .nn import linear_batch
 from .nn import linear_on_cat
+from .nn import precompute_stage
+from .patch_functors import StagePatchFunctor
+from .patch_functors import apply_stage_patch
+from .patch_functors import remove_stage_patch
 from .ops import ln_modulate_quant
 from .utils import check_quantized
 
@@ -46,5 +50,9 @@ __all__ = [
     "group_sibling_linears_",
     "linear_batch",
     "linear_on_cat",
+    "precompute_stage",
+    "StagePatchFunctor",
+    "apply_stage_patch",
+    "remove_stage_patch",
     "ln_modulate_quant",
 ]

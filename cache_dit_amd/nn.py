@@ -69,6 +69,8 @@ class _Fp8LinearBase(nn.Linear):
 
   weight_scale: torch.Tensor
   share_input_quant: bool = False
+  #: (input key, output, stream, capture id) left by precompute_stage, or None
+  _precomputed = None
   epilogue: int
   scale_mode: str
   quant_type: str
@@ -232,6 +234,10 @@ class Fp8DynamicLinear(_Fp8LinearBase):
         if self.sibling_group is not None or self.share_input_quant:
           _note_inference_bypass(type(self).__name__)
       else:
+        if self._precomputed is not None:
+          out = _take_precomputed(self, x)
+          if out is not None:
+            return out
         if _recorder is not None:
           _recorder.note(self, x)
         if self.sibling_group is not None:
@@ -268,6 +274,10 @@ class Fp8WeightOnlyLinear(_Fp8LinearBase):
         if self.sibling_group is not None:
           _note_inference_bypass(type(self).__name__)
       else:
+        if self._precomputed is not None:
+          out = _take_precomputed(self, x)
+          if out is not None:
+            return out
         if _recorder is not None:
           _recorder.note(self, x)
         if self.sibling_group is not None:
@@ -446,6 +456,68 @@ def linear_batch(pairs):
       act[0], act[1] = q, s
     ops.gemm_rowwise_batched_into(acts)
   return result
+
+
+#: Linears that hold an output computed ahead by precompute_stage (dropped at the next stage)
+_precomputed_holders: list = []
+
+
+def _stream_state(x2: torch.Tensor):
+  capture_id = (_native.stream_capture_id(ops._stream_ptr(x2))
+                if torch.cuda.is_current_stream_capturing() else 0)
+  return (x2.device.index, ops._stream_ptr(x2)), capture_id
+
+
+def _take_precomputed(lin: "_Fp8LinearBase", x: torch.Tensor):
+  """The output precompute_stage left on `lin`, if `x` is the very activation it was computed
+  from (same buffer, unmodified, same stream and graph capture); None otherwise. Either way
+  the stash is emptied: an output is handed out once."""
+  key, out, stream, capture_id = lin._precomputed
+  lin._precomputed = None
+  x2 = ops._as_rows(x)
+  if key.matches(x2) and (stream, capture_id) == _stream_state(x2):
+    return out.view(*x.shape[:-1], lin.out_features)
+  return None
+
+
+def precompute_stage(pairs) -> bool:
+  """Runs `linear_batch(pairs)` now and leaves every output on its Linear, to be returned
+  when that Linear is next called with the very same activation. For code that knows which
+  Linears an unmodified module is about to call on which tensors (a forward pre-hook on an
+  attention module sees `hidden_states` and `encoder_hidden_states` before the module's own
+  code calls to_q / to_k / to_v and add_q_proj / add_k_proj / add_v_proj one by one): the
+  stage then costs one quantizer launch and one GEMM launch, and the module's code stays as
+  it is. A Linear that is called with anything else computes as usual, so a wrong guess
+  costs time, not correctness. Outputs nobody collects are dropped when the next stage is
+  precomputed. Returns False (nothing done) where linear_batch would not batch: a compiled
+  graph, inference-mode tensors, Linears of other types or of mixed types. Not thread-safe,
+  like the sibling groups."""
+  if torch.compiler.is_compiling():
+    return False
+  for lin in _precomputed_holders:
+    lin._precomputed = None
+  _precomputed_holders.clear()
+  flat = [lin for _, lins in pairs for lin in lins]
+  if not flat:
+    return False
+  first = flat[0]
+  if (type(first) not in (Fp8DynamicLinear, Fp8WeightOnlyLinear) or len(flat) > _native.MAX_GROUP
+      or len(pairs) > _native.MAX_ACTS or len({id(lin) for lin in flat}) != len(flat)
+      or any(type(lin) is not type(first) or lin.in_features != first.in_features
+             or lin._scale_mode_id != first._scale_mode_id or lin.sibling_group is not None
+             for lin in flat)
+      or any(not x.is_cuda or x.dtype != torch.bfloat16 or x.is_inference()
+             or x.shape[-1] != first.in_features for x, _ in pairs)):
+    return False
+  outs = linear_batch(pairs)
+  for (x, lins), ys in zip(pairs, outs):
+    x2 = ops._as_rows(x)
+    stream, capture_id = _stream_state(x2)
+    key = _InputKey(x2)
+    for lin, y in zip(lins, ys):
+      lin._precomputed = (key, y.view(-1, lin.out_features), stream, capture_id)
+      _precomputed_holders.append(lin)
+  return True
 
 
 def linear_on_cat(linear: nn.Module, xs) -> torch.Tensor:

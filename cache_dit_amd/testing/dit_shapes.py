@@ -97,21 +97,6 @@ def _ln(x, eps=1e-6):
   return F.layer_norm(x.float(), (x.shape[-1], ), eps=eps).to(x.dtype)
 
 
-class _ModulatedNorm:
-  """Mixin of the modules that compute `layer_norm(x) * (1 + scale) + shift` for quantized
-  Linears. With `fused_norm_quant` set (see fuse_norm_quant) the expression runs as one
-  HIP kernel that also delivers the FP8 codes to those Linears."""
-  fused_norm_quant = False
-  fused_norm_materialize = True
-
-  def _modulated(self, x, shift, scale):
-    if self.fused_norm_quant and x.is_cuda:
-      from .. import ops
-      return ops.ln_modulate_quant(x, shift, scale, eps=1e-6,
-                                   materialize=self.fused_norm_materialize)
-    return _ln(x) * (1 + scale) + shift
-
-
 class TimeEmbed(nn.Module):
   """timestep (+ pooled text) -> conditioning vector; names contain `embed`, so the
   default exclude list leaves these Linears alone when quantizing the whole model."""
@@ -134,36 +119,64 @@ class TimeEmbed(nn.Module):
 
 
 # ------------------------------------------------------------------------------- FLUX
+# Module attributes, forward signatures and return conventions are those of diffusers'
+# FluxTransformer2DModel blocks (the block forwards the reference adapts in
+# src/cache_dit/caching/patch_functors/functor_flux.py:48-80), so that code written against a
+# diffusers block -- the stage patchers of cache_dit_amd.patch_functors -- runs on these.
 
 
-class AdaLayerNormZero(_ModulatedNorm, nn.Module):
+class AdaLayerNormZero(nn.Module):
+  """diffusers' AdaLayerNormZero as FLUX uses it: `forward(x, emb=temb)` returns the modulated
+  norm and (gate_msa, shift_mlp, scale_mlp, gate_mlp)."""
 
-  def __init__(self, dim: int, chunks: int):
+  def __init__(self, dim: int):
     super().__init__()
-    self.chunks = chunks
-    self.linear = nn.Linear(dim, chunks * dim)
+    self.silu = nn.SiLU()
+    self.linear = nn.Linear(dim, 6 * dim)
+    self.norm = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
 
-  def forward(self, x, temb):
-    mods = self.linear(F.silu(temb)).unsqueeze(1).chunk(self.chunks, dim=-1)
-    shift, scale = mods[0], mods[1]
-    return self._modulated(x, shift, scale), mods[2:]
-
-
-def _batch(pairs):
-  from ..nn import linear_batch
-  return linear_batch(pairs)
+  def forward(self, x, timestep=None, class_labels=None, hidden_dtype=None, emb=None):
+    emb = self.linear(self.silu(emb))
+    shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = emb.chunk(6, dim=1)
+    x = self.norm(x) * (1 + scale_msa[:, None]) + shift_msa[:, None]
+    return x, gate_msa, shift_mlp, scale_mlp, gate_mlp
 
 
-def _ff_pair(ff_a: "FeedForward", xa, ff_b: "FeedForward", xb):
-  """Two FeedForwards on independent inputs, their Linears launched pairwise."""
-  (ha, ), (hb, ) = _batch([(xa, [ff_a.net[0].proj]), (xb, [ff_b.net[0].proj])])
-  ha, hb = ff_a.net[0].act(ha), ff_b.net[0].act(hb)  # identity once fused into the epilogue
-  (ya, ), (yb, ) = _batch([(ha, [ff_a.net[2]]), (hb, [ff_b.net[2]])])
-  return ya, yb
+class AdaLayerNormZeroSingle(nn.Module):
+  """diffusers' AdaLayerNormZeroSingle: `forward(x, emb=temb)` -> (modulated norm, gate)."""
+
+  def __init__(self, dim: int):
+    super().__init__()
+    self.silu = nn.SiLU()
+    self.linear = nn.Linear(dim, 3 * dim)
+    self.norm = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
+
+  def forward(self, x, emb=None):
+    emb = self.linear(self.silu(emb))
+    shift_msa, scale_msa, gate_msa = emb.chunk(3, dim=1)
+    x = self.norm(x) * (1 + scale_msa[:, None]) + shift_msa[:, None]
+    return x, gate_msa
+
+
+class AdaLayerNormContinuous(nn.Module):
+  """diffusers' AdaLayerNormContinuous (norm_out): scale first, then shift."""
+
+  def __init__(self, dim: int):
+    super().__init__()
+    self.silu = nn.SiLU()
+    self.linear = nn.Linear(dim, 2 * dim)
+    self.norm = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
+
+  def forward(self, x, conditioning_embedding):
+    emb = self.linear(self.silu(conditioning_embedding).to(x.dtype))
+    scale, shift = emb.chunk(2, dim=1)
+    return self.norm(x) * (1 + scale)[:, None, :] + shift[:, None, :]
 
 
 class FluxAttention(nn.Module):
-  batch_streams = False  # see batch_streams(): image- and text-stream Linears in one launch
+  """Joint (added_kv) or plain self-attention with per-head RMS norms of q and k; text
+  tokens first. `forward(hidden_states, encoder_hidden_states=None, image_rotary_emb=None)`
+  returns (image part, text part) for joint attention, one tensor otherwise."""
 
   def __init__(self, dim: int, heads: int, joint: bool):
     super().__init__()
@@ -179,89 +192,83 @@ class FluxAttention(nn.Module):
       self.norm_added_q, self.norm_added_k = RMSNorm(hd), RMSNorm(hd)
       self.to_add_out = nn.Linear(dim, dim)
 
-  def forward(self, hidden, encoder=None, rope=None, qkv=None):
-    if qkv is not None:  # computed by the caller together with other Linears on `hidden`
-      q, k, v = qkv
-    elif self.joint and self.batch_streams:
-      (q, k, v), (eq, ek, ev) = _batch([(hidden, [self.to_q, self.to_k, self.to_v]),
-                                        (encoder, [self.add_q_proj, self.add_k_proj, self.add_v_proj])])
-    else:
-      q, k, v = self.to_q(hidden), self.to_k(hidden), self.to_v(hidden)
-      if self.joint:
-        eq, ek, ev = self.add_q_proj(encoder), self.add_k_proj(encoder), self.add_v_proj(encoder)
+  def forward(self, hidden_states, encoder_hidden_states=None, image_rotary_emb=None, **kwargs):
+    q, k, v = self.to_q(hidden_states), self.to_k(hidden_states), self.to_v(hidden_states)
     q = self.norm_q(_heads(q, self.heads))
     k = self.norm_k(_heads(k, self.heads))
     v = _heads(v, self.heads)
     if self.joint:
+      eq = self.add_q_proj(encoder_hidden_states)
+      ek = self.add_k_proj(encoder_hidden_states)
+      ev = self.add_v_proj(encoder_hidden_states)
       eq = self.norm_added_q(_heads(eq, self.heads))
       ek = self.norm_added_k(_heads(ek, self.heads))
       ev = _heads(ev, self.heads)
       q, k, v = torch.cat([eq, q], 2), torch.cat([ek, k], 2), torch.cat([ev, v], 2)
-    if rope is not None:
-      q, k = apply_rope(q, rope), apply_rope(k, rope)
+    if image_rotary_emb is not None:
+      q, k = apply_rope(q, image_rotary_emb), apply_rope(k, image_rotary_emb)
     o = _merge(F.scaled_dot_product_attention(q, k, v))
     if not self.joint:
       return o
-    n_txt = encoder.shape[1]
-    if self.batch_streams:
-      (a, ), (ca, ) = _batch([(o[:, n_txt:], [self.to_out[0]]), (o[:, :n_txt], [self.to_add_out])])
-      return self.to_out[1](a), ca
-    return self.to_out[1](self.to_out[0](o[:, n_txt:])), self.to_add_out(o[:, :n_txt])
+    n_txt = encoder_hidden_states.shape[1]
+    encoder_part, hidden_part = o.split_with_sizes([n_txt, o.shape[1] - n_txt], dim=1)
+    hidden_part = self.to_out[1](self.to_out[0](hidden_part))
+    return hidden_part, self.to_add_out(encoder_part)
 
 
-class FluxTransformerBlock(_ModulatedNorm, nn.Module):
+class FluxTransformerBlock(nn.Module):
   """Double-stream block: 14 Linears (7 per stream)."""
 
   def __init__(self, dim: int, heads: int, mlp: int):
     super().__init__()
-    self.norm1, self.norm1_context = AdaLayerNormZero(dim, 6), AdaLayerNormZero(dim, 6)
+    self.norm1, self.norm1_context = AdaLayerNormZero(dim), AdaLayerNormZero(dim)
     self.attn = FluxAttention(dim, heads, joint=True)
-    self.ff, self.ff_context = FeedForward(dim, mlp), FeedForward(dim, mlp)
+    self.norm2 = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
+    self.ff = FeedForward(dim, mlp)
+    self.norm2_context = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
+    self.ff_context = FeedForward(dim, mlp)
 
-  def forward(self, hidden, encoder, temb, rope):
-    nh, (gate_msa, shift_mlp, scale_mlp, gate_mlp) = self.norm1(hidden, temb)
-    ne, (c_gate_msa, c_shift_mlp, c_scale_mlp, c_gate_mlp) = self.norm1_context(encoder, temb)
-    a, ca = self.attn(nh, ne, rope)
-    hidden = hidden + gate_msa * a
-    encoder = encoder + c_gate_msa * ca
-    if self.attn.batch_streams:
-      f, cf = _ff_pair(self.ff, self._modulated(hidden, shift_mlp, scale_mlp), self.ff_context,
-                       self._modulated(encoder, c_shift_mlp, c_scale_mlp))
-    else:
-      f = self.ff(self._modulated(hidden, shift_mlp, scale_mlp))
-      cf = self.ff_context(self._modulated(encoder, c_shift_mlp, c_scale_mlp))
-    hidden = hidden + gate_mlp * f
-    encoder = encoder + c_gate_mlp * cf
-    return encoder, hidden
+  def forward(self, hidden_states, encoder_hidden_states, temb, image_rotary_emb=None,
+              joint_attention_kwargs=None):
+    norm_hidden_states, gate_msa, shift_mlp, scale_mlp, gate_mlp = self.norm1(hidden_states, emb=temb)
+    norm_encoder_hidden_states, c_gate_msa, c_shift_mlp, c_scale_mlp, c_gate_mlp = self.norm1_context(
+        encoder_hidden_states, emb=temb)
+    attn_output, context_attn_output = self.attn(hidden_states=norm_hidden_states,
+                                                 encoder_hidden_states=norm_encoder_hidden_states,
+                                                 image_rotary_emb=image_rotary_emb,
+                                                 **(joint_attention_kwargs or {}))
+    hidden_states = hidden_states + gate_msa.unsqueeze(1) * attn_output
+    norm_hidden_states = self.norm2(hidden_states)
+    norm_hidden_states = norm_hidden_states * (1 + scale_mlp[:, None]) + shift_mlp[:, None]
+    hidden_states = hidden_states + gate_mlp.unsqueeze(1) * self.ff(norm_hidden_states)
+    encoder_hidden_states = encoder_hidden_states + c_gate_msa.unsqueeze(1) * context_attn_output
+    norm_encoder_hidden_states = self.norm2_context(encoder_hidden_states)
+    norm_encoder_hidden_states = norm_encoder_hidden_states * (1 + c_scale_mlp[:, None]) + c_shift_mlp[:, None]
+    encoder_hidden_states = encoder_hidden_states + c_gate_mlp.unsqueeze(1) * self.ff_context(
+        norm_encoder_hidden_states)
+    return encoder_hidden_states, hidden_states
 
 
 class FluxSingleTransformerBlock(nn.Module):
-  """Single-stream block: 6 Linears; `proj_mlp` is followed by GELU(tanh)."""
+  """Single-stream block on the concatenated [text | image] tokens: 6 Linears; `proj_mlp` is
+  followed by GELU(tanh)."""
 
   def __init__(self, dim: int, heads: int, mlp: int):
     super().__init__()
-    self.norm = AdaLayerNormZero(dim, 3)
+    self.norm = AdaLayerNormZeroSingle(dim)
     self.proj_mlp = nn.Linear(dim, mlp)
     self.act_mlp = nn.GELU(approximate="tanh")
     self.attn = FluxAttention(dim, heads, joint=False)
     self.proj_out = nn.Linear(dim + mlp, dim)
-    self.fuse_cat = False  # fuse_cat_quant: proj_out quantizes [attn | mlp] without the copy
-    self.batch_siblings = False  # batch_streams(single_blocks=True): proj_mlp + q/k/v in one launch
 
-  def forward(self, hidden, temb, rope):
-    normed, (gate, ) = self.norm(hidden, temb)
-    if self.batch_siblings:
-      (mlp, q, k, v), = _batch([(normed, [self.proj_mlp, self.attn.to_q, self.attn.to_k,
-                                          self.attn.to_v])])
-      mlp = self.act_mlp(mlp)
-      attn = self.attn(normed, rope=rope, qkv=(q, k, v))
-    else:
-      mlp = self.act_mlp(self.proj_mlp(normed))
-      attn = self.attn(normed, rope=rope)
-    if self.fuse_cat:
-      from ..nn import linear_on_cat
-      return hidden + gate * linear_on_cat(self.proj_out, [attn, mlp])
-    return hidden + gate * self.proj_out(torch.cat([attn, mlp], dim=2))
+  def forward(self, hidden_states, temb, image_rotary_emb=None, joint_attention_kwargs=None):
+    residual = hidden_states
+    norm_hidden_states, gate = self.norm(hidden_states, emb=temb)
+    mlp_hidden_states = self.act_mlp(self.proj_mlp(norm_hidden_states))
+    attn_output = self.attn(hidden_states=norm_hidden_states, image_rotary_emb=image_rotary_emb,
+                            **(joint_attention_kwargs or {}))
+    hidden_states = torch.cat([attn_output, mlp_hidden_states], dim=2)
+    return residual + gate.unsqueeze(1) * self.proj_out(hidden_states)
 
 
 class FluxLikeTransformer(nn.Module):
@@ -278,7 +285,7 @@ class FluxLikeTransformer(nn.Module):
         [FluxTransformerBlock(dim, heads, mlp) for _ in range(n_double)])
     self.single_transformer_blocks = nn.ModuleList(
         [FluxSingleTransformerBlock(dim, heads, mlp) for _ in range(n_single)])
-    self.norm_out = AdaLayerNormZero(dim, 2)
+    self.norm_out = AdaLayerNormContinuous(dim)
     self.proj_out = nn.Linear(dim, in_channels)
 
   def forward(self, hidden_states, encoder_hidden_states, pooled_projections, timestep):
@@ -288,12 +295,13 @@ class FluxLikeTransformer(nn.Module):
     n_txt, n_img = encoder.shape[1], hidden.shape[1]
     rope = rope_table(n_txt + n_img, self.dim // self.heads, hidden.device)
     for blk in self.transformer_blocks:
-      encoder, hidden = blk(hidden, encoder, temb, rope)
+      encoder, hidden = blk(hidden_states=hidden, encoder_hidden_states=encoder, temb=temb,
+                            image_rotary_emb=rope)
     hidden = torch.cat([encoder, hidden], dim=1)
     for blk in self.single_transformer_blocks:
-      hidden = blk(hidden, temb, rope)
+      hidden = blk(hidden_states=hidden, temb=temb, image_rotary_emb=rope)
     hidden = hidden[:, n_txt:]
-    hidden, _ = self.norm_out(hidden, temb)
+    hidden = self.norm_out(hidden, temb)
     return self.proj_out(hidden)
 
 
@@ -311,37 +319,45 @@ def flux_like_inputs(device, n_img=4096, n_txt=512, in_channels=64, text_dim=409
 # ------------------------------------------------------------------------------- Qwen-Image
 
 
-class QwenImageTransformerBlock(_ModulatedNorm, nn.Module):
-  """12 quantized Linears + `img_mod.1` / `txt_mod.1`, which the default exclude
-  pattern "mod" skips."""
+class QwenImageTransformerBlock(nn.Module):
+  """12 quantized Linears + `img_mod.1` / `txt_mod.1`, which the default exclude pattern
+  "mod" skips. Attributes, `_modulate` and the forward signature follow diffusers'
+  QwenImageTransformerBlock (the block the reference adapts in
+  src/cache_dit/caching/patch_functors/functor_qwen_image_controlnet.py:43-117)."""
 
   def __init__(self, dim: int, heads: int, mlp: int):
     super().__init__()
     self.img_mod = nn.Sequential(nn.SiLU(), nn.Linear(dim, 6 * dim))
-    self.txt_mod = nn.Sequential(nn.SiLU(), nn.Linear(dim, 6 * dim))
+    self.img_norm1 = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
     self.attn = FluxAttention(dim, heads, joint=True)
-    self.img_mlp, self.txt_mlp = FeedForward(dim, mlp), FeedForward(dim, mlp)
+    self.img_norm2 = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
+    self.img_mlp = FeedForward(dim, mlp)
+    self.txt_mod = nn.Sequential(nn.SiLU(), nn.Linear(dim, 6 * dim))
+    self.txt_norm1 = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
+    self.txt_norm2 = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
+    self.txt_mlp = FeedForward(dim, mlp)
 
-  def _modulate(self, x, shift, scale):
-    return self._modulated(x, shift, scale)
+  def _modulate(self, x, mod_params):
+    shift, scale, gate = mod_params.chunk(3, dim=-1)
+    return x * (1 + scale.unsqueeze(1)) + shift.unsqueeze(1), gate.unsqueeze(1)
 
-  def forward(self, hidden, encoder, temb, rope):
-    i1, i2 = self.img_mod(temb).unsqueeze(1).chunk(2, dim=-1)
-    t1, t2 = self.txt_mod(temb).unsqueeze(1).chunk(2, dim=-1)
-    (si1, sc1, g1), (si2, sc2, g2) = i1.chunk(3, dim=-1), i2.chunk(3, dim=-1)
-    (ti1, tc1, tg1), (ti2, tc2, tg2) = t1.chunk(3, dim=-1), t2.chunk(3, dim=-1)
-    a, ca = self.attn(self._modulate(hidden, si1, sc1), self._modulate(encoder, ti1, tc1), rope)
-    hidden = hidden + g1 * a
-    encoder = encoder + tg1 * ca
-    if self.attn.batch_streams:
-      f, cf = _ff_pair(self.img_mlp, self._modulate(hidden, si2, sc2), self.txt_mlp,
-                       self._modulate(encoder, ti2, tc2))
-    else:
-      f = self.img_mlp(self._modulate(hidden, si2, sc2))
-      cf = self.txt_mlp(self._modulate(encoder, ti2, tc2))
-    hidden = hidden + g2 * f
-    encoder = encoder + tg2 * cf
-    return encoder, hidden
+  def forward(self, hidden_states, encoder_hidden_states, encoder_hidden_states_mask=None, temb=None,
+              image_rotary_emb=None, joint_attention_kwargs=None):
+    img_mod1, img_mod2 = self.img_mod(temb).chunk(2, dim=-1)
+    txt_mod1, txt_mod2 = self.txt_mod(temb).chunk(2, dim=-1)
+    img_modulated, img_gate1 = self._modulate(self.img_norm1(hidden_states), img_mod1)
+    txt_modulated, txt_gate1 = self._modulate(self.txt_norm1(encoder_hidden_states), txt_mod1)
+    img_attn_output, txt_attn_output = self.attn(hidden_states=img_modulated,
+                                                 encoder_hidden_states=txt_modulated,
+                                                 image_rotary_emb=image_rotary_emb,
+                                                 **(joint_attention_kwargs or {}))
+    hidden_states = hidden_states + img_gate1 * img_attn_output
+    encoder_hidden_states = encoder_hidden_states + txt_gate1 * txt_attn_output
+    img_modulated2, img_gate2 = self._modulate(self.img_norm2(hidden_states), img_mod2)
+    hidden_states = hidden_states + img_gate2 * self.img_mlp(img_modulated2)
+    txt_modulated2, txt_gate2 = self._modulate(self.txt_norm2(encoder_hidden_states), txt_mod2)
+    encoder_hidden_states = encoder_hidden_states + txt_gate2 * self.txt_mlp(txt_modulated2)
+    return encoder_hidden_states, hidden_states
 
 
 class QwenImageLikeTransformer(nn.Module):
@@ -356,7 +372,7 @@ class QwenImageLikeTransformer(nn.Module):
     self.time_text_embed = TimeEmbed(dim)
     self.transformer_blocks = nn.ModuleList(
         [QwenImageTransformerBlock(dim, heads, mlp) for _ in range(n_layers)])
-    self.norm_out = AdaLayerNormZero(dim, 2)
+    self.norm_out = AdaLayerNormContinuous(dim)
     self.proj_out = nn.Linear(dim, in_channels)
 
   def forward(self, hidden_states, encoder_hidden_states, timestep):
@@ -365,8 +381,9 @@ class QwenImageLikeTransformer(nn.Module):
     temb = self.time_text_embed(timestep)
     rope = rope_table(encoder.shape[1] + hidden.shape[1], self.dim // self.heads, hidden.device)
     for blk in self.transformer_blocks:
-      encoder, hidden = blk(hidden, encoder, temb, rope)
-    hidden, _ = self.norm_out(hidden, temb)
+      encoder, hidden = blk(hidden_states=hidden, encoder_hidden_states=encoder,
+                            encoder_hidden_states_mask=None, temb=temb, image_rotary_emb=rope)
+    hidden = self.norm_out(hidden, temb)
     return self.proj_out(hidden)
 
 
@@ -384,6 +401,9 @@ def qwen_image_like_inputs(device, n_img=6889, n_txt=256, in_channels=64, text_d
 
 
 class WanAttention(nn.Module):
+  """`forward(hidden_states, encoder_hidden_states=None, rotary_emb=None)`: self-attention,
+  or cross-attention to the text when `encoder_hidden_states` is given (diffusers'
+  WanAttention; reference: src/cache_dit/distributed/transformers/wan.py:69-160)."""
 
   def __init__(self, dim: int, heads: int):
     super().__init__()
@@ -392,32 +412,45 @@ class WanAttention(nn.Module):
     self.to_out = nn.ModuleList([nn.Linear(dim, dim), nn.Dropout(0.0)])
     self.norm_q, self.norm_k = RMSNorm(dim), RMSNorm(dim)  # full width, before the head split
 
-  def forward(self, hidden, context=None, rope=None):
-    src = hidden if context is None else context
-    q = _heads(self.norm_q(self.to_q(hidden)), self.heads)
+  def forward(self, hidden_states, encoder_hidden_states=None, attention_mask=None, rotary_emb=None,
+              **kwargs):
+    src = hidden_states if encoder_hidden_states is None else encoder_hidden_states
+    q = _heads(self.norm_q(self.to_q(hidden_states)), self.heads)
     k = _heads(self.norm_k(self.to_k(src)), self.heads)
     v = _heads(self.to_v(src), self.heads)
-    if rope is not None:
-      q, k = apply_rope(q, rope), apply_rope(k, rope)
+    if rotary_emb is not None:
+      q, k = apply_rope(q, rotary_emb), apply_rope(k, rotary_emb)
     o = _merge(F.scaled_dot_product_attention(q, k, v))
     return self.to_out[1](self.to_out[0](o))
 
 
-class WanTransformerBlock(_ModulatedNorm, nn.Module):
-  """10 Linears: self-attention, cross-attention to the text, GELU-tanh FFN."""
+class WanTransformerBlock(nn.Module):
+  """10 Linears: self-attention, cross-attention to the text, GELU-tanh FFN. Attributes and
+  the forward signature follow diffusers' WanTransformerBlock (the block the reference adapts
+  in src/cache_dit/caching/patch_functors/functor_wan_vace.py:40-90); the two modulations are
+  done in bf16 tensor ops here (diffusers computes them in fp32 and rounds once)."""
 
   def __init__(self, dim: int, heads: int, ffn: int):
     super().__init__()
-    self.attn1, self.attn2 = WanAttention(dim, heads), WanAttention(dim, heads)
+    self.norm1 = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
+    self.attn1 = WanAttention(dim, heads)
+    self.attn2 = WanAttention(dim, heads)
     self.norm2 = nn.LayerNorm(dim, eps=1e-6)
     self.ffn = FeedForward(dim, ffn)
+    self.norm3 = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
     self.scale_shift_table = nn.Parameter(torch.randn(1, 6, dim) / dim**0.5)
 
-  def forward(self, hidden, context, temb6, rope):
-    sh1, sc1, g1, sh2, sc2, g2 = (self.scale_shift_table + temb6).chunk(6, dim=1)
-    hidden = hidden + g1 * self.attn1(self._modulated(hidden, sh1, sc1), rope=rope)
-    hidden = hidden + self.attn2(self.norm2(hidden), context)
-    return hidden + g2 * self.ffn(self._modulated(hidden, sh2, sc2))
+  def forward(self, hidden_states, encoder_hidden_states, temb, rotary_emb=None):
+    shift_msa, scale_msa, gate_msa, c_shift_msa, c_scale_msa, c_gate_msa = (
+        self.scale_shift_table + temb).chunk(6, dim=1)
+    norm_hidden_states = self.norm1(hidden_states) * (1 + scale_msa) + shift_msa
+    attn_output = self.attn1(hidden_states=norm_hidden_states, rotary_emb=rotary_emb)
+    hidden_states = hidden_states + attn_output * gate_msa
+    norm_hidden_states = self.norm2(hidden_states)
+    hidden_states = hidden_states + self.attn2(hidden_states=norm_hidden_states,
+                                               encoder_hidden_states=encoder_hidden_states)
+    norm_hidden_states = self.norm3(hidden_states) * (1 + c_scale_msa) + c_shift_msa
+    return hidden_states + self.ffn(norm_hidden_states) * c_gate_msa
 
 
 class WanLikeTransformer(nn.Module):
@@ -443,7 +476,7 @@ class WanLikeTransformer(nn.Module):
     context = self.condition_embedder["text_embedder"](encoder_hidden_states)
     rope = rope_table(hidden.shape[1], self.dim // self.heads, hidden.device)
     for blk in self.blocks:
-      hidden = blk(hidden, context, temb6, rope)
+      hidden = blk(hidden_states=hidden, encoder_hidden_states=context, temb=temb6, rotary_emb=rope)
     return self.proj_out(_ln(hidden))
 
 
@@ -480,52 +513,51 @@ def fuse_gelu_epilogues(model: nn.Module) -> int:
   return n
 
 
+def _restage(model: nn.Module, **changes) -> None:
+  """(Re)applies the stage patch functor with the options accumulated on `model`."""
+  from ..patch_functors import StagePatchFunctor
+  opts = model.__dict__.setdefault("_stage_opts", {
+      "batch_stages": False, "single_blocks": False, "fuse_cat": False, "fuse_norm_quant": False,
+      "materialize": True})
+  opts.update(changes)
+  if any(opts[k] for k in ("batch_stages", "fuse_cat", "fuse_norm_quant")):
+    StagePatchFunctor().apply(model, **opts)
+  else:
+    StagePatchFunctor().remove(model)
+
+
 def batch_streams(model: nn.Module, enable: bool = True, single_blocks: bool = False) -> int:
-  """Switches the double-stream blocks of `model` (FLUX, Qwen-Image) to forwards that hand
-  the image-stream and the text-stream Linears of a stage to linear_batch: one GEMM launch
-  per stage instead of one per Linear, the small text-stream GEMMs riding along with the
-  large image-stream ones. single_blocks=True does the same for proj_mlp + q/k/v of FLUX
-  single blocks (in eager code group_sibling_linears_ finds those by itself; a compiled
-  graph needs the explicit call). Outputs are bit-identical. Returns the number of
-  double-stream attention modules switched."""
-  n = 0
-  for m in model.modules():
-    if isinstance(m, FluxAttention) and m.joint:
-      m.batch_streams = bool(enable)
-      n += 1
-    if isinstance(m, FluxSingleTransformerBlock):
-      m.batch_siblings = bool(enable) and single_blocks
-  return n
+  """Patches `model` (cache_dit_amd.patch_functors.StagePatchFunctor) so that the Linears of
+  every stage of a block run as one launch: the image-stream and the text-stream Linears of
+  a double-stream block (FLUX, Qwen-Image), the query next to key / value of a cross
+  attention (Wan); single_blocks=True also proj_mlp + q/k/v of FLUX single blocks. The
+  model's own forwards stay as they are. Outputs are bit-identical. Returns the number of
+  double-stream attention modules."""
+  _restage(model, batch_stages=bool(enable), single_blocks=bool(enable) and single_blocks)
+  return sum(isinstance(m, FluxAttention) and m.joint for m in model.modules())
 
 
 def fuse_cat_quant(model: nn.Module, enable: bool = True) -> int:
-  """Switches the single-stream blocks of `model` to `linear_on_cat`: proj_out's quantizer
-  reads the attention output and the MLP activation in place instead of their torch.cat
-  copy. Outputs are bit-identical. Returns the number of blocks switched."""
-  n = 0
-  for m in model.modules():
-    if isinstance(m, FluxSingleTransformerBlock):
-      m.fuse_cat = bool(enable)
-      n += 1
-  return n
+  """Single-stream blocks of `model`: proj_out's quantizer reads the attention output and the
+  MLP activation in place instead of their torch.cat copy (`nn.linear_on_cat`, through the
+  stage patch functor). Outputs are bit-identical. Returns the number of such blocks."""
+  _restage(model, fuse_cat=bool(enable))
+  return sum(isinstance(m, FluxSingleTransformerBlock) for m in model.modules())
 
 
 def fuse_norm_quant(model: nn.Module, enable: bool = True, materialize: bool = True) -> int:
-  """Switches every modulated LayerNorm of `model` to the kernel that also quantizes
-  (ops.ln_modulate_quant). Pair it with share_activation_quant_ on the Linears so that
-  they pick the delivered codes up. materialize=False also drops the bf16 write of the
-  modulated activation: valid here because only quantized Linears read it. Returns the
-  number of modules switched."""
+  """Every modulated LayerNorm inside the repeated blocks of `model` runs as the kernel that
+  also quantizes (ops.ln_modulate_quant, through the stage patch functor), and the Linears of
+  the blocks pick the delivered codes up. materialize=False also drops the bf16 write of the
+  modulated activation: valid here because only quantized Linears read it. Returns the number
+  of modules whose forward computes a modulated norm (FLUX double block: norm1, norm1_context
+  and the block itself; single block: norm; Qwen-Image and Wan blocks: the block)."""
+  _restage(model, fuse_norm_quant=bool(enable), materialize=bool(materialize))
   n = 0
-  blocks = getattr(model, "_repeated_blocks", [])
-  for blk in model.modules():
-    if type(blk).__name__ not in blocks:
-      continue  # outside the repeated blocks (norm_out) the consumer is an unquantized Linear
-    for m in blk.modules():
-      if isinstance(m, _ModulatedNorm):
-        m.fused_norm_quant = bool(enable)
-        m.fused_norm_materialize = bool(materialize)
-        n += 1
+  for m in model.modules():
+    name = type(m).__name__
+    n += {"FluxTransformerBlock": 3, "FluxSingleTransformerBlock": 1, "QwenImageTransformerBlock": 1,
+          "WanTransformerBlock": 1}.get(name, 0)
   return n
 
 
