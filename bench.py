@@ -719,19 +719,19 @@ def dit_forward_ms(device, iters=5):
       note_err = ""
   del model
   torch.cuda.empty_cache()
-  return ms, graph_ms, ("float8_per_row, GELU-tanh fused into the producing Linear, sibling Linears "
-                        "grouped on one shared quantization, image- and text-stream Linears of a "
-                        "stage batched into one launch, quantizer fused into the modulated "
-                        "LayerNorms and reading proj_out's two sources in place; bf16 SDPA attention, RMS norms, RoPE and residual glue in eager "
-                        "PyTorch ops" + note_err)
+  return ms, graph_ms, ("float8_per_row on the unmodified synthetic model + apply_stage_patch: "
+                        "GELU-tanh fused into the producing Linear, the Linears of a stage (image "
+                        "and text stream, proj_mlp + q/k/v) one quantizer and one batched GEMM "
+                        "launch, quantizer fused into the modulated LayerNorms and reading "
+                        "proj_out's two sources in place; bf16 SDPA attention, RMS norms, RoPE "
+                        "and residual glue in eager PyTorch ops" + note_err)
 
 
 def dit_forward_compiled_ms(device, iters=5):
   """The same transformer with its blocks compiled by torch.compile (regional compilation,
-  fullgraph): every converted Linear is one registered op, the Linears of a stage one
-  batched op (cdit::linear_w8a8_batch), so Inductor fuses the element-wise glue around
-  them. Returns (ms, seconds spent compiling, cosine against the eager forward) or
-  (None, None, note)."""
+  fullgraph): every converted Linear is one registered op, so Inductor fuses the
+  element-wise glue around them. Returns (ms, seconds spent compiling, cosine against the
+  eager forward) or (None, None, note)."""
   try:
     import torch
     import cache_dit_amd
@@ -741,7 +741,8 @@ def dit_forward_compiled_ms(device, iters=5):
       model = dit_shapes.FluxLikeTransformer().to(torch.bfloat16)
     cache_dit_amd.quantize(model, cache_dit_amd.QuantizeConfig(quant_type="float8_per_row"))
     dit_shapes.fuse_gelu_epilogues(model)
-    dit_shapes.batch_streams(model, single_blocks=True)
+    # (no stage patch here: a traced graph takes none of its stateful shortcuts, and its
+    # per-module hooks would make every block a compilation of its own)
     inputs = dit_shapes.flux_like_inputs(device)
     with torch.no_grad():
       want = model(**inputs)
@@ -958,7 +959,10 @@ def main():
                       "proj_mlp + q/k/v) share its quantization, and the independent Linears of "
                       "one stage of a block (image stream + text stream) run as one quantizer "
                       "launch and one batched GEMM launch (two where the tile cost model splits "
-                      "the stage), bit-identical to running each Linear on its own",
+                      "the stage), bit-identical to running each Linear on its own. This is the "
+                      "launch pattern cache_dit_amd.apply_stage_patch gives an unmodified model "
+                      "(hooks on its attention modules, rebound block forwards); plain "
+                      "quantize() alone gives ungrouped_*, group_sibling_linears_ grouped_*",
           "quant_type": "float8_per_row",
           "launch": launch_mode,
           "linears_per_step": n_layers,

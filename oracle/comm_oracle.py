@@ -61,9 +61,34 @@ def qkv_permute_quant(x: torch.Tensor) -> torch.Tensor:
 
 def qkv_permute_dequant(quant_x: torch.Tensor) -> torch.Tensor:
   """_fp8_comm_qkv_dequant_permute_kernel (_float8_comm.py:116-148): e4m3 [S, B, N, D + 4]
-  -> bf16 [B, S, N, D]."""
+  -> bf16 [B, S, N, D], x[b, s] = dequant(quant_x[s, b]): the inverse of qkv_permute_quant's
+  permutation, which is what the output's declared shape says.
+
+  DEVIATION for B > 1, parity unpinned there: the reference kernel as written stores the
+  dequantized row of program `bs_id = s * B + b` at `x_ptr + bs_id * x.stride(1)`
+  (_float8_comm.py:130-139; the wrapper passes x.stride(1) of the [B, S, N, D] output,
+  _ops_registery.py:160-170), i.e. at flat row s * B + b of a buffer whose flat row b * S + s
+  is x[b, s]. For B = 1 the two agree; for B > 1 and S > 1 the reference leaves the rows in
+  [S, B] order inside a tensor declared [B, S, N, D], so that dequant(quant(x)[p]) is not
+  x[:, :, p]. Its own test (tests/kernels/test_triton_ops.py:132-160, B = 2) only asks that
+  the result be nearer to slice p than to the other slices, which both layouts satisfy.
+  This restatement, and the HIP kernel, implement the true permutation (round trip =
+  identity up to quantization error); `qkv_permute_dequant_as_written` below restates the
+  literal behaviour for comparison."""
   S, B, N, D4 = quant_x.shape
   D = D4 - 4
   scale = quant_x[..., D:].contiguous().view(torch.float32)  # [S, B, N, 1]
   x = quant_x[..., :D].to(torch.float32) * scale
   return x.to(torch.bfloat16).permute(1, 0, 2, 3).contiguous()
+
+
+def qkv_permute_dequant_as_written(quant_x: torch.Tensor) -> torch.Tensor:
+  """The reference kernel's literal store pattern (see qkv_permute_dequant): flat row
+  s * B + b of the [B, S, N, D] output receives dequant(quant_x[s, b]). Equal to
+  qkv_permute_dequant for B = 1 only. Not used by the product; kept so that a test can state
+  which of the two layouts this build follows."""
+  S, B, N, D4 = quant_x.shape
+  D = D4 - 4
+  scale = quant_x[..., D:].contiguous().view(torch.float32)
+  x = (quant_x[..., :D].to(torch.float32) * scale).to(torch.bfloat16)  # [S, B, N, D]
+  return x.reshape(S * B, N, D).reshape(B, S, N, D).contiguous()

@@ -102,3 +102,29 @@ def test_reference_round_trip_qkv_tracks_selected_slice():
     assert d.shape == (2, 4, 5, 64) and d.dtype == torch.bfloat16
     assert min(range(3), key=lambda i: dist[i]) == p
     assert dist[p] < 0.05
+
+
+def test_permute_dequant_layout_for_more_than_one_batch_element():
+  """Which layout the restatement (and the HIP kernel) follow where the reference's kernel as
+  written and the declared output shape disagree (B > 1, S > 1): the true permutation, under
+  which quant -> dequant is the identity up to quantization error on x[:, :, p]. The literal
+  store pattern of the reference agrees for B = 1 and scrambles rows otherwise; parity is
+  unpinned for B > 1 (the reference's own test passes under both)."""
+  g = torch.Generator().manual_seed(0)
+  for B, S in ((1, 5), (2, 4), (3, 2)):
+    x = torch.randn(B, S, 3, 5, 64, generator=g).to(torch.bfloat16)
+    qx = co.qkv_permute_quant(x)
+    for p in range(3):
+      want = x[:, :, p].float()
+      back = co.qkv_permute_dequant(qx[p]).float()
+      literal = co.qkv_permute_dequant_as_written(qx[p]).float()
+      assert back.shape == want.shape == literal.shape
+      assert (back - want).abs().max() <= 0.07 * want.abs().max()       # half an e4m3 step at most
+      if B == 1:
+        assert torch.equal(literal, back)
+      else:
+        assert (literal - want).abs().max() > 0.5 * want.abs().max()     # rows in [S, B] order
+        # the reference's own (loose) criterion holds for both layouts
+        for cand in (back, literal):
+          d = [(cand - x[:, :, r].float()).abs().mean().item() for r in range(3)]
+          assert min(range(3), key=lambda r: d[r]) == p
