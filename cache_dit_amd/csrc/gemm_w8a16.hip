@@ -774,16 +774,6 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n,
     // 64 contiguous bytes, lanes 4r .. 4r+3 on row r. They are issued while the next
     // block is computed, the last block's after the two copies of the epilogue join.
     const int bp_addr = 4 * (16 * (lane & 3) + (lane >> 2));
-    // Whole lines (wave tiles whose width is a multiple of 64 columns): two neighbouring
-    // column blocks are stored together, 8 lanes on the 128 contiguous bytes of a row and 8
-    // rows per store instruction, so that no 128-byte line leaves in two halves. After the
-    // permlane16_swap (lane bit 4 now says which 16 bytes, the register which half of the 32
-    // rows) the two blocks trade words between the halves of every 16-lane row (DPP
-    // row_ror:8 under a bank mask: lane bit 3 now says which block, the register which 8
-    // rows), and ds_bpermute_b32 hands lane L = 8 row + piece the words of lane
-    // 32 ((piece >> 1) & 1) + 16 (piece & 1) + 8 (piece >> 2) + row.
-    constexpr bool FULL_LINE = C::WN % 64 == 0;
-    const int bp_line = 4 * (32 * ((lane >> 1) & 1) + 16 * (lane & 1) + 8 * ((lane >> 2) & 1) + (lane >> 3));
     // Buffer stores: the descriptor of a block covers the rows of it that exist (the
     // hardware drops lanes beyond), lanes whose columns do not exist get an offset
     // beyond any descriptor -- no bounds branches, no 64-bit address arithmetic per store.
@@ -800,121 +790,60 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n,
     uint8_t* const out_wave = reinterpret_cast<uint8_t*>(cur_out) +
                               ((int64_t)(m0 + wm * C::WM) * cur_ldo + (n0 + wn * C::WN)) * 2;
     const int rows_wave = m_of(cur_act) - (m0 + wm * C::WM);
-    const uint32_t out_lane = FULL_LINE
-                                  ? ((uint32_t)(lane >> 3) * (uint32_t)cur_ldo + 8u * (lane & 7)) * 2
-                                  : ((uint32_t)(lane >> 2) * (uint32_t)cur_ldo + 8u * (lane & 3)) * 2;
+    const uint32_t out_lane = ((uint32_t)(lane >> 2) * (uint32_t)cur_ldo + 8u * (lane & 3)) * 2;
     const uint32_t half_block = 16u * (uint32_t)cur_ldo * 2;
-    const uint32_t rows8 = 8u * (uint32_t)cur_ldo * 2;
-    constexpr int NOFF = FULL_LINE ? TN / 2 : TN;  // column offsets: per pair of blocks or per block
-    uint32_t out_off[NOFF];
+    uint32_t out_off[TN];
 #pragma unroll
-    for (int j = 0; j < NOFF; ++j) {
-      if constexpr (FULL_LINE) {
-        out_off[j] = n0 + wn * C::WN + 64 * j + 8 * (lane & 7) < cur_N ? out_lane + 128 * j : kNoColumn;
-      } else {
-        out_off[j] = n0 + wn * C::WN + 32 * j + 8 * (lane & 3) < cur_N ? out_lane + 64 * j : kNoColumn;
-      }
-    }
-    auto block_rsrc = [&](int i) {
-      const int rows = __builtin_amdgcn_readfirstlane(min(max(rows_wave - 32 * i, 0), 32));
-      return __builtin_amdgcn_make_buffer_rsrc(out_wave + (int64_t)(32 * i) * cur_ldo * 2, 0,
-                                               rows * cur_ldo * 2, 0x00020000);
-    };
-    uint32_t moved[FULL_LINE ? 16 : 8];
-    // FULL_LINE: (i, jp) is a pair of blocks, four stores of 8 rows; else (i, j) one block,
-    // two stores of 16 rows
+    for (int j = 0; j < TN; ++j)
+      out_off[j] = n0 + wn * C::WN + 32 * j + 8 * (lane & 3) < cur_N ? out_lane + 64 * j : kNoColumn;
+    uint32_t moved[8];
     auto store_moved = [&](int i, int j) {
-      const __amdgpu_buffer_rsrc_t block = block_rsrc(i);
-      if constexpr (FULL_LINE) {
-#pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4)
-          __builtin_amdgcn_raw_buffer_store_b128(
-              v4u{moved[4 * s4], moved[4 * s4 + 1], moved[4 * s4 + 2], moved[4 * s4 + 3]}, block,
-              (int)(out_off[j] + s4 * rows8), 0, 2);
-      } else {
-        __builtin_amdgcn_raw_buffer_store_b128(v4u{moved[0], moved[1], moved[2], moved[3]}, block,
-                                               (int)out_off[j], 0, 2);
-        __builtin_amdgcn_raw_buffer_store_b128(v4u{moved[4], moved[5], moved[6], moved[7]}, block,
-                                               (int)(out_off[j] + half_block), 0, 2);
-      }
+      const int rows = __builtin_amdgcn_readfirstlane(min(max(rows_wave - 32 * i, 0), 32));
+      const __amdgpu_buffer_rsrc_t block = __builtin_amdgcn_make_buffer_rsrc(
+          out_wave + (int64_t)(32 * i) * cur_ldo * 2, 0, rows * cur_ldo * 2, 0x00020000);
+      __builtin_amdgcn_raw_buffer_store_b128(v4u{moved[0], moved[1], moved[2], moved[3]}, block,
+                                             (int)out_off[j], 0, 2);
+      __builtin_amdgcn_raw_buffer_store_b128(v4u{moved[4], moved[5], moved[6], moved[7]}, block,
+                                             (int)(out_off[j] + half_block), 0, 2);
     };
     auto epilogue = [&](auto gelu_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
-      // packed bf16 words of block (i, j): 8 per lane (16 consecutive columns of one row)
-      auto block_words = [&](int i, int j, uint32_t (&pk)[8]) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
         const uint32_t bw[8] = {bi[j][0].x, bi[j][0].y, bi[j][0].z, bi[j][0].w,
                                 bi[j][1].x, bi[j][1].y, bi[j][1].z, bi[j][1].w};
 #pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const float b0 = __uint_as_float(bw[r >> 1] << 16);
-          const float b1 = __uint_as_float(bw[r >> 1] & 0xffff0000u);
-          float a0, a1;
-          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a0) : "a"(acc[i][j][r]));
-          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a1) : "a"(acc[i][j][r + 1]));
-          float v0 = __fmaf_rn(a0, bs[j][r >> 2][r & 3], b0);
-          float v1 = __fmaf_rn(a1, bs[j][r >> 2][(r + 1) & 3], b1);
-          if constexpr (GELU) {
-            v0 = gelu_tanh(v0);
-            v1 = gelu_tanh(v1);
+        for (int i = 0; i < TM; ++i) {
+          uint32_t pk[8];
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            const float b0 = __uint_as_float(bw[r >> 1] << 16);
+            const float b1 = __uint_as_float(bw[r >> 1] & 0xffff0000u);
+            float a0, a1;
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a0) : "a"(acc[i][j][r]));
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a1) : "a"(acc[i][j][r + 1]));
+            float v0 = __fmaf_rn(a0, bs[j][r >> 2][r & 3], b0);
+            float v1 = __fmaf_rn(a1, bs[j][r >> 2][(r + 1) & 3], b1);
+            if constexpr (GELU) {
+              v0 = gelu_tanh(v0);
+              v1 = gelu_tanh(v1);
+            }
+            pk[r >> 1] = pack_bf16x2(v0, v1);
           }
-          pk[r >> 1] = pack_bf16x2(v0, v1);
-        }
-      };
-      if constexpr (FULL_LINE) {
-#pragma unroll
-        for (int jp = 0; jp < TN / 2; ++jp) {
-#pragma unroll
-          for (int i = 0; i < TM; ++i) {
-            uint32_t pk0[8], pk1[8];
-            block_words(i, 2 * jp, pk0);
-            block_words(i, 2 * jp + 1, pk1);
-            // the previous pair's words have had this pair's arithmetic to arrive
-            __builtin_amdgcn_sched_barrier(0);
-            if (i > 0) {
-              store_moved(i - 1, jp);
-            } else if (jp > 0) {
-              store_moved(TM - 1, jp - 1);
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-              const auto s0 = __builtin_amdgcn_permlane16_swap(pk0[k], pk0[4 + k], false, false);
-              const auto s1 = __builtin_amdgcn_permlane16_swap(pk1[k], pk1[4 + k], false, false);
-#pragma unroll
-              for (int a = 0; a < 2; ++a) {  // rows 0-15 and 16-31 of the block
-                const int w0 = (int)s0[a], w1 = (int)s1[a];
-                // row_ror:8 = 0x128; bank mask 0xc: lanes 8-15 of a row of 16 take the other
-                // half's word, lanes 0-7 keep `old`; 0x3 the other way round
-                const int p = __builtin_amdgcn_update_dpp(w0, w1, 0x128, 0xf, 0xc, false);
-                const int q = __builtin_amdgcn_update_dpp(w1, w0, 0x128, 0xf, 0x3, false);
-                moved[4 * (2 * a) + k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_line, p);
-                moved[4 * (2 * a + 1) + k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_line, q);
-              }
-            }
-            __builtin_amdgcn_sched_barrier(0);
+          // the previous block's words have had this block's arithmetic to arrive
+          __builtin_amdgcn_sched_barrier(0);
+          if (i > 0) {
+            store_moved(i - 1, j);
+          } else if (j > 0) {
+            store_moved(TM - 1, j - 1);
           }
-        }
-      } else {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-#pragma unroll
-          for (int i = 0; i < TM; ++i) {
-            uint32_t pk[8];
-            block_words(i, j, pk);
-            // the previous block's words have had this block's arithmetic to arrive
-            __builtin_amdgcn_sched_barrier(0);
-            if (i > 0) {
-              store_moved(i - 1, j);
-            } else if (j > 0) {
-              store_moved(TM - 1, j - 1);
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-              const auto sw = __builtin_amdgcn_permlane16_swap(pk[k], pk[4 + k], false, false);
-              moved[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_addr, (int)sw[0]);
-              moved[4 + k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_addr, (int)sw[1]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
+          for (int k = 0; k < 4; ++k) {
+            const auto sw = __builtin_amdgcn_permlane16_swap(pk[k], pk[4 + k], false, false);
+            moved[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_addr, (int)sw[0]);
+            moved[4 + k] = (uint32_t)__builtin_amdgcn_ds_bpermute(bp_addr, (int)sw[1]);
           }
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     };
@@ -923,7 +852,7 @@ gemm_w8a16_wide(GemmArgs g, int tiles_m, int tiles_n,
     } else {
       epilogue(std::false_type{});
     }
-    store_moved(TM - 1, FULL_LINE ? TN / 2 - 1 : TN - 1);
+    store_moved(TM - 1, TN - 1);
     if (next_tile >= ntiles) break;
     m0 = nm0;
     n0 = nn0;

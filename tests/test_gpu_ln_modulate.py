@@ -79,6 +79,27 @@ def test_strided_rows_zero_variance_and_errors():
     torch.ops.cdit.ln_modulate_quant(const.view(3, 1, 256), zero.repeat(2, 1), zero.repeat(2, 1))
 
 
+@pytest.mark.parametrize("K", [512, 3072, 8200])
+def test_rows_with_a_large_offset(K):
+  """Rows whose mean is far larger than their spread (mean^2 > 4 var): E[x^2] - mean^2 would
+  cancel, so the kernel recomputes the variance around the mean from its registers. Mixed
+  with ordinary rows in one launch so that both paths run inside the same workgroups."""
+  import cache_dit_amd.ops  # noqa: F401
+  g = torch.Generator().manual_seed(K)
+  x = torch.randn(96, K, generator=g)
+  x[0::3] = x[0::3] + 3.0
+  x[1::3] = x[1::3] * 3.0 - 11.0
+  x[4] = torch.where(torch.arange(K) % 2 == 0, 128.0, 129.0)  # two adjacent bf16 values
+  shift = (torch.randn(K, generator=g) * 0.5).to(torch.bfloat16)
+  scale = (torch.randn(K, generator=g) * 0.3).to(torch.bfloat16)
+  x = x.to(torch.bfloat16)
+  y, q, s = torch.ops.cdit.ln_modulate_quant(x.cuda(), shift.cuda(), scale.cuda())
+  torch.cuda.synchronize()
+  _check_y(y, to.ln_modulate(x, shift, scale, 1e-6), shift)
+  q_ref, s_ref = to.quantize_rowwise(y.cpu())
+  assert (bits_u8(q) == bits_u8(q_ref)).all() and (bits_u32(s) == bits_u32(s_ref)).all()
+
+
 def test_codes_are_handed_to_the_consuming_linears():
   """A FLUX-shaped model with the fused producer: the Linears fed by a modulated norm
   launch no quantizer of their own, the output stays within the cosine bar of the
