@@ -821,6 +821,12 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
     constexpr int OB = OUT == CDIT_DT_F32 ? 4 : 2;  // bytes per output element
     constexpr uint32_t kNoColumn = 0x80000000u;
     constexpr int kStoreOnce = 2;  // cache policy of the output stores: non-temporal (written once)
+    // Where a wave tile has whole-line pairs and a half-line pair (96 columns), the half lines
+    // are stored with the plain policy unless the epilogue is the long one (GELU): the other
+    // half of such a line comes from the other wave of the row, and a non-temporal half can
+    // leave the L2 before it arrives. Measured at 4608 x 3072 x 12288, alternating builds:
+    // 2 % faster than all stores non-temporal (which in turn beats all stores plain) without
+    // GELU, 2-3 % slower with it, where the two waves' stores lie further apart in time.
     uint16_t* cur_out = g.out;
     int64_t cur_ldo = g.ldo;
     int cur_epilogue = g.epilogue;
@@ -877,7 +883,8 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
     // row is being computed, so the latency of the permutation is not waited for; the
     // last row's after the two copies of the epilogue have joined
     uint32_t moved[NH > 0 ? NH : 1][4], moved_a[LP > 0 ? LP : 1][4], moved_b[LP > 0 ? LP : 1][4];
-    auto store_moved = [&](int i) {
+    auto store_moved = [&](int i, auto half_policy_tag) {
+      constexpr int kHalfPolicy = decltype(half_policy_tag)::value;
       const __amdgpu_buffer_rsrc_t row = out_row_of(i);
 #pragma unroll
       for (int v = 0; v < LP; ++v) {
@@ -891,10 +898,11 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
 #pragma unroll
       for (int h = 0; h < NH; ++h)
         __builtin_amdgcn_raw_buffer_store_b128(
-            v4u{moved[h][0], moved[h][1], moved[h][2], moved[h][3]}, row, (int)out_off[h], 0, kStoreOnce);
+            v4u{moved[h][0], moved[h][1], moved[h][2], moved[h][3]}, row, (int)out_off[h], 0, kHalfPolicy);
     };
     auto epilogue = [&](auto gelu_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
+      constexpr std::integral_constant<int, (LP > 0 && !GELU) ? 0 : kStoreOnce> half_policy{};
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
         const __amdgpu_buffer_rsrc_t out_row = out_row_of(i);
@@ -939,7 +947,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
         if constexpr (PERMUTE) {
           // the previous row's words have had this row's arithmetic to arrive
           __builtin_amdgcn_sched_barrier(0);
-          if (i > 0) store_moved(i - 1);
+          if (i > 0) store_moved(i - 1, half_policy);
 #pragma unroll
           for (int v = 0; v < LP; ++v)
 #pragma unroll
@@ -966,7 +974,8 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
     } else {
       epilogue(std::false_type{});
     }
-    if constexpr (PERMUTE) store_moved(TM - 1);
+    // (one copy of the last row's stores for both epilogues, all non-temporal)
+    if constexpr (PERMUTE) store_moved(TM - 1, std::integral_constant<int, kStoreOnce>{});
     if (next_tile >= ntiles) break;
     m0 = nm0;
     n0 = nn0;
