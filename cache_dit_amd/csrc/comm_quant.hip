@@ -69,6 +69,37 @@ __device__ __forceinline__ uint2 load8(const uint8_t* src, int align) {
   return uint2{(uint32_t)s[0] | ((uint32_t)s[1] << 16), (uint32_t)s[2] | ((uint32_t)s[3] << 16)};
 }
 
+// Division of a row index by a launch constant (N, B, S of the permuted layouts): the
+// compiler's 64-bit division costs more instructions than the row's arithmetic. For
+// n < 2^31 and 2^(s-1) < d <= 2^s: n / d = (n * mul) >> (31 + s) with mul = floor(2^(31+s) / d)
+// + 1 (mul * d exceeds 2^(31+s) by at most d, so the error term n * d / 2^(31+s) stays below
+// one), which is one v_mul_hi_u32 and a shift. d = 1 is passed as mul = 0.
+struct FastDiv {
+  uint32_t d, mul, shift;
+};
+FastDiv make_fastdiv(uint32_t d) {
+  if (d <= 1) return FastDiv{1u, 0u, 0u};
+  uint32_t s = 0;
+  while ((1ull << s) < d) ++s;
+  return FastDiv{d, (uint32_t)((1ull << (31 + s)) / d + 1ull), s - 1};
+}
+__device__ __forceinline__ uint32_t fd_div(uint32_t n, FastDiv f) {
+  return f.mul ? __umulhi(n, f.mul) >> f.shift : n;
+}
+
+// max over each group of G adjacent lanes (G = 8, 16, 32), the same in every lane of the
+// group: DPP inside rows of 16 lanes, one crossbar step for G = 32.
+template <int G>
+__device__ __forceinline__ uint32_t group_max_u32(uint32_t v) {
+  auto mx = [](uint32_t a, uint32_t b) { return a > b ? a : b; };
+  v = mx(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  v = mx(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  v = mx(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, false));  // row_half_mirror
+  if constexpr (G >= 16) v = mx(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xf, 0xf, false));  // row_mirror
+  if constexpr (G >= 32) v = mx(v, (uint32_t)__shfl_xor((int)v, 16, 64));
+  return v;
+}
+
 __device__ __forceinline__ int align_of(const void* p) {
   const uintptr_t a = reinterpret_cast<uintptr_t>(p);
   return (a & 7) == 0 ? 8 : (a & 3) == 0 ? 4 : (a & 1) == 0 ? 2 : 1;
@@ -105,15 +136,26 @@ __device__ __forceinline__ void quant_row(const uint16_t* __restrict__ xr, uint8
     for (int k = lane; k < H; k += 64) amax = fmaxf(amax, __uint_as_float((uint32_t)(xr[k] & 0x7fffu) << 16));
   }
   amax = wave_max_f32_nonneg(amax);
+  // (a NaN in the row has the largest bit pattern and arrives here as the amax)
+  const bool finite_row = (__float_as_uint(amax) & 0x7fffffffu) < 0x7f800000u;
   float scale, inv = 0.0f;
+  bool plain;  // wave-uniform: the clamp is a no-op and, for SCALE 1, the fast division is exact
   if constexpr (SCALE == 0) {
     amax = fmaxf(amax, 1e-4f);
     scale = amax / kFp8Max;
     inv = 1.0f / scale;
+    // |x| <= amax: |x * inv| <= 448 (1 + 2^-22) < 464, where the conversion still rounds to 448
+    plain = finite_row;
   } else {
-    scale = fmaxf(amax / kFp8Max, 1e-6f);
+    const float raw = amax / kFp8Max;
+    scale = fmaxf(raw, 1e-6f);
+    inv = 1.0f / scale;
+    // scale = fl(amax / 448) inside the window: the case the fast division is proven on
+    // (tests/native/divcheck.c, fp32 scales); a floored scale takes the compiler's division
+    plain = finite_row && scale == raw && scale_in_fast_window(scale);
   }
   auto q = [&](float x) {
+    if (plain) return SCALE == 0 ? x * inv : div_scale<true>(x, scale, inv);
     const float y = SCALE == 0 ? x * inv : x / scale;
     return y != y ? y : fminf(fmaxf(y, -kFp8Max), kFp8Max);
   };
@@ -263,32 +305,26 @@ __global__ __launch_bounds__(64) void comm_per_token_dequant(const uint8_t* __re
 // channels contiguous, as the reference kernel assumes).
 template <int CH>
 __global__ __launch_bounds__(64) void comm_qkv_permute_quant(
-    const uint16_t* __restrict__ x, uint8_t* __restrict__ y, int B, int S, int P, int N, int D,
-    int64_t sb, int64_t ss, int64_t sp, bool vec) {
+    const uint16_t* __restrict__ x, uint8_t* __restrict__ y, uint32_t rows, FastDiv dN, FastDiv dB,
+    FastDiv dS, int D, int64_t sb, int64_t ss, int64_t sp, bool vec) {
   const int lane = threadIdx.x;
-  const int64_t rows = (int64_t)P * S * B * N;
-  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
-    const int n = (int)(r % N);
-    const int64_t t = r / N;
-    const int b = (int)(t % B);
-    const int s = (int)((t / B) % S);
-    const int p = (int)(t / ((int64_t)B * S));
-    quant_row<1, CH>(x + b * sb + s * ss + p * sp + (int64_t)n * D, y + r * (D + 4), D, vec, lane);
+  for (uint32_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    const uint32_t t = fd_div(r, dN), n = r - t * dN.d;
+    const uint32_t u = fd_div(t, dB), b = t - u * dB.d;
+    const uint32_t p = fd_div(u, dS), s = u - p * dS.d;
+    quant_row<1, CH>(x + b * sb + s * ss + p * sp + (int64_t)n * D, y + (int64_t)r * (D + 4), D, vec, lane);
   }
 }
 
 // quant_x [S,B,N,D+4] (byte strides for s, b, n) -> x [B,S,N,D] contiguous bf16.
 __global__ __launch_bounds__(64) void comm_qkv_permute_dequant(
-    const uint8_t* __restrict__ qx, uint16_t* __restrict__ x, int S, int B, int N, int D, int64_t qs,
-    int64_t qb, int64_t qn, bool vec) {
+    const uint8_t* __restrict__ qx, uint16_t* __restrict__ x, uint32_t rows, FastDiv dN, FastDiv dS,
+    int D, int64_t qs, int64_t qb, int64_t qn, bool vec) {
   const int lane = threadIdx.x;
-  const int64_t rows = (int64_t)B * S * N;
-  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {  // r = (b * S + s) * N + n
-    const int n = (int)(r % N);
-    const int64_t t = r / N;
-    const int s = (int)(t % S);
-    const int b = (int)(t / S);
-    dequant_row<1>(qx + s * qs + b * qb + n * qn, x + r * D, D, vec, lane);
+  for (uint32_t r = blockIdx.x; r < rows; r += gridDim.x) {  // r = (b * S + s) * N + n
+    const uint32_t t = fd_div(r, dN), n = r - t * dN.d;
+    const uint32_t b = fd_div(t, dS), s = t - b * dS.d;
+    dequant_row<1>(qx + s * qs + b * qb + n * qn, x + (int64_t)r * D, D, vec, lane);
   }
 }
 
@@ -296,29 +332,19 @@ __global__ __launch_bounds__(64) void comm_qkv_permute_dequant(
 // G = D / 8 lanes (rounded up to a power of two), so a wavefront takes 64 / G rows at a
 // time and the amax is reduced inside each group of G lanes.
 template <int G>
-__device__ __forceinline__ float group_max_nonneg(float v) {
-#pragma unroll
-  for (int o = 1; o < G; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
-}
-
-template <int G>
 __global__ __launch_bounds__(64) void comm_qkv_permute_quant_grouped(
-    const uint16_t* __restrict__ x, uint8_t* __restrict__ y, int B, int S, int P, int N, int D,
-    int64_t sb, int64_t ss, int64_t sp) {
+    const uint16_t* __restrict__ x, uint8_t* __restrict__ y, uint32_t rows, FastDiv dN, FastDiv dB,
+    FastDiv dS, int D, int64_t sb, int64_t ss, int64_t sp) {
   constexpr int RPW = 64 / G;  // rows per wavefront
   const int lane = threadIdx.x, j = lane % G, sub = lane / G;
   const int nchunks = D >> 3;
-  const int64_t rows = (int64_t)P * S * B * N;
-  for (int64_t r0 = (int64_t)blockIdx.x * RPW; r0 < rows; r0 += (int64_t)gridDim.x * RPW) {
-    const int64_t r = r0 + sub;
+  for (uint32_t r0 = blockIdx.x * RPW; r0 < rows; r0 += gridDim.x * RPW) {
+    const uint32_t r = r0 + sub;
     const bool row_ok = r < rows, active = row_ok && j < nchunks;
-    const int64_t rc = row_ok ? r : rows - 1;
-    const int n = (int)(rc % N);
-    const int64_t t = rc / N;
-    const int b = (int)(t % B);
-    const int s = (int)((t / B) % S);
-    const int p = (int)(t / ((int64_t)B * S));
+    const uint32_t rc = row_ok ? r : rows - 1;
+    const uint32_t t = fd_div(rc, dN), n = rc - t * dN.d;
+    const uint32_t u = fd_div(t, dB), b = t - u * dB.d;
+    const uint32_t p = fd_div(u, dS), s = u - p * dS.d;
     const uint16_t* xr = x + b * sb + s * ss + p * sp + (int64_t)n * D;
     const uint4 v = active ? reinterpret_cast<const uint4*>(xr)[j] : make_uint4(0, 0, 0, 0);
     uint32_t m = 0;
@@ -326,16 +352,29 @@ __global__ __launch_bounds__(64) void comm_qkv_permute_quant_grouped(
     m = absmax2(m, v.y);
     m = absmax2(m, v.z);
     m = absmax2(m, v.w);
-    const float amax = group_max_nonneg<G>(__uint_as_float(fold2(m) << 16));
-    const float scale = fmaxf(amax / kFp8Max, 1e-6f);
-    auto q = [&](float f) {
-      const float yv = f / scale;
-      return yv != yv ? yv : fminf(fmaxf(yv, -kFp8Max), kFp8Max);
-    };
+    const uint32_t mbits = group_max_u32<G>(fold2(m));  // bf16 pattern of the row's max |x|
+    const float raw = __uint_as_float(mbits << 16) / kFp8Max;
+    const float scale = fmaxf(raw, 1e-6f);
+    const float inv = 1.0f / scale;
+    // The proven fast division where every row of the wavefront has a finite amax and an
+    // unfloored scale inside the window (scale = fl(amax / 448); tests/native/divcheck.c),
+    // the compiler's division and the clamp for the whole wavefront otherwise.
+    const bool plain = mbits < 0x7f80u && scale == raw && scale_in_fast_window(scale);
+    uint32_t lo, hi;
+    if (__builtin_amdgcn_ballot_w64(!plain) == 0) {
+      auto q = [&](float f) { return div_scale<true>(f, scale, inv); };
+      lo = cvt4_fp8(q(bf16_lo(v.x)), q(bf16_hi(v.x)), q(bf16_lo(v.y)), q(bf16_hi(v.y)));
+      hi = cvt4_fp8(q(bf16_lo(v.z)), q(bf16_hi(v.z)), q(bf16_lo(v.w)), q(bf16_hi(v.w)));
+    } else {
+      auto q = [&](float f) {
+        const float yv = f / scale;
+        return yv != yv ? yv : fminf(fmaxf(yv, -kFp8Max), kFp8Max);
+      };
+      lo = cvt4_fp8(q(bf16_lo(v.x)), q(bf16_hi(v.x)), q(bf16_lo(v.y)), q(bf16_hi(v.y)));
+      hi = cvt4_fp8(q(bf16_lo(v.z)), q(bf16_hi(v.z)), q(bf16_lo(v.w)), q(bf16_hi(v.w)));
+    }
     if (active) {
-      uint8_t* yr = y + rc * (D + 4);  // 4-byte aligned: D % 8 == 0 and y is
-      const uint32_t lo = cvt4_fp8(q(bf16_lo(v.x)), q(bf16_hi(v.x)), q(bf16_lo(v.y)), q(bf16_hi(v.y)));
-      const uint32_t hi = cvt4_fp8(q(bf16_lo(v.z)), q(bf16_hi(v.z)), q(bf16_lo(v.w)), q(bf16_hi(v.w)));
+      uint8_t* yr = y + (int64_t)rc * (D + 4);  // 4-byte aligned: D % 8 == 0 and y is
       reinterpret_cast<uint32_t*>(yr + 8 * j)[0] = lo;
       reinterpret_cast<uint32_t*>(yr + 8 * j)[1] = hi;
       if (j == 0) *reinterpret_cast<float*>(yr + D) = scale;
@@ -345,19 +384,16 @@ __global__ __launch_bounds__(64) void comm_qkv_permute_quant_grouped(
 
 template <int G>
 __global__ __launch_bounds__(64) void comm_qkv_permute_dequant_grouped(
-    const uint8_t* __restrict__ qx, uint16_t* __restrict__ x, int S, int B, int N, int D, int64_t qs,
-    int64_t qb, int64_t qn) {
+    const uint8_t* __restrict__ qx, uint16_t* __restrict__ x, uint32_t rows, FastDiv dN, FastDiv dS,
+    int D, int64_t qs, int64_t qb, int64_t qn) {
   constexpr int RPW = 64 / G;
   const int lane = threadIdx.x, j = lane % G, sub = lane / G;
   const int nchunks = D >> 3;
-  const int64_t rows = (int64_t)B * S * N;
-  for (int64_t r0 = (int64_t)blockIdx.x * RPW; r0 < rows; r0 += (int64_t)gridDim.x * RPW) {
-    const int64_t r = r0 + sub;  // (b * S + s) * N + n
+  for (uint32_t r0 = blockIdx.x * RPW; r0 < rows; r0 += gridDim.x * RPW) {
+    const uint32_t r = r0 + sub;  // (b * S + s) * N + n
     if (r >= rows || j >= nchunks) continue;
-    const int n = (int)(r % N);
-    const int64_t t = r / N;
-    const int s = (int)(t % S);
-    const int b = (int)(t / S);
+    const uint32_t t = fd_div(r, dN), n = r - t * dN.d;
+    const uint32_t b = fd_div(t, dS), s = t - b * dS.d;
     const uint8_t* xr = qx + s * qs + b * qb + n * qn;
     const float scale = *reinterpret_cast<const float*>(xr + D);
     const uint32_t w0 = reinterpret_cast<const uint32_t*>(xr + 8 * j)[0];
@@ -370,7 +406,7 @@ __global__ __launch_bounds__(64) void comm_qkv_permute_dequant_grouped(
     o.y = pair(__builtin_amdgcn_cvt_f32_fp8((int)w0, 2), __builtin_amdgcn_cvt_f32_fp8((int)w0, 3));
     o.z = pair(__builtin_amdgcn_cvt_f32_fp8((int)w1, 0), __builtin_amdgcn_cvt_f32_fp8((int)w1, 1));
     o.w = pair(__builtin_amdgcn_cvt_f32_fp8((int)w1, 2), __builtin_amdgcn_cvt_f32_fp8((int)w1, 3));
-    reinterpret_cast<uint4*>(x + r * D)[j] = o;
+    reinterpret_cast<uint4*>(x + (int64_t)r * D)[j] = o;
   }
 }
 
@@ -410,12 +446,17 @@ int launch_comm_qkv_permute_quant(const void* x, int B, int S, int P, int N, int
   const bool vec = D % 8 == 0 && D <= kMaxChunks * 512 && sb % 8 == 0 && ss % 8 == 0 && sp % 8 == 0 &&
                    reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 4 == 0;
   const int64_t rows = (int64_t)P * S * B * N;
+  if (rows >= (int64_t)1 << 31) {
+    set_error("cdit_fp8_comm_qkv_permute_quant: %lld head rows, at most 2^31 - 1", (long long)rows);
+    return CDIT_EINVAL;
+  }
+  const FastDiv dN = make_fastdiv((uint32_t)N), dB = make_fastdiv((uint32_t)B), dS = make_fastdiv((uint32_t)S);
   if (vec && D <= 256) {
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     uint8_t* yp = static_cast<uint8_t*>(y);
 #define CDIT_QKV_Q(G)                                                                            \
   hipLaunchKernelGGL(comm_qkv_permute_quant_grouped<G>, dim3(grid_for((rows + 64 / G - 1) / (64 / G))), \
-                     dim3(64), 0, stream, xp, yp, B, S, P, N, D, sb, ss, sp)
+                     dim3(64), 0, stream, xp, yp, (uint32_t)rows, dN, dB, dS, D, sb, ss, sp)
     if (D <= 64) CDIT_QKV_Q(8);
     else if (D <= 128) CDIT_QKV_Q(16);
     else CDIT_QKV_Q(32);
@@ -426,8 +467,8 @@ int launch_comm_qkv_permute_quant(const void* x, int B, int S, int P, int N, int
 #define CDIT_QKV_ROW(CH)                                                                          \
   if (need <= CH) {                                                                               \
     hipLaunchKernelGGL(comm_qkv_permute_quant<CH>, dim3(grid_for(rows)), dim3(64), 0, stream,      \
-                       static_cast<const uint16_t*>(x), static_cast<uint8_t*>(y), B, S, P, N, D, sb, \
-                       ss, sp, vec);                                                              \
+                       static_cast<const uint16_t*>(x), static_cast<uint8_t*>(y), (uint32_t)rows,  \
+                       dN, dB, dS, D, sb, ss, sp, vec);                                           \
     return 0;                                                                                     \
   }
   CDIT_QKV_ROW(1) CDIT_QKV_ROW(4) CDIT_QKV_ROW(32)
@@ -440,12 +481,17 @@ int launch_comm_qkv_permute_dequant(const void* qx, int S, int B, int N, int D, 
   const bool vec = D % 8 == 0 && qs % 4 == 0 && qb % 4 == 0 && qn % 4 == 0 &&
                    reinterpret_cast<uintptr_t>(qx) % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
   const int64_t rows = (int64_t)B * S * N;
+  if (rows >= (int64_t)1 << 31) {
+    set_error("cdit_fp8_comm_qkv_permute_dequant: %lld head rows, at most 2^31 - 1", (long long)rows);
+    return CDIT_EINVAL;
+  }
+  const FastDiv dN = make_fastdiv((uint32_t)N), dS = make_fastdiv((uint32_t)S);
   if (vec && D <= 256) {
     const uint8_t* qp = static_cast<const uint8_t*>(qx);
     uint16_t* xp = static_cast<uint16_t*>(x);
 #define CDIT_QKV_D(G)                                                                              \
   hipLaunchKernelGGL(comm_qkv_permute_dequant_grouped<G>, dim3(grid_for((rows + 64 / G - 1) / (64 / G))), \
-                     dim3(64), 0, stream, qp, xp, S, B, N, D, qs, qb, qn)
+                     dim3(64), 0, stream, qp, xp, (uint32_t)rows, dN, dS, D, qs, qb, qn)
     if (D <= 64) CDIT_QKV_D(8);
     else if (D <= 128) CDIT_QKV_D(16);
     else CDIT_QKV_D(32);
@@ -453,8 +499,8 @@ int launch_comm_qkv_permute_dequant(const void* qx, int S, int B, int N, int D, 
     return 0;
   }
   hipLaunchKernelGGL(comm_qkv_permute_dequant, dim3(grid_for(rows)), dim3(64), 0, stream,
-                     static_cast<const uint8_t*>(qx), static_cast<uint16_t*>(x), S, B, N, D, qs, qb, qn,
-                     vec);
+                     static_cast<const uint8_t*>(qx), static_cast<uint16_t*>(x), (uint32_t)rows, dN, dS, D,
+                     qs, qb, qn, vec);
   return 0;
 }
 

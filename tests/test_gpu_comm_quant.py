@@ -69,6 +69,37 @@ def test_qkv_permute_quant_and_dequant_bit_exact(shape):
     assert torch.equal(d.cpu().view(torch.int16), d_ref.view(torch.int16))
 
 
+@pytest.mark.parametrize("D", [64, 128, 256, 512])
+def test_qkv_permute_quant_over_the_range_of_row_magnitudes(D):
+  """Head rows from far below the 1e-6 floor of the scale to the top of the bf16 range,
+  neighbours in one wavefront: the kernel's exact fast division (rows whose scale is
+  amax / 448 inside its proven window) and its fallback (floored or very large scales)
+  must both give the oracle's codes, whichever the other rows of the wavefront take."""
+  from cache_dit_amd import comm_quant as cq
+  B, S, P, N = 1, 23, 3, 6
+  g = torch.Generator().manual_seed(D)
+  x = torch.randn(B, S, P, N, D, generator=g)
+  mags = torch.tensor([1e-30, 1e-9, 3e-7, 4.4e-4, 4.6e-4, 1e-3, 1.0, 77.0, 1e9, 1e30, 3e38])
+  pick = torch.randint(0, len(mags), (B, S, P, N, 1), generator=g)
+  x = (x * mags[pick]).clamp(-3e38, 3e38).to(torch.bfloat16)
+  q = cq.fp8_comm_qkv_permute_quant(x.cuda())
+  q_ref = co.qkv_permute_quant(x)
+  assert (bits_u8(q) == bits_u8(q_ref)).all()
+  for p in range(P):
+    d = cq.fp8_comm_qkv_permute_dequant(q[p])
+    assert torch.equal(d.cpu().view(torch.int16), co.qkv_permute_dequant(q_ref[p]).view(torch.int16))
+
+
+def test_per_token_quant_over_the_range_of_row_magnitudes():
+  from cache_dit_amd import comm_quant as cq
+  g = torch.Generator().manual_seed(5)
+  x = torch.randn(64, 1536, generator=g)
+  mags = torch.tensor([1e-30, 1e-9, 1e-5, 9e-5, 1.1e-4, 1.0, 1e9, 1e30, 3e38])
+  x = (x * mags[torch.randint(0, len(mags), (64, 1), generator=g)]).clamp(-3e38, 3e38).to(torch.bfloat16)
+  q = cq.fp8_comm_per_token_quant(x.cuda())
+  assert (bits_u8(q) == bits_u8(co.per_token_quant(x))).all()
+
+
 def test_qkv_permute_quant_takes_a_strided_input():
   """x as a view of a packed [B, S, 3 * N * D] qkv projection output with padding."""
   from cache_dit_amd import comm_quant as cq
