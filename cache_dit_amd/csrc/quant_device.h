@@ -96,10 +96,13 @@ __device__ __forceinline__ float clamp448(float y) {
 template <bool FAST>
 __device__ __forceinline__ float div_scale(float x, float s, float r) {
   if constexpr (FAST) {
+    // Markstein's correction of q0 = x r, written with the residual negated: d = q0 s - x is
+    // the exact negative of the usual x - q0 s, so q = q0 - d r is the same correctly rounded
+    // quotient for every non-zero x, and for x = -0 (q0 = -0, d = +0) it is (-0) + (-0) = -0
+    // where the usual form gives +0: the sign of a zero survives without a copysign.
     const float q0 = x * r;
-    const float e = __fmaf_rn(-q0, s, x);
-    const float q = __fmaf_rn(e, r, q0);
-    return __uint_as_float((__float_as_uint(q) & 0x7fffffffu) | (__float_as_uint(x) & 0x80000000u));
+    const float d = __fmaf_rn(q0, s, -x);
+    return __fmaf_rn(-d, r, q0);
   } else {
     return x / s;
   }

@@ -14,8 +14,8 @@
 // correctly rounded one: a bare reciprocal multiply flips about 1e-4 of the
 // codes. Per element the kernel therefore refines q0 = x*r (r = 1/scale,
 // correctly rounded, computed once per row) with the exact residual:
-//   e = fma(-q0, scale, x);  q = fma(e, r, q0);  q = copysign(q, x)
-// (Markstein's correction; the copysign restores -0 for x = -0). That this
+//   d = fma(q0, scale, -x);  q = fma(-d, r, q0)
+// (Markstein's correction with the residual negated, which keeps the sign of x = -0). That this
 // reproduces x/scale down to the e4m3 code has been verified exhaustively on
 // the CPU for every (x, amax) pair of bf16 values with |x| <= amax, in both
 // scale modes, whenever 2^-100 <= scale < 2^101 (tests/native/divcheck.c);

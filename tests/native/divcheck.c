@@ -43,8 +43,13 @@ int main(int argc, char** argv) {
           const float x = oracle_bf16_to_f32((uint16_t)(xb | (sg << 15)));
           const float ref = x / s;
           const float q0 = x * r;
-          const float e = fmaf(-q0, s, x);
-          const float q1 = copysignf(fmaf(e, r, q0), x);
+          /* the kernel's form: the residual negated, no copysign (keeps the sign of -0).
+           * The empty asm hides where d comes from: gcc -O1 and above otherwise rewrites
+           * -fma(a, b, c) as fma(-a, b, -c), which is not the same operation for a zero
+           * result (it turns this form back into the usual one and -0 into +0). */
+          float d = fmaf(q0, s, -x);
+          __asm__ volatile("" : "+x"(d));
+          const float q1 = fmaf(-d, r, q0);
           ++checked;
           /* the kernel's fast path does not clamp: the raw quotient must encode like
            * the oracle's clamped one (it stays below the tie at 464) */
