@@ -24,6 +24,16 @@ __device__ __forceinline__ float round_to_bf16(float f) {
   return __uint_as_float(u & 0xffff0000u);
 }
 
+// two fp32 -> packed bf16 pair, round to nearest even (v_cvt_pk_bf16_f32: one
+// instruction for what round_to_bf16 spells out in five integer operations per value;
+// a NaN keeps its sign and payload bits here, round_to_bf16 returns the canonical one)
+__device__ __forceinline__ uint32_t pk_bf16(float lo, float hi) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+  const v2f v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf));
+}
+
 // max over the wavefront of an unsigned value (order independent, exact). Four
 // DPP steps reduce each row of 16 lanes (xor 1, xor 2, half mirror, mirror), then
 // the four row results are read into scalars.

@@ -401,15 +401,6 @@ __device__ __forceinline__ uint32_t bf16_bits(float f) {
   return __float_as_uint(round_to_bf16(f)) >> 16;
 }
 
-// two fp32 -> packed bf16 pair, round to nearest even (v_cvt_pk_bf16_f32: one
-// instruction for what round_to_bf16 spells out in five integer operations per value)
-__device__ __forceinline__ uint32_t pk_bf16(float lo, float hi) {
-  typedef float v2f __attribute__((ext_vector_type(2)));
-  typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
-  const v2f v = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf));
-}
-
 // y bits of one element: x, scale, shift as fp32 (exact widenings of bf16 values)
 __device__ __forceinline__ uint32_t modulate1(float x, float mean, float rstd, float sc, float sh) {
   const float n = round_to_bf16((x - mean) * rstd);

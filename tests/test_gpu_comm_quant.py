@@ -100,6 +100,33 @@ def test_per_token_quant_over_the_range_of_row_magnitudes():
   assert (bits_u8(q) == bits_u8(co.per_token_quant(x))).all()
 
 
+def _same_bf16_up_to_nan(got, want):
+  """Bit for bit, except that a NaN only has to be a NaN (its sign and payload are whatever
+  the converting hardware or library leaves)."""
+  nan = torch.isnan(want)
+  assert torch.equal(torch.isnan(got), nan)
+  assert torch.equal(got.view(torch.int16)[~nan], want.view(torch.int16)[~nan])
+
+
+def test_dequant_of_arbitrary_code_bytes_including_nan_codes():
+  """The dequantizers take whatever bytes arrive: every code value, the two NaN codes among
+  them, next to rows without any in the same wavefront."""
+  from cache_dit_amd import comm_quant as cq
+  g = torch.Generator().manual_seed(11)
+  for H in (64, 1536, 3072):
+    raw = torch.randint(0, 256, (37, H + 2), dtype=torch.uint8, generator=g)
+    raw[::3] &= 0x77  # rows without a NaN code (the low seven bits never all ones)
+    raw[:, H:] = torch.tensor([0x80, 0x3c], dtype=torch.uint8)  # scale 2^-6 (bf16 0x3c80), low byte first
+    q = raw.view(FP8)
+    _same_bf16_up_to_nan(cq.fp8_comm_per_token_dequant(q.cuda()).cpu(), co.per_token_dequant(q))
+  for D in (64, 128, 512):
+    raw = torch.randint(0, 256, (5, 2, 3, D + 4), dtype=torch.uint8, generator=g)
+    raw[::2] &= 0x77
+    raw[..., D:] = torch.tensor([0, 0, 0x80, 0x3c], dtype=torch.uint8)  # fp32 scale 2^-6
+    q = raw.view(FP8)
+    _same_bf16_up_to_nan(cq.fp8_comm_qkv_permute_dequant(q.cuda()).cpu(), co.qkv_permute_dequant(q))
+
+
 def test_qkv_permute_quant_takes_a_strided_input():
   """x as a view of a packed [B, S, 3 * N * D] qkv projection output with padding."""
   from cache_dit_amd import comm_quant as cq
