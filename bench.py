@@ -504,7 +504,16 @@ def headline_kernels(device):
       i = it["i"] = (it["i"] + 1) % nbuf
       ops.w8a16_into(xs[i], ws[i], wsc, b, outs[i & 1], 0)
 
-    w_ms = _time_events(w8a16, 30, 5)
+    # (settled clocks as for the FP8 GEMM: blocks of 50 launches until two in a row agree to
+    # 0.5 %, at most 2 s, then the median of three blocks)
+    t_start, prev = time.perf_counter(), _time_events(w8a16, 50, 20)
+    while time.perf_counter() - t_start < 2.0:
+      cur = _time_events(w8a16, 50, 0)
+      settled = abs(cur - prev) <= 0.005 * prev
+      prev = cur
+      if settled and time.perf_counter() - t_start > 0.5:
+        break
+    w_ms = sorted(_time_events(w8a16, 50, 0) for _ in range(3))[1]
     res["w8a16_ms"] = w_ms
     res["w8a16_tflops"] = 2.0 * M * K * N / w_ms / 1e9
     res["w8a16_frac_bf16_peak"] = res["w8a16_tflops"] / BF16_PEAK_TFLOPS

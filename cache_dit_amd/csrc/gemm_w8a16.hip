@@ -1140,7 +1140,9 @@ TileChoice choose_variant(Tiles tiles, WideOk wide_ok) {
       const int64_t t = tiles(bm, bn), full = t / cus, rem = t % cus;
       return (full * 10 * cus + (rem ? 4 * cus + 6 * rem : 0)) * bm * bn * pen;
     };
-    const int64_t c8 = cost(256, 192, 103), c7 = cost(256, 256, 100);
+    // (256 x 192 against 256 x 256, measured: 0.98 at 4608 x 3072 x 12288, 0.955 at N = 15360,
+    // 1.03 at 4096 x 3072 x 12288, 1.05 at N = 9216; a penalty of 2 % puts all four on the right side)
+    const int64_t c8 = cost(256, 192, 102), c7 = cost(256, 256, 100);
     return c8 < c7 ? TileChoice{8, c8} : TileChoice{7, c7};
   }
   // Smaller problems: whole rounds over the CUs times tile area, the small tiles
