@@ -274,6 +274,20 @@ def test_full_flux_shaped_step_cosine():
   assert torch.isfinite(y.float()).all()
   assert c_ref >= 0.999, c_ref
   assert c_bf16 >= 0.99, c_bf16
+  # The stage patch on this unmodified model at full size: the launches of a forward are
+  # those of the step the benchmark times as its headline (per step 152 quantizer launches,
+  # 114 batched GEMM calls -- 171 launches where the tile cost model splits a stage --, 38
+  # proj_out and 76 M = 1 Linears), and the output keeps its bits.
+  from test_gpu_patch_functors import _Launches
+  with torch.no_grad():
+    y_plain = model(**inputs)
+    cache_dit.apply_stage_patch(model)
+    with _Launches() as staged:
+      y_staged = model(**inputs)
+    cache_dit.remove_stage_patch(model)
+  assert torch.equal(y_staged, y_plain)
+  assert staged.n["batched"] == 19 * 4 + 38 and staged.n["single"] == 19 * 2 + 38 * 2
+  assert staged.n["shared_quant"] + staged.n["cat2"] == 152 and staged.n["cat2"] == 38
 
 
 def _full_size_step(model_cls, inputs_fn, n_quantized, n_skipped):
