@@ -702,8 +702,8 @@ def dit_forward_ms(device, iters=5):
   cache_dit_amd.quantize(model, cache_dit_amd.QuantizeConfig(quant_type="float8_per_row"))
   dit_shapes.fuse_gelu_epilogues(model)
   inputs = flux_like_inputs(device)
-  # the model's block and attention code stays as it is: the stage patch functor hooks the
-  # attention modules and rebinds the block forwards (cache_dit_amd.patch_functors)
+  # the model's block and attention code stays as it is: the stage patch functor rebinds the
+  # forwards of the blocks and of their attention modules (cache_dit_amd.patch_functors)
   cache_dit_amd.apply_stage_patch(model, batch_stages=True, single_blocks=True, fuse_cat=True,
                                   fuse_norm_quant=True, materialize=False)
   graph_ms = None
@@ -737,10 +737,10 @@ def dit_forward_ms(device, iters=5):
 
 
 def dit_forward_compiled_ms(device, iters=5):
-  """The same transformer with its blocks compiled by torch.compile (regional compilation,
-  fullgraph): every converted Linear is one registered op, so Inductor fuses the
-  element-wise glue around them. Returns (ms, seconds spent compiling, cosine against the
-  eager forward) or (None, None, note)."""
+  """The same transformer, stage-patched, with its blocks compiled by torch.compile (regional
+  compilation, fullgraph): every stage is one registered batch op, every other converted
+  Linear one op, so Inductor fuses the element-wise glue around them. Returns (ms, seconds
+  spent compiling, cosine against the eager forward) or (None, None, note)."""
   try:
     import torch
     import cache_dit_amd
@@ -750,11 +750,12 @@ def dit_forward_compiled_ms(device, iters=5):
       model = dit_shapes.FluxLikeTransformer().to(torch.bfloat16)
     cache_dit_amd.quantize(model, cache_dit_amd.QuantizeConfig(quant_type="float8_per_row"))
     dit_shapes.fuse_gelu_epilogues(model)
-    # (no stage patch here: a traced graph takes none of its stateful shortcuts, and its
-    # per-module hooks would make every block a compilation of its own)
     inputs = dit_shapes.flux_like_inputs(device)
     with torch.no_grad():
       want = model(**inputs)
+      # (inside the traced graph the rebound forwards emit one batch op per stage; the fused
+      # norms stay tensor ops there, which Inductor fuses itself)
+      cache_dit_amd.apply_stage_patch(model)
       t0 = time.perf_counter()
       for blk in list(model.transformer_blocks) + list(model.single_transformer_blocks):
         blk.compile(fullgraph=True)

@@ -229,7 +229,12 @@ class Fp8DynamicLinear(_Fp8LinearBase):
     # memory its graphs are captured into), and so do inference-mode tensors, which carry
     # no version counter to tell a modified buffer by
     stateless = torch.compiler.is_compiling()
-    if not stateless:
+    if stateless:
+      if self._precomputed is not None:
+        out = _take_precomputed_traced(self, x)
+        if out is not None:
+          return out
+    else:
       if x.is_inference():
         if self.sibling_group is not None or self.share_input_quant:
           _note_inference_bypass(type(self).__name__)
@@ -269,7 +274,12 @@ class Fp8WeightOnlyLinear(_Fp8LinearBase):
 
   def forward(self, x: torch.Tensor) -> torch.Tensor:
     self._check_input(x)
-    if not torch.compiler.is_compiling():  # as in Fp8DynamicLinear
+    if torch.compiler.is_compiling():  # as in Fp8DynamicLinear
+      if self._precomputed is not None:
+        out = _take_precomputed_traced(self, x)
+        if out is not None:
+          return out
+    else:
       if x.is_inference():
         if self.sibling_group is not None:
           _note_inference_bypass(type(self).__name__)
@@ -480,6 +490,28 @@ def _take_precomputed(lin: "_Fp8LinearBase", x: torch.Tensor):
   return None
 
 
+def _take_precomputed_traced(lin: "_Fp8LinearBase", x: torch.Tensor):
+  """Inside a traced graph a stash is (activation, output) and is taken when `x` is that very
+  tensor object (the tracer follows objects, not storage); emptied either way."""
+  stash = lin._precomputed
+  lin._precomputed = None
+  if len(stash) == 2 and stash[0] is x:
+    return stash[1]
+  return None
+
+
+def _stage_batchable(pairs, flat, first, traced: bool) -> bool:
+  if (type(first) not in (Fp8DynamicLinear, Fp8WeightOnlyLinear) or len(flat) > _native.MAX_GROUP
+      or len(pairs) > _native.MAX_ACTS
+      or any(flat[i] is flat[j] for i in range(len(flat)) for j in range(i))
+      or any(type(lin) is not type(first) or lin.in_features != first.in_features
+             or lin._scale_mode_id != first._scale_mode_id or lin.sibling_group is not None
+             for lin in flat)):
+    return False
+  return not any(not x.is_cuda or x.dtype != torch.bfloat16 or x.shape[-1] != first.in_features
+                 or (not traced and x.is_inference()) for x, _ in pairs)
+
+
 def precompute_stage(pairs) -> bool:
   """Runs `linear_batch(pairs)` now and leaves every output on its Linear, to be returned
   when that Linear is next called with the very same activation. For code that knows which
@@ -489,25 +521,27 @@ def precompute_stage(pairs) -> bool:
   stage then costs one quantizer launch and one GEMM launch, and the module's code stays as
   it is. A Linear that is called with anything else computes as usual, so a wrong guess
   costs time, not correctness. Outputs nobody collects are dropped when the next stage is
-  precomputed. Returns False (nothing done) where linear_batch would not batch: a compiled
-  graph, inference-mode tensors, Linears of other types or of mixed types. Not thread-safe,
-  like the sibling groups."""
-  if torch.compiler.is_compiling():
-    return False
-  for lin in _precomputed_holders:
-    lin._precomputed = None
-  _precomputed_holders.clear()
+  precomputed. Returns False (nothing done) where linear_batch would not batch:
+  inference-mode tensors, Linears of other types or of mixed types. Inside a traced graph
+  (torch.compile) the stage becomes the one traceable batch op and an output goes to the
+  Linear call that receives the same tensor object; whoever stashes there also clears what
+  is left (`release_precomputed`). Not thread-safe, like the sibling groups."""
   flat = [lin for _, lins in pairs for lin in lins]
   if not flat:
     return False
   first = flat[0]
-  if (type(first) not in (Fp8DynamicLinear, Fp8WeightOnlyLinear) or len(flat) > _native.MAX_GROUP
-      or len(pairs) > _native.MAX_ACTS or len({id(lin) for lin in flat}) != len(flat)
-      or any(type(lin) is not type(first) or lin.in_features != first.in_features
-             or lin._scale_mode_id != first._scale_mode_id or lin.sibling_group is not None
-             for lin in flat)
-      or any(not x.is_cuda or x.dtype != torch.bfloat16 or x.is_inference()
-             or x.shape[-1] != first.in_features for x, _ in pairs)):
+  if torch.compiler.is_compiling():
+    if not _stage_batchable(pairs, flat, first, True):
+      return False
+    outs = linear_batch(pairs)
+    for (x, lins), ys in zip(pairs, outs):
+      for lin, y in zip(lins, ys):
+        lin._precomputed = (x, y)
+    return True
+  for lin in _precomputed_holders:
+    lin._precomputed = None
+  _precomputed_holders.clear()
+  if not _stage_batchable(pairs, flat, first, False):
     return False
   outs = linear_batch(pairs)
   for (x, lins), ys in zip(pairs, outs):
@@ -518,6 +552,13 @@ def precompute_stage(pairs) -> bool:
       lin._precomputed = (key, y.view(-1, lin.out_features), stream, capture_id)
       _precomputed_holders.append(lin)
   return True
+
+
+def release_precomputed(linears) -> None:
+  """Drops what precompute_stage left on `linears` and nobody collected."""
+  for lin in linears:
+    if lin is not None and lin._precomputed is not None:
+      lin._precomputed = None
 
 
 def linear_on_cat(linear: nn.Module, xs) -> torch.Tensor:

@@ -10,16 +10,19 @@ diffusers' attribute names (`norm1`, `attn.to_q`, `attn.add_q_proj`, `attn.to_ou
 `attn.to_add_out`, `ff.net[0].proj`, `ff.net[2]`, `proj_mlp`, `proj_out`, `img_mod`, `attn1` ...)
 and block forward signatures. Three mechanisms, from least to most intrusive:
 
-  * forward pre-hooks on the attention modules. The hook sees `hidden_states` and
-    `encoder_hidden_states` before the module's own code (diffusers: its attention
-    processor) calls to_q / to_k / to_v and add_q_proj / add_k_proj / add_v_proj one after
-    the other, computes all of them with `nn.precompute_stage` and leaves each output on its
-    Linear, which returns it when called with that very activation. The attention code itself
-    (norms, RoPE, SDPA, whatever processor is installed) is not touched. A second hook on
-    `to_out[0]` does the same for the output projections of a joint attention, whose two
-    inputs are the two parts of one split tensor.
-  * rebound block forwards, adapted from the diffusers block forwards, for what hooks cannot
-    do: the two FeedForwards of a double-stream block run at different points of the original
+  * a wrapper bound as `forward` of the attention modules (an instance attribute; the class
+    and its processor stay as they are). It sees `hidden_states` and `encoder_hidden_states`
+    before the module's own code (diffusers: its attention processor) calls to_q / to_k /
+    to_v and add_q_proj / add_k_proj / add_v_proj one after the other, computes all of them
+    with `nn.precompute_stage` and leaves each output on its Linear, which returns it when
+    called with that very activation. The attention code itself (norms, RoPE, SDPA, whatever
+    processor is installed) is not touched. A second wrapper on `to_out[0]` does the same for
+    the output projections of a joint attention, whose two inputs are the two parts of one
+    split tensor. (Wrappers rather than forward hooks: a hook handle carries a process-wide
+    serial number, which a graph tracer guards on, so that every block would be compiled
+    separately.)
+  * rebound block forwards, adapted from the diffusers block forwards, for what these
+    wrappers cannot do: the two FeedForwards of a double-stream block run at different points of the original
     forward (the text stream's input does not exist yet when the image stream's runs), so
     the forward is reordered to put both modulated inputs side by side; a FLUX single block
     precomputes proj_mlp next to q/k/v and lets proj_out's quantizer read
@@ -30,8 +33,10 @@ and block forward signatures. Three mechanisms, from least to most intrusive:
 
 Outputs are bit-identical to the unpatched model in the first two cases (the kernels give the
 same bits batched or not; the reordering moves whole tensor ops, not arithmetic inside them).
-Everything falls back to the plain behaviour where nothing can be batched: a compiled graph,
-inference-mode tensors, Linears that were not converted.
+Everything falls back to the plain behaviour where nothing can be batched: inference-mode
+tensors, Linears that were not converted. Inside a traced graph (torch.compile of the patched
+blocks) a stage is the one traceable batch op; the fused norms and the joint output
+projections keep their plain form there.
 """
 from __future__ import annotations
 
@@ -59,57 +64,58 @@ def _quantized(*mods) -> bool:
   return all(isinstance(m, _QUANT) for m in mods)
 
 
-# ------------------------------------------------------------------ attention: hooks
+# ------------------------------------------------------------------ attention modules
 
 
-def _attention_stage_hook(attn: nn.Module, args, kwargs):
-  """Forward pre-hook of an attention module (diffusers' Attention / FluxAttention /
+_STAGE_LINEARS = ("to_q", "to_k", "to_v", "add_q_proj", "add_k_proj", "add_v_proj")
+
+
+def _attention_forward(self, *args, **kwargs):
+  """Bound as `forward` of an attention module (diffusers' Attention / FluxAttention /
   WanAttention interface: `hidden_states`, `encoder_hidden_states` first, by position or
-  keyword). Computes the projections of the stage ahead and stashes them."""
-  if torch.compiler.is_compiling() or not getattr(attn, "_cdit_stage_batch", False):
-    return None
+  keyword). Computes the projections of the stage ahead, leaves each output on its Linear
+  and runs the module's own forward, whose code (processor, norms, RoPE, SDPA) then calls
+  the Linears one by one and finds the outputs."""
+  if not getattr(self, "_cdit_stage_batch", False):
+    return self._cdit_orig_forward(*args, **kwargs)
   hidden = kwargs.get("hidden_states", args[0] if args else None)
   encoder = kwargs.get("encoder_hidden_states", args[1] if len(args) > 1 else None)
-  if not isinstance(hidden, torch.Tensor):
-    return None
-  q, k, v = attn.to_q, attn.to_k, attn.to_v
-  if q._precomputed is not None:
-    return None  # the block's forward already put this stage together (proj_mlp + q/k/v)
-  add_q = getattr(attn, "add_q_proj", None)
-  if add_q is not None and isinstance(encoder, torch.Tensor):
-    attn._cdit_n_txt = encoder.shape[1]
-    cnn.precompute_stage([(hidden, [q, k, v]), (encoder, [add_q, attn.add_k_proj, attn.add_v_proj])])
+  q, k, v = self.to_q, self.to_k, self.to_v
+  add_q = getattr(self, "add_q_proj", None)
+  if not isinstance(hidden, torch.Tensor) or q._precomputed is not None:
+    pass  # (the block's forward already put this stage together: proj_mlp + q/k/v)
+  elif add_q is not None and isinstance(encoder, torch.Tensor):
+    self._cdit_n_txt = encoder.shape[1]
+    cnn.precompute_stage([(hidden, [q, k, v]), (encoder, [add_q, self.add_k_proj, self.add_v_proj])])
   elif isinstance(encoder, torch.Tensor):  # cross-attention: the query on one activation, k / v on the other
     cnn.precompute_stage([(hidden, [q]), (encoder, [k, v])])
   else:
     cnn.precompute_stage([(hidden, [q, k, v])])
-  return None
+  out = self._cdit_orig_forward(*args, **kwargs)
+  # what the module's code did not collect (it was called with other tensors) is dropped here
+  cnn.release_precomputed([q, k, v, add_q, getattr(self, "add_k_proj", None), getattr(self, "add_v_proj", None)])
+  return out
 
 
-def _joint_out_hook(attn: nn.Module):
-  """Forward pre-hook for `attn.to_out[0]` of a joint attention: its input is the image part
-  of the attention output, split off one tensor whose first `n_txt` tokens go to
+def _joint_out_forward(self, x):
+  """Bound as `forward` of `attn.to_out[0]` of a joint attention: its input is the image
+  part of the attention output, split off one tensor whose first `n_txt` tokens go to
   `attn.to_add_out` next. Both projections are computed here; the text part is addressed as
   the rows in front of the image part in the same storage. Whatever to_add_out is then called
-  with, it only takes the stashed output if that is exactly this memory, unmodified."""
-
-  def hook(to_out0: nn.Module, args):
-    if torch.compiler.is_compiling() or not getattr(attn, "_cdit_stage_batch", False):
-      return None
-    x = args[0] if args else None
+  with, it only takes the stashed output if that is exactly this memory, unmodified. (Eager
+  code only: a traced graph has no storage to address, the two Linears stay two ops there.)"""
+  attn = self._cdit_joint_attn[0]
+  if not torch.compiler.is_compiling() and getattr(attn, "_cdit_stage_batch", False):
     n_txt = getattr(attn, "_cdit_n_txt", 0)
     # (one batch element: with more, the rows of a part are not contiguous and every Linear
     # call works on a copy of its own, which no stash can be keyed on)
-    if (not isinstance(x, torch.Tensor) or x.dim() != 3 or n_txt <= 0 or x._base is None
-        or x.shape[0] != 1 or x.stride(2) != 1 or x.stride(1) != x.shape[2]
-        or x.storage_offset() < n_txt * x.stride(1)):
-      return None
-    front = x.as_strided((x.shape[0], n_txt, x.shape[2]), x.stride(),
-                         x.storage_offset() - n_txt * x.stride(1))
-    cnn.precompute_stage([(x, [to_out0]), (front, [attn.to_add_out])])
-    return None
-
-  return hook
+    if (isinstance(x, torch.Tensor) and x.dim() == 3 and n_txt > 0 and x._base is not None
+        and x.shape[0] == 1 and x.stride(2) == 1 and x.stride(1) == x.shape[2]
+        and x.storage_offset() >= n_txt * x.stride(1)):
+      front = x.as_strided((x.shape[0], n_txt, x.shape[2]), x.stride(),
+                           x.storage_offset() - n_txt * x.stride(1))
+      cnn.precompute_stage([(x, [self]), (front, [attn.to_add_out])])
+  return self._cdit_orig_forward(x)
 
 
 # ------------------------------------------------------------------ pieces of the block forwards
@@ -119,8 +125,9 @@ def _modulated_norm(block, norm: nn.Module, x, shift, scale):
   """`norm(x) * (1 + scale) + shift` for a LayerNorm without affine parameters: as bf16 tensor
   ops, or as the kernel that also hands the FP8 codes to the consuming Linears."""
   o = _opts(block)
-  if (o.get("fuse_norm") and x.is_cuda and x.dtype == torch.bfloat16 and isinstance(norm, nn.LayerNorm)
-      and norm.weight is None and norm.bias is None):
+  # (a traced graph keeps the tensor ops: its compiler fuses them, and nothing is handed over there)
+  if (o.get("fuse_norm") and not torch.compiler.is_compiling() and x.is_cuda and x.dtype == torch.bfloat16
+      and isinstance(norm, nn.LayerNorm) and norm.weight is None and norm.bias is None):
     return ops.ln_modulate_quant(x, shift, scale, eps=norm.eps, materialize=o.get("materialize", True))
   return norm(x) * (1 + scale) + shift
 
@@ -263,7 +270,7 @@ def _qwen_image_forward(self, hidden_states, encoder_hidden_states, encoder_hidd
 # Adapted from diffusers' WanTransformerBlock.forward
 # (src/diffusers/models/transformers/transformer_wan.py), the forward the reference adapts in
 # src/cache_dit/caching/patch_functors/functor_wan_vace.py:40-90. One stream: the stages are the
-# attention modules' own (hooks); the block forward is only rebound for the fused modulated
+# attention modules' own (their wrappers); the block forward is only rebound for the fused modulated
 # norms, which are computed as bf16 tensor ops (diffusers does these two in fp32 and rounds
 # once, so this rebinding is offered for models that accept the bf16 form).
 
@@ -290,7 +297,7 @@ class StagePatchFunctor:
   src/cache_dit/caching/patch_functors/functor_base.py:20-50); `remove(transformer)` undoes
   it. Blocks are recognised by class name, attention modules by their `to_q / to_k / to_v`.
 
-  batch_stages     one quantizer + one GEMM launch per stage (hooks and rebound forwards)
+  batch_stages     one quantizer + one GEMM launch per stage (rebound forwards)
   single_blocks    also precompute proj_mlp + q/k/v of FLUX single blocks as one stage (eager
                    code can leave this to nn.group_sibling_linears_; a rebound forward does
                    not need the discovery run)
@@ -320,8 +327,8 @@ class StagePatchFunctor:
             fuse_cat: bool = True, fuse_norm_quant: bool = False, materialize: bool = True) -> nn.Module:
     if batch_stages and any(isinstance(m, _QUANT) and m.sibling_group is not None
                             for m in transformer.modules()):
-      logger.warning("stage patch: sibling groups are removed (a stage is computed by the hooks "
-                     "and rebound forwards instead)")
+      logger.warning("stage patch: sibling groups are removed (a stage is computed by the rebound "
+                     "forwards instead)")
       cnn.group_sibling_linears_(transformer, enable=False)
     n_blocks = n_attn = 0
     batch_of = {}  # attention module -> whether its owning block batches stages
@@ -335,8 +342,8 @@ class StagePatchFunctor:
             "fuse_norm": bool(fuse_norm_quant),
             "materialize": bool(materialize),
             # (looked up here: the rebound forwards may run inside a traced graph)
-            "attn_takes_mask": (hasattr(block, "attn") and "encoder_hidden_states_mask"
-                                in inspect.signature(block.attn.forward).parameters),
+            "attn_takes_mask": (hasattr(block, "attn") and "encoder_hidden_states_mask" in inspect.signature(
+                block.attn.__dict__.get("_cdit_orig_forward") or block.attn.forward).parameters),
         }
         block._cdit_stage_opts = opts
         rebind = (opts["fuse_norm"] if name in self.NORM_ONLY_BLOCKS else
@@ -355,13 +362,12 @@ class StagePatchFunctor:
     for attn in transformer.modules():
       if all(isinstance(getattr(attn, a, None), _QUANT) for a in ("to_q", "to_k", "to_v")):
         attn._cdit_stage_batch = batch_of.get(id(attn), bool(batch_stages))
-        if "_cdit_stage_hooks" not in attn.__dict__:
-          handles = [attn.register_forward_pre_hook(_attention_stage_hook, with_kwargs=True)]
-          to_out = getattr(attn, "to_out", None)
-          if (getattr(attn, "to_add_out", None) is not None and to_out is not None
-              and _quantized(to_out[0], attn.to_add_out)):
-            handles.append(to_out[0].register_forward_pre_hook(_joint_out_hook(attn)))
-          attn._cdit_stage_hooks = handles
+        self._rebind(attn, _attention_forward)
+        to_out = getattr(attn, "to_out", None)
+        if (getattr(attn, "to_add_out", None) is not None and to_out is not None
+            and _quantized(to_out[0], attn.to_add_out)):
+          to_out[0].__dict__["_cdit_joint_attn"] = (attn, )  # (a tuple: not registered as a submodule)
+          self._rebind(to_out[0], _joint_out_forward)
         n_attn += 1
     transformer._cdit_stage_patched = True
     logger.info(f"stage patch: {n_blocks} blocks, {n_attn} attention modules of "
@@ -373,8 +379,7 @@ class StagePatchFunctor:
       self._rebind(m, None)
       m.__dict__.pop("_cdit_stage_opts", None)
       m.__dict__.pop("_cdit_stage_batch", None)
-      for h in m.__dict__.pop("_cdit_stage_hooks", []):
-        h.remove()
+      m.__dict__.pop("_cdit_joint_attn", None)
     transformer.__dict__.pop("_cdit_stage_patched", None)
     return transformer
 

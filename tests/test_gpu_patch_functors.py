@@ -78,7 +78,7 @@ def test_flux_blocks_patched_in_place_run_stage_by_stage(quant_type):
     # the model's code is what it was: the class forwards are untouched, the instances rebound
     assert type(double).forward is ds.FluxTransformerBlock.forward
     assert type(single).forward is ds.FluxSingleTransformerBlock.forward
-    assert type(double.attn).forward is ds.FluxAttention.forward and "forward" not in double.attn.__dict__
+    assert type(double.attn).forward is ds.FluxAttention.forward and not double.attn._forward_pre_hooks
     with _Launches() as staged:
       y1 = model(**inputs)
     assert torch.equal(y1, y0)
@@ -100,7 +100,8 @@ def test_flux_blocks_patched_in_place_run_stage_by_stage(quant_type):
       assert torch.isfinite(y2.float()).all() and cosine(y2, y0) >= 0.9999
     cache_dit.remove_stage_patch(model)
     assert "forward" not in double.__dict__ and "forward" not in single.__dict__
-    assert not double.attn._forward_pre_hooks and not double.attn.to_out[0]._forward_pre_hooks
+    assert "forward" not in double.attn.__dict__ and "forward" not in double.attn.to_out[0].__dict__
+    assert "_cdit_joint_attn" not in double.attn.to_out[0].__dict__
     with _Launches() as again:
       assert torch.equal(model(**inputs), y0)
     assert again.n["batched"] == 0
@@ -236,3 +237,44 @@ def test_precompute_stage_wrong_guesses_cost_time_not_correctness():
   with torch.inference_mode():
     assert not cache_dit.precompute_stage([(x.clone(), lins[:2])])
   assert torch.equal(lins[0](x), want[0])
+
+
+def test_patched_blocks_traced_by_torch_compile_keep_the_stages():
+  """The patched blocks under torch.compile(fullgraph=True): every stage the wrappers and
+  rebound forwards put together is ONE batch op in the traced graph (counted with a backend
+  that only inspects the graph and runs it as it is), all blocks of a class share one
+  compiled graph, and the output equals the eager forward's."""
+  import cache_dit_amd as cache_dit
+  try:
+    import torch._dynamo as dynamo
+  except Exception as e:
+    pytest.skip(f"no graph tracer: {str(e)[:80]}")
+  model, inputs = _flux(n_double=3, n_single=3)
+  seen = []
+
+  def inspect_only(gm, example_inputs):
+    ops_in_graph = [str(n.target) for n in gm.graph.nodes if n.op == "call_function"]
+    seen.append({"batch": sum("linear_w8a8_batch" in t for t in ops_in_graph),
+                 "single": sum(t.startswith("cdit.linear_w8a8.") or t == "cdit.linear_w8a8" or
+                               "cdit.linear_w8a8.default" in t for t in ops_in_graph),
+                 "cat2": sum("linear_w8a8_cat2" in t for t in ops_in_graph)})
+    return gm.forward
+
+  with torch.no_grad():
+    y0 = model(**inputs)
+    cache_dit.apply_stage_patch(model)
+    assert torch.equal(model(**inputs), y0)
+    dynamo.reset()
+    for blocks in (model.transformer_blocks, model.single_transformer_blocks):
+      for i in range(len(blocks)):
+        blocks[i] = torch.compile(blocks[i], backend=inspect_only, fullgraph=True)
+    y1 = model(**inputs)
+  # one graph per block class (the blocks of a class share it); double block: q/k/v of both
+  # streams, the two ff.net.0.proj, the two ff.net.2 as batch ops, its two output projections
+  # and two M = 1 Linears single; single block: proj_mlp + q/k/v one batch op, proj_out
+  # reading its two sources, the M = 1 Linear
+  assert len(seen) == 2, seen
+  assert seen[0] == {"batch": 3, "single": 4, "cat2": 0}, seen
+  assert seen[1] == {"batch": 1, "single": 1, "cat2": 1}, seen
+  assert torch.equal(y1, y0)
+  assert all(m._precomputed is None for m in model.modules() if hasattr(m, "_precomputed"))
