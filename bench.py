@@ -519,6 +519,20 @@ def headline_kernels(device):
     res["w8a16_frac_bf16_peak"] = res["w8a16_tflops"] / BF16_PEAK_TFLOPS
   except Exception as e:
     res["w8a16_note"] = str(e)[:120]
+  # the per-tensor quantizer (float8_per_tensor and the policy's fallback pass): three launches
+  # (zero the amax word, amax over the tensor, cast), the tensor read twice: 5MK + 4M bytes
+  try:
+    amax_ws = torch.zeros(1, dtype=torch.int32, device=device)
+
+    def pt_tensor():
+      i = it["i"] = (it["i"] + 1) % nbuf
+      ops.quant_tensorwise_into(xs[i], qs[i], ss[i], amax_ws, 0)
+
+    pt_ms = sorted(_time_events(pt_tensor, 100, 20 if k == 0 else 0) for k in range(3))[1]
+    res["per_tensor_quant_ms"] = pt_ms
+    res["per_tensor_quant_gbps"] = (5.0 * K + 4) * M / pt_ms / 1e6
+  except Exception as e:
+    res["per_tensor_quant_note"] = str(e)[:120]
   # the FP8 comm quantizers (scale packed behind each row) on an activation of the headline
   # size and on its q/k/v as [B, S, 3, heads, head_dim]; GB/s over their algorithmic bytes
   try:
