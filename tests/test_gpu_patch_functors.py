@@ -278,3 +278,45 @@ def test_patched_blocks_traced_by_torch_compile_keep_the_stages():
   assert seen[1] == {"batch": 1, "single": 1, "cat2": 1}, seen
   assert torch.equal(y1, y0)
   assert all(m._precomputed is None for m in model.modules() if hasattr(m, "_precomputed"))
+
+
+def test_patched_qwen_image_and_wan_blocks_trace_without_graph_breaks():
+  """The other two block families under torch.compile(fullgraph=True) with the stage patch:
+  one graph per block class, the stages as batch ops, the eager forward's bits."""
+  import cache_dit_amd as cache_dit
+  from cache_dit_amd.testing import dit_shapes as ds
+  try:
+    import torch._dynamo as dynamo
+  except Exception as e:
+    pytest.skip(f"no graph tracer: {str(e)[:80]}")
+  torch.manual_seed(0)
+  qwen = ds.QwenImageLikeTransformer(dim=256, heads=2, mlp=512, n_layers=3, in_channels=64,
+                                     text_dim=128).to(torch.bfloat16).cuda()
+  cache_dit.quantize(qwen, cache_dit.QuantizeConfig())
+  ds.fuse_gelu_epilogues(qwen)
+  qin = ds.qwen_image_like_inputs("cuda", n_img=200, n_txt=24, in_channels=64, text_dim=128)
+  wan = ds.WanLikeTransformer(dim=256, heads=2, ffn=512, n_layers=3, in_channels=64,
+                              text_dim=128).to(torch.bfloat16).cuda()
+  cache_dit.quantize(wan, cache_dit.QuantizeConfig())
+  win = ds.wan_like_inputs("cuda", n_tokens=200, n_txt=48, in_channels=64, text_dim=128)
+  for model, inputs, batch_ops in ((qwen, qin, 3), (wan, win, 2)):
+    seen = []
+
+    def inspect_only(gm, example_inputs, seen=seen):
+      seen.append(sum("linear_w8a8_batch" in str(n.target) for n in gm.graph.nodes
+                      if n.op == "call_function"))
+      return gm.forward
+
+    blocks = next(m for m in model.children() if isinstance(m, torch.nn.ModuleList))
+    with torch.no_grad():
+      y0 = model(**inputs)
+      cache_dit.apply_stage_patch(model)
+      dynamo.reset()
+      for i in range(len(blocks)):
+        blocks[i] = torch.compile(blocks[i], backend=inspect_only, fullgraph=True)
+      y1 = model(**inputs)
+    # Qwen-Image: q/k/v of both streams and the two pairs of MLP Linears (its joint output
+    # projections rest on storage addresses and stay two ops in a traced graph); Wan: q/k/v of
+    # the self-attention, the query next to k / v of the cross-attention
+    assert seen == [batch_ops], seen
+    assert torch.equal(y1, y0)
