@@ -22,9 +22,10 @@ and block forward signatures. Three mechanisms, from least to most intrusive:
     serial number, which a graph tracer guards on, so that every block would be compiled
     separately.)
   * rebound block forwards, adapted from the diffusers block forwards, for what these
-    wrappers cannot do: the two FeedForwards of a double-stream block run at different points of the original
-    forward (the text stream's input does not exist yet when the image stream's runs), so
-    the forward is reordered to put both modulated inputs side by side; a FLUX single block
+    wrappers cannot do: the two FeedForwards of a double-stream block run at different
+    points of the original forward (the text stream's input does not exist yet when the
+    image stream's runs), so the forward is reordered to put both modulated inputs side by
+    side; a FLUX single block
     precomputes proj_mlp next to q/k/v and lets proj_out's quantizer read
     `[attn_output | mlp_hidden_states]` in place (`nn.linear_on_cat`).
   * optionally (`fuse_norm_quant=True`) the modulated LayerNorms
@@ -65,9 +66,6 @@ def _quantized(*mods) -> bool:
 
 
 # ------------------------------------------------------------------ attention modules
-
-
-_STAGE_LINEARS = ("to_q", "to_k", "to_v", "add_q_proj", "add_k_proj", "add_v_proj")
 
 
 def _attention_forward(self, *args, **kwargs):
