@@ -517,6 +517,23 @@ def headline_kernels(device):
     res["w8a16_ms"] = w_ms
     res["w8a16_tflops"] = 2.0 * M * K * N / w_ms / 1e9
     res["w8a16_frac_bf16_peak"] = res["w8a16_tflops"] / BF16_PEAK_TFLOPS
+    # comparators on the same box: the vendor library's plain bf16 GEMM on a bf16 copy of the
+    # weights, and the form the weight-only mode replaces (dequantize with tensor ops, then
+    # that GEMM)
+    wb = [ws[i].to(torch.bfloat16) for i in range(2)]
+
+    def blas_bf16():
+      i = it["i"] = (it["i"] + 1) % nbuf
+      torch.nn.functional.linear(xs[i], wb[i & 1], b)
+
+    def dequant_then_gemm():
+      i = it["i"] = (it["i"] + 1) % nbuf
+      w = (ws[i].to(torch.float32) * wsc[:, None]).to(torch.bfloat16)
+      torch.nn.functional.linear(xs[i], w, b)
+
+    res["hipblaslt_bf16_tflops"] = 2.0 * M * K * N / _time_events(blas_bf16, 30, 10) / 1e9
+    res["w8a16_dequant_then_gemm_ms"] = _time_events(dequant_then_gemm, 20, 5)
+    del wb
   except Exception as e:
     res["w8a16_note"] = str(e)[:120]
   # the per-tensor quantizer (float8_per_tensor and the policy's fallback pass): three launches
