@@ -444,12 +444,57 @@ def headline_kernels(device):
       "quant_ms_before_gemm_legs": list(quant_before),
       "quant_ms_after_gemm_legs": list(quant_after),
   }
+  # Where the workgroups of such a launch finish, by XCD (the measurement instance of the same
+  # kernel: cdit_debug_gemm_stamps): the clocks of the eight XCDs differ under the power
+  # limit, the launch ends with the slowest; whether handing tiles out dynamically could
+  # help is a matter of that spread against one tile's time.
+  from cache_dit_amd import _native
+  L, stream = _native.load(), torch.cuda.current_stream().cuda_stream
+  try:
+    import ctypes
+    stamps = torch.zeros(4 * 256, dtype=torch.int64, device=device)
+    n_wg = ctypes.c_int(0)
+    per_xcd, last_xcd, tile_us, launch_us = {}, {}, [], []
+    for rep in range(12):
+      for _ in range(25):  # keeps the part in the power-limited state the timed legs run in
+        gemm()
+      i = it["i"] = (it["i"] + 1) % nbuf
+      _native.check(L.cdit_debug_gemm_stamps(qs[i].data_ptr(), ss[i].data_ptr(), ws[i].data_ptr(),
+                                              wsc.data_ptr(), b.data_ptr(), outs[i & 1].data_ptr(),
+                                              M, N, K, K, K, N, stamps.data_ptr(), ctypes.byref(n_wg),
+                                              stream))
+      torch.cuda.synchronize()
+      if rep < 2:
+        continue  # (warm-up)
+      st = stamps.view(-1, 4)[:n_wg.value].cpu()
+      t0 = int(st[:, 0].min())
+      end_us = (st[:, 1] - t0).double() / 100.0  # 100 MHz ticks
+      launch_us.append(float(end_us.max()))
+      tile_us.append(float(((st[:, 1] - st[:, 0]).double() / st[:, 3].double()).mean() / 100.0))
+      for x in sorted(set(st[:, 2].tolist())):
+        per_xcd.setdefault(int(x), []).append(float(end_us[st[:, 2] == x].mean()))
+        last_xcd.setdefault(int(x), []).append(float(end_us[st[:, 2] == x].max()))
+    xcd_last = {x: sum(v) / len(v) for x, v in last_xcd.items()}
+    xcd_mean = {x: sum(v) / len(v) for x, v in per_xcd.items()}
+    t_tile = sum(tile_us) / len(tile_us)
+    finish = {
+        "mean_finish_us_by_xcd": [round(xcd_mean[x], 2) for x in sorted(xcd_mean)],
+        "last_finish_us_by_xcd": [round(xcd_last[x], 2) for x in sorted(xcd_last)],
+        "launch_us": round(sum(launch_us) / len(launch_us), 2),
+        "tile_us": round(t_tile, 2),
+        "tiles_per_workgroup": float(st[:, 3].double().mean()),
+        "spread_fastest_to_slowest_xcd_in_tiles": round((max(xcd_mean.values()) - min(xcd_mean.values())) / t_tile, 3),
+        "note": "10 launches of the 288x192 kernel with per-workgroup time stamps, each behind 25 "
+                "ordinary launches; finish = end of a workgroup after the first start, averaged per "
+                "XCD; a tile = a workgroup's time / its tiles",
+    }
+  except Exception as e:
+    finish = {"note": f"unavailable: {str(e)[:120]}"}
+  res["xcd_finish_times"] = finish
   # What bounds the quantizer at this size: the fixed cost of a launch of M one-wavefront
   # workgroups. The same kernel with K = 0 (4608 workgroups that only write their scale)
   # and on a single row, next to the 42 MB case; rocprofv3 --kernel-trace of this command
   # gives the matching device-side durations (profiles/).
-  from cache_dit_amd import _native
-  L, stream = _native.load(), torch.cuda.current_stream().cuda_stream
 
   def quant_raw(rows, cols):
     def fn():

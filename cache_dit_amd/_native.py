@@ -50,6 +50,7 @@ EXPORTS = (
     "cdit_debug_set_gemm_variant",
     "cdit_debug_set_quant_hints",
     "cdit_debug_mfma_only",
+    "cdit_debug_gemm_stamps",
     "cdit_stream_capture_id",
 )
 
@@ -77,6 +78,9 @@ def _bind(L: ctypes.CDLL) -> None:
   L.cdit_debug_set_quant_hints.argtypes = [ci]
   L.cdit_debug_mfma_only.restype = ci
   L.cdit_debug_mfma_only.argtypes = [vp, ci, ci, ci, ctypes.POINTER(ctypes.c_double), vp]
+  L.cdit_debug_gemm_stamps.restype = ci
+  L.cdit_debug_gemm_stamps.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp,
+                                       ctypes.POINTER(ci), vp]
   L.cdit_fp8_quant_rowwise.restype = ci
   L.cdit_fp8_quant_rowwise.argtypes = [vp, i64, i64, i64, vp, i64, vp, ci, vp]
   L.cdit_fp8_quant_rowwise_cat2.restype = ci

@@ -174,6 +174,38 @@ int cdit_debug_mfma_only(void* out_f32, int blocks, int iters, int random_operan
   return rc ? rc : after_launch(fn);
 }
 
+int cdit_debug_gemm_stamps(const void* a_q, const float* a_scale, const void* b_q, const float* b_scale,
+                           const void* bias, void* out, int64_t M, int64_t N, int64_t K, int64_t lda,
+                           int64_t ldb, int64_t ldo, void* stamps_u64, int* workgroups, void* stream) {
+  const char* fn = "cdit_debug_gemm_stamps";
+  int rc = check_gemm(fn, a_q, b_q, b_scale, bias, out, M, N, K, lda, ldb, ldo, 0, CDIT_DT_BF16, false);
+  if (rc) return rc;
+  if (!a_scale || !stamps_u64 || M == 0 || N == 0) {
+    set_error("%s: a_scale or stamps is null, or an empty problem", fn);
+    return CDIT_EINVAL;
+  }
+  rc = check_arch();
+  if (rc) return rc;
+  GemmArgs g;
+  g.a = a_q;
+  g.a_scale = a_scale;
+  g.b = static_cast<const uint8_t*>(b_q);
+  g.b_scale = b_scale;
+  g.bias = static_cast<const uint16_t*>(bias);
+  g.out = static_cast<uint16_t*>(out);
+  g.M = (int)M;
+  g.N = (int)N;
+  g.K = (int)K;
+  g.lda = lda;
+  g.ldb = ldb;
+  g.ldo = ldo;
+  g.epilogue = 0;
+  g.out_dtype = CDIT_DT_BF16;
+  rc = launch_gemm_fp8_stamps(g, static_cast<unsigned long long*>(stamps_u64), workgroups,
+                              static_cast<hipStream_t>(stream));
+  return rc ? rc : after_launch(fn);
+}
+
 // consumer_follows: the codes are read by a GEMM launched right behind (the fused
 // Linear entry point): the quantizer then keeps its loads and stores cacheable.
 static int quant_rowwise_impl(const char* fn, const void* x_bf16, int64_t M, int64_t K,

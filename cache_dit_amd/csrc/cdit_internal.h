@@ -97,6 +97,9 @@ struct GemmGroup {
 
 // variant < 0: choose by shape.
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream);
+// the 288 x 192 kernel with per-workgroup time stamps (measurement only; gemm_fp8.hip)
+int launch_gemm_fp8_stamps(const GemmArgs& g, unsigned long long* stamps, int* workgroups,
+                           hipStream_t stream);
 // All members of `grp` in one launch (K, lda, ldb and the output dtype from `common`; its other
 // fields are ignored). 0: launched; -1: not taken (shape, alignment or variant without a
 // grouped form); else a CDIT_E* code.

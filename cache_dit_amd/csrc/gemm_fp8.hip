@@ -422,12 +422,23 @@ struct NoGroup {};
 // the bf16 instances carry no trace of the others. GROUPED: the launch walks the tiles
 // of a GemmGroup (the B-side fields of `g` are then unused); the instances without it
 // are unchanged by its existence.
-template <class C, int OUT = CDIT_DT_BF16, bool GROUPED = false>
+// STAMPS (a measurement instance, never launched by the operator entry points): every
+// workgroup leaves four 64-bit words at stamps + 4 * blockIdx.x -- the constant-rate wall
+// clock (100 MHz) at its start and after its last store has been issued and its DMA has
+// drained, the id of the XCD it ran on and the number of tiles it took -- so that the spread
+// of the finish times over the XCDs can be read off a real launch.
+struct StampArgs {
+  unsigned long long* stamps;
+};
+template <class C, int OUT = CDIT_DT_BF16, bool GROUPED = false, bool STAMPS = false>
 __global__ __launch_bounds__(C::THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void
 gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
-              std::conditional_t<GROUPED, GemmGroup, NoGroup> grp) {
+              std::conditional_t<GROUPED, GemmGroup, std::conditional_t<STAMPS, StampArgs, NoGroup>> grp) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int tid = threadIdx.x;
+  unsigned long long stamp_start = 0;
+  int stamp_tiles = 0;
+  if constexpr (STAMPS) stamp_start = wall_clock64();
   const int lane = tid & 63;
   // wave-uniform on purpose: LDS-DMA destinations (M0) then come from scalar code
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -976,6 +987,7 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
     }
     // (one copy of the last row's stores for both epilogues, all non-temporal)
     if constexpr (PERMUTE) store_moved(TM - 1, std::integral_constant<int, kStoreOnce>{});
+    if constexpr (STAMPS) ++stamp_tiles;
     if (next_tile >= ntiles) break;
     m0 = nm0;
     n0 = nn0;
@@ -984,6 +996,20 @@ gemm_fp8_wide(GemmArgs g, int tiles_m, int tiles_n,
   }
   // the zero-record DMA of the last D steps must not outlive the workgroup
   wait_vm<0>();
+  if constexpr (STAMPS) {
+    typedef unsigned int u2v __attribute__((ext_vector_type(2)));
+    const unsigned long long stamp_end = wall_clock64();
+    // HW_REG_XCC_ID (register 20), bits 3:0
+    const unsigned xcc = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11));
+    const __amdgpu_buffer_rsrc_t sb = __builtin_amdgcn_make_buffer_rsrc(grp.stamps + 4 * blockIdx.x, 0, 32, 0x00020000);
+    // (thread 0 writes; every other thread's offset lies beyond the 32 bytes. 8-byte stores:
+    // the 16-byte buffer stores of this kernel are the output's, and are counted)
+    const int off = tid == 0 ? 0 : 64;
+    __builtin_amdgcn_raw_buffer_store_b64(u2v{(unsigned)stamp_start, (unsigned)(stamp_start >> 32)}, sb, off, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b64(u2v{(unsigned)stamp_end, (unsigned)(stamp_end >> 32)}, sb, off + 8, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b64(u2v{xcc, 0u}, sb, off + 16, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b64(u2v{(unsigned)stamp_tiles, 0u}, sb, off + 24, 0, 0);
+  }
 }
 
 template <class C, int OUT = CDIT_DT_BF16>
@@ -1002,6 +1028,27 @@ int launch_wide(const GemmArgs& g, hipStream_t stream) {
   // one persistent workgroup per CU (its LDS and registers fill the CU)
   hipLaunchKernelGGL((gemm_fp8_wide<C, OUT>), dim3(ntiles < cus ? ntiles : cus), dim3(C::THREADS),
                      C::LDS_BYTES, stream, g, tiles_m, tiles_n, NoGroup{});
+  return 0;
+}
+
+// The measurement instance of the same kernel (StampArgs above).
+template <class C>
+int launch_wide_stamps(const GemmArgs& g, unsigned long long* stamps, int* workgroups, hipStream_t stream) {
+  static bool lds_allowed[64];
+  if (int rc = allow_dynamic_lds(
+          reinterpret_cast<const void*>(&gemm_fp8_wide<C, CDIT_DT_BF16, false, true>), C::LDS_BYTES,
+          lds_allowed))
+    return rc;
+  const int cus = cu_count();
+  if (cus <= 0) {
+    set_error("cannot query the CU count of the current device");
+    return CDIT_EHIP;
+  }
+  const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
+  const int ntiles = tiles_m * tiles_n, wgs = ntiles < cus ? ntiles : cus;
+  if (workgroups) *workgroups = wgs;
+  hipLaunchKernelGGL((gemm_fp8_wide<C, CDIT_DT_BF16, false, true>), dim3(wgs), dim3(C::THREADS),
+                     C::LDS_BYTES, stream, g, tiles_m, tiles_n, StampArgs{stamps});
   return 0;
 }
 
@@ -1488,6 +1535,16 @@ template <class Tiles, class WideOk>
 TileChoice choose_bf16_variant(Tiles tiles, WideOk wide_ok);
 template <class WideOk>
 int launch_bf16_variant(const GemmArgs& g, int variant, WideOk wide_ok, hipStream_t stream);
+
+int launch_gemm_fp8_stamps(const GemmArgs& g, unsigned long long* stamps, int* workgroups,
+                           hipStream_t stream) {
+  if (!tiled_ok(g) || g.out_dtype != CDIT_DT_BF16 || g.K < 128 * 3 || g.M <= 16) {
+    set_error("cdit_debug_gemm_stamps: the 288 x 192 kernel takes bf16 outputs, aligned operands, "
+              "K >= 384 and M > 16");
+    return CDIT_EINVAL;
+  }
+  return launch_wide_stamps<V14>(g, stamps, workgroups, stream);
+}
 
 int launch_gemm_fp8(const GemmArgs& g, int variant, hipStream_t stream) {
   if (!tiled_ok(g) || variant == 100) {

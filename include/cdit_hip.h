@@ -389,6 +389,21 @@ int cdit_debug_set_quant_hints(int hints);
 int cdit_debug_mfma_only(void* out_f32, int blocks, int iters, int random_operands, double* flop,
                          void* stream);
 
+/*
+ * Measurement aid, not part of the operator interface (no counterpart in the reference):
+ * cdit_fp8_gemm_rowwise (bf16 output, no epilogue flags) on the 288 x 192 tile kernel, built
+ * with time stamps: every workgroup (one per CU, at most one per tile; their number goes to
+ * *workgroups, host memory, may be null) leaves four 64-bit words at stamps_u64 + 4 * its
+ * index: the constant-rate wall clock (100 MHz ticks) at its start and at its end, the id
+ * of the XCD it ran on, and the number of tiles it computed. stamps_u64: device memory for
+ * 4 * 256 words at least. The output is the GEMM's. What bench.py derives from it: how far
+ * the workgroups' finish times lie apart by XCD, in units of one tile's time, which is what
+ * decides whether handing tiles out dynamically could shorten a launch.
+ */
+int cdit_debug_gemm_stamps(const void* a_q, const float* a_scale, const void* b_q, const float* b_scale,
+                           const void* bias, void* out, int64_t M, int64_t N, int64_t K, int64_t lda,
+                           int64_t ldb, int64_t ldo, void* stamps_u64, int* workgroups, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -670,3 +670,44 @@ def test_scales_and_bias_at_odd_offsets():
   aligned = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
   ops.gemm_rowwise_into(a, s_a[1:].clone(), w, s_w[1:].clone(), b[1:].clone(), aligned, 0)
   assert torch.equal(out, aligned) or max_rel_err(out, aligned.cpu()) <= REL_TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(4608, 12288, 3072), (1000, 840, 512)])
+def test_measurement_instance_with_time_stamps_gives_the_same_bits(M, N, K):
+  """cdit_debug_gemm_stamps runs the 288 x 192 kernel with four stamps per workgroup added:
+  the output must be the ordinary kernel's bit for bit, every workgroup that the launcher
+  reports must have written a start before its end, a hardware XCD id below 8 and a tile
+  count, and the tile counts must add up to the tiles of the problem."""
+  import ctypes
+  from cache_dit_amd import _native
+  L = _native.load()
+  g = torch.Generator().manual_seed(M + K)
+  a = (torch.randn(M, K, generator=g) * 40).cuda().to(FP8)
+  w = (torch.randn(N, K, generator=g) * 40).cuda().to(FP8)
+  sa = (torch.rand(M, 1, generator=g) + 0.5).cuda()
+  sw = (torch.rand(1, N, generator=g) * 1e-3).cuda()
+  b = torch.randn(N, generator=g).to(torch.bfloat16).cuda()
+  ref = torch.full((M, N), 7.0, dtype=torch.bfloat16, device="cuda")
+  out = torch.full((M, N), -7.0, dtype=torch.bfloat16, device="cuda")
+  _native.set_gemm_variant(14)
+  _native.check(L.cdit_fp8_gemm_rowwise(a.data_ptr(), sa.data_ptr(), w.data_ptr(), sw.data_ptr(),
+                                        b.data_ptr(), ref.data_ptr(), M, N, K, K, K, N, 0, 1, None))
+  stamps = torch.zeros(4 * 512, dtype=torch.int64, device="cuda")
+  n_wg = ctypes.c_int(0)
+  _native.check(L.cdit_debug_gemm_stamps(a.data_ptr(), sa.data_ptr(), w.data_ptr(), sw.data_ptr(),
+                                         b.data_ptr(), out.data_ptr(), M, N, K, K, K, N,
+                                         stamps.data_ptr(), ctypes.byref(n_wg), None))
+  torch.cuda.synchronize()
+  assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+  assert 0 < n_wg.value <= 512
+  st = stamps.view(-1, 4).cpu()
+  used, rest = st[:n_wg.value], st[n_wg.value:]
+  assert (rest == 0).all()
+  assert (used[:, 1] > used[:, 0]).all() and (used[:, 0] > 0).all()
+  assert ((used[:, 2] >= 0) & (used[:, 2] < 8)).all()
+  assert int(used[:, 3].sum()) == ((M + 287) // 288) * ((N + 191) // 192)
+  # too small for this kernel: refused with a message, nothing launched
+  rc = L.cdit_debug_gemm_stamps(a.data_ptr(), sa.data_ptr(), w.data_ptr(), sw.data_ptr(),
+                                b.data_ptr(), out.data_ptr(), 16, N, K, K, K, N,
+                                stamps.data_ptr(), ctypes.byref(n_wg), None)
+  assert rc != 0 and b"288 x 192" in L.cdit_last_error()

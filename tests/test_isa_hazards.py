@@ -158,18 +158,20 @@ def test_output_stores_are_unconditional(wide_kernels):
   branch); for 16-bit outputs the stores of the last row of blocks follow the join."""
   counted = 0
   for name, code in wide_kernels.items():
-    m = re.search(r"gemm_fp8_wideINS0_7CfgWideILi(\d+)ELi(\d+)ELi\d+ELi\d+ELb[01]EEELi(\d)E", name)
+    m = re.search(r"gemm_fp8_wideINS0_7CfgWideILi(\d+)ELi(\d+)ELi\d+ELi\d+ELb[01]EEELi(\d)ELb[01]ELb([01])E", name)
     if not m:
       continue
     bm, bn, out = int(m.group(1)), int(m.group(2)), int(m.group(3))
+    # (the measurement instance leaves its time stamps with two more 16-byte stores)
+    stamp_stores = 2 if m.group(4) == "1" else 0
     per_row = bn // 64 * (2 if out == 2 else 1)
     expect = bm // 32 * per_row
     shared = 0 if out == 2 else per_row
     assert not any(l.startswith("global_store") for l in code), name
     code = labeled[name]
     stores = [i for i, l in enumerate(code) if l.startswith("buffer_store_dwordx4")]
-    assert len(stores) == 2 * (expect - shared) + shared, \
-        f"{name}: {len(stores)} output stores, expected 2 * {expect - shared} + {shared}"
+    assert len(stores) == 2 * (expect - shared) + shared + stamp_stores, \
+        f"{name}: {len(stores)} output stores, expected 2 * {expect - shared} + {shared} + {stamp_stores}"
     # no store under a lane mask (a store that may be skipped) or in a loop over the
     # values of a descriptor: none lies between an exec-conditional branch and its target
     label_at = {m.group(1): i for i, l in enumerate(code) for m in [re.match(r"(\.\w+):", l)] if m}
