@@ -1047,7 +1047,7 @@ def main():
                       "launch and one batched GEMM launch (two where the tile cost model splits "
                       "the stage), bit-identical to running each Linear on its own. This is the "
                       "launch pattern cache_dit_amd.apply_stage_patch gives an unmodified model "
-                      "(hooks on its attention modules, rebound block forwards); plain "
+                      "(rebound forwards of its attention modules and blocks); plain "
                       "quantize() alone gives ungrouped_*, group_sibling_linears_ grouped_*",
           "quant_type": "float8_per_row",
           "launch": launch_mode,
