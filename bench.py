@@ -362,6 +362,68 @@ def measured_traffic(kernel_key):
     return None
 
 
+class _BoardPower:
+  """Samples the board power the amdgpu driver reports for the GPU (hwmon power1_input or
+  power1_average, microwatts; a reading the driver smooths over a few hundred ms) from a thread
+  while a leg runs. `cap_w` is the power limit the driver enforces (power1_cap). Best effort:
+  without the files every figure is None."""
+
+  def __init__(self, device_index=0, period=0.02):
+    import glob
+    self.period, self.samples, self._stop, self._thread = period, [], False, None
+    self.path = self.cap_w = None
+    cards = sorted(glob.glob("/sys/class/drm/card[0-9]*/device/hwmon/hwmon*"))
+    cards = [c for c in cards if any(os.path.exists(os.path.join(c, f)) for f in ("power1_input", "power1_average"))]
+    if len(cards) > 1:  # several GPUs visible: the one whose PCI address is the torch device's
+      try:
+        import torch
+        pr = torch.cuda.get_device_properties(device_index)
+        addr = f"{pr.pci_domain_id:04x}:{pr.pci_bus_id:02x}:{pr.pci_device_id:02x}.0"
+        cards = [c for c in cards if addr in os.path.realpath(c)] or cards[:0]
+      except Exception:
+        cards = cards[:0]
+    if cards:
+      for f in ("power1_input", "power1_average"):
+        if os.path.exists(os.path.join(cards[0], f)):
+          self.path = os.path.join(cards[0], f)
+          break
+      try:
+        with open(os.path.join(cards[0], "power1_cap")) as fh:
+          self.cap_w = int(fh.read()) / 1e6
+      except (OSError, ValueError):
+        pass
+
+  def _run(self):
+    while not self._stop:
+      try:
+        with open(self.path) as fh:
+          self.samples.append((time.perf_counter(), int(fh.read()) / 1e6))
+      except (OSError, ValueError):
+        pass
+      time.sleep(self.period)
+
+  def __enter__(self):
+    if self.path:
+      import threading
+      self._thread = threading.Thread(target=self._run, daemon=True)
+      self._thread.start()
+    return self
+
+  def __exit__(self, *exc):
+    self._stop = True
+    if self._thread:
+      self._thread.join()
+
+  def settled_w(self, since=None):
+    """Mean of the last quarter of the samples taken (after `since`): the smoothed reading
+    needs about half a second of steady load to arrive."""
+    w = [v for t, v in self.samples if since is None or t >= since]
+    if not w:
+      return None
+    tail = w[-max(1, len(w) // 4):]
+    return sum(tail) / len(tail)
+
+
 def _time_events(fn, iters, warmup):
   """Average duration in ms of fn() over `iters` calls, HIP events on the current
   stream (the stream the kernels are launched on)."""
@@ -421,15 +483,27 @@ def headline_kernels(device):
     return blocks[2], blocks[0], blocks[-1]
 
   quant_before = quant_median_ms()
-  t_start, prev = time.perf_counter(), _time_events(gemm, 100, 100)
-  while time.perf_counter() - t_start < 4.0:
-    cur = _time_events(gemm, 100, 0)
-    settled = abs(cur - prev) <= 0.005 * prev
-    prev = cur
-    if settled and time.perf_counter() - t_start > 1.5:
-      break
-  gemm_ms = _time_events(gemm, 100, 10)
-  gemm_gelu_ms = _time_events(gemm_gelu, 100, 10)
+  power = _BoardPower(torch.device(device).index or 0)
+  idle_w = None
+  if power.path:
+    time.sleep(0.3)
+    try:
+      with open(power.path) as fh:
+        idle_w = int(fh.read()) / 1e6  # (between legs: not a cold idle)
+    except (OSError, ValueError):
+      pass
+  with power:
+    t_start, prev = time.perf_counter(), _time_events(gemm, 100, 100)
+    while time.perf_counter() - t_start < 4.0:
+      cur = _time_events(gemm, 100, 0)
+      settled = abs(cur - prev) <= 0.005 * prev
+      prev = cur
+      if settled and time.perf_counter() - t_start > 1.5:
+        break
+    gemm_ms = _time_events(gemm, 100, 10)
+    gemm_w = power.settled_w()
+    gemm_max_w = max((v for _, v in power.samples), default=None)
+    gemm_gelu_ms = _time_events(gemm_gelu, 100, 10)
   quant_after = quant_median_ms()
   quant_ms = quant_after[0]
   res = {
@@ -443,6 +517,11 @@ def headline_kernels(device):
       # median, fastest and slowest of five blocks of 100 back-to-back launches (ms)
       "quant_ms_before_gemm_legs": list(quant_before),
       "quant_ms_after_gemm_legs": list(quant_after),
+      # board power as the amdgpu driver reports it (hwmon), sampled every 20 ms while the
+      # GEMM legs ran: the settled reading against the limit the driver enforces
+      "board_power": {"cap_w": power.cap_w, "gemm_w": gemm_w, "gemm_max_w": gemm_max_w,
+                      "before_gemm_legs_w": idle_w,
+                      "source": power.path},
   }
   # Where the workgroups of such a launch finish, by XCD (the measurement instance of the same
   # kernel: cdit_debug_gemm_stamps): the clocks of the eight XCDs differ under the power
@@ -665,6 +744,14 @@ def mfma_only_ceiling(device):
 
     times = sorted(_time_events(fn, 1, 2 if k == 0 else 0) for k in range(3))
     res[key] = flop.value / times[1] / 1e9
+    # the same loop held for 0.6 s (40 launches) with the board power sampled: the smoothed
+    # reading needs that long; the rate of the last 10 launches next to it
+    with _BoardPower(torch.device(device).index or 0) as power:
+      _time_events(fn, 30, 0)
+      sustained_ms = _time_events(fn, 10, 0)
+    res[key.replace("_tflops", "_sustained_tflops")] = flop.value / sustained_ms / 1e9
+    res[key.replace("_tflops", "_board_w")] = power.settled_w()
+    res["board_cap_w"] = power.cap_w
   res["note"] = ("loop of v_mfma_f32_16x16x128_f8f6f4 on register operands, 256 workgroups x 4 "
                  "wavefronts, 16 independent accumulators, no memory traffic; HIP events")
   return res
@@ -1000,6 +1087,9 @@ def main():
       # rate the power-limited part sustains on random e4m3 operands, and the GEMM against it
       "mfma_only_tflops": ceiling["random_operands_tflops"],
       "frac_of_mfma_only": head["gemm_tflops"] / ceiling["random_operands_tflops"],
+      # board power the driver reports while this kernel runs back to back, and its limit
+      "board_power_w": head["board_power"]["gemm_max_w"],
+      "board_power_cap_w": head["board_power"]["cap_w"],
   }
   roofline_quant = {
       "kernel": "quant_rowwise_regs at M=4608 K=3072",
