@@ -1045,7 +1045,8 @@ int launch_wide_stamps(const GemmArgs& g, unsigned long long* stamps, int* workg
     return CDIT_EHIP;
   }
   const int tiles_m = (g.M + C::BM - 1) / C::BM, tiles_n = (g.N + C::BN - 1) / C::BN;
-  const int ntiles = tiles_m * tiles_n, wgs = ntiles < cus ? ntiles : cus;
+  // (the caller's buffer holds the stamps of 256 workgroups)
+  const int ntiles = tiles_m * tiles_n, wgs = std::min(ntiles, std::min(cus, 256));
   if (workgroups) *workgroups = wgs;
   hipLaunchKernelGGL((gemm_fp8_wide<C, CDIT_DT_BF16, false, true>), dim3(wgs), dim3(C::THREADS),
                      C::LDS_BYTES, stream, g, tiles_m, tiles_n, StampArgs{stamps});
