@@ -135,10 +135,10 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t bytes_buf(const void* base, in
 // bytes of the row and its last SH bytes go out in 2- and 4-byte stores.
 template <int SCALE, int CH, int SH>
 __device__ __forceinline__ void store_codes_plain(const uint4 (&v)[CH], uint8_t* __restrict__ yr, int H,
-                                                  float scale, float inv, int lane) {
+                                                  float scale, float inv, Recip rc, int lane) {
   const int nchunks = H >> 3;
   const __amdgpu_buffer_rsrc_t rb = bytes_buf(yr - SH, SH + H);
-  auto q = [&](float x) { return SCALE == 0 ? x * inv : div_scale<true>(x, scale, inv); };
+  auto q = [&](float x) { return SCALE == 0 ? x * inv : div_scale<true>(x, scale, rc); };
   uint32_t carry_lo = 0, carry_hi = 0;
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
@@ -224,6 +224,7 @@ __device__ __forceinline__ void quant_row(const uint16_t* __restrict__ xr, uint8
   // (a NaN in the row has the largest bit pattern and arrives here as the amax)
   const bool finite_row = (__float_as_uint(amax) & 0x7fffffffu) < 0x7f800000u;
   float scale, inv = 0.0f;
+  Recip rc{};
   bool plain;  // wave-uniform: the clamp is a no-op and, for SCALE 1, the fast division is exact
   if constexpr (SCALE == 0) {
     amax = fmaxf(amax, 1e-4f);
@@ -234,23 +235,23 @@ __device__ __forceinline__ void quant_row(const uint16_t* __restrict__ xr, uint8
   } else {
     const float raw = amax / kFp8Max;
     scale = fmaxf(raw, 1e-6f);
-    inv = 1.0f / scale;
+    rc = make_recip(scale);
     // scale = fl(amax / 448) inside the window: the case the fast division is proven on
     // (tests/native/divcheck.c, fp32 scales); a floored scale takes the compiler's division
     plain = finite_row && scale == raw && scale_in_fast_window(scale);
   }
   auto q = [&](float x) {
-    if (plain) return SCALE == 0 ? x * inv : div_scale<true>(x, scale, inv);
+    if (plain) return SCALE == 0 ? x * inv : div_scale<true>(x, scale, rc);
     const float y = SCALE == 0 ? x * inv : x / scale;
     return y != y ? y : fminf(fmaxf(y, -kFp8Max), kFp8Max);
   };
   const int sh = (int)(reinterpret_cast<uintptr_t>(yr) & 7);  // wave-uniform
   if (vec && plain && (sh & 1) == 0) {
     switch (sh) {
-      case 0: store_codes_plain<SCALE, CH, 0>(v, yr, H, scale, inv, lane); break;
-      case 2: store_codes_plain<SCALE, CH, 2>(v, yr, H, scale, inv, lane); break;
-      case 4: store_codes_plain<SCALE, CH, 4>(v, yr, H, scale, inv, lane); break;
-      default: store_codes_plain<SCALE, CH, 6>(v, yr, H, scale, inv, lane); break;
+      case 0: store_codes_plain<SCALE, CH, 0>(v, yr, H, scale, inv, rc, lane); break;
+      case 2: store_codes_plain<SCALE, CH, 2>(v, yr, H, scale, inv, rc, lane); break;
+      case 4: store_codes_plain<SCALE, CH, 4>(v, yr, H, scale, inv, rc, lane); break;
+      default: store_codes_plain<SCALE, CH, 6>(v, yr, H, scale, inv, rc, lane); break;
     }
     // the scale behind the codes, from lane 0 (H is even here: 2- resp. 4-byte aligned)
     const __amdgpu_buffer_rsrc_t sb = bytes_buf(yr + H, 4);
@@ -551,14 +552,14 @@ __global__ __launch_bounds__(64 * kGroupedWaves) void comm_qkv_permute_quant_gro
       const uint32_t mbits = group_max_u32<G>(fold2(m));  // bf16 pattern of the row's max |x|
       const float raw = __uint_as_float(mbits << 16) / kFp8Max;
       const float scale = fmaxf(raw, 1e-6f);
-      const float inv = 1.0f / scale;
+      const Recip rc = make_recip(scale);
       // The proven fast division where every row of the wavefront has a finite amax and an
       // unfloored scale inside the window (scale = fl(amax / 448); tests/native/divcheck.c),
       // the compiler's division and the clamp for the whole wavefront otherwise.
       const bool plain = mbits < 0x7f80u && scale == raw && scale_in_fast_window(scale);
       uint32_t lo, hi;
       if (__builtin_amdgcn_ballot_w64(!plain) == 0) {
-        auto q = [&](float f) { return div_scale<true>(f, scale, inv); };
+        auto q = [&](float f) { return div_scale<true>(f, scale, rc); };
         lo = cvt4_fp8(q(bf16_lo(v[u].x)), q(bf16_hi(v[u].x)), q(bf16_lo(v[u].y)), q(bf16_hi(v[u].y)));
         hi = cvt4_fp8(q(bf16_lo(v[u].z)), q(bf16_hi(v[u].z)), q(bf16_lo(v[u].w)), q(bf16_hi(v[u].w)));
       } else {

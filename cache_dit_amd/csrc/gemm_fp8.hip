@@ -1220,7 +1220,7 @@ __global__ __launch_bounds__(256) void linear_fp8_skinny_fused(GemmArgs g, uint8
     if (threadIdx.x == 0) row_s[m] = s;
     uint2* dst = reinterpret_cast<uint2*>(codes + m * pitch);
     if (scale_in_fast_window(s)) {  // uniform
-      const float rcp = 1.0f / s;
+      const Recip rcp = make_recip(s);
       for (int c = threadIdx.x; c < nchunks; c += 256) {
         const uint4 v = xr[c];
         dst[c] = uint2{quant4<true>(v.x, v.y, s, rcp), quant4<true>(v.z, v.w, s, rcp)};
@@ -1228,7 +1228,7 @@ __global__ __launch_bounds__(256) void linear_fp8_skinny_fused(GemmArgs g, uint8
     } else {
       for (int c = threadIdx.x; c < nchunks; c += 256) {
         const uint4 v = xr[c];
-        dst[c] = uint2{quant4<false>(v.x, v.y, s, 0.0f), quant4<false>(v.z, v.w, s, 0.0f)};
+        dst[c] = uint2{quant4<false>(v.x, v.y, s, Recip{}), quant4<false>(v.z, v.w, s, Recip{})};
       }
     }
     __syncthreads();  // codes of row m complete; wave_amax free for the next row
@@ -1356,7 +1356,7 @@ __global__ __launch_bounds__(64 * kRow1Waves) void linear_fp8_row1(GemmArgs g, u
     for (int i = 1; i < WAVES; ++i) amax = max(amax, wave_amax[i]);
     as = row_scale(amax, scale_mode);
     const bool fast = scale_in_fast_window(as);  // uniform
-    const float rcp = 1.0f / as;
+    const Recip rcp = make_recip(as);
     uint2* dst = reinterpret_cast<uint2*>(codes);
 #pragma unroll
     for (int p = 0; p < PP; ++p) {
@@ -1365,7 +1365,7 @@ __global__ __launch_bounds__(64 * kRow1Waves) void linear_fp8_row1(GemmArgs g, u
       if (fast) {
         code = uint2{quant4<true>(v[p].x, v[p].y, as, rcp), quant4<true>(v[p].z, v[p].w, as, rcp)};
       } else {
-        code = uint2{quant4<false>(v[p].x, v[p].y, as, 0.0f), quant4<false>(v[p].z, v[p].w, as, 0.0f)};
+        code = uint2{quant4<false>(v[p].x, v[p].y, as, Recip{}), quant4<false>(v[p].z, v[p].w, as, Recip{})};
       }
       if (c >= nchunks) code = uint2{0u, 0u};
       if (c < CHK * 128) dst[c] = code;

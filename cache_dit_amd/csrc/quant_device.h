@@ -102,17 +102,30 @@ __device__ __forceinline__ float clamp448(float y) {
   return y != y ? y : fminf(fmaxf(y, -kFp8Max), kFp8Max);
 }
 
-// x / s with s > 0 finite. FAST: r = 1/s correctly rounded, s inside the window.
+// 1 / s of the fast path as an unevaluated sum hi + lo of two fp32 values: hi is the fp32
+// value at or just below 1 / s (the correctly rounded reciprocal, stepped down by one unit in
+// the last place when it lies above), lo >= 0 the remainder (1 - s hi) / s to fp32 accuracy.
+// Worked out once per row.
+struct Recip {
+  float hi, lo;
+};
+__device__ __forceinline__ Recip make_recip(float s) {
+  const float r = 1.0f / s;
+  const float hi = __fmaf_rn(-s, r, 1.0f) < 0.0f ? __uint_as_float(__float_as_uint(r) - 1u) : r;
+  return Recip{hi, __fmaf_rn(-s, hi, 1.0f) * r};
+}
+
+// x / s with s > 0 finite. FAST (s inside the window, r = make_recip(s)): x hi + x lo in a
+// multiply and an FMA. The sum hi + lo carries 1 / s to about 48 bits, so the result is
+// x / s rounded once, up to a double rounding of the small term: not always the fp32
+// quotient of the division, but always a value that converts to the same e4m3 code -- the
+// roundings of that conversion lie 2^20 times further apart than those of fp32, and an exact
+// tie of the conversion is reproduced exactly (tests/native/divcheck.c checks every input
+// pair). With lo >= 0 both terms carry the sign of x, so x = -0 gives -0.
 template <bool FAST>
-__device__ __forceinline__ float div_scale(float x, float s, float r) {
+__device__ __forceinline__ float div_scale(float x, float s, Recip r) {
   if constexpr (FAST) {
-    // Markstein's correction of q0 = x r, written with the residual negated: d = q0 s - x is
-    // the exact negative of the usual x - q0 s, so q = q0 - d r is the same correctly rounded
-    // quotient for every non-zero x, and for x = -0 (q0 = -0, d = +0) it is (-0) + (-0) = -0
-    // where the usual form gives +0: the sign of a zero survives without a copysign.
-    const float q0 = x * r;
-    const float d = __fmaf_rn(q0, s, -x);
-    return __fmaf_rn(-d, r, q0);
+    return __fmaf_rn(x, r.hi, x * r.lo);
   } else {
     return x / s;
   }
@@ -129,7 +142,7 @@ __device__ __forceinline__ bool scale_in_fast_window(float s) {
 // below the tie at 464 where the e4m3 conversion would stop rounding to 448
 // (tests/native/divcheck.c checks the unclamped quotient of every input pair).
 template <bool FAST>
-__device__ __forceinline__ uint32_t quant4(uint32_t w0, uint32_t w1, float s, float r) {
+__device__ __forceinline__ uint32_t quant4(uint32_t w0, uint32_t w1, float s, Recip r) {
   float a = div_scale<FAST>(bf16_lo(w0), s, r);
   float b = div_scale<FAST>(bf16_hi(w0), s, r);
   float c = div_scale<FAST>(bf16_lo(w1), s, r);

@@ -10,12 +10,13 @@
 // Arithmetic follows torchao's _choose_scale_float8 / _quantize_affine_float8
 // as cache-dit calls them (src/cache_dit/quantization/torchao/quantize_ao.py:54-70):
 // amax in bf16, scale = amax/448 (optionally rounded to bf16), zero scale -> 1,
-// q = cast(clamp(float(x)/scale, +-448)). The quotient must be the IEEE
-// correctly rounded one: a bare reciprocal multiply flips about 1e-4 of the
-// codes. Per element the kernel therefore refines q0 = x*r (r = 1/scale,
-// correctly rounded, computed once per row) with the exact residual:
-//   d = fma(q0, scale, -x);  q = fma(-d, r, q0)
-// (Markstein's correction with the residual negated, which keeps the sign of x = -0). That this
+// q = cast(clamp(float(x)/scale, +-448)). The codes must be those of the IEEE
+// division: a bare reciprocal multiply flips about 1e-4 of them. Per row the
+// kernel therefore works out 1/scale as an unevaluated sum hi + lo of two fp32
+// values (make_recip) and per element
+//   q = fma(x, hi, x * lo)
+// which is x/scale rounded once up to a double rounding of the small term, and
+// keeps the sign of x = -0. That this
 // reproduces x/scale down to the e4m3 code has been verified exhaustively on
 // the CPU for every (x, amax) pair of bf16 values with |x| <= amax, in both
 // scale modes, whenever 2^-100 <= scale < 2^101 (tests/native/divcheck.c);
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(64) void quant_rowwise_regs(
     if (lane == 0) *s_row = s;
     uint2* qr = reinterpret_cast<uint2*>(q_row);
     if (scale_in_fast_window(s)) {  // wave-uniform
-      const float r = 1.0f / s;
+      const Recip r = make_recip(s);
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
         const int idx = c * 64 + lane;
@@ -116,8 +117,8 @@ __global__ __launch_bounds__(64) void quant_rowwise_regs(
       for (int idx = lane; idx < nchunks; idx += 64) {
         const uint4 w = xr[idx];
         uint2 o;
-        o.x = quant4<false>(w.x, w.y, s, 0.0f);
-        o.y = quant4<false>(w.z, w.w, s, 0.0f);
+        o.x = quant4<false>(w.x, w.y, s, Recip{});
+        o.y = quant4<false>(w.z, w.w, s, Recip{});
         qr[idx] = o;
       }
     }
@@ -182,7 +183,7 @@ __global__ __launch_bounds__(64 * WAVES) void quant_rowwise_split2(
     if (threadIdx.x == 0) *s_row = s;
     uint2* qr = reinterpret_cast<uint2*>(q_row);
     if (scale_in_fast_window(s)) {  // uniform
-      const float r = 1.0f / s;
+      const Recip r = make_recip(s);
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
         const int idx = (WAVES * c + wave) * 64 + lane;
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(64 * WAVES) void quant_rowwise_split2(
 #pragma unroll 1
       for (int idx = threadIdx.x; idx < nchunks; idx += 64 * WAVES) {
         const uint4 w = xr[idx];
-        qr[idx] = uint2{quant4<false>(w.x, w.y, s, 0.0f), quant4<false>(w.z, w.w, s, 0.0f)};
+        qr[idx] = uint2{quant4<false>(w.x, w.y, s, Recip{}), quant4<false>(w.z, w.w, s, Recip{})};
       }
     }
   }
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(64 * WAVES) void quant_rowwise_cat_regs(
     if (threadIdx.x == 0) scale[row] = s;
     uint2* qr = reinterpret_cast<uint2*>(q + row * ld_q);
     if (scale_in_fast_window(s)) {  // uniform
-      const float r = 1.0f / s;
+      const Recip r = make_recip(s);
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
         const int idx = (WAVES * c + wave) * 64 + lane;
@@ -266,7 +267,7 @@ __global__ __launch_bounds__(64 * WAVES) void quant_rowwise_cat_regs(
 #pragma unroll 1
       for (int idx = threadIdx.x; idx < nchunks; idx += 64 * WAVES) {
         const uint4 w = load(idx);
-        qr[idx] = uint2{quant4<false>(w.x, w.y, s, 0.0f), quant4<false>(w.z, w.w, s, 0.0f)};
+        qr[idx] = uint2{quant4<false>(w.x, w.y, s, Recip{}), quant4<false>(w.z, w.w, s, Recip{})};
       }
     }
   }
@@ -346,7 +347,7 @@ __global__ __launch_bounds__(64) void quant_tensorwise_cast(
   const int lane = threadIdx.x & 63;
   const float s = row_scale(*amax_ws, scale_mode);
   const bool fast = scale_in_fast_window(s);
-  const float r = 1.0f / s;
+  const Recip r = make_recip(s);
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
     if (lane == 0) scale[row] = s;
     const uint16_t* xr = x + row * ld_x;
@@ -367,8 +368,8 @@ __global__ __launch_bounds__(64) void quant_tensorwise_cast(
         for (int idx = lane; idx < (K >> 3); idx += 64) {
           const uint4 w = xv[idx];
           uint2 o;
-          o.x = quant4<false>(w.x, w.y, s, 0.0f);
-          o.y = quant4<false>(w.z, w.w, s, 0.0f);
+          o.x = quant4<false>(w.x, w.y, s, Recip{});
+          o.y = quant4<false>(w.z, w.w, s, Recip{});
           qv[idx] = o;
         }
       }
@@ -435,7 +436,7 @@ __global__ __launch_bounds__(64) void quant_tensorwise_cast_rows(
   const int lane = threadIdx.x & 63;
   const float s = row_scale(*amax_ws, scale_mode);
   const bool fast = scale_in_fast_window(s);
-  const float r = 1.0f / s;
+  const Recip r = make_recip(s);
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
     if (lane == 0) scale[row] = s;
     const __amdgpu_buffer_rsrc_t xb = __builtin_amdgcn_make_buffer_rsrc(
@@ -454,7 +455,7 @@ __global__ __launch_bounds__(64) void quant_tensorwise_cast_rows(
 #pragma unroll 1
       for (int c = 0; c < CH; ++c)
         __builtin_amdgcn_raw_buffer_store_b64(
-            u2v{quant4<false>(w[c][0], w[c][1], s, 0.0f), quant4<false>(w[c][2], w[c][3], s, 0.0f)}, qb,
+            u2v{quant4<false>(w[c][0], w[c][1], s, Recip{}), quant4<false>(w[c][2], w[c][3], s, Recip{})}, qb,
             8 * (c * 64 + lane), 0, 2);
     }
   }
@@ -717,7 +718,7 @@ __global__ __launch_bounds__(64 * WAVES) void ln_modulate_quant_rows(
                                           threadIdx.x == 0 ? 0 : 4, 0, kCached);
     u2v o[CH];
     if (scale_in_fast_window(s)) {  // uniform
-      const float r = 1.0f / s;
+      const Recip r = make_recip(s);
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
         uint32_t p[2] = {0u, 0u};

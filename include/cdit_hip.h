@@ -87,7 +87,7 @@ int cdit_device_arch(char* buf, int buf_len);
  *   q[m,k]   = e4m3fn_rne(clamp(float(x[m,k]) / scale[m], -448, 448))
  *
  * x: bf16 [M,K], leading dimension ld_x; q: e4m3 bytes [M,K], leading
- * dimension ld_q; scale: fp32 [M]. The division is IEEE correctly rounded.
+ * dimension ld_q; scale: fp32 [M]. The codes are those of the IEEE division.
  * M == 0 or K == 0 is a no-op that returns CDIT_OK. NaN/Inf inputs are outside
  * the bit-exact contract.
  */

@@ -1,5 +1,5 @@
-"""The quantizer kernel divides with one reciprocal per row plus two FMAs per
-element. tests/native/divcheck.c proves on the CPU, exhaustively over every bf16
+"""The quantizer kernel divides with a two-term reciprocal per row plus a multiply and an
+FMA per element. tests/native/divcheck.c proves on the CPU, exhaustively over every bf16
 amax and every bf16 x with |x| <= amax in both scale modes, that this yields the
 same e4m3 code as the IEEE division of the oracle."""
 import os
