@@ -585,6 +585,16 @@ __global__ __launch_bounds__(64 * WAVES) void ln_modulate_quant_rows(
 
   float t_f[CH][8], sh_f[CH][8];  // modulation vectors of the current modulation row
   int cur_mod = -1;
+  auto widen_mod = [&](int c, const u4v& sh, const u4v& sc) {
+    const bool valid = idx[c] < nchunks;  // beyond K: t = 0, so that y = 0 there
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      t_f[c][2 * e] = valid ? round_bf16_wide(1.0f + bf16_lo(sc[e])) : 0.0f;
+      t_f[c][2 * e + 1] = valid ? round_bf16_wide(1.0f + bf16_hi(sc[e])) : 0.0f;
+      sh_f[c][2 * e] = bf16_lo(sh[e]);
+      sh_f[c][2 * e + 1] = bf16_hi(sh[e]);
+    }
+  };
   auto load_mod = [&](int mod) {
     const __amdgpu_buffer_rsrc_t shb = row_buf(shift, (int64_t)mod * ld_mod * 2, K * 2);
     const __amdgpu_buffer_rsrc_t scb = row_buf(scale_mod, (int64_t)mod * ld_mod * 2, K * 2);
@@ -592,14 +602,7 @@ __global__ __launch_bounds__(64 * WAVES) void ln_modulate_quant_rows(
     for (int c = 0; c < CH; ++c) {
       const u4v sh = __builtin_amdgcn_raw_buffer_load_b128(shb, idx[c] * 16, 0, kCached);
       const u4v sc = __builtin_amdgcn_raw_buffer_load_b128(scb, idx[c] * 16, 0, kCached);
-      const bool valid = idx[c] < nchunks;  // beyond K: t = 0, so that y = 0 there
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        t_f[c][2 * e] = valid ? round_bf16_wide(1.0f + bf16_lo(sc[e])) : 0.0f;
-        t_f[c][2 * e + 1] = valid ? round_bf16_wide(1.0f + bf16_hi(sc[e])) : 0.0f;
-        sh_f[c][2 * e] = bf16_lo(sh[e]);
-        sh_f[c][2 * e + 1] = bf16_hi(sh[e]);
-      }
+      widen_mod(c, sh, sc);
     }
     cur_mod = mod;
   };
@@ -749,7 +752,25 @@ __global__ __launch_bounds__(64 * WAVES) void ln_modulate_quant_rows(
   };
 
   u4v va[CH], vb[CH];
-  load_row(row0, va);
+  // The modulation vectors first: they come from the L2 (every workgroup reads the same two)
+  // and are widened while the first row is still on its way from memory.
+  {
+    const __amdgpu_buffer_rsrc_t xb = row_buf(x, (int64_t)row0 * ld_x * 2, K * 2);
+    const int mod = row0 / rows_per_mod;
+    const __amdgpu_buffer_rsrc_t shb = row_buf(shift, (int64_t)mod * ld_mod * 2, K * 2);
+    const __amdgpu_buffer_rsrc_t scb = row_buf(scale_mod, (int64_t)mod * ld_mod * 2, K * 2);
+    u4v sh[CH], sc[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      sh[c] = __builtin_amdgcn_raw_buffer_load_b128(shb, idx[c] * 16, 0, kCached);
+      sc[c] = __builtin_amdgcn_raw_buffer_load_b128(scb, idx[c] * 16, 0, kCached);
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) va[c] = __builtin_amdgcn_raw_buffer_load_b128(xb, idx[c] * 16, 0, kCached);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) widen_mod(c, sh[c], sc[c]);
+    cur_mod = mod;
+  }
   {
     // As many stores as a row issues, every lane beyond its descriptor (nothing is written):
     // the first row then meets the same sequence of accesses in flight as every later one,
@@ -1054,7 +1075,10 @@ int launch_ln_modulate_quant(const void* x, int64_t M, int64_t K, int64_t ld_x, 
     const int64_t cus = cu_count_or(256);
     // (measured at 4608 x 3072: 16.1 us with 16 wavefronts' worth of workgroups per CU, 15.2
     // with 20 or 24; four wavefronts of two chunks per row instead of two of three: 17.4-17.7)
-    const int64_t target = cus * 24 / waves;
+    // (32760 x 5120: 104.7 us with 48 wavefronts' worth per CU, 11 rows each, against 107.8
+    // with 24; with fewer than eight rows per workgroup the smaller number wins)
+    int64_t target = cus * 48 / waves;
+    if (M < 8 * target) target = cus * 24 / waves;
     const int rows_per_wg = (int)((M + target - 1) / target);
     const dim3 rgrid((unsigned)((M + rows_per_wg - 1) / rows_per_wg));
 #define CDIT_LNQ_LAUNCH(W, CH, WY)                                                              \
